@@ -1,0 +1,265 @@
+#!/usr/bin/env python3
+"""Benchmark of the group-quantized linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--skip-extra] [--skip-cpu]
+
+A "step" is one decode token's worth of q4f16_1 GEMVs at Llama-3-8B shapes, batch 1:
+32 layers x (fused qkv 6144x4096, o_proj 4096x4096, fused gate_up 28672x4096, down 4096x14336)
+plus lm_head 128256x4096 = 129 launches that stream 4.23 GB of distinct packed weights and
+scales (every layer owns its own tensors, so nothing is re-read from cache between launches).
+Inputs are resident in HBM before the timed region.  `value` is the algorithmic GB/s of the whole
+step (weights + scales + activations + outputs, each counted once) measured with HIP events on the
+launch stream; the step is replayed from a HIP graph unless --no-graph is given.
+
+The JSON line also carries
+  roofline      the dominant kernel (the gate_up GEMV, 52 % of a step's bytes) timed on its own
+                over the 32 distinct gate_up weight sets;
+  cpu_baseline  the C restatement of the reference's fused dequantize-matmul loop nest on the
+                host cores (a reported baseline, not the target);
+  extra         per-shape GEMV GB/s for batch 1/4/8 and prefill GEMM TFLOP/s at M = 2048.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "mlc-llm_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+BITS, G = 4, 32
+LAYERS = 32
+SHAPES = {  # name: (N, K)
+    "qkv": (6144, 4096),
+    "o_proj": (4096, 4096),
+    "gate_up": (28672, 4096),
+    "down": (4096, 14336),
+}
+LM_HEAD = (128256, 4096)
+
+
+def gemv_bytes(n: int, k: int, b: int = 1) -> int:
+    ng = -(-k // G)
+    return n * 4 * ng * 4 + n * ng * 2 + b * k * 2 + b * n * 2
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--skip-extra", action="store_true")
+    ap.add_argument("--skip-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.stderr.write("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1\n")
+        return 2
+
+    import numpy as np
+    import torch
+
+    import mlc_llm_amd as gq
+    from mlc_llm_amd import ops
+
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py needs a GPU\n")
+        return 1
+    if not os.path.exists(gq._lib.LIB_PATH):
+        import __graft_entry__
+
+        __graft_entry__.build()
+    gq._lib.call("mi355gq_check_device")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    # ---------------------------------------------------------------- synthetic model, quantized on the GPU
+    def make_weight(n, k, seed):
+        g = torch.Generator(device=dev).manual_seed(seed)
+        w = (torch.randn((n, k), generator=g, device=dev, dtype=torch.float32) * 0.02).half()
+        return ops.quantize(w, BITS, G)
+
+    layers = []
+    for layer in range(LAYERS):
+        layers.append({name: make_weight(n, k, 1000 * layer + i) for i, (name, (n, k)) in enumerate(SHAPES.items())})
+    lm_head = make_weight(*LM_HEAD, 999_999)
+    gx = torch.Generator(device=dev).manual_seed(1)
+    x_in = {k: torch.randn((8, k), generator=gx, device=dev).half() for k in (4096, 14336)}
+    outs = {name: torch.empty((8, n), dtype=torch.float16, device=dev) for name, (n, _) in SHAPES.items()}
+    out_lm = torch.empty((8, LM_HEAD[0]), dtype=torch.float16, device=dev)
+    torch.cuda.synchronize()
+
+    def run_linear(name, qw, qs, b, out):
+        n, k = qw.shape[0], (LM_HEAD[1] if name == "lm_head" else SHAPES[name][1])
+        ops.linear(x_in[k][:b], qw, qs, BITS, G, None, torch.float16, out[:b])
+
+    def decode_step(b=1):
+        for lw in layers:
+            for name in SHAPES:
+                run_linear(name, lw[name][0], lw[name][1], b, outs[name])
+        run_linear("lm_head", lm_head[0], lm_head[1], b, out_lm)
+
+    step_bytes = LAYERS * sum(gemv_bytes(n, k) for n, k in SHAPES.values()) + gemv_bytes(*LM_HEAD)
+    launches_per_step = LAYERS * len(SHAPES) + 1
+
+    # ---------------------------------------------------------------- parity gate before timing
+    from oracle import c_oracle
+    from oracle import gq_oracle as o
+
+    s4 = o.SCHEMES["q4f16_1"]
+    qw0, qs0 = layers[0]["o_proj"]
+    qw0_h, qs0_h = qw0.cpu().numpy().view(np.uint32), qs0.cpu().numpy()
+    x1_h = x_in[4096][:1].cpu().numpy()
+    run_linear("o_proj", qw0, qs0, 1, outs["o_proj"])
+    err, bound, rel = o.check_linear(outs["o_proj"][:1].float().cpu().numpy(),
+                                     o.linear_fp32(x1_h, qw0_h, qs0_h, s4), x1_h, 4096)
+    if not (err <= bound and rel <= 2e-3):
+        sys.stderr.write(f"parity check failed before timing: err {err} bound {bound} rel {rel}\n")
+        return 1
+
+    # ---------------------------------------------------------------- timed region: K decode steps
+    def timed(fn, iters, warmup, use_graph):
+        """ms per call of fn, HIP events on the current (launch) stream."""
+        if use_graph:
+            fn()  # eager once: lazy init must not happen under capture
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                fn()
+            call = graph.replay
+        else:
+            call = fn
+        for _ in range(warmup):
+            call()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    use_graph = not args.no_graph
+    t_wall0 = time.perf_counter()
+    ms_step = timed(decode_step, args.steps, args.warmup, use_graph)
+    value = step_bytes / (ms_step * 1e-3) / 1e9
+
+    # ---------------------------------------------------------------- roofline of the dominant kernel
+    def gate_up_sweep():
+        for lw in layers:
+            run_linear("gate_up", lw["gate_up"][0], lw["gate_up"][1], 1, outs["gate_up"])
+
+    ms_sweep = timed(gate_up_sweep, max(5, args.steps), 2, use_graph)
+    us_gate_up = ms_sweep * 1e3 / LAYERS
+    gu_bytes = gemv_bytes(*SHAPES["gate_up"])
+    achieved = gu_bytes / (us_gate_up * 1e-6) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "gemv_gate_up_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath, encoding="utf-8") as f:
+            traffic = json.load(f).get("hbm_bytes_per_launch")
+    roofline = {
+        "bound": "hbm", "kernel": "gq::gemv_dot2_kernel<4,1,R> on gate_up 28672x4096, batch 1",
+        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+        "bytes_per_launch": gu_bytes, "us_per_launch": round(us_gate_up, 3),
+    }
+
+    # ---------------------------------------------------------------- extra: per shape, batch 1/4/8, prefill GEMM
+    extra = {}
+    if not args.skip_extra:
+        per_shape = {}
+        for name, (n, k) in list(SHAPES.items()) + [("lm_head", LM_HEAD)]:
+            for b in (1, 4, 8):
+                if name == "lm_head":
+                    # 8 launches on the one lm_head (296 MB: larger than the 256 MB infinity cache)
+                    def sweep(b=b):
+                        for _ in range(8):
+                            run_linear("lm_head", lm_head[0], lm_head[1], b, out_lm)
+                    cnt = 8
+                else:
+                    def sweep(name=name, b=b):
+                        for lw in layers:
+                            run_linear(name, lw[name][0], lw[name][1], b, outs[name])
+                    cnt = LAYERS
+                us = timed(sweep, 5, 1, use_graph) * 1e3 / cnt
+                gbs = gemv_bytes(n, k, b) / (us * 1e-6) / 1e9
+                per_shape[f"{name}_b{b}"] = {"us": round(us, 2), "GB/s": round(gbs, 1),
+                                             "frac_hbm": round(gbs / HBM_PEAK_GBS, 3)}
+        extra["gemv"] = per_shape
+        gemm = {}
+        m = 2048
+        xm = {k: torch.randn((m, k), generator=gx, device=dev).half() for k in (4096, 14336)}
+        for name, (n, k) in list(SHAPES.items()) + [("lm_head", LM_HEAD)]:
+            qw, qs = lm_head if name == "lm_head" else layers[0][name]
+            ym = torch.empty((m, n), dtype=torch.float16, device=dev)
+
+            def call(qw=qw, qs=qs, k=k, ym=ym):
+                ops.linear(xm[k], qw, qs, BITS, G, None, torch.float16, ym)
+            ms = timed(call, 5, 2, False)
+            tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+            gemm[f"{name}_m{m}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
+                                    "frac_mfma": round(tf / MFMA_F16_PEAK_TFLOPS, 3)}
+            del ym
+        extra["prefill_gemm"] = gemm
+        extra["decode_tokens_per_s_linear_only"] = round(1e3 / ms_step, 1)
+
+    # ---------------------------------------------------------------- CPU baseline (bounded sample)
+    cpu = None
+    if not args.skip_cpu:
+        n, k = SHAPES["gate_up"]
+        qw_h = layers[0]["gate_up"][0].cpu().numpy().view(np.uint32)
+        qs_h = layers[0]["gate_up"][1].cpu().numpy()
+        scratch = np.empty(k, np.float32)
+        out_h = np.empty((1, n), np.float32)
+        c_oracle.linear(x1_h, qw_h, qs_h, BITS, G, None, scratch, out_h)  # warm-up + parity
+        run_linear("gate_up", *layers[0]["gate_up"], 1, outs["gate_up"])
+        gpu_y = outs["gate_up"][:1].float().cpu().numpy()
+        cerr = float(np.abs(gpu_y - out_h).max())
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 10.0:
+            c_oracle.linear(x1_h, qw_h, qs_h, BITS, G, None, scratch, out_h)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        cpu = {
+            "value": round(gu_bytes / dt / 1e9, 2), "unit": "GB/s", "cores": c_oracle.num_threads(),
+            "kind": "port",
+            "sample": f"gate_up 28672x4096 q4f16_1 GEMV, batch 1, {reps} calls in 10 s "
+                      "(C restatement of the reference loop nest, OpenMP over N; TVM's llvm build "
+                      "is not available offline)",
+            "us_per_call": round(dt * 1e6, 1), "max_abs_diff_vs_gpu": cerr,
+        }
+
+    line = {
+        "metric": "q4f16_1 dequant-GEMV GB/s (% of HBM peak), Llama-3-8B decode; prefill TFLOP/s",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16 in/out, f32 accumulate, u32 packed int4",
+        "data": "synthetic",
+        "config": {
+            "workload": "Llama-3-8B q4f16_1 decode linears, batch 1: 32 x (qkv 6144x4096, o 4096x4096, "
+                        "gate_up 28672x4096, down 4096x14336) + lm_head 128256x4096 "
+                        "(BASELINE configs[1], B=1)",
+            "launches_per_step": launches_per_step, "bytes_per_step": step_bytes,
+            "hip_graph": use_graph, "group_size": G, "bits": BITS,
+        },
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "extra": extra,
+        "wall_s": round(time.perf_counter() - t_wall0, 1),
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,167 @@
+/*
+ * mi355gq — MI355X (gfx950) kernels for MLC-LLM group-quantized weights, C ABI.
+ *
+ * Every entry point takes raw device pointers, sizes and a hipStream_t (passed
+ * as void*), launches asynchronously on that stream and returns MI355GQ_OK or a
+ * negative code; mi355gq_last_error() then holds a thread-local message.
+ * Nothing allocates, nothing retains pointers, nothing synchronises: outputs
+ * (and workspaces, where named) are owned by the caller, exactly as Relax
+ * `call_dps_packed` hands them over (destination-passing style, see the
+ * reference's python/mlc_llm/op/ft_gemm.py:72-92 and op/cutlass.py:71-77).
+ *
+ * Layouts are the reference's, unchanged (python/mlc_llm/quantization/
+ * group_quantization.py:342-347, 574-580): NK layout,
+ *   q_weight uint32 [N, nw]  nw = (G / E) * ceil(K / G),  E = 32 / bits
+ *   q_scale  fp16   [N, ng]  ng = ceil(K / G)
+ * q4f16_1: bits = 4, G = 32;  q3f16_1: bits = 3, G = 40.  fp16 = IEEE binary16.
+ * All tensors are dense row-major; q_weight rows must be 16-byte aligned
+ * (always true for a 16-byte aligned base because nw is a multiple of 4).
+ */
+#ifndef MI355GQ_H_
+#define MI355GQ_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define MI355GQ_API __attribute__((visibility("default")))
+#else
+#define MI355GQ_API
+#endif
+
+#define MI355GQ_VERSION 100
+
+enum {
+  MI355GQ_OK = 0,
+  MI355GQ_ERR_ARG = -1,         /* bad pointer / size / scheme / alignment */
+  MI355GQ_ERR_HIP = -2,         /* a HIP call failed; message holds hipGetErrorString */
+  MI355GQ_ERR_UNSUPPORTED = -3, /* valid request this build has no kernel for */
+  MI355GQ_ERR_WORKSPACE = -4    /* caller's workspace is too small */
+};
+
+enum { MI355GQ_F16 = 0, MI355GQ_F32 = 1 };             /* output dtype */
+enum { MI355GQ_ROUND_HALF_AWAY = 0, MI355GQ_ROUND_HALF_EVEN = 1 };
+enum { MI355GQ_I32 = 0, MI355GQ_I64 = 1 };             /* indptr dtype */
+
+typedef void* mi355gq_stream_t; /* hipStream_t */
+
+MI355GQ_API int mi355gq_version(void);
+/* Thread-local message of the last failing call on this thread ("" if none). */
+MI355GQ_API const char* mi355gq_last_error(void);
+/* 0 when the current HIP device is gfx950, MI355GQ_ERR_UNSUPPORTED otherwise. */
+MI355GQ_API int mi355gq_check_device(void);
+
+/* Tuning/diagnostic knob (process-global, not thread-safe against running calls):
+ * "gemv_rows_per_wave", "gemv_variant", "gemm_variant" ... ; value < 0 restores the default. */
+MI355GQ_API int mi355gq_set_option(const char* name, int value);
+
+/*
+ * GroupQuantize.quantize_weight, NK layout (replaces the Relax function built at
+ * python/mlc_llm/quantization/group_quantization.py:188-306 and utils.py:136-188).
+ * w fp16 [rows, K] -> q_weight uint32 [rows, nw], q_scale fp16 [rows, ng]. Bit-exact.
+ */
+MI355GQ_API int mi355gq_quantize(const void* w, int64_t rows, int64_t K, int bits, int group_size,
+                     int round_mode, void* q_weight, void* q_scale, mi355gq_stream_t stream);
+
+/*
+ * GroupQuantize._dequantize (group_quantization.py:155-186, utils.py:15-48):
+ * out fp16 [rows, K] = (unpack(q_weight) - m) * q_scale, evaluated for k < K only. Bit-exact.
+ */
+MI355GQ_API int mi355gq_dequantize(const void* q_weight, const void* q_scale, int64_t rows, int64_t K,
+                       int bits, int group_size, void* out, mi355gq_stream_t stream);
+
+/*
+ * GroupQuantizeEmbedding.forward (group_quantization.py:486-522, fused by
+ * compiler_pass/fuse_dequantize_take.py:14-49): out fp16 [T, K] = dequantize(row ids[t]).
+ * ids int32 [T], each in [0, num_rows) (not checked on the device: out-of-range ids are
+ * clamped to the table like a safe gather, never read out of bounds).
+ */
+MI355GQ_API int mi355gq_embedding_take(const void* ids, int64_t T, const void* q_weight, const void* q_scale,
+                           int64_t num_rows, int64_t K, int bits, int group_size, void* out,
+                           mi355gq_stream_t stream);
+
+/*
+ * GroupQuantizeLinear.forward / GroupQuantizeEmbedding.lm_head_forward
+ * (group_quantization.py:390-437, 524-556), i.e. the fused_dequantize*_NT_matmul kernels
+ * (compiler_pass/fuse_dequantize_matmul_ewise.py, fuse_transpose_matmul.py:64-143):
+ *   y[M, N] = x[M, K] . dequantize(q_weight, q_scale)[N, K]^T (+ bias[N])
+ * x fp16, bias fp16 or NULL, y fp16 (MI355GQ_F16) or fp32 (MI355GQ_F32); fp32 accumulation.
+ * M <= 8 runs the decode GEMV, larger M the MFMA GEMM (the regime split of
+ * compiler_pass/low_batch_specialization.py:22-57).
+ * workspace: device scratch, may be NULL with workspace_bytes = 0 when
+ * mi355gq_linear_workspace_bytes() returns 0 for the shape.
+ */
+MI355GQ_API int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size);
+MI355GQ_API int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                   int64_t M, int64_t N, int64_t K, int bits, int group_size, int out_dtype,
+                   void* y, void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream);
+
+/*
+ * moe_matmul.dequantize_gemv (python/mlc_llm/op/moe_matmul.py:77-176), single-token MoE:
+ *   out[e, :] = x[x_rows == 1 ? 0 : e, :] . dequantize(W[expert_ids[e]])^T,  e < top_k
+ * x fp16 [x_rows, K] with x_rows in {1, top_k}; expert_ids int32 [1, top_k];
+ * q_weight uint32 [num_experts, N, nw]; q_scale fp16 [num_experts, N, ng]; out fp16 [top_k, N].
+ */
+MI355GQ_API int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                     const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N,
+                     int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream);
+
+/*
+ * moe_matmul.dequantize_group_gemm (op/moe_matmul.py:562-768):
+ *   out[r, :] = x[r, :] . dequantize(W[e])^T  for indptr[e] <= r < indptr[e+1]
+ * x fp16 [rows, K] already gathered in expert order; indptr [num_experts + 1], int32 or int64
+ * (indptr[0] = 0); out fp16 [rows, N].  Rows outside every segment are left untouched.
+ */
+MI355GQ_API int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                           const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
+                           int64_t K, int bits, int group_size, void* out,
+                           mi355gq_stream_t stream);
+
+/* ---- routing glue of the MoE layer (python/mlc_llm/op/moe_misc.py) ---- */
+
+/* gating_softmax_topk, norm_topk_prob = True (moe_misc.py:135-235): logits fp16 [T, num_experts]
+ * -> weights fp16 [T, top_k] (softmax over the selected logits, fp32 maths), ids int32 [T, top_k].
+ * Ties keep the lower expert index. top_k <= 8, num_experts <= 256. */
+MI355GQ_API int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
+                                void* weights, void* ids, mi355gq_stream_t stream);
+
+/* moe_cumsum (moe_misc.py:371-450): ids int32 [T, top_k] -> cumsum int32 [num_experts * T],
+ * inclusive prefix sum of the expert-major token mask. */
+MI355GQ_API int mi355gq_moe_cumsum(const void* ids, int64_t T, int64_t top_k, int64_t num_experts,
+                       void* cumsum, mi355gq_stream_t stream);
+
+/* get_indices (moe_misc.py:453-525): cumsum int32 [num_experts * T], ids int32 [T, top_k]
+ * -> reverse_indices, token_indices int32 [T * top_k]. */
+MI355GQ_API int mi355gq_moe_get_indices(const void* cumsum, const void* ids, int64_t T, int64_t top_k,
+                            int64_t num_experts, void* reverse_indices, void* token_indices, mi355gq_stream_t stream);
+
+/* get_indptr (moe_misc.py:528-605): inclusive = 0 -> [num_experts + 1] with leading 0,
+ * inclusive = 1 -> [num_experts]; out_dtype MI355GQ_I32 or MI355GQ_I64. */
+MI355GQ_API int mi355gq_moe_get_indptr(const void* cumsum, int64_t num_experts, int64_t T, int inclusive,
+                           int out_dtype, void* indptr, mi355gq_stream_t stream);
+
+/* relax take(x, indices, axis=0) as used at model/mixtral/mixtral_model.py:107:
+ * out fp16 [R, H] = x[indices[r], :]. */
+MI355GQ_API int mi355gq_take_rows(const void* x, const void* indices, int64_t R, int64_t H, int64_t x_rows,
+                      void* out, mi355gq_stream_t stream);
+
+/* scatter_output (moe_misc.py:608-645): out[indices[r], :] = x[r, :], fp16 [R, H]. */
+MI355GQ_API int mi355gq_moe_scatter_output(const void* x, const void* indices, int64_t R, int64_t H,
+                               void* out, mi355gq_stream_t stream);
+
+/* split + silu(x1) * x3 (mixtral_model.py:66-68): x fp16 [R, 2I] -> out fp16 [R, I]. */
+MI355GQ_API int mi355gq_silu_mul(const void* x, int64_t R, int64_t I, void* out, mi355gq_stream_t stream);
+
+/* weights * experts' outputs, summed over top_k (mixtral_model.py:111-115, moe_misc.moe_sum
+ * :14-32): y fp16 [T, top_k, H], weights fp16 [T, top_k] -> out fp16 [T, H]; fp16 product,
+ * fp16 left-to-right sum, as the reference's elementwise ops do. */
+MI355GQ_API int mi355gq_moe_combine(const void* y, const void* weights, int64_t T, int64_t top_k, int64_t H,
+                        void* out, mi355gq_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355GQ_H_ */

@@ -1,0 +1,354 @@
+// C ABI of libmi355gq.so: argument validation, error reporting, dispatch to the launchers.
+// Declarations (with the reference interface each entry replaces) live in include/mi355gq.h.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/mi355gq.h"
+#include "gq_internal.hpp"
+
+namespace gq {
+Options& options() {
+  static Options o;
+  return o;
+}
+}  // namespace gq
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_result(hipError_t e, const char* what) {
+  if (e == hipSuccess) return MI355GQ_OK;
+  return fail(MI355GQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
+
+// q4f16_1-like (bits 4, G = 32) and q3f16_1-like (bits 3, G = 40): a group is 4 storage words
+int check_scheme(int bits, int group_size) {
+  if (bits != 4 && bits != 3)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "bits=%d: only int4 and int3 group quantization is built", bits);
+  const int e = 32 / bits;
+  if (group_size <= 0 || group_size % e != 0)
+    return fail(MI355GQ_ERR_ARG, "group_size=%d is not a multiple of %d elements per storage word",
+                group_size, e);
+  if (group_size != 4 * e)
+    return fail(MI355GQ_ERR_UNSUPPORTED,
+                "group_size=%d with bits=%d: kernels are built for 4 storage words per group "
+                "(q4f16_1: 32, q3f16_1: 40)", group_size, bits);
+  return MI355GQ_OK;
+}
+
+#define GQ_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) return fail(MI355GQ_ERR_ARG, __VA_ARGS__); \
+  } while (0)
+
+#define GQ_CHECK(expr)        \
+  do {                        \
+    const int rc_ = (expr);   \
+    if (rc_ != MI355GQ_OK) return rc_; \
+  } while (0)
+
+hipStream_t as_stream(mi355gq_stream_t s) { return static_cast<hipStream_t>(s); }
+
+constexpr int64_t kMaxDim = int64_t(1) << 31;
+
+}  // namespace
+
+extern "C" {
+
+int mi355gq_version(void) { return MI355GQ_VERSION; }
+
+const char* mi355gq_last_error(void) { return g_err; }
+
+int mi355gq_check_device(void) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_result(e, "hipGetDevice");
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return hip_result(e, "hipGetDeviceProperties");
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "device %d is %s; this library holds gfx950 code only", dev,
+                prop.gcnArchName);
+  return MI355GQ_OK;
+}
+
+int mi355gq_set_option(const char* name, int value) {
+  GQ_REQUIRE(name != nullptr, "option name is null");
+  gq::Options& o = gq::options();
+  if (!strcmp(name, "gemv_rows_per_wave")) o.gemv_rows_per_wave = value;
+  else if (!strcmp(name, "gemv_variant")) o.gemv_variant = value;
+  else if (!strcmp(name, "gemm_variant")) o.gemm_variant = value;
+  else if (!strcmp(name, "gemv_split")) o.gemv_split = value;
+  else return fail(MI355GQ_ERR_ARG, "unknown option '%s'", name);
+  return MI355GQ_OK;
+}
+
+int mi355gq_quantize(const void* w, int64_t rows, int64_t K, int bits, int group_size,
+                     int round_mode, void* q_weight, void* q_scale, mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(rows >= 0 && K >= 0 && rows < kMaxDim && K < kMaxDim, "quantize: bad shape [%lld, %lld]",
+             (long long)rows, (long long)K);
+  GQ_REQUIRE(round_mode == MI355GQ_ROUND_HALF_AWAY || round_mode == MI355GQ_ROUND_HALF_EVEN,
+             "quantize: round_mode=%d", round_mode);
+  if (rows == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(w && q_weight && q_scale, "quantize: null pointer");
+  GQ_REQUIRE(aligned16(w) && aligned16(q_weight) && aligned2(q_scale),
+             "quantize: w and q_weight must be 16-byte aligned");
+  return hip_result(gq::launch_quantize(static_cast<const uint16_t*>(w), rows, K, bits, group_size,
+                                        round_mode, static_cast<uint32_t*>(q_weight),
+                                        static_cast<uint16_t*>(q_scale), as_stream(stream)),
+                    "quantize launch");
+}
+
+int mi355gq_dequantize(const void* q_weight, const void* q_scale, int64_t rows, int64_t K,
+                       int bits, int group_size, void* out, mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(rows >= 0 && K >= 0 && rows < kMaxDim && K < kMaxDim, "dequantize: bad shape");
+  if (rows == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(q_weight && q_scale && out, "dequantize: null pointer");
+  GQ_REQUIRE(aligned16(q_weight) && aligned16(out) && aligned2(q_scale),
+             "dequantize: q_weight and out must be 16-byte aligned");
+  return hip_result(gq::launch_dequantize(nullptr, rows, static_cast<const uint32_t*>(q_weight),
+                                          static_cast<const uint16_t*>(q_scale), rows, K, bits,
+                                          group_size, static_cast<uint16_t*>(out), as_stream(stream)),
+                    "dequantize launch");
+}
+
+int mi355gq_embedding_take(const void* ids, int64_t T, const void* q_weight, const void* q_scale,
+                           int64_t num_rows, int64_t K, int bits, int group_size, void* out,
+                           mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(T >= 0 && K >= 0 && num_rows >= 0 && T < kMaxDim && K < kMaxDim,
+             "embedding_take: bad shape");
+  if (T == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(num_rows > 0, "embedding_take: empty table");
+  GQ_REQUIRE(ids && q_weight && q_scale && out, "embedding_take: null pointer");
+  GQ_REQUIRE(aligned4(ids) && aligned16(q_weight) && aligned16(out),
+             "embedding_take: q_weight and out must be 16-byte aligned");
+  return hip_result(
+      gq::launch_dequantize(static_cast<const int32_t*>(ids), T,
+                            static_cast<const uint32_t*>(q_weight),
+                            static_cast<const uint16_t*>(q_scale), num_rows, K, bits, group_size,
+                            static_cast<uint16_t*>(out), as_stream(stream)),
+      "embedding_take launch");
+}
+
+int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
+  (void)M; (void)N; (void)K; (void)bits; (void)group_size;
+  return 0;  // no kernel of this build needs scratch
+}
+
+int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                   int64_t M, int64_t N, int64_t K, int bits, int group_size, int out_dtype,
+                   void* y, void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
+  (void)workspace;
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
+             "linear: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  GQ_REQUIRE(out_dtype == MI355GQ_F16 || out_dtype == MI355GQ_F32, "linear: out_dtype=%d", out_dtype);
+  GQ_REQUIRE(workspace_bytes >= 0, "linear: negative workspace size");
+  if (M == 0 || N == 0) return MI355GQ_OK;
+  GQ_REQUIRE(y != nullptr, "linear: y is null");
+  GQ_REQUIRE(K == 0 || (x && q_weight && q_scale), "linear: null pointer");
+  GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned2(q_scale) && aligned4(y) &&
+                 aligned2(bias),
+             "linear: x and q_weight must be 16-byte aligned");
+  if (M <= 8) {
+    gq::GemvArgs a{};
+    a.x = static_cast<const uint16_t*>(x);
+    a.q_weight = static_cast<const uint32_t*>(q_weight);
+    a.q_scale = static_cast<const uint16_t*>(q_scale);
+    a.bias = static_cast<const uint16_t*>(bias);
+    a.y = y;
+    a.expert_ids = nullptr;
+    a.M = M; a.N = N; a.K = K; a.slots = 1; a.x_slot_stride = 0; a.num_experts = 1;
+    a.bits = bits; a.group_size = group_size; a.out_f32 = out_dtype == MI355GQ_F32;
+    return hip_result(gq::launch_gemv(a, as_stream(stream)), "gemv launch");
+  }
+  gq::GemmArgs g{};
+  g.x = static_cast<const uint16_t*>(x);
+  g.q_weight = static_cast<const uint32_t*>(q_weight);
+  g.q_scale = static_cast<const uint16_t*>(q_scale);
+  g.bias = static_cast<const uint16_t*>(bias);
+  g.y = y;
+  g.indptr = nullptr; g.indptr_i64 = 0;
+  g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
+  g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
+  return hip_result(gq::launch_gemm(g, as_stream(stream)), "gemm launch");
+}
+
+int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                     const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N,
+                     int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(top_k >= 0 && top_k <= 65535 && N >= 0 && K >= 0 && N < kMaxDim && K < kMaxDim &&
+                 num_experts > 0 && num_experts < kMaxDim,
+             "moe_gemv: bad shape");
+  GQ_REQUIRE(x_rows == 1 || x_rows == top_k, "moe_gemv: x has %lld rows, expected 1 or top_k=%lld",
+             (long long)x_rows, (long long)top_k);
+  if (top_k == 0 || N == 0) return MI355GQ_OK;
+  GQ_REQUIRE(x && q_weight && q_scale && expert_ids && out, "moe_gemv: null pointer");
+  GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned4(expert_ids) && aligned2(out),
+             "moe_gemv: x and q_weight must be 16-byte aligned");
+  GQ_REQUIRE(x_rows == 1 || (K % 8) == 0, "moe_gemv: K must be a multiple of 8 when x has top_k rows");
+  gq::GemvArgs a{};
+  a.x = static_cast<const uint16_t*>(x);
+  a.q_weight = static_cast<const uint32_t*>(q_weight);
+  a.q_scale = static_cast<const uint16_t*>(q_scale);
+  a.bias = nullptr;
+  a.y = out;
+  a.expert_ids = static_cast<const int32_t*>(expert_ids);
+  a.M = 1; a.N = N; a.K = K; a.slots = top_k; a.x_slot_stride = x_rows == 1 ? 0 : K;
+  a.num_experts = num_experts;
+  a.bits = bits; a.group_size = group_size; a.out_f32 = 0;
+  return hip_result(gq::launch_gemv(a, as_stream(stream)), "moe_gemv launch");
+}
+
+int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                           const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
+                           int64_t K, int bits, int group_size, void* out,
+                           mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(rows >= 0 && N >= 0 && K >= 0 && rows < kMaxDim && N < kMaxDim && K < kMaxDim &&
+                 num_experts > 0 && num_experts <= 65536,
+             "moe_group_gemm: bad shape");
+  GQ_REQUIRE(indptr_dtype == MI355GQ_I32 || indptr_dtype == MI355GQ_I64,
+             "moe_group_gemm: indptr_dtype=%d", indptr_dtype);
+  if (rows == 0 || N == 0) return MI355GQ_OK;
+  GQ_REQUIRE(x && q_weight && q_scale && indptr && out, "moe_group_gemm: null pointer");
+  GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned16(out) &&
+                 (indptr_dtype == MI355GQ_I32 ? aligned4(indptr)
+                                              : (reinterpret_cast<uintptr_t>(indptr) & 7u) == 0),
+             "moe_group_gemm: x, q_weight and out must be 16-byte aligned");
+  gq::GemmArgs g{};
+  g.x = static_cast<const uint16_t*>(x);
+  g.q_weight = static_cast<const uint32_t*>(q_weight);
+  g.q_scale = static_cast<const uint16_t*>(q_scale);
+  g.bias = nullptr;
+  g.y = out;
+  g.indptr = indptr; g.indptr_i64 = indptr_dtype == MI355GQ_I64;
+  g.rows = rows; g.N = N; g.K = K; g.num_experts = num_experts;
+  g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
+  return hip_result(gq::launch_gemm(g, as_stream(stream)), "moe_group_gemm launch");
+}
+
+int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
+                                void* weights, void* ids, mi355gq_stream_t stream) {
+  GQ_REQUIRE(T >= 0 && T < kMaxDim, "gating_softmax_topk: bad T");
+  GQ_REQUIRE(num_experts >= 1 && num_experts <= 256, "gating_softmax_topk: num_experts=%lld (1..256)",
+             (long long)num_experts);
+  GQ_REQUIRE(top_k >= 1 && top_k <= 8 && top_k <= num_experts,
+             "gating_softmax_topk: top_k=%lld (1..min(8, num_experts))", (long long)top_k);
+  if (T == 0) return MI355GQ_OK;
+  GQ_REQUIRE(logits && weights && ids, "gating_softmax_topk: null pointer");
+  return hip_result(gq::launch_topk_softmax(static_cast<const uint16_t*>(logits), T,
+                                            static_cast<int>(num_experts), static_cast<int>(top_k),
+                                            static_cast<uint16_t*>(weights),
+                                            static_cast<int32_t*>(ids), as_stream(stream)),
+                    "gating_softmax_topk launch");
+}
+
+int mi355gq_moe_cumsum(const void* ids, int64_t T, int64_t top_k, int64_t num_experts,
+                       void* cumsum, mi355gq_stream_t stream) {
+  GQ_REQUIRE(T >= 0 && T < kMaxDim && top_k >= 1 && top_k <= 64, "moe_cumsum: bad shape");
+  GQ_REQUIRE(num_experts >= 1 && num_experts <= 256, "moe_cumsum: num_experts=%lld (1..256)",
+             (long long)num_experts);
+  GQ_REQUIRE(T * num_experts < kMaxDim, "moe_cumsum: T * num_experts overflows int32");
+  if (T == 0) return MI355GQ_OK;
+  GQ_REQUIRE(ids && cumsum, "moe_cumsum: null pointer");
+  return hip_result(gq::launch_moe_cumsum(static_cast<const int32_t*>(ids), T,
+                                          static_cast<int>(top_k), static_cast<int>(num_experts),
+                                          static_cast<int32_t*>(cumsum), as_stream(stream)),
+                    "moe_cumsum launch");
+}
+
+int mi355gq_moe_get_indices(const void* cumsum, const void* ids, int64_t T, int64_t top_k,
+                            int64_t num_experts, void* reverse_indices, void* token_indices,
+                            mi355gq_stream_t stream) {
+  GQ_REQUIRE(T >= 0 && T < kMaxDim && top_k >= 1 && top_k <= 64 && num_experts >= 1 &&
+                 num_experts < kMaxDim && T * top_k < kMaxDim,
+             "moe_get_indices: bad shape");
+  if (T == 0) return MI355GQ_OK;
+  GQ_REQUIRE(cumsum && ids && reverse_indices && token_indices, "moe_get_indices: null pointer");
+  return hip_result(
+      gq::launch_get_indices(static_cast<const int32_t*>(cumsum), static_cast<const int32_t*>(ids),
+                             T, static_cast<int>(top_k), static_cast<int>(num_experts),
+                             static_cast<int32_t*>(reverse_indices),
+                             static_cast<int32_t*>(token_indices), as_stream(stream)),
+      "moe_get_indices launch");
+}
+
+int mi355gq_moe_get_indptr(const void* cumsum, int64_t num_experts, int64_t T, int inclusive,
+                           int out_dtype, void* indptr, mi355gq_stream_t stream) {
+  GQ_REQUIRE(num_experts >= 1 && num_experts < kMaxDim && T >= 1 && T < kMaxDim,
+             "moe_get_indptr: bad shape (needs T >= 1)");
+  GQ_REQUIRE(out_dtype == MI355GQ_I32 || out_dtype == MI355GQ_I64, "moe_get_indptr: out_dtype=%d",
+             out_dtype);
+  GQ_REQUIRE(cumsum && indptr, "moe_get_indptr: null pointer");
+  return hip_result(gq::launch_get_indptr(static_cast<const int32_t*>(cumsum), num_experts, T,
+                                          inclusive != 0, out_dtype == MI355GQ_I64, indptr,
+                                          as_stream(stream)),
+                    "moe_get_indptr launch");
+}
+
+int mi355gq_take_rows(const void* x, const void* indices, int64_t R, int64_t H, int64_t x_rows,
+                      void* out, mi355gq_stream_t stream) {
+  GQ_REQUIRE(R >= 0 && H >= 0 && x_rows >= 0 && R < kMaxDim && H < kMaxDim, "take_rows: bad shape");
+  if (R == 0 || H == 0) return MI355GQ_OK;
+  GQ_REQUIRE(x && indices && out, "take_rows: null pointer");
+  return hip_result(gq::launch_take_rows(static_cast<const uint16_t*>(x),
+                                         static_cast<const int32_t*>(indices), R, H, x_rows,
+                                         static_cast<uint16_t*>(out), 0, as_stream(stream)),
+                    "take_rows launch");
+}
+
+int mi355gq_moe_scatter_output(const void* x, const void* indices, int64_t R, int64_t H, void* out,
+                               mi355gq_stream_t stream) {
+  GQ_REQUIRE(R >= 0 && H >= 0 && R < kMaxDim && H < kMaxDim, "moe_scatter_output: bad shape");
+  if (R == 0 || H == 0) return MI355GQ_OK;
+  GQ_REQUIRE(x && indices && out, "moe_scatter_output: null pointer");
+  return hip_result(gq::launch_take_rows(static_cast<const uint16_t*>(x),
+                                         static_cast<const int32_t*>(indices), R, H, R,
+                                         static_cast<uint16_t*>(out), 1, as_stream(stream)),
+                    "moe_scatter_output launch");
+}
+
+int mi355gq_silu_mul(const void* x, int64_t R, int64_t I, void* out, mi355gq_stream_t stream) {
+  GQ_REQUIRE(R >= 0 && I >= 0 && R < kMaxDim && I < kMaxDim, "silu_mul: bad shape");
+  if (R == 0 || I == 0) return MI355GQ_OK;
+  GQ_REQUIRE(x && out, "silu_mul: null pointer");
+  return hip_result(gq::launch_silu_mul(static_cast<const uint16_t*>(x), R, I,
+                                        static_cast<uint16_t*>(out), as_stream(stream)),
+                    "silu_mul launch");
+}
+
+int mi355gq_moe_combine(const void* y, const void* weights, int64_t T, int64_t top_k, int64_t H,
+                        void* out, mi355gq_stream_t stream) {
+  GQ_REQUIRE(T >= 0 && H >= 0 && T < kMaxDim && H < kMaxDim && top_k >= 1 && top_k <= 64,
+             "moe_combine: bad shape");
+  if (T == 0 || H == 0) return MI355GQ_OK;
+  GQ_REQUIRE(y && weights && out, "moe_combine: null pointer");
+  return hip_result(gq::launch_moe_combine(static_cast<const uint16_t*>(y),
+                                           static_cast<const uint16_t*>(weights), T,
+                                           static_cast<int>(top_k), H, static_cast<uint16_t*>(out),
+                                           as_stream(stream)),
+                    "moe_combine launch");
+}
+
+}  // extern "C"

@@ -1,0 +1,65 @@
+// Shared device helpers for the gfx950 group-quantization kernels.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gq {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+
+// Compile-time facts of one scheme (group_quantization.py:57-61 of the reference).
+template <int BITS>
+struct Scheme {
+  static constexpr int kBits = BITS;
+  static constexpr int kElem = 32 / BITS;              // values per uint32: 8 | 10
+  static constexpr int kMaxInt = (1 << (BITS - 1)) - 1;  // 7 | 3
+  static constexpr uint32_t kMask = (1u << BITS) - 1u;
+};
+
+__device__ __forceinline__ half2_t as_half2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ __forceinline__ uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
+
+// fp32-accumulating dot of two half pairs: v_dot2_f32_f16.
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(as_half2(a), as_half2(b), c, false);
+}
+
+// (a & mask) | bits : v_and_or_b32
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bits) {
+  return (a & mask) | bits;
+}
+
+__device__ __forceinline__ float h2f(uint16_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, h));
+}
+// round-to-nearest-even float -> half (v_cvt_f16_f32 under the default rounding mode)
+__device__ __forceinline__ uint16_t f2h(float f) {
+  return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
+}
+
+// Sum over the 64 lanes of a wave; every lane ends up with the total.
+// quad_perm and row-mirror steps are DPP moves, the two widest steps cross rows via bpermute.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v);  // row_half_mirror: lane i <-> 7-i inside each 8
+  v += dpp_f<0x140>(v);  // row_mirror: lane i <-> 15-i inside each 16
+  v += __shfl_xor(v, 16, kWave);
+  v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+}  // namespace gq

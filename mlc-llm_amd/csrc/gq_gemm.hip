@@ -1,0 +1,303 @@
+// Prefill GEMM and MoE grouped GEMM: y[m, n] = sum_k x[m, k] * dequant(W)[n, k] on fp16 MFMA.
+//
+// Replaces the TVM-generated fused_dequantize*_NT_matmul kernel for M > 8
+// (python/mlc_llm/quantization/group_quantization.py:390-437 through
+// compiler_pass/low_batch_specialization.py:44-57) and moe_matmul.dequantize_group_gemm
+// (python/mlc_llm/op/moe_matmul.py:562-768; the indptr segment walk of :653-679 is the
+// tile-to-expert mapping below).
+//
+// MFMA-bound.  A workgroup (4 waves) owns a BM x BN output tile and walks K in tiles of two
+// quantisation groups.  Per K tile:
+//  * activations go global -> registers -> LDS unchanged (16-byte chunks);
+//  * packed weights go global -> registers (one 128-bit load = one group), are dequantised in
+//    registers exactly as the reference does (fp16 (q - m), then one fp16 multiply by the scale)
+//    and are written to LDS in natural k order;
+//  * both LDS tiles are k-contiguous with rows padded by 16 bytes, which makes every
+//    ds_read_b128 / ds_write_b128 of 16 consecutive lanes hit 64 distinct banks;
+//  * each wave feeds v_mfma_f32_32x32x16_f16 from 16-byte LDS fragments, fp32 accumulators;
+//  * global loads of tile t+1 are issued before the MFMAs of tile t, dequantisation and the LDS
+//    stores of t+1 after them (two LDS stages, one barrier per tile).
+#include "gq_common.hpp"
+#include "gq_internal.hpp"
+
+namespace gq {
+
+template <int BITS>
+struct GemmTraits;
+template <>
+struct GemmTraits<4> {
+  static constexpr int G = 32;
+};
+template <>
+struct GemmTraits<3> {
+  static constexpr int G = 40;
+};
+
+struct GemmParams {
+  const uint16_t* x;
+  const uint32_t* qw;
+  const uint16_t* qs;
+  const uint16_t* bias;
+  void* y;
+  const void* indptr;
+  int64_t expert_w_stride, expert_s_stride;
+  int rows, N, K, ng, nw;
+  int num_experts;
+  int out_f32, indptr_i64;
+};
+
+// One group (4 storage words) -> G halves in natural k order, (q - m) * s with fp16 rounding.
+template <int BITS>
+__device__ __forceinline__ void dequant_group(const uint4 w4, const uint16_t scale_bits,
+                                              uint32_t* __restrict__ out /* G/2 half pairs */) {
+  constexpr uint32_t kMagic = 0x64006400u;  // 1024.0 in both halves
+  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+  const _Float16 s = __builtin_bit_cast(_Float16, scale_bits);
+  const half2_t s2 = {s, s};
+  if (BITS == 4) {
+    const half2_t off = {static_cast<_Float16>(-1031.0f), static_cast<_Float16>(-1031.0f)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t t1 = w[i] >> 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // byte j of w -> low half (field 2j in its low nibble), byte j of w>>4 -> high half
+        const uint32_t sel = 0x0c000c00u | ((4u + j) << 16) | static_cast<uint32_t>(j);
+        const uint32_t r = and_or(__builtin_amdgcn_perm(t1, w[i], sel), 0x000f000fu, kMagic);
+        out[4 * i + j] = as_u32((as_half2(r) + off) * s2);
+      }
+    }
+  } else {
+    const half2_t off = {static_cast<_Float16>(-1027.0f), static_cast<_Float16>(-1027.0f)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 5; ++j) {
+        const uint32_t t = w[i] >> (6 * j);
+        const uint32_t r = and_or(t << 13, 0x00070000u, and_or(t, 0x00000007u, kMagic));
+        out[5 * i + j] = as_u32((as_half2(r) + off) * s2);
+      }
+    }
+  }
+}
+
+template <int BITS, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
+  using T = GemmTraits<BITS>;
+  constexpr int G = T::G;
+  constexpr int BK = 2 * G;            // 64 | 80
+  constexpr int KSTEPS = BK / 16;      // MFMA k = 16
+  constexpr int CPR = BK / 8;          // 16-byte chunks per tile row
+  constexpr int LDA = BK + 8;          // padded row, in halves
+  constexpr int WAVES_N = BN / WN;
+  static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_CHUNKS = BM * CPR / 256;  // 16-byte chunks of x per thread per tile
+  constexpr int W_GROUPS = BN * 2 / 256;    // groups of W per thread per tile
+  static_assert(BM * CPR % 256 == 0 && BN * 2 % 256 == 0, "tile / thread mismatch");
+
+  extern __shared__ uint4 smem[];
+  uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
+  // stage s: A at s*(BM+BN)*LDA, W right after A
+  auto a_tile = [&](int s) { return lds + s * (BM + BN) * LDA; };
+  auto w_tile = [&](int s) { return lds + s * (BM + BN) * LDA + BM * LDA; };
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+
+  // ---- which rows / which expert does this workgroup own
+  int seg_lo = 0, seg_hi = p.rows, mt = blockIdx.y, expert = 0;
+  if (p.indptr != nullptr) {
+    int t = blockIdx.y;
+    bool found = false;
+    for (int e = 0; e < p.num_experts; ++e) {
+      int64_t lo, hi;
+      if (p.indptr_i64) {
+        lo = static_cast<const int64_t*>(p.indptr)[e];
+        hi = static_cast<const int64_t*>(p.indptr)[e + 1];
+      } else {
+        lo = static_cast<const int32_t*>(p.indptr)[e];
+        hi = static_cast<const int32_t*>(p.indptr)[e + 1];
+      }
+      lo = lo < 0 ? 0 : (lo > p.rows ? p.rows : lo);  // a corrupt indptr must not leave the tensors
+      hi = hi < lo ? lo : (hi > p.rows ? p.rows : hi);
+      const int tiles = static_cast<int>((hi - lo + BM - 1) / BM);
+      if (t < tiles) {
+        seg_lo = static_cast<int>(lo);
+        seg_hi = static_cast<int>(hi);
+        mt = t;
+        expert = e;
+        found = true;
+        break;
+      }
+      t -= tiles;
+    }
+    if (!found) return;  // uniform over the workgroup
+  }
+  const int m0 = seg_lo + mt * BM;
+  if (m0 >= seg_hi) return;
+  const int n0 = blockIdx.x * BN;
+  const uint32_t* qw = p.qw + expert * p.expert_w_stride;
+  const uint16_t* qs = p.qs + expert * p.expert_s_stride;
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  uint4 a_reg[A_CHUNKS];
+  uint4 w_reg[W_GROUPS];
+  uint16_t s_reg[W_GROUPS];
+  const bool k_vec = (p.K & 7) == 0;
+
+  auto load_tile = [&](int kt) {
+    const int k_base = kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx / CPR, c = idx - r * CPR;
+      const int row = m0 + r, k = k_base + 8 * c;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (row < seg_hi && k < p.K) {
+        const uint16_t* src = p.x + static_cast<int64_t>(row) * p.K + k;
+        if (k_vec) {
+          v = *reinterpret_cast<const uint4*>(src);
+        } else {
+          uint16_t e[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) e[q] = (k + q < p.K) ? src[q] : uint16_t(0);
+          v.x = e[0] | (uint32_t(e[1]) << 16); v.y = e[2] | (uint32_t(e[3]) << 16);
+          v.z = e[4] | (uint32_t(e[5]) << 16); v.w = e[6] | (uint32_t(e[7]) << 16);
+        }
+      }
+      a_reg[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < W_GROUPS; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx >> 1, gsel = idx & 1;
+      const int row = min(n0 + r, p.N - 1);
+      const int g = 2 * kt + gsel;
+      if (g < p.ng) {
+        w_reg[i] = *reinterpret_cast<const uint4*>(qw + static_cast<int64_t>(row) * p.nw + 4 * g);
+        s_reg[i] = qs[static_cast<int64_t>(row) * p.ng + g];
+      } else {
+        w_reg[i] = make_uint4(0, 0, 0, 0);
+        s_reg[i] = 0;  // scale +0.0: the whole group dequantises to (-m) * 0 = -0.0
+      }
+    }
+  };
+
+  auto store_tile = [&](int s) {
+    uint16_t* at = a_tile(s);
+    uint16_t* wt = w_tile(s);
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx / CPR, c = idx - r * CPR;
+      *reinterpret_cast<uint4*>(at + r * LDA + 8 * c) = a_reg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < W_GROUPS; ++i) {
+      const int idx = tid + 256 * i;
+      const int r = idx >> 1, gsel = idx & 1;
+      uint32_t d[G / 2];
+      dequant_group<BITS>(w_reg[i], s_reg[i], d);
+      uint4* dst = reinterpret_cast<uint4*>(wt + r * LDA + gsel * G);
+#pragma unroll
+      for (int c = 0; c < G / 8; ++c) dst[c] = make_uint4(d[4 * c], d[4 * c + 1], d[4 * c + 2], d[4 * c + 3]);
+    }
+  };
+
+  const int nk = (p.ng + 1) / 2;
+  if (nk > 0) {
+    load_tile(0);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  const int frag_row = lane & 31, frag_k = 8 * (lane >> 5);
+  for (int kt = 0; kt < nk; ++kt) {
+    const int s = kt & 1;
+    if (kt + 1 < nk) load_tile(kt + 1);
+    const uint16_t* at = a_tile(s) + (wm0 + frag_row) * LDA + frag_k;
+    const uint16_t* wt = w_tile(s) + (wn0 + frag_row) * LDA + frag_k;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      half8_t af[TM], bf[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA + ks * 16);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bf[j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA + ks * 16);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) store_tile(s ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: D[i][j] of a 32x32 tile sits in lane (j + 32*((i/4)%2)), register 4*(i/8) + i%4
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn0 + j * 32 + (lane & 31);
+      const float b = (p.bias != nullptr && col < p.N) ? h2f(p.bias[col]) : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < seg_hi && col < p.N) {
+          const float v = acc[i][j][r] + b;
+          const int64_t o = static_cast<int64_t>(row) * p.N + col;
+          if (p.out_f32) static_cast<float*>(p.y)[o] = v;
+          else static_cast<uint16_t*>(p.y)[o] = f2h(v);
+        }
+      }
+    }
+  }
+}
+
+template <int BITS, int BM, int BN, int WM, int WN>
+static hipError_t launch_cfg(const GemmParams& p, hipStream_t s) {
+  constexpr int BK = 2 * GemmTraits<BITS>::G;
+  constexpr int LDA = BK + 8;
+  constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
+  auto kern = gemm_kernel<BITS, BM, BN, WM, WN>;
+  if (lds > 65536) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(lds));
+    if (e != hipSuccess) return e;
+  }
+  const int m_tiles = p.indptr ? (p.rows + BM - 1) / BM + p.num_experts : (p.rows + BM - 1) / BM;
+  const dim3 grid((p.N + BN - 1) / BN, m_tiles);
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
+  GemmParams p;
+  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.y = a.y;
+  p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64;
+  p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
+  p.ng = static_cast<int>((a.K + a.group_size - 1) / a.group_size);
+  p.nw = 4 * p.ng;
+  p.expert_w_stride = a.N * p.nw;
+  p.expert_s_stride = a.N * p.ng;
+  p.num_experts = static_cast<int>(a.num_experts);
+  p.out_f32 = a.out_f32;
+  if (a.rows == 0 || a.N == 0) return hipSuccess;
+  if (a.bits == 4) return launch_cfg<4, 128, 128, 64, 64>(p, s);
+  return launch_cfg<3, 128, 128, 64, 64>(p, s);
+}
+
+}  // namespace gq

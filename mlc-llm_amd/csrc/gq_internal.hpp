@@ -1,0 +1,68 @@
+// Internal launcher interface between the C ABI layer (gq_api.hip) and the kernel files.
+// Launchers assume validated arguments and return the hipError_t of the launch.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gq {
+
+struct Options {
+  int gemv_rows_per_wave = -1;  // -1: heuristic
+  int gemv_variant = -1;        // -1: heuristic, 0: dot2 kernel, 1: mfma kernel
+  int gemm_variant = -1;
+  int gemv_split = -1;
+};
+Options& options();
+
+struct GemvArgs {
+  const uint16_t* x;        // [x_rows, K] fp16
+  const uint32_t* q_weight; // [experts?, N, nw]
+  const uint16_t* q_scale;  // [experts?, N, ng]
+  const uint16_t* bias;     // [N] or null
+  void* y;                  // [M or slots, N]
+  const int32_t* expert_ids;  // null for a plain linear; else [slots]
+  int64_t M;                // batch rows of a plain linear (1..8); 1 for MoE slots
+  int64_t N, K;
+  int64_t slots;            // 1 for a plain linear, top_k for MoE
+  int64_t x_slot_stride;    // elements between x rows of consecutive slots (0 or K)
+  int64_t num_experts;
+  int bits, group_size;
+  int out_f32;
+};
+hipError_t launch_gemv(const GemvArgs& a, hipStream_t s);
+
+struct GemmArgs {
+  const uint16_t* x;        // [rows, K]
+  const uint32_t* q_weight; // [experts, N, nw]
+  const uint16_t* q_scale;  // [experts, N, ng]
+  const uint16_t* bias;     // [N] or null (plain linear only)
+  void* y;                  // [rows, N]
+  const void* indptr;       // null for a plain linear
+  int indptr_i64;
+  int64_t rows, N, K, num_experts;
+  int bits, group_size, out_f32;
+};
+hipError_t launch_gemm(const GemmArgs& a, hipStream_t s);
+
+hipError_t launch_quantize(const uint16_t* w, int64_t rows, int64_t K, int bits, int group_size,
+                           int round_mode, uint32_t* qw, uint16_t* qs, hipStream_t s);
+hipError_t launch_dequantize(const int32_t* ids, int64_t out_rows, const uint32_t* qw,
+                             const uint16_t* qs, int64_t table_rows, int64_t K, int bits,
+                             int group_size, uint16_t* out, hipStream_t s);
+
+hipError_t launch_topk_softmax(const uint16_t* logits, int64_t T, int ne, int k, uint16_t* w,
+                               int32_t* ids, hipStream_t s);
+hipError_t launch_moe_cumsum(const int32_t* ids, int64_t T, int k, int ne, int32_t* cumsum,
+                             hipStream_t s);
+hipError_t launch_get_indices(const int32_t* cumsum, const int32_t* ids, int64_t T, int k, int ne,
+                              int32_t* rev, int32_t* tok, hipStream_t s);
+hipError_t launch_get_indptr(const int32_t* cumsum, int64_t ne, int64_t T, int inclusive,
+                             int out_i64, void* indptr, hipStream_t s);
+hipError_t launch_take_rows(const uint16_t* x, const int32_t* idx, int64_t R, int64_t H,
+                            int64_t x_rows, uint16_t* out, int scatter, hipStream_t s);
+hipError_t launch_silu_mul(const uint16_t* x, int64_t R, int64_t I, uint16_t* out, hipStream_t s);
+hipError_t launch_moe_combine(const uint16_t* y, const uint16_t* w, int64_t T, int k, int64_t H,
+                              uint16_t* out, hipStream_t s);
+
+}  // namespace gq

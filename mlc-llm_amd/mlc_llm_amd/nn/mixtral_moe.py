@@ -1,0 +1,55 @@
+"""MixtralMoE.forward over group-quantized experts.
+
+Mirror of python/mlc_llm/model/mixtral/mixtral_model.py:32-117 of the reference, with the
+router logits supplied by the caller (the router `gate` is an unquantized nn.Linear there,
+quantization/utils.py:57-59, and is outside this path).
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .. import ops
+from ..op import moe_misc
+from ..quantization import GroupQuantize, GroupQuantizeMixtralExperts
+
+
+class MixtralMoE(nn.Module):
+    """Mixture of experts with group-quantized e1_e3 / e2 expert stacks."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_local_experts: int,
+                 num_experts_per_tok: int, config: GroupQuantize, device=None):
+        super().__init__()
+        self.num_experts_per_tok = num_experts_per_tok
+        self.num_local_experts = num_local_experts
+        self.intermediate_size = intermediate_size
+        self.e1_e3 = GroupQuantizeMixtralExperts(num_local_experts, hidden_size,
+                                                 2 * intermediate_size, config, device=device)
+        self.e2 = GroupQuantizeMixtralExperts(num_local_experts, intermediate_size, hidden_size,
+                                              config, device=device)
+
+    def _expert_forward(self, x: torch.Tensor, indptr: torch.Tensor) -> torch.Tensor:
+        x1_x3 = self.e1_e3(x, indptr)
+        return self.e2(ops.silu_mul(x1_x3), indptr)
+
+    def forward(self, x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+        """x fp16 [batch, seq, hidden]; gate fp16 [batch * seq, num_local_experts] router logits."""
+        experts_per_tok = self.num_experts_per_tok
+        local_experts = self.num_local_experts
+        batch_size, seq_len, hidden_size = x.shape
+        num_tokens = batch_size * seq_len
+        x = x.reshape(num_tokens, hidden_size).contiguous()
+        expert_weights, expert_indices = moe_misc.gating_softmax_topk(gate, experts_per_tok)
+        if num_tokens == 1:
+            x = self._expert_forward(x, expert_indices)
+        else:
+            cumsum = moe_misc.moe_cumsum(expert_indices, local_experts)
+            reverse_indices, token_indices = moe_misc.get_indices(cumsum, expert_indices)
+            indptr = moe_misc.get_indptr(cumsum, local_experts, num_tokens, inclusive=False,
+                                         out_dtype="int32")
+            x = ops.take_rows(x, token_indices)
+            x = self._expert_forward(x, indptr)
+            x = moe_misc.scatter_output(x, reverse_indices)
+        x = ops.moe_combine(x.reshape(num_tokens, experts_per_tok, hidden_size), expert_weights)
+        return x.reshape(batch_size, seq_len, hidden_size)

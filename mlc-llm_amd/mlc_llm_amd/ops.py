@@ -1,0 +1,246 @@
+"""Destination-passing operators over torch ROCm tensors.
+
+Each function plays the role the Relax VM plays around `call_dps_packed`: it
+checks shapes and dtypes, allocates the output tensor(s) and hands raw pointers
+plus the current HIP stream to the C ABI.  uint32 storage is held in int32
+torch tensors (same bits; torch's uint32 support on device is partial).
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _chk(t: torch.Tensor, dtype, name: str) -> torch.Tensor:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a torch.Tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise ValueError(f"{name}: must live on the GPU (got {t.device})")
+    dtypes = dtype if isinstance(dtype, tuple) else (dtype,)
+    if t.dtype not in dtypes:
+        raise TypeError(f"{name}: dtype {t.dtype}, expected {dtypes}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
+    return t
+
+
+_STORAGE = (torch.int32, torch.uint32)
+
+
+def num_group(k: int, group_size: int) -> int:
+    return -(-k // group_size)
+
+
+def num_storage(k: int, bits: int, group_size: int) -> int:
+    return (group_size // (32 // bits)) * num_group(k, group_size)
+
+
+def quantize(w: torch.Tensor, bits: int, group_size: int, round_mode: int = _lib.ROUND_HALF_AWAY
+             ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """w fp16 [..., K] -> (q_weight int32-as-uint32 [..., nw], q_scale fp16 [..., ng])."""
+    _chk(w, torch.float16, "w")
+    k = w.shape[-1]
+    rows = w.numel() // k if k else 0
+    lead = tuple(w.shape[:-1])
+    qw = torch.empty((*lead, num_storage(k, bits, group_size)), dtype=torch.int32, device=w.device)
+    qs = torch.empty((*lead, num_group(k, group_size)), dtype=torch.float16, device=w.device)
+    _lib.call("mi355gq_quantize", w.data_ptr(), rows, k, bits, group_size, round_mode,
+              qw.data_ptr(), qs.data_ptr(), _stream())
+    return qw, qs
+
+
+def dequantize(q_weight: torch.Tensor, q_scale: torch.Tensor, k: int, bits: int, group_size: int
+               ) -> torch.Tensor:
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    lead = tuple(q_weight.shape[:-1])
+    _check_qshapes(q_weight, q_scale, lead, k, bits, group_size)
+    rows = 1
+    for d in lead:
+        rows *= d
+    out = torch.empty((*lead, k), dtype=torch.float16, device=q_weight.device)
+    _lib.call("mi355gq_dequantize", q_weight.data_ptr(), q_scale.data_ptr(), rows, k, bits,
+              group_size, out.data_ptr(), _stream())
+    return out
+
+
+def _check_qshapes(q_weight, q_scale, lead, k, bits, group_size):
+    nw, ng = num_storage(k, bits, group_size), num_group(k, group_size)
+    if tuple(q_weight.shape) != (*lead, nw):
+        raise ValueError(f"q_weight shape {tuple(q_weight.shape)}, expected {(*lead, nw)}")
+    if tuple(q_scale.shape) != (*lead, ng):
+        raise ValueError(f"q_scale shape {tuple(q_scale.shape)}, expected {(*lead, ng)}")
+
+
+def embedding_take(ids: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, k: int,
+                   bits: int, group_size: int) -> torch.Tensor:
+    _chk(ids, torch.int32, "ids")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    num = q_weight.shape[0]
+    _check_qshapes(q_weight, q_scale, (num,), k, bits, group_size)
+    t = ids.numel()
+    out = torch.empty((*ids.shape, k), dtype=torch.float16, device=q_weight.device)
+    _lib.call("mi355gq_embedding_take", ids.data_ptr(), t, q_weight.data_ptr(), q_scale.data_ptr(),
+              num, k, bits, group_size, out.data_ptr(), _stream())
+    return out
+
+
+def linear(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits: int,
+           group_size: int, bias: Optional[torch.Tensor] = None, out_dtype=torch.float16,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[..., N] = x[..., K] . dequantize(q_weight, q_scale)^T (+ bias)."""
+    _chk(x, torch.float16, "x")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    k = x.shape[-1]
+    n = q_weight.shape[0]
+    _check_qshapes(q_weight, q_scale, (n,), k, bits, group_size)
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    if bias is not None:
+        _chk(bias, torch.float16, "bias")
+        if tuple(bias.shape) != (n,):
+            raise ValueError(f"bias shape {tuple(bias.shape)}, expected {(n,)}")
+    if out_dtype not in (torch.float16, torch.float32):
+        raise TypeError(f"out_dtype {out_dtype}")
+    if out is None:
+        out = torch.empty((*x.shape[:-1], n), dtype=out_dtype, device=x.device)
+    else:
+        _chk(out, out_dtype, "out")
+    ws_bytes = _lib.lib().mi355gq_linear_workspace_bytes(m, n, k, bits, group_size)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    _lib.call("mi355gq_linear", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(),
+              bias.data_ptr() if bias is not None else None, m, n, k, bits, group_size,
+              _lib.F32 if out_dtype == torch.float32 else _lib.F16, out.data_ptr(),
+              ws.data_ptr() if ws is not None else None, ws_bytes, _stream())
+    return out
+
+
+def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
+             expert_ids: torch.Tensor, bits: int, group_size: int) -> torch.Tensor:
+    _chk(x, torch.float16, "x")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    _chk(expert_ids, torch.int32, "expert_ids")
+    if x.dim() != 2 or expert_ids.dim() != 2 or expert_ids.shape[0] != 1:
+        raise ValueError("moe_gemv: x must be [1|k, K] and expert_ids [1, k]")
+    ne, n, _ = q_weight.shape
+    k = x.shape[1]
+    _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
+    top_k = expert_ids.shape[1]
+    out = torch.empty((top_k, n), dtype=torch.float16, device=x.device)
+    _lib.call("mi355gq_moe_gemv", x.data_ptr(), x.shape[0], q_weight.data_ptr(),
+              q_scale.data_ptr(), expert_ids.data_ptr(), top_k, ne, n, k, bits, group_size,
+              out.data_ptr(), _stream())
+    return out
+
+
+def moe_group_gemm(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
+                   indptr: torch.Tensor, bits: int, group_size: int) -> torch.Tensor:
+    _chk(x, torch.float16, "x")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    _chk(indptr, (torch.int32, torch.int64), "indptr")
+    ne, n, _ = q_weight.shape
+    rows, k = x.shape
+    _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
+    if tuple(indptr.shape) != (ne + 1,):
+        raise ValueError(f"indptr shape {tuple(indptr.shape)}, expected {(ne + 1,)}")
+    out = torch.zeros((rows, n), dtype=torch.float16, device=x.device)
+    _lib.call("mi355gq_moe_group_gemm", x.data_ptr(), rows, q_weight.data_ptr(),
+              q_scale.data_ptr(), indptr.data_ptr(),
+              _lib.I64 if indptr.dtype == torch.int64 else _lib.I32, ne, n, k, bits, group_size,
+              out.data_ptr(), _stream())
+    return out
+
+
+def gating_softmax_topk(logits: torch.Tensor, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    _chk(logits, torch.float16, "logits")
+    t, ne = logits.shape
+    w = torch.empty((t, top_k), dtype=torch.float16, device=logits.device)
+    ids = torch.empty((t, top_k), dtype=torch.int32, device=logits.device)
+    _lib.call("mi355gq_gating_softmax_topk", logits.data_ptr(), t, ne, top_k, w.data_ptr(),
+              ids.data_ptr(), _stream())
+    return w, ids
+
+
+def moe_cumsum(expert_indices: torch.Tensor, num_local_experts: int) -> torch.Tensor:
+    _chk(expert_indices, torch.int32, "expert_indices")
+    t, k = expert_indices.shape
+    out = torch.empty((num_local_experts * t,), dtype=torch.int32, device=expert_indices.device)
+    _lib.call("mi355gq_moe_cumsum", expert_indices.data_ptr(), t, k, num_local_experts,
+              out.data_ptr(), _stream())
+    return out
+
+
+def get_indices(cumsum: torch.Tensor, expert_indices: torch.Tensor
+                ) -> Tuple[torch.Tensor, torch.Tensor]:
+    _chk(cumsum, torch.int32, "cumsum")
+    _chk(expert_indices, torch.int32, "expert_indices")
+    t, k = expert_indices.shape
+    ne = cumsum.numel() // t if t else 1
+    rev = torch.zeros((t * k,), dtype=torch.int32, device=cumsum.device)
+    tok = torch.zeros((t * k,), dtype=torch.int32, device=cumsum.device)
+    _lib.call("mi355gq_moe_get_indices", cumsum.data_ptr(), expert_indices.data_ptr(), t, k, ne,
+              rev.data_ptr(), tok.data_ptr(), _stream())
+    return rev, tok
+
+
+def get_indptr(cumsum: torch.Tensor, num_local_experts: int, batch_size: int, inclusive: bool,
+               out_dtype=torch.int32) -> torch.Tensor:
+    _chk(cumsum, torch.int32, "cumsum")
+    n = num_local_experts if inclusive else num_local_experts + 1
+    out = torch.empty((n,), dtype=out_dtype, device=cumsum.device)
+    _lib.call("mi355gq_moe_get_indptr", cumsum.data_ptr(), num_local_experts, batch_size,
+              int(inclusive), _lib.I64 if out_dtype == torch.int64 else _lib.I32, out.data_ptr(),
+              _stream())
+    return out
+
+
+def take_rows(x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    _chk(x, torch.float16, "x")
+    _chk(indices, torch.int32, "indices")
+    r, h = indices.numel(), x.shape[1]
+    out = torch.zeros((r, h), dtype=torch.float16, device=x.device)
+    _lib.call("mi355gq_take_rows", x.data_ptr(), indices.data_ptr(), r, h, x.shape[0],
+              out.data_ptr(), _stream())
+    return out
+
+
+def scatter_output(x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    _chk(x, torch.float16, "x")
+    _chk(indices, torch.int32, "indices")
+    r, h = x.shape
+    out = torch.zeros_like(x)
+    _lib.call("mi355gq_moe_scatter_output", x.data_ptr(), indices.data_ptr(), r, h,
+              out.data_ptr(), _stream())
+    return out
+
+
+def silu_mul(x: torch.Tensor) -> torch.Tensor:
+    _chk(x, torch.float16, "x")
+    r, two_i = x.shape
+    out = torch.empty((r, two_i // 2), dtype=torch.float16, device=x.device)
+    _lib.call("mi355gq_silu_mul", x.data_ptr(), r, two_i // 2, out.data_ptr(), _stream())
+    return out
+
+
+def moe_combine(y: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+    """y fp16 [T, k, H], weights fp16 [T, k] -> fp16 [T, H]."""
+    _chk(y, torch.float16, "y")
+    _chk(weights, torch.float16, "weights")
+    t, k, h = y.shape
+    out = torch.empty((t, h), dtype=torch.float16, device=y.device)
+    _lib.call("mi355gq_moe_combine", y.data_ptr(), weights.data_ptr(), t, k, h, out.data_ptr(),
+              _stream())
+    return out

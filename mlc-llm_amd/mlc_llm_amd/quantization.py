@@ -1,0 +1,342 @@
+"""Host-side mirror of the reference's group-quantization interface, over torch tensors.
+
+Same names, argument meaning and error behaviour as
+python/mlc_llm/quantization/group_quantization.py and quantization.py of the
+reference; the arithmetic runs in the HIP library through `ops`.
+
+* GroupQuantize            <- group_quantization.py:27-63  (+ quantize_weight :188-233,
+                              quantize_model :65-153)
+* QUANTIZATION             <- quantization.py:47-90 (the group-quant float16 entries)
+* GroupQuantizeLinear      <- group_quantization.py:309-449
+* GroupQuantizeEmbedding   <- group_quantization.py:452-556
+* GroupQuantizeMixtralExperts <- group_quantization.py:559-660
+* MixtralExperts           <- nn/expert.py:9-33 (parameter holder that quantize_model replaces)
+* QuantizeMapping          <- loader/mapping.py (param_map / map_func)
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from functools import partial
+from typing import Callable, Dict, List, Literal, Optional
+
+import torch
+from torch import nn
+
+from . import _lib, ops
+
+_DTYPE_BITS = {"int3": 3, "int4": 4, "int8": 8, "uint32": 32}
+_TORCH_DTYPE = {"float16": torch.float16, "float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+@dataclasses.dataclass
+class QuantizeMapping:
+    """param_map: fp name -> quantized names; map_func: fp name -> quantize function."""
+
+    param_map: Dict[str, List[str]]
+    map_func: Dict[str, Callable]
+
+
+def is_final_fc(name: str) -> bool:
+    """quantization/utils.py:51-54 of the reference."""
+    return name in ["head", "lm_head", "lm_head.linear", "embed_out"]
+
+
+def is_moe_gate(name: str, node: nn.Linear) -> bool:
+    """quantization/utils.py:57-59 of the reference."""
+    return name.endswith("gate") and isinstance(node.out_features, int) and node.out_features <= 256
+
+
+@dataclasses.dataclass
+class GroupQuantize:
+    """Configuration for group quantization (same fields as the reference dataclass)."""
+
+    name: str
+    kind: str
+    group_size: int
+    quantize_dtype: Literal["int3", "int4", "int8"]
+    storage_dtype: Literal["uint32"]
+    model_dtype: Literal["float16", "float32", "bfloat16"]
+    linear_weight_layout: Literal["KN", "NK"]
+    quantize_embedding: bool = True
+    quantize_final_fc: bool = True
+
+    num_elem_per_storage: int = 0
+    num_storage_per_group: int = 0
+    max_int_value: int = 0
+    tensor_parallel_shards: int = 0
+    # tie rule of round() in quantize_weight: "half_away" is what TVM's llvm/rocm targets emit
+    round_mode: Literal["half_away", "half_even"] = "half_away"
+
+    def __post_init__(self):
+        assert self.kind == "group-quant"
+        assert self.quantize_dtype in ("int3", "int4", "int8")
+        assert self.storage_dtype.startswith("uint")
+        assert self.model_dtype in _TORCH_DTYPE
+        qbits = _DTYPE_BITS[self.quantize_dtype]
+        sbits = _DTYPE_BITS[self.storage_dtype]
+        if sbits < qbits:
+            raise ValueError("Storage unit should be greater or equal to quantized element")
+        self.num_elem_per_storage = sbits // qbits
+        if self.group_size % self.num_elem_per_storage != 0:
+            raise ValueError("Group size should be divisible by numbers of elements per storage")
+        self.num_storage_per_group = self.group_size // self.num_elem_per_storage
+        self.max_int_value = (2 ** (qbits - 1)) - 1
+        self.linear_quant_axis = 0 if self.linear_weight_layout == "KN" else 1
+
+    @property
+    def bits(self) -> int:
+        return _DTYPE_BITS[self.quantize_dtype]
+
+    def _require_built(self):
+        if self.model_dtype != "float16" or self.linear_weight_layout != "NK":
+            raise NotImplementedError(
+                f"{self.name}: only float16 / NK-layout group quantization has gfx950 kernels"
+            )
+
+    def quantize_weight(self, weight: torch.Tensor, axis: int = -1, output_transpose: bool = False
+                        ) -> List[torch.Tensor]:
+        """Quantize `weight` along `axis` (must be the last axis): [q_weight, q_scale]."""
+        self._require_built()
+        axis = axis if axis >= 0 else weight.dim() + axis
+        if axis != weight.dim() - 1:
+            raise NotImplementedError("quantize_weight: only the last axis is supported (NK layout)")
+        if output_transpose:
+            raise NotImplementedError("quantize_weight: output_transpose belongs to the KN layouts")
+        mode = _lib.ROUND_HALF_AWAY if self.round_mode == "half_away" else _lib.ROUND_HALF_EVEN
+        qw, qs = ops.quantize(weight.contiguous(), self.bits, self.group_size, mode)
+        return [qw, qs]
+
+    def dequantize_weight(self, q_weight: torch.Tensor, q_scale: torch.Tensor, in_features: int
+                          ) -> torch.Tensor:
+        """GroupQuantize._dequantize over the last axis, out_shape [..., in_features]."""
+        self._require_built()
+        return ops.dequantize(q_weight, q_scale, in_features, self.bits, self.group_size)
+
+    def quantize_model(self, model: nn.Module, quant_map: QuantizeMapping, name_prefix: str
+                       ) -> nn.Module:
+        """Replace Linear / Embedding / MixtralExperts by their quantized twins, record names."""
+        config = self
+
+        def visit(prefix: str, module: nn.Module) -> nn.Module:
+            for child_name, child in list(module.named_children()):
+                name = f"{prefix}.{child_name}" if prefix else child_name
+                new = replace(name, child)
+                if new is not child:
+                    setattr(module, child_name, new)
+            return module
+
+        def replace(name: str, node: nn.Module) -> nn.Module:
+            if getattr(node, "no_quantization", False):
+                return node
+            if (
+                isinstance(node, nn.Linear)
+                and (not is_final_fc(name) or config.quantize_final_fc)
+                and not is_moe_gate(name, node)
+            ):
+                weight_name = f"{name}.weight"
+                quant_map.param_map[weight_name] = [f"{name}.q_weight", f"{name}.q_scale"]
+                quant_map.map_func[weight_name] = partial(
+                    config.quantize_weight, output_transpose=config.linear_weight_layout == "KN"
+                )
+                return GroupQuantizeLinear.from_linear(node, config)
+            if isinstance(node, nn.Embedding) and config.quantize_embedding:
+                weight_name = f"{name}.weight"
+                quant_map.param_map[weight_name] = [f"{name}.q_weight", f"{name}.q_scale"]
+                quant_map.map_func[weight_name] = config.quantize_weight
+                return GroupQuantizeEmbedding.from_embedding(node, config)
+            if isinstance(node, MixtralExperts):
+                weight_name = f"{name}.weight"
+                quant_map.param_map[weight_name] = [f"{name}.q_weight", f"{name}.q_scale"]
+                quant_map.map_func[weight_name] = config.quantize_weight
+                return GroupQuantizeMixtralExperts.from_mixtral_experts(node, config)
+            return visit(name, node)
+
+        return visit(name_prefix, model)
+
+
+def _ceildiv(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+def _storage_param(shape, device) -> nn.Parameter:
+    return nn.Parameter(torch.zeros(shape, dtype=torch.int32, device=device), requires_grad=False)
+
+
+def _float_param(shape, dtype, device) -> nn.Parameter:
+    return nn.Parameter(torch.zeros(shape, dtype=dtype, device=device), requires_grad=False)
+
+
+class GroupQuantizeLinear(nn.Module):
+    """An nn.Linear with group-quantized weight: q_weight [N, nw], q_scale [N, ng] (NK)."""
+
+    def __init__(self, in_features: int, out_features: int, config: GroupQuantize,
+                 bias: bool = True, out_dtype: Optional[str] = None, device=None) -> None:
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.out_dtype = out_dtype
+        self.config = config
+        num_group = _ceildiv(in_features, config.group_size)
+        num_shards = config.tensor_parallel_shards
+        if num_shards > 1 and (in_features * num_shards // config.group_size) % num_shards != 0:
+            raise ValueError(
+                f"The linear dimension {in_features * num_shards} has "
+                f"{in_features * num_shards // config.group_size} groups under group size "
+                f"{config.group_size}. The groups cannot be evenly distributed on "
+                f"{num_shards} GPUs.\n"
+                "Possible solutions: reduce number of GPUs, or use quantization with smaller "
+                "group size."
+            )
+        model_dtype = _TORCH_DTYPE[config.model_dtype]
+        if config.linear_weight_layout == "KN":
+            self.q_weight = _storage_param(
+                (config.num_storage_per_group * num_group, out_features), device)
+            self.q_scale = _float_param((num_group, out_features), model_dtype, device)
+        else:
+            self.q_weight = _storage_param(
+                (out_features, config.num_storage_per_group * num_group), device)
+            self.q_scale = _float_param((out_features, num_group), model_dtype, device)
+        if bias:
+            bias_dtype = model_dtype if out_dtype is None else _TORCH_DTYPE[out_dtype]
+            self.bias = _float_param((out_features,), bias_dtype, device)
+        else:
+            self.bias = None
+
+    @staticmethod
+    def from_linear(src: nn.Linear, config: GroupQuantize) -> "GroupQuantizeLinear":
+        out_features, in_features = src.weight.shape
+        return GroupQuantizeLinear(
+            in_features=in_features,
+            out_features=out_features,
+            config=config,
+            bias=getattr(src, "bias", None) is not None,
+            out_dtype=getattr(src, "out_dtype", None),
+            device=src.weight.device,
+        )
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        self.config._require_built()
+        out_dtype = torch.float16 if self.out_dtype is None else _TORCH_DTYPE[self.out_dtype]
+        bias = self.bias
+        if bias is not None and bias.dtype != torch.float16:
+            # fp32 bias with fp32 output: added after the kernel, as the reference's `x + bias`
+            y = ops.linear(x, self.q_weight, self.q_scale, self.config.bits,
+                           self.config.group_size, None, out_dtype)
+            return y + bias
+        return ops.linear(x, self.q_weight, self.q_scale, self.config.bits,
+                          self.config.group_size, bias, out_dtype)
+
+
+class GroupQuantizeEmbedding(nn.Module):
+    """An nn.Embedding with group-quantized table, usable as tied lm_head."""
+
+    def __init__(self, num: int, dim: int, config: GroupQuantize, device=None):
+        super().__init__()
+        self.num = num
+        self.dim = dim
+        self.config = config
+        num_group = _ceildiv(dim, config.group_size)
+        self.q_weight = _storage_param((num, config.num_storage_per_group * num_group), device)
+        self.q_scale = _float_param((num, num_group), _TORCH_DTYPE[config.model_dtype], device)
+
+    @staticmethod
+    def from_embedding(embedding: nn.Embedding, config: GroupQuantize) -> "GroupQuantizeEmbedding":
+        num, dim = embedding.weight.shape
+        return GroupQuantizeEmbedding(num, dim, config, device=embedding.weight.device)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        self.config._require_built()
+        ids = x.reshape(-1).to(torch.int32).contiguous()
+        out = ops.embedding_take(ids, self.q_weight, self.q_scale, self.dim, self.config.bits,
+                                 self.config.group_size)
+        return out.reshape(*x.shape, self.dim)
+
+    def lm_head_forward(self, x: torch.Tensor) -> torch.Tensor:
+        """Dequantize the table and multiply: logits in float32."""
+        self.config._require_built()
+        return ops.linear(x, self.q_weight, self.q_scale, self.config.bits, self.config.group_size,
+                          None, torch.float32)
+
+
+class MixtralExperts(nn.Module):
+    """Unquantized expert stack [num_local_experts, out_features, in_features] (holder only)."""
+
+    def __init__(self, num_local_experts, in_features, out_features, tensor_parallel_shards=1,
+                 device=None):
+        super().__init__()
+        self.num_local_experts = num_local_experts
+        self.in_features = in_features
+        self.out_features = out_features
+        self.tensor_parallel_shards = tensor_parallel_shards
+        self.weight = nn.Parameter(
+            torch.zeros((num_local_experts, out_features, in_features), dtype=torch.float16,
+                        device=device), requires_grad=False)
+
+
+class GroupQuantizeMixtralExperts(nn.Module):
+    """MixtralExperts with group-quantized weights [Ne, N, nw] / [Ne, N, ng]."""
+
+    def __init__(self, num_local_experts, in_features, out_features, config: GroupQuantize,
+                 device=None):
+        super().__init__()
+        self.num_local_experts = num_local_experts
+        self.in_features = in_features
+        self.out_features = out_features
+        self.config = config
+        num_group = _ceildiv(in_features, config.group_size)
+        self.q_weight = _storage_param(
+            (num_local_experts, out_features, config.num_storage_per_group * num_group), device)
+        self.q_scale = _float_param((num_local_experts, out_features, num_group),
+                                    _TORCH_DTYPE[config.model_dtype], device)
+        self.quantize_dtype = config.quantize_dtype
+        self.group_size = config.group_size
+        self.dtype = config.model_dtype
+        if config.linear_weight_layout == "KN":
+            raise NotImplementedError("GroupQuantizeMixtralExperts does not support KN layout now.")
+
+    @staticmethod
+    def from_mixtral_experts(src: MixtralExperts, config: GroupQuantize
+                             ) -> "GroupQuantizeMixtralExperts":
+        return GroupQuantizeMixtralExperts(
+            num_local_experts=src.num_local_experts,
+            in_features=src.in_features,
+            out_features=src.out_features,
+            config=config,
+            device=src.weight.device,
+        )
+
+    def forward(self, x: torch.Tensor, indptr: torch.Tensor) -> torch.Tensor:
+        """2-D `indptr` [1, k] holds the selected expert ids (single token); 1-D is a true indptr."""
+        assert x.dim() == 2
+        if indptr.dim() == 2:
+            assert indptr.shape[0] == 1
+            return ops.moe_gemv(x, self.q_weight, self.q_scale, indptr, self.config.bits,
+                                self.group_size)
+        assert indptr.dim() == 1
+        return ops.moe_group_gemm(x, self.q_weight, self.q_scale, indptr, self.config.bits,
+                                  self.group_size)
+
+
+def _group(name: str, group_size: int, qdtype: str, layout: str, model_dtype: str = "float16"):
+    return GroupQuantize(
+        name=name,
+        kind="group-quant",
+        group_size=group_size,
+        quantize_dtype=qdtype,
+        storage_dtype="uint32",
+        model_dtype=model_dtype,
+        linear_weight_layout=layout,
+        quantize_embedding=True,
+        quantize_final_fc=True,
+    )
+
+
+# The group-quant entries of the reference registry (quantization.py:47-90).  The KN-layout
+# entries are listed so that names resolve; their kernels are not built (NotImplementedError).
+QUANTIZATION: Dict[str, GroupQuantize] = {
+    "q3f16_0": _group("q3f16_0", 40, "int3", "KN"),
+    "q3f16_1": _group("q3f16_1", 40, "int3", "NK"),
+    "q4f16_0": _group("q4f16_0", 32, "int4", "KN"),
+    "q4f16_1": _group("q4f16_1", 32, "int4", "NK"),
+}

@@ -1,0 +1,343 @@
+"""CPU oracle (numpy) for MLC-LLM's group-quantized linear path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package imports this module;
+it exists so that tests, the smoke check and the benchmark's CPU leg can verify
+the HIP kernels.  It restates, operation for operation, the tensor-expression
+definitions of the reference (paths relative to the reference checkout):
+
+* python/mlc_llm/quantization/group_quantization.py:235-306  (_quantize)
+* python/mlc_llm/quantization/group_quantization.py:155-186  (_dequantize)
+* python/mlc_llm/quantization/utils.py:15-48                 (convert_uint_to_float)
+* python/mlc_llm/quantization/utils.py:136-188               (pack_weight)
+* python/mlc_llm/op/moe_matmul.py:77-176, 562-768            (MoE dequant GEMV / group GEMM)
+* python/mlc_llm/op/moe_misc.py:14-32, 35-60, 135-235, 371-645 (routing ops)
+* python/mlc_llm/model/mixtral/mixtral_model.py:64-117       (MixtralMoE.forward)
+
+The arithmetic of the reference is produced by TVM, which is not part of the
+reference checkout.  Two behaviours therefore rest on TVM's documented lowering
+rather than on a run of the reference, and are PARITY UNPINNED:
+
+* the tie rule of ``round`` inside ``_quantize`` (half-away-from-zero on the
+  llvm / rocm targets; exposed here as ``round_mode``);
+* the result for an all-zero group (0/0 = NaN flows through compare+select
+  ``max``/``min`` and yields q = 0).
+
+Also PARITY UNPINNED (no reference test or golden vector exists): the MoE
+kernels (dequantize_gemv, dequantize_group_gemm) and the routing operators,
+apart from the worked ``moe_cumsum`` example in the reference docstring
+(op/moe_misc.py:399-427), which tests/ replays as a known answer.
+
+Everything else (field order, offset, scale indexing, padded K) is pinned in
+tests/ against the reference's own numpy test twins and hand-derived vectors.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+
+F16 = np.float16
+F32 = np.float32
+U32 = np.uint32
+
+
+@dataclass(frozen=True)
+class Scheme:
+    """Parameters of one GroupQuantize instance (group_quantization.py:27-63)."""
+
+    name: str
+    bits: int
+    group_size: int
+
+    @property
+    def elem_per_storage(self) -> int:  # :57
+        return 32 // self.bits
+
+    @property
+    def storage_per_group(self) -> int:  # :60
+        return self.group_size // self.elem_per_storage
+
+    @property
+    def max_int(self) -> int:  # :61
+        return (1 << (self.bits - 1)) - 1
+
+    def num_group(self, k: int) -> int:
+        return -(-k // self.group_size)
+
+    def num_storage(self, k: int) -> int:
+        return self.storage_per_group * self.num_group(k)
+
+
+# quantization/quantization.py:58-68 and :80-90
+SCHEMES = {
+    "q4f16_1": Scheme("q4f16_1", 4, 32),
+    "q3f16_1": Scheme("q3f16_1", 3, 40),
+}
+
+
+def _round(t32: np.ndarray, round_mode: str) -> np.ndarray:
+    """round() of a float32 array holding fp16-representable values."""
+    if round_mode == "half_away":  # llvm.round / __ocml_round_f16
+        return np.trunc(t32 + np.copysign(F32(0.5), t32))
+    if round_mode == "half_even":  # CUDA hrint
+        return np.rint(t32)
+    raise ValueError(f"unknown round_mode {round_mode!r}")
+
+
+def quantize_values(w: np.ndarray, scheme: Scheme, round_mode: str = "half_away"):
+    """max-abs scale and integer codes, before packing.
+
+    w: float16 [..., K] (quantisation axis last, NK layout).
+    Returns (q uint32 [..., K], scale float16 [..., ng]).
+    Every floating-point operation is a single correctly-rounded fp16 op, in the
+    order of group_quantization.py:250-287.
+    """
+    assert w.dtype == F16
+    g, m = scheme.group_size, scheme.max_int
+    k = w.shape[-1]
+    ng = scheme.num_group(k)
+    lead = w.shape[:-1]
+    pad = ng * g - k
+    absw = np.abs(w)
+    if pad:
+        # padded lanes hold min_value(fp16) (:262) and never win the max
+        absw = np.concatenate([absw, np.full((*lead, pad), -65504.0, F16)], axis=-1)
+    max_abs = absw.reshape(*lead, ng, g).max(axis=-1)  # :250-267 (exact)
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        scale = (max_abs / F16(m)).astype(F16)  # :268-272 fp16 divide
+        s_full = np.repeat(scale, g, axis=-1)[..., :k]
+        t = (w / s_full).astype(F16)  # :279-280 fp16 divide
+        t = (t + F16(m)).astype(F16)  # :281 fp16 add
+        r = _round(t.astype(F32), round_mode)  # :278
+        r = np.where(r > 0, r, F32(0))  # :277-283 max = select(a > b, a, b); NaN -> 0
+        r = np.where(r < 2 * m, r, F32(2 * m))  # :276,285 min = select(a < b, a, b)
+    return r.astype(U32), scale  # :286 cast to storage dtype
+
+
+def pack(q: np.ndarray, scheme: Scheme, num_storage: int | None = None) -> np.ndarray:
+    """utils.py:136-188: LSB-first packing with zero padding beyond K."""
+    assert q.dtype == U32
+    e, b = scheme.elem_per_storage, scheme.bits
+    k = q.shape[-1]
+    nw = scheme.num_storage(k) if num_storage is None else num_storage
+    lead = q.shape[:-1]
+    qp = np.zeros((*lead, nw * e), U32)
+    qp[..., :k] = q
+    qp = qp.reshape(*lead, nw, e)
+    out = np.zeros((*lead, nw), U32)
+    for r in range(e):
+        out += qp[..., r] << U32(r * b)
+    return out
+
+
+def quantize(w: np.ndarray, scheme: Scheme, round_mode: str = "half_away"):
+    """GroupQuantize.quantize_weight for the NK layout: (q_weight, q_scale)."""
+    q, scale = quantize_values(w, scheme, round_mode)
+    return pack(q, scheme), scale
+
+
+def unpack(q_weight: np.ndarray, scheme: Scheme, k: int) -> np.ndarray:
+    """utils.py:31-47 (non-ft_reorder branch): integer codes, uint32 [..., K]."""
+    assert q_weight.dtype == U32
+    e, b = scheme.elem_per_storage, scheme.bits
+    j = np.arange(k)
+    words = q_weight[..., j // e]
+    return (words >> ((j % e) * b).astype(U32)) & U32((1 << b) - 1)
+
+
+def dequantize(q_weight: np.ndarray, q_scale: np.ndarray, scheme: Scheme, k: int) -> np.ndarray:
+    """group_quantization.py:176-185: fp16 subtract (exact) then fp16 multiply."""
+    assert q_scale.dtype == F16
+    u = unpack(q_weight, scheme, k).astype(F16)
+    d = (u - F16(scheme.max_int)).astype(F16)
+    s = q_scale[..., np.arange(k) // scheme.group_size]
+    return (d * s).astype(F16)
+
+
+def linear_fp32(x, q_weight, q_scale, scheme: Scheme, bias=None) -> np.ndarray:
+    """fp32 dequant-then-matmul: the yardstick the output tolerance is quoted against.
+
+    x fp16 [M, K]; returns float64 [M, N] (exact products of fp16 values, summed in
+    float64, so the yardstick itself carries no accumulation error).
+    """
+    k = x.shape[-1]
+    w = dequantize(q_weight, q_scale, scheme, k).astype(np.float64)
+    y = x.astype(np.float64) @ w.T
+    if bias is not None:
+        y = y + bias.astype(np.float64)
+    return y
+
+
+def embedding_take(ids, q_weight, q_scale, scheme: Scheme, k: int) -> np.ndarray:
+    """GroupQuantizeEmbedding.forward (group_quantization.py:486-522)."""
+    return dequantize(q_weight[ids], q_scale[ids], scheme, k)
+
+
+# --------------------------------------------------------------------------- MoE routing
+
+
+def gating_softmax_topk(x: np.ndarray, k: int):
+    """moe_misc.py:135-235 with norm_topk_prob=True.
+
+    Top-k by insertion with strict '>' (ties keep the lower expert index,
+    :42-60), then softmax over the k selected logits in fp32, cast to x.dtype.
+    """
+    t, ne = x.shape
+    # running top-k starts at min_value(dtype) (:35-39); the reference leaves the
+    # index slots uninitialised, which only matters if fewer than k logits exceed it
+    vals = np.full((t, k), float(np.finfo(x.dtype).min), np.float64)
+    idx = np.zeros((t, k), np.int32)
+    for row in range(t):
+        for e in range(ne):
+            v = float(x[row, e])
+            for i in range(k):
+                if v > vals[row, i]:
+                    vals[row, i + 1 :] = vals[row, i:-1].copy()
+                    idx[row, i + 1 :] = idx[row, i:-1].copy()
+                    vals[row, i] = v
+                    idx[row, i] = e
+                    break
+    v32 = vals.astype(F32)
+    mx = v32.max(axis=1, keepdims=True)
+    ex = np.exp(v32 - mx, dtype=F32)
+    den = ex[:, 0].copy()
+    for i in range(1, k):  # left-to-right sum as in _nested_sum (:183-187)
+        den = den + ex[:, i]
+    return (ex / den[:, None]).astype(x.dtype), idx
+
+
+def moe_cumsum(expert_indices: np.ndarray, num_local_experts: int) -> np.ndarray:
+    """moe_misc.py:371-450: inclusive cumsum of the expert-major mask."""
+    t = expert_indices.shape[0]
+    mask = np.zeros((t, num_local_experts), np.int32)
+    for b in range(t):
+        for e in expert_indices[b]:
+            mask[b, e] = 1
+    return np.cumsum(mask.T.reshape(-1), dtype=np.int64).astype(np.int32)
+
+
+def get_indices(cumsum: np.ndarray, expert_indices: np.ndarray):
+    """moe_misc.py:453-525: (reverse_indices, token_indices)."""
+    t, k = expert_indices.shape
+    rev = np.zeros(t * k, np.int32)
+    tok = np.zeros(t * k, np.int32)
+    for b in range(t):
+        for j in range(k):
+            e = int(expert_indices[b, j])
+            pos = int(cumsum[e * t + b]) - 1
+            rev[pos] = b * k + j
+            tok[pos] = b
+    return rev, tok
+
+
+def get_indptr(cumsum, num_local_experts: int, batch_size: int, inclusive: bool, dtype=np.int32):
+    """moe_misc.py:528-605.  inclusive=False gives Ne+1 entries with a leading 0."""
+    if inclusive:
+        return np.array(
+            [cumsum[(i + 1) * batch_size - 1] for i in range(num_local_experts)], dtype
+        )
+    out = np.zeros(num_local_experts + 1, dtype)
+    for i in range(1, num_local_experts + 1):
+        out[i] = cumsum[i * batch_size - 1]
+    return out
+
+
+def scatter_output(x: np.ndarray, indices: np.ndarray) -> np.ndarray:
+    """moe_misc.py:608-645: out[indices[i]] = x[i]."""
+    out = np.zeros_like(x)
+    out[indices] = x
+    return out
+
+
+# --------------------------------------------------------------------------- MoE matmuls
+
+
+def moe_dequantize_gemv_fp32(x, q_weight, q_scale, expert_ids, scheme: Scheme) -> np.ndarray:
+    """moe_matmul.py:147-176 in exact arithmetic: float64 [k, N].
+
+    x fp16 [1|k, K]; expert_ids int32 [1, k]; q_weight [Ne, N, nw]; q_scale [Ne, N, ng].
+    """
+    kk = expert_ids.shape[1]
+    kdim = x.shape[1]
+    outs = []
+    for e in range(kk):
+        xe = x[0 if x.shape[0] == 1 else e]
+        ex = int(expert_ids[0, e])
+        w = dequantize(q_weight[ex], q_scale[ex], scheme, kdim).astype(np.float64)
+        outs.append(w @ xe.astype(np.float64))
+    return np.stack(outs)
+
+
+def dequantize_group_gemm_fp32(x, q_weight, q_scale, indptr, scheme: Scheme) -> np.ndarray:
+    """moe_matmul.py:632-722 in exact arithmetic: float64 [rows, N]."""
+    ne, n, _ = q_weight.shape
+    kdim = x.shape[1]
+    out = np.zeros((x.shape[0], n), np.float64)
+    for e in range(ne):
+        lo, hi = int(indptr[e]), int(indptr[e + 1])
+        if hi > lo:
+            w = dequantize(q_weight[e], q_scale[e], scheme, kdim).astype(np.float64)
+            out[lo:hi] = x[lo:hi].astype(np.float64) @ w.T
+    return out
+
+
+def silu_mul_f16(x1_x3: np.ndarray) -> np.ndarray:
+    """mixtral_model.py:66-68: split in two halves, silu(x1) * x3, all in fp16.
+
+    silu(x) = x * sigmoid(x) is evaluated in float32 and rounded once to fp16,
+    then multiplied by x3 in fp16.  (The reference's own rounding points inside
+    silu depend on TVM's legalisation: PARITY UNPINNED, compared with a 2-ulp
+    tolerance.)
+    """
+    h = x1_x3.shape[-1] // 2
+    x1, x3 = x1_x3[..., :h], x1_x3[..., h:]
+    x32 = x1.astype(F32)
+    silu = (x32 / (F32(1) + np.exp(-x32))).astype(F16)
+    return (silu * x3).astype(F16)
+
+
+def mixtral_moe(x, gate_logits, w13, s13, w2, s2, scheme: Scheme, top_k: int = 2):
+    """MixtralMoE.forward (mixtral_model.py:64-117) given the router logits.
+
+    Expert matmuls are evaluated exactly (float64) and rounded to fp16 where the
+    reference stores fp16 tensors; elementwise glue is fp16.  Returns fp16 [T, H].
+    """
+    t, hdim = x.shape
+    ne = w13.shape[0]
+    weights, ids = gating_softmax_topk(gate_logits, top_k)
+    if t == 1:
+        y = moe_dequantize_gemv_fp32(x, w13, s13, ids, scheme).astype(F16)
+        y = silu_mul_f16(y)
+        y = moe_dequantize_gemv_fp32(y, w2, s2, ids, scheme).astype(F16)
+    else:
+        cs = moe_cumsum(ids, ne)
+        rev, tok = get_indices(cs, ids)
+        indptr = get_indptr(cs, ne, t, inclusive=False)
+        xs = x[tok]
+        y = dequantize_group_gemm_fp32(xs, w13, s13, indptr, scheme).astype(F16)
+        y = silu_mul_f16(y)
+        y = dequantize_group_gemm_fp32(y, w2, s2, indptr, scheme).astype(F16)
+        y = scatter_output(y, rev)
+    y = (y.reshape(t, top_k, hdim) * weights.reshape(t, top_k, 1)).astype(F16)
+    out = y[:, 0]
+    for j in range(1, top_k):  # moe_sum (moe_misc.py:14-32)
+        out = (out + y[:, j]).astype(F16)
+    return out
+
+
+# --------------------------------------------------------------------------- tolerance
+
+
+def linear_tolerance(x: np.ndarray, k: int) -> float:
+    """max-abs bound for fp16 matmul outputs: 1e-2 * |x|_inf * sqrt(K) / 64."""
+    return 1e-2 * float(np.abs(x.astype(np.float64)).max()) * float(np.sqrt(k)) / 64.0
+
+
+def check_linear(y, ref64: np.ndarray, x: np.ndarray, k: int):
+    """Returns (max_abs_err, bound, rel_l2).  Pass iff err <= bound and rel_l2 <= 2e-3."""
+    y64 = np.asarray(y, dtype=np.float64)
+    err = float(np.abs(y64 - ref64).max()) if y64.size else 0.0
+    den = float(np.linalg.norm(ref64))
+    rel = float(np.linalg.norm(y64 - ref64) / den) if den > 0 else 0.0
+    return err, linear_tolerance(x, k), rel

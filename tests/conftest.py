@@ -1,0 +1,48 @@
+"""pytest configuration: the `gpu` marker and import paths.
+
+`-m "not gpu"`: oracle against golden vectors and known answers, host logic, and that the
+C-ABI library loads and exports every declared symbol (no kernels run).
+`-m gpu`: parity of the HIP kernels, called through the C ABI, against the oracle.
+"""
+
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.join(ROOT, "mlc-llm_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run on the GPU box)")
+
+
+def pytest_collection_modifyitems(config, items):
+    try:
+        import torch
+
+        has_gpu = torch.cuda.is_available()
+    except Exception:  # pragma: no cover
+        has_gpu = False
+    if has_gpu:
+        return
+    skip = pytest.mark.skip(reason="no GPU in this environment")
+    for item in items:
+        if "gpu" in item.keywords:
+            item.add_marker(skip)
+
+
+@pytest.fixture(scope="session")
+def golden():
+    import numpy as np
+
+    def load(name):
+        with np.load(os.path.join(GOLDEN, name + ".npz")) as z:
+            return {k: z[k] for k in z.files}
+
+    return load

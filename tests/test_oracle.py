@@ -1,0 +1,357 @@
+"""Pins the CPU oracle (oracle/gq_oracle.py and oracle/gq_oracle.c).
+
+What pins what:
+* field order / offset / scale indexing / padded K: hand-derived words, and the numpy
+  formulation the reference's own test uses (tests/python/quantization/
+  test_group_quantization.py:54-81 builds the expected dequantized matrix by repeat + indices;
+  `_dequant_by_repeat` below follows that formulation, which differs from the oracle's gather);
+* packing: exhaustive field enumeration, inverse of unpack, zero padding, top bits of int3;
+* scale and codes: closed-form groups whose exact answer is known without running any
+  quantizer, constructed ties, invariants, and the reference test's own loose check
+  (test_group_quantization.py:20-51, 84-108) on its shapes;
+* the C restatement must agree bit for bit with the numpy one;
+* routing: the worked example in the reference docstring (op/moe_misc.py:399-427) and brute force;
+* golden fixtures freeze all of it.
+"""
+
+import numpy as np
+import pytest
+
+from oracle import c_oracle
+from oracle import gq_oracle as o
+
+Q4, Q3 = o.SCHEMES["q4f16_1"], o.SCHEMES["q3f16_1"]
+REF_SHAPES = [("q3f16_1", (2, 13)), ("q3f16_1", (16, 120)), ("q4f16_1", (2, 13)), ("q4f16_1", (16, 128))]
+
+
+def test_scheme_constants():
+    # group_quantization.py:57-61 for the two registry entries (quantization.py:58-68, 80-90)
+    assert (Q4.elem_per_storage, Q4.storage_per_group, Q4.max_int) == (8, 4, 7)
+    assert (Q3.elem_per_storage, Q3.storage_per_group, Q3.max_int) == (10, 4, 3)
+    assert (Q4.num_group(4096), Q4.num_storage(4096)) == (128, 512)
+    assert (Q4.num_group(14336), Q4.num_storage(14336)) == (448, 1792)
+    assert (Q3.num_group(4096), Q3.num_storage(4096)) == (103, 412)
+    assert (Q3.num_group(11008), Q3.num_storage(11008)) == (276, 1104)
+    assert (Q3.num_group(13), Q3.num_storage(13)) == (1, 4)
+
+
+def test_unpack_known_words():
+    # nibble r of 0x76543210 is r; LSB first
+    qw = np.array([[0x76543210, 0xFEDCBA98, 0, 0]], np.uint32)
+    assert o.unpack(qw, Q4, 16).tolist() == [list(range(16))]
+    # int3: field r sits at bit 3r, 10 fields, bits 30-31 unused
+    word = sum((r % 8) << (3 * r) for r in range(10))
+    qw3 = np.array([[word, 0xFFFFFFFF, 0, 0]], np.uint32)
+    assert o.unpack(qw3, Q3, 20).tolist() == [[0, 1, 2, 3, 4, 5, 6, 7, 0, 1] + [7] * 10]
+
+
+def test_dequantize_known_values():
+    # (q - 7) * s and (q - 3) * s with s exactly representable
+    qw = np.array([[0x76543210, 0xFEDCBA98, 0, 0]], np.uint32)
+    d = o.dequantize(qw, np.array([[0.5]], np.float16), Q4, 32)
+    assert d[0, :16].tolist() == [(q - 7) * 0.5 for q in range(16)]
+    assert (d[0, 16:] == -3.5).all()
+    word = sum((r % 8) << (3 * r) for r in range(10))
+    d3 = o.dequantize(np.array([[word, 0, 0, 0]], np.uint32), np.array([[2.0]], np.float16), Q3, 13)
+    assert d3[0].tolist() == [(q - 3) * 2.0 for q in [0, 1, 2, 3, 4, 5, 6, 7, 0, 1, 0, 0, 0]]
+
+
+def test_dequantize_rounds_product_to_fp16():
+    # 7 * s needs more than 11 significant bits for s = 1 + 2^-10: fp16 product must round
+    s = np.float16(1 + 2**-10)
+    qw = np.array([[14, 0, 0, 0]], np.uint32)  # q = 14 -> (14 - 7) = 7
+    d = o.dequantize(qw, np.array([[s]], np.float16), Q4, 1)
+    exact = 7 * float(s)
+    assert float(d[0, 0]) == float(np.float16(exact)) and float(d[0, 0]) != exact
+
+
+def _dequant_by_repeat(s, weight, scale, out_shape):
+    """The formulation of the reference test's expected value (repeat words and scales)."""
+    mask = (1 << s.bits) - 1
+    wr = np.repeat(weight, s.elem_per_storage, axis=-1)
+    sr = np.repeat(scale, s.group_size, axis=-1)
+    j = np.indices(wr.shape)[1]
+    wb = (wr >> ((j % s.elem_per_storage) * s.bits).astype(np.uint32)) & np.uint32(mask)
+    assert wb.shape[1] <= sr.shape[1]
+    return ((wb.astype(np.float32) - s.max_int) * sr[..., : wb.shape[1]].astype(np.float32))[
+        : out_shape[0], : out_shape[1]]
+
+
+@pytest.mark.parametrize("name,shape", REF_SHAPES)
+def test_dequantize_matches_reference_test_formulation(name, shape):
+    # test_group_quantization.py:111-146: random full-range words, random scales, rtol/atol 1e-3
+    s = o.SCHEMES[name]
+    rng = np.random.default_rng(7)
+    n, k = shape
+    qw = rng.integers(0, 2**32, (n, s.num_storage(k)), dtype=np.uint64).astype(np.uint32)
+    qs = rng.random((n, s.num_group(k))).astype(np.float16)
+    got = o.dequantize(qw, qs, s, k).astype(np.float32)
+    want = _dequant_by_repeat(s, qw, qs, shape)
+    np.testing.assert_allclose(got, want, rtol=1e-3, atol=1e-3)
+    # and exactly: the fp32 product of two halves rounded once to half
+    assert (got == want.astype(np.float16).astype(np.float32)).all()
+
+
+@pytest.mark.parametrize("s", [Q4, Q3])
+def test_pack_unpack_exhaustive_fields(s):
+    e, b = s.elem_per_storage, s.bits
+    for pos in range(e):
+        for val in range(1 << b):
+            q = np.zeros((1, s.group_size), np.uint32)
+            q[0, pos] = val
+            packed = o.pack(q, s)
+            assert packed.shape == (1, 4)
+            assert int(packed[0, 0]) == val << (pos * b) and not packed[0, 1:].any()
+            assert (o.unpack(packed, s, s.group_size) == q).all()
+    rng = np.random.default_rng(1)
+    q = rng.integers(0, 1 << b, (5, 3 * s.group_size - 7)).astype(np.uint32)
+    packed = o.pack(q, s)
+    assert (o.unpack(packed, s, q.shape[1]) == q).all()
+    # zero padding beyond K, and bits 30-31 of int3 words stay clear
+    full = o.unpack(packed, s, packed.shape[1] * e)
+    assert not full[:, q.shape[1]:].any()
+    if b == 3:
+        assert not (packed >> np.uint32(30)).any()
+
+
+@pytest.mark.parametrize("s", [Q4, Q3])
+def test_quantize_closed_form_group(s):
+    # w = (q - m) * 2^-6 with the extremes present: scale is exactly 2^-6 and q comes back exactly,
+    # whatever the tie rule
+    m, g = s.max_int, s.group_size
+    rng = np.random.default_rng(3)
+    q = rng.integers(0, 2 * m + 1, (4, 2 * g)).astype(np.int64)
+    q[:, 0] = 2 * m
+    q[:, g] = 0
+    w = ((q - m) * 2.0**-6).astype(np.float16)
+    for mode in ("half_away", "half_even"):
+        qw, qs = o.quantize(w, s, mode)
+        assert (qs == np.float16(2.0**-6)).all()
+        assert (o.unpack(qw, s, 2 * g) == q).all()
+        assert (o.dequantize(qw, qs, s, 2 * g) == w).all()
+
+
+@pytest.mark.parametrize("s", [Q4, Q3])
+def test_quantize_ties_follow_round_mode(s):
+    m, g = s.max_int, s.group_size
+    w = np.zeros((1, g), np.float16)
+    w[0, 0] = m * 2.0**-6  # fixes scale = 2^-6
+    w[0, 1] = 0.5 * 2.0**-6  # t = m + 0.5
+    w[0, 2] = 1.5 * 2.0**-6  # t = m + 1.5
+    w[0, 3] = -0.5 * 2.0**-6  # t = m - 0.5
+    away = o.unpack(o.quantize(w, s, "half_away")[0], s, g)[0]
+    even = o.unpack(o.quantize(w, s, "half_even")[0], s, g)[0]
+    assert away[:4].tolist() == [2 * m, m + 1, m + 2, m]
+    exp_even = [2 * m] + [int(np.rint(v)) for v in (m + 0.5, m + 1.5, m - 0.5)]
+    assert even[:4].tolist() == exp_even
+    assert away[:4].tolist() != even[:4].tolist()
+
+
+@pytest.mark.parametrize("s", [Q4, Q3])
+def test_quantize_invariants_and_zero_group(s):
+    rng = np.random.default_rng(5)
+    k = 5 * s.group_size - 11
+    w = (rng.standard_normal((32, k)) * 0.02).astype(np.float16)
+    w[3, : s.group_size] = 0
+    qw, qs = o.quantize(w, s)
+    q = o.unpack(qw, s, k).astype(np.int64)
+    assert q.min() >= 0 and q.max() <= 2 * s.max_int
+    assert not q[3, : s.group_size].any() and qs[3, 0] == 0  # 0/0 -> NaN -> 0
+    # scale is the correctly rounded fp16 quotient max|w| / m
+    g = s.group_size
+    for n in (0, 7):
+        for gi in range(qs.shape[1]):
+            grp = w[n, gi * g: (gi + 1) * g]
+            mx = np.abs(grp).max()
+            assert qs[n, gi] == np.float16(np.float32(mx) / np.float32(s.max_int))
+            # the element of largest magnitude lands on an end of the range
+            j = int(np.abs(grp.astype(np.float32)).argmax())
+            assert q[n, gi * g + j] in (0, 2 * s.max_int) or mx == 0
+            # monotone in w inside a group
+            order = np.argsort(grp.astype(np.float32), kind="stable")
+            assert (np.diff(q[n, gi * g: gi * g + len(grp)][order]) >= 0).all()
+    # reconstruction error is at most half a step (plus fp16 rounding of the quotient)
+    d = o.dequantize(qw, qs, s, k).astype(np.float32)
+    step = np.repeat(qs.astype(np.float32), g, axis=1)[:, :k]
+    assert (np.abs(d - w.astype(np.float32)) <= 0.5 * step * 1.04 + 1e-6).all()
+
+
+def _quantize_np_float64(s, w):
+    """The loose numpy check of the reference test (test_group_quantization.py:20-51)."""
+    g, m = s.group_size, s.max_int
+    n, k = w.shape
+    wp = np.pad(w.astype(np.float64), ((0, 0), (0, (-k) % g)))
+    wr = wp.reshape(n, -1, g)
+    mx = np.maximum(np.abs(wr).max(-1), 1e-4)
+    scale = mx / m
+    q = np.clip(np.round(wr / scale[..., None]) + m, 0, 2 * m)
+    return q.reshape(n, -1)[:, :k], scale
+
+
+@pytest.mark.parametrize("name,shape", REF_SHAPES)
+def test_quantize_within_reference_test_tolerance(name, shape):
+    # test_group_quantization.py:84-108: uniform[0,1) weights; scales rtol/atol 1e-3; dequantized
+    # values atol 0.2 (int4) / 0.4 (int3)
+    s = o.SCHEMES[name]
+    w = np.random.default_rng(11).random(shape).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    q_ref, scale_ref = _quantize_np_float64(s, w)
+    np.testing.assert_allclose(qs.astype(np.float64), scale_ref, rtol=1e-3, atol=1e-3)
+    got = o.dequantize(qw, qs, s, shape[1]).astype(np.float64)
+    want = (q_ref - s.max_int) * np.repeat(scale_ref, s.group_size, axis=1)[:, : shape[1]]
+    np.testing.assert_allclose(got, want, rtol=1e-2 if s.bits == 3 else 1e-3,
+                               atol=0.4 if s.bits == 3 else 0.2)
+
+
+@pytest.mark.parametrize("s", [Q4, Q3])
+def test_c_oracle_matches_numpy_oracle(s):
+    rng = np.random.default_rng(13)
+    for shape in [(2, 13), (16, 4 * s.group_size), (9, 1000)]:
+        w = (rng.standard_normal(shape) * 0.02).astype(np.float16)
+        w[0, : min(shape[1], s.group_size)] = 0
+        for mode, name in ((0, "half_away"), (1, "half_even")):
+            qw, qs = o.quantize(w, s, name)
+            cw, cs = c_oracle.quantize(w, s.bits, s.group_size, mode)
+            assert (qw == cw).all() and (qs.view(np.uint16) == cs.view(np.uint16)).all()
+        d = o.dequantize(qw, qs, s, shape[1])
+        cd = c_oracle.dequantize(qw, qs, shape[1], s.bits, s.group_size)
+        assert (d.view(np.uint16) == cd.view(np.uint16)).all()
+        x = rng.standard_normal((3, shape[1])).astype(np.float16)
+        err, bound, rel = o.check_linear(c_oracle.linear(x, qw, qs, s.bits, s.group_size),
+                                         o.linear_fp32(x, qw, qs, s), x, shape[1])
+        assert err <= bound and rel <= 1e-5
+
+
+def test_c_oracle_half_conversion_exhaustive():
+    lib = c_oracle.lib()
+    allh = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    f = allh.view(np.float16).astype(np.float32)
+    for h in range(0, 65536, 5):
+        v = lib.gqo_h2f(h)
+        assert v == f[h] or (np.isnan(v) and np.isnan(f[h]))
+    rng = np.random.default_rng(17)
+    xs = rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 20000)
+    xs = np.concatenate([xs, np.array([65519.99, 65520, 65504, 6e-8, 2.9802322e-8, 2.9802326e-8,
+                                       0.0, -0.0, 1.00048828125, 1.00146484375], np.float32)])
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16).view(np.uint16)
+    for v, w_ in zip(xs, want):
+        assert lib.gqo_f2h(float(v)) == w_
+
+
+def test_linear_special_cases():
+    # scale 1: the quantized matmul is an integer matmul; identity activations return the matrix
+    rng = np.random.default_rng(19)
+    for s in (Q4, Q3):
+        k = 2 * s.group_size
+        q = rng.integers(0, 2 * s.max_int + 1, (6, k)).astype(np.uint32)
+        qw = o.pack(q, s)
+        qs = np.ones((6, 2), np.float16)
+        x = rng.integers(-4, 5, (3, k)).astype(np.float16)
+        want = x.astype(np.int64) @ (q.astype(np.int64) - s.max_int).T
+        assert (o.linear_fp32(x, qw, qs, s) == want).all()
+        eye = np.eye(k, dtype=np.float16)
+        assert (o.linear_fp32(eye, qw, qs, s).T == o.dequantize(qw, qs, s, k)).all()
+
+
+def test_moe_cumsum_docstring_example():
+    # op/moe_misc.py:399-427 of the reference
+    ids = np.array([[0, 1], [1, 2], [3, 4], [2, 5]], np.int32)
+    want = np.array([[1, 1, 1, 1], [2, 3, 3, 3], [3, 4, 4, 5], [5, 5, 6, 6], [6, 6, 7, 7], [7, 7, 7, 8]])
+    cs = o.moe_cumsum(ids, 6)
+    assert (cs.reshape(6, 4) == want).all()
+    assert o.get_indptr(cs, 6, 4, False).tolist() == [0, 1, 3, 5, 6, 7, 8]
+    assert o.get_indptr(cs, 6, 4, True).tolist() == [1, 3, 5, 6, 7, 8]
+    rev, tok = o.get_indices(cs, ids)
+    # slots ordered by (expert, token): e0:{t0} e1:{t0,t1} e2:{t1,t3} e3:{t2} e4:{t2} e5:{t3}
+    assert tok.tolist() == [0, 0, 1, 1, 3, 2, 2, 3]
+    assert rev.tolist() == [0, 1, 2, 3, 6, 4, 5, 7]
+
+
+def test_routing_brute_force_properties():
+    rng = np.random.default_rng(23)
+    t, ne, k = 37, 8, 2
+    logits = rng.standard_normal((t, ne)).astype(np.float16)
+    logits[4, :] = 0.25  # full tie: lowest indices, in order
+    w, ids = o.gating_softmax_topk(logits, k)
+    assert ids[4].tolist() == [0, 1]
+    for r in range(t):
+        order = sorted(range(ne), key=lambda e: (-float(logits[r, e]), e))[:k]
+        assert ids[r].tolist() == order
+        v = logits[r, order].astype(np.float64)
+        p = np.exp(v - v.max())
+        np.testing.assert_allclose(w[r].astype(np.float64), p / p.sum(), atol=6e-4)
+    cs = o.moe_cumsum(ids, ne)
+    rev, tok = o.get_indices(cs, ids)
+    indptr = o.get_indptr(cs, ne, t, False)
+    assert indptr[0] == 0 and indptr[-1] == t * k and (np.diff(indptr) >= 0).all()
+    assert sorted(rev.tolist()) == list(range(t * k))  # a permutation
+    for e in range(ne):
+        seg = tok[indptr[e]: indptr[e + 1]]
+        assert (np.diff(seg) > 0).all()  # stable by token inside an expert
+        assert all(e in ids[b] for b in seg)
+    x = rng.standard_normal((t * k, 5)).astype(np.float16)
+    flat = np.repeat(np.arange(t), k)
+    assert (flat[rev] == tok).all()
+    assert (o.scatter_output(x[rev], rev) == x).all()  # scatter undoes the gather
+
+
+def test_group_gemm_and_moe_gemv_against_dense():
+    rng = np.random.default_rng(29)
+    s = Q4
+    ne, n, k = 3, 10, 64
+    w = (rng.standard_normal((ne, n, k)) * 0.05).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    x = rng.standard_normal((7, k)).astype(np.float16)
+    indptr = np.array([0, 3, 3, 7], np.int32)
+    y = o.dequantize_group_gemm_fp32(x, qw, qs, indptr, s)
+    wd = o.dequantize(qw, qs, s, k).astype(np.float64)
+    assert np.allclose(y[:3], x[:3].astype(np.float64) @ wd[0].T)
+    assert np.allclose(y[3:], x[3:].astype(np.float64) @ wd[2].T)
+    yc = c_oracle.group_gemm(x, qw, qs, indptr, s.bits, s.group_size)
+    assert np.allclose(yc, y, atol=1e-4)
+    ids = np.array([[2, 0]], np.int32)
+    g = o.moe_dequantize_gemv_fp32(x[:1], qw, qs, ids, s)
+    assert np.allclose(g[0], wd[2] @ x[0].astype(np.float64)) and np.allclose(g[1], wd[0] @ x[0].astype(np.float64))
+    g2 = o.moe_dequantize_gemv_fp32(x[:2], qw, qs, ids, s)
+    assert np.allclose(g2[1], wd[0] @ x[1].astype(np.float64))
+
+
+def test_golden_fixtures_reproduce(golden):
+    import glob
+    import os
+
+    from conftest import GOLDEN
+
+    names = sorted(os.path.basename(p)[:-4] for p in glob.glob(os.path.join(GOLDEN, "*.npz")))
+    assert len(names) >= 20
+    for name in names:
+        z = golden(name)
+        if name.startswith("quant_"):
+            s = o.SCHEMES[name.split("_")[1] + "_1"]
+            for mode in ("half_away", "half_even"):
+                qw, qs = o.quantize(z["w"], s, mode)
+                assert (qw == z[f"q_weight_{mode}"]).all()
+                assert (qs.view(np.uint16) == z[f"q_scale_{mode}"].view(np.uint16)).all()
+            k = z["w"].shape[1]
+            d = o.dequantize(z["q_weight_half_away"], z["q_scale_half_away"], s, k)
+            assert (d.view(np.uint16) == z["dequant"].view(np.uint16)).all()
+            assert np.array_equal(o.linear_fp32(z["x"], z["q_weight_half_away"], z["q_scale_half_away"], s), z["y"])
+        elif name.startswith("dequant_"):
+            s = o.SCHEMES[name.split("_")[1] + "_1"]
+            k = z["dequant"].shape[1]
+            d = o.dequantize(z["q_weight"], z["q_scale"], s, k)
+            assert (d.view(np.uint16) == z["dequant"].view(np.uint16)).all()
+        elif name.startswith("routing_"):
+            t, ne = z["logits"].shape
+            k = z["ids"].shape[1]
+            w, ids = o.gating_softmax_topk(z["logits"], k)
+            assert (ids == z["ids"]).all() and (w.view(np.uint16) == z["weights"].view(np.uint16)).all()
+            cs = o.moe_cumsum(ids, ne)
+            assert (cs == z["cumsum"]).all()
+            rev, tok = o.get_indices(cs, ids)
+            assert (rev == z["reverse_indices"]).all() and (tok == z["token_indices"]).all()
+            assert (o.get_indptr(cs, ne, t, False) == z["indptr"]).all()
+        elif name.startswith("moe_"):
+            y = o.mixtral_moe(z["x"], z["logits"], z["q13"], z["s13"], z["q2"], z["s2"], Q4, 2)
+            assert (y.view(np.uint16) == z["y"].view(np.uint16)).all()
