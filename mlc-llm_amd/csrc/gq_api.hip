@@ -169,7 +169,9 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
   GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned2(q_scale) && aligned4(y) &&
                  aligned2(bias),
              "linear: x and q_weight must be 16-byte aligned");
-  if (M <= 8) {
+  // regimes: M <= 2 register GEMV; 3..16 MFMA skinny kernel (q4) or LDS GEMV up to 8 (q3); else GEMM
+  const bool use_gemv = M <= 2 || (M <= 8 && (bits != 4 || gq::options().gemm_variant == 2));
+  if (use_gemv) {
     gq::GemvArgs a{};
     a.x = static_cast<const uint16_t*>(x);
     a.q_weight = static_cast<const uint32_t*>(q_weight);
@@ -190,6 +192,10 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
   g.indptr = nullptr; g.indptr_i64 = 0;
   g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
   g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
+  if (M <= 16 && bits == 4 && gq::options().gemm_variant != 1) {
+    const hipError_t e = gq::launch_skinny(g, static_cast<int>(M), as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "skinny launch");
+  }
   return hip_result(gq::launch_gemm(g, as_stream(stream)), "gemm launch");
 }
 
@@ -245,6 +251,11 @@ int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, co
   g.indptr = indptr; g.indptr_i64 = indptr_dtype == MI355GQ_I64;
   g.rows = rows; g.N = N; g.K = K; g.num_experts = num_experts;
   g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
+  // few rows in total: every expert is a skinny problem bound by streaming its weights
+  if (rows <= 128 && bits == 4 && gq::options().gemm_variant != 1) {
+    const hipError_t e = gq::launch_skinny(g, static_cast<int>(rows), as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "moe skinny launch");
+  }
   return hip_result(gq::launch_gemm(g, as_stream(stream)), "moe_group_gemm launch");
 }
 

@@ -32,9 +32,13 @@ __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
   return __builtin_amdgcn_fdot2(as_half2(a), as_half2(b), c, false);
 }
 
-// (a & mask) | bits : v_and_or_b32
+// (a & mask) | bits as ONE v_and_or_b32.  A VOP3 instruction takes a single 32-bit literal, so the
+// compiler splits the two-constant form into v_and + v_or; keeping the mask in a VGPR and the OR
+// bits in an SGPR makes the fused form encodable (both constants are loop invariant).
 __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t bits) {
-  return (a & mask) | bits;
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(mask), "s"(bits));
+  return r;
 }
 
 __device__ __forceinline__ float h2f(uint16_t h) {
@@ -59,6 +63,24 @@ __device__ __forceinline__ float wave_sum(float v) {
   v += dpp_f<0x140>(v);  // row_mirror: lane i <-> 15-i inside each 16
   v += __shfl_xor(v, 16, kWave);
   v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+// Sum over the 64 lanes with DPP only; the total is valid in lane 63 alone.
+// row_bcast15 adds lane 15 of the previous row into rows 1 and 3, row_bcast31 adds lane 31
+// (rows 0+1) into rows 2 and 3.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_masked_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL,
+                                                                ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum_last(float v) {
+  v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  v += dpp_f<0x141>(v);  // row_half_mirror
+  v += dpp_f<0x140>(v);  // row_mirror: every lane now holds its row's sum
+  v += dpp_masked_f<0x142, 0xA>(v);  // row_bcast15
+  v += dpp_masked_f<0x143, 0xC>(v);  // row_bcast31
   return v;
 }
 

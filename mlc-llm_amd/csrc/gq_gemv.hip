@@ -20,39 +20,9 @@
 //    (conflict-free ds_read_b128); values beyond K are staged as 0, which also neutralises the
 //    zero padding fields of the last q3 group;
 //  * the per-row sum over lanes is a DPP/bpermute wave reduction.
-#include "gq_common.hpp"
-#include "gq_internal.hpp"
+#include "gq_gemv_common.hpp"
 
 namespace gq {
-
-template <int BITS>
-struct GemvTraits;
-template <>
-struct GemvTraits<4> {
-  static constexpr int G = 32;   // values per group
-  static constexpr int CH = 4;   // 16-byte x chunks per group (8 halves each)
-};
-template <>
-struct GemvTraits<3> {
-  static constexpr int G = 40;
-  static constexpr int CH = 5;
-};
-
-struct GemvParams {
-  const uint16_t* x;
-  const uint32_t* qw;
-  const uint16_t* qs;
-  const uint16_t* bias;
-  void* y;
-  const int32_t* expert_ids;
-  int64_t x_slot_stride;
-  int64_t expert_w_stride;  // N * nw
-  int64_t expert_s_stride;  // N * ng
-  int N, K, ng, nw;
-  int num_experts;
-  int gc;  // groups staged per LDS chunk (multiple of 64)
-  int out_f32;
-};
 
 // Stage groups [gbase, gbase + gcount) of NB activation rows into LDS (permuted) + corr terms.
 template <int BITS, int NB>
@@ -117,40 +87,6 @@ __device__ __forceinline__ void stage_x(const uint16_t* __restrict__ x, int K, i
     c += dpp_f<0xB1>(c);
     c += dpp_f<0x4E>(c);
     if (live && word == 0) corr[b * gc + gl] = c;
-  }
-}
-
-// sum_k x_k * (field_k - m) for one group, given the 4 storage words and the staged x pairs
-template <int BITS>
-__device__ __forceinline__ float group_dot(const uint4 w4, const uint32_t* __restrict__ xr,
-                                           float corr) {
-  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
-  constexpr uint32_t kMagic = 0x64006400u;
-  if (BITS == 4) {
-    float lo = 0.f, hi = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t w8 = w[i] >> 8;
-      lo = dot2(and_or(w[i], 0x000f000fu, kMagic), xr[4 * i + 0], lo);
-      hi = dot2(and_or(w[i], 0x00f000f0u, kMagic), xr[4 * i + 1], hi);
-      lo = dot2(and_or(w8, 0x000f000fu, kMagic), xr[4 * i + 2], lo);
-      hi = dot2(and_or(w8, 0x00f000f0u, kMagic), xr[4 * i + 3], hi);
-    }
-    return fmaf(hi, 0.0625f, lo) - corr;
-  } else {
-    float a1 = 0.f, a8 = 0.f, a64 = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
-      const uint32_t t = (w[i] & 0x0000ffffu) | ((w[i] << 1) & 0xffff0000u);
-      const uint32_t t9 = t >> 9;
-      a1 = dot2(and_or(t, 0x00070007u, kMagic), xr[5 * i + 0], a1);
-      a8 = dot2(and_or(t, 0x00380038u, kMagic), xr[5 * i + 1], a8);
-      a64 = dot2(and_or(t, 0x01c001c0u, kMagic), xr[5 * i + 2], a64);
-      a1 = dot2(and_or(t9, 0x00070007u, kMagic), xr[5 * i + 3], a1);
-      a8 = dot2(and_or(t9, 0x00380038u, kMagic), xr[5 * i + 4], a8);
-    }
-    return fmaf(a64, 0.015625f, fmaf(a8, 0.125f, a1)) - corr;
   }
 }
 
@@ -289,6 +225,25 @@ static hipError_t launch_nb(const GemvParams& p, int slots, int nb, int R, hipSt
   }
 }
 
+hipError_t launch_gemv_lds(const GemvParams& p_in, int bits, int nb, int slots, hipStream_t s) {
+  GemvParams p = p_in;
+  const int ch = bits == 4 ? 4 : 5;
+  // LDS chunk: whole K if it fits 64 KiB, else the largest multiple of 64 groups that does
+  int gc = (p.ng + 63) & ~63;
+  const int cap = (65536 / (nb * (ch * 16 + 4))) & ~63;
+  if (gc > cap) gc = cap < 64 ? 64 : cap;
+  p.gc = gc;
+  int R = options().gemv_rows_per_wave;
+  if (R != 1 && R != 2 && R != 4) {
+    // enough waves to cover the 256 CUs a few times over, else fewer rows per wave
+    const int64_t waves4 = (static_cast<int64_t>(p.N) + 3) / 4 * slots;
+    R = waves4 >= 4096 ? 4 : (waves4 >= 1024 ? 2 : 1);
+    if (nb > 4 && R > 2) R = 2;  // register budget
+  }
+  if (bits == 4) return launch_nb<4>(p, slots, nb, R, s);
+  return launch_nb<3>(p, slots, nb, R, s);
+}
+
 hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
   GemvParams p;
   p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.y = a.y;
@@ -301,23 +256,16 @@ hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
   p.expert_s_stride = a.N * p.ng;
   p.num_experts = static_cast<int>(a.num_experts);
   p.out_f32 = a.out_f32;
-  const int nb = static_cast<int>(a.M);
-  const int ch = a.bits == 4 ? 4 : 5;
-  // LDS chunk: whole K if it fits 64 KiB, else the largest multiple of 64 groups that does
-  int gc = (p.ng + 63) & ~63;
-  const int cap = (65536 / (nb * (ch * 16 + 4))) & ~63;
-  if (gc > cap) gc = cap < 64 ? 64 : cap;
-  p.gc = gc;
-  int R = options().gemv_rows_per_wave;
-  if (R != 1 && R != 2 && R != 4) {
-    // enough waves to cover the 256 CUs a few times over, else fewer rows per wave
-    const int64_t waves4 = (a.N + 3) / 4 * a.slots;
-    R = waves4 >= 4096 ? 4 : (waves4 >= 1024 ? 2 : 1);
-    if (nb > 4 && R > 2) R = 2;  // register budget
-  }
+  p.gc = 0;
   if (a.N == 0 || a.slots == 0) return hipSuccess;
-  if (a.bits == 4) return launch_nb<4>(p, static_cast<int>(a.slots), nb, R, s);
-  return launch_nb<3>(p, static_cast<int>(a.slots), nb, R, s);
+  const int nb = static_cast<int>(a.M);
+  const int slots = static_cast<int>(a.slots);
+  const int variant = options().gemv_variant;  // -1 auto, 0 LDS-staged kernel, 1 register kernel
+  if (variant != 0) {
+    const hipError_t e = launch_gemv_reg(p, a.bits, nb, slots, s);
+    if (e != hipErrorNotSupported) return e;
+  }
+  return launch_gemv_lds(p, a.bits, nb, slots, s);
 }
 
 }  // namespace gq

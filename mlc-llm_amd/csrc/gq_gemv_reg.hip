@@ -1,0 +1,300 @@
+// Decode GEMV, register-resident activations, persistent waves (the batch-1 workhorse).
+//
+// Same arithmetic as gq_gemv.hip (see there for the unpack trick); different data movement:
+//  * a lane is pinned to the quantisation groups {lane + 64*i, i < ITERS} of every row it
+//    visits, so its slice of x (ITERS * G halves, already in the pair order the masks produce)
+//    and the matching correction terms stay in VGPRs for the whole kernel;
+//  * x is read from global memory once per workgroup (staged through LDS with a single barrier
+//    at kernel start) rather than once per wave: with thousands of waves the re-reads of x
+//    through L2 would otherwise rival the weight stream itself;
+//  * a wave walks the row sets {w, w + W, w + 2W, ...} (R rows per set, W waves in the grid) and
+//    keeps the R * ITERS 128-bit loads of the next set in flight while it reduces the current
+//    one, so each lane always has a full set of loads outstanding;
+//  * the grid is sized to a few waves per SIMD (not one block per row block): fewer, longer
+//    lived waves stream HBM better than thousands of short ones.
+#include "gq_gemv_common.hpp"
+
+namespace gq {
+
+// x pairs of one group in the order the unpack masks produce them, from the natural-order halves.
+// v_perm_b32 picks the two 16-bit lanes directly: byte selectors 0-3 address S1, 4-7 address S0.
+template <int BITS>
+__device__ __forceinline__ float permute_group(const uint32_t* __restrict__ n /* G/2 natural pairs */,
+                                               uint32_t* __restrict__ xr /* G/2 permuted pairs */) {
+  constexpr uint32_t kLoLo = 0x05040100u;  // (lo16(S1), lo16(S0))
+  constexpr uint32_t kHiHi = 0x07060302u;  // (hi16(S1), hi16(S0))
+  constexpr uint32_t kLoHi = 0x07060100u;  // (lo16(S1), hi16(S0))
+  constexpr uint32_t kHiLo = 0x05040302u;  // (hi16(S1), lo16(S0))
+  float c = 0.f;
+  if (BITS == 4) {
+    // word w holds x[8w..8w+7] as pairs (0,1)(2,3)(4,5)(6,7); wanted (0,4)(1,5)(2,6)(3,7).
+    // Fields 1,3,5,7 come out of the mask times 16: their 1024 shrinks to 64 after rescaling.
+    const uint32_t c_lo = 0x64076407u;  // (1031, 1031)
+    const uint32_t c_hi = 0x54705470u;  // (71, 71)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      xr[4 * w + 0] = __builtin_amdgcn_perm(n[4 * w + 2], n[4 * w + 0], kLoLo);
+      xr[4 * w + 1] = __builtin_amdgcn_perm(n[4 * w + 2], n[4 * w + 0], kHiHi);
+      xr[4 * w + 2] = __builtin_amdgcn_perm(n[4 * w + 3], n[4 * w + 1], kLoLo);
+      xr[4 * w + 3] = __builtin_amdgcn_perm(n[4 * w + 3], n[4 * w + 1], kHiHi);
+      c = dot2(xr[4 * w + 0], c_lo, c);
+      c = dot2(xr[4 * w + 1], c_hi, c);
+      c = dot2(xr[4 * w + 2], c_lo, c);
+      c = dot2(xr[4 * w + 3], c_hi, c);
+    }
+  } else {
+    // word w holds x[10w..10w+9] as 5 natural pairs; wanted (j, j+5); pair j sits at mantissa
+    // bit 3*(j mod 3), so its 1024 becomes 1024, 128 or 16 after rescaling (+ m = 3).
+    const uint32_t c1 = 0x64036403u;   // (1027, 1027)
+    const uint32_t c8 = 0x58185818u;   // (131, 131)
+    const uint32_t c64 = 0x4cc04cc0u;  // (19, 19)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t* r = n + 5 * w;
+      xr[5 * w + 0] = __builtin_amdgcn_perm(r[2], r[0], kLoHi);
+      xr[5 * w + 1] = __builtin_amdgcn_perm(r[3], r[0], kHiLo);
+      xr[5 * w + 2] = __builtin_amdgcn_perm(r[3], r[1], kLoHi);
+      xr[5 * w + 3] = __builtin_amdgcn_perm(r[4], r[1], kHiLo);
+      xr[5 * w + 4] = __builtin_amdgcn_perm(r[4], r[2], kLoHi);
+      c = dot2(xr[5 * w + 0], c1, c);
+      c = dot2(xr[5 * w + 1], c8, c);
+      c = dot2(xr[5 * w + 2], c64, c);
+      c = dot2(xr[5 * w + 3], c1, c);
+      c = dot2(xr[5 * w + 4], c8, c);
+    }
+  }
+  return c;
+}
+
+template <int BITS, int NB, int R, int ITERS>
+__global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int nsets) {
+  using T = GemvTraits<BITS>;
+  constexpr int G = T::G;
+  constexpr int HP = G / 2;  // half pairs of x per group
+  // 16-byte x chunks each of the 256 threads stages: NB * ITERS * 64 groups * G/8 chunks / 256
+  constexpr int XS = (NB * ITERS * 64 * (G / 8) + 255) / 256;
+
+  extern __shared__ uint4 smem[];  // x as [NB][ng * G] halves, zero beyond K
+  const int kpad = p.ng * G;
+
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * 4;
+  const int slot = blockIdx.y;
+
+  const uint16_t* x = p.x + slot * p.x_slot_stride;
+  const uint32_t* qw = p.qw;
+  const uint16_t* qs = p.qs;
+  if (p.expert_ids != nullptr) {
+    int e = p.expert_ids[slot];
+    e = e < 0 ? 0 : (e >= p.num_experts ? p.num_experts - 1 : e);
+    qw += e * p.expert_w_stride;
+    qs += e * p.expert_s_stride;
+  }
+
+  // ---- x chunks go out first: waiting for them later must not wait for the weight loads,
+  //      and the load counter retires in issue order
+  const int chunks = NB * (kpad / 8);
+  const bool vec = (p.K & 7) == 0;
+  uint4 xv[XS];
+  bool xok[XS];
+#pragma unroll
+  for (int i = 0; i < XS; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    const int b = c / (kpad / 8);
+    const int k = (c - b * (kpad / 8)) * 8;
+    xok[i] = vec && c < chunks && k + 8 <= p.K;
+    // always a valid 16-byte load (x itself when the chunk is out of range); zeroed at store time
+    const uint16_t* src = xok[i] ? x + static_cast<int64_t>(b) * p.K + k : x;
+    xv[i] = *reinterpret_cast<const uint4*>(src);
+  }
+
+  // ---- this lane's groups (clamped so that every address is valid)
+  int gidx[ITERS];
+  bool gok[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int g = it * 64 + lane;
+    gok[it] = g < p.ng;
+    gidx[it] = gok[it] ? g : p.ng - 1;
+  }
+
+  // ---- weight / scale / bias loads of one row set.  Branch-free on purpose: the wait-count
+  //      insertion only keeps "the other buffer's loads may stay in flight" across the loop when
+  //      every path issues the same loads.  A set past the end reads one cached line instead.
+  uint4 wa[R][ITERS], wb[R][ITERS];
+  uint32_t sa[R][ITERS], sb[R][ITERS];  // fp16 bits, kept 32 bits wide so that the in-flight values are never re-packed
+  uint32_t ba = 0, bb = 0;
+  auto issue = [&](int set, uint4 (&wn)[R][ITERS], uint32_t (&sn)[R][ITERS], uint32_t& bn) {
+    const bool live = set < nsets;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int row = min(set * R + r, p.N - 1);  // rows past N are computed and dropped
+      const uint32_t* wr = qw + static_cast<int64_t>(row) * p.nw;
+      const uint16_t* sr = qs + static_cast<int64_t>(row) * p.ng;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        wn[r][it] = *reinterpret_cast<const uint4*>(live ? wr + 4 * gidx[it] : qw);
+        sn[r][it] = *(live ? sr + gidx[it] : qs);
+      }
+    }
+    // lane r carries the bias of row r of the set (read back with readlane at store time)
+    const int brow = min(set * R + min(lane, R - 1), p.N - 1);
+    bn = *((live && p.bias != nullptr) ? p.bias + brow : qs);
+  };
+  int set_a = gw, set_b = gw + nwaves;
+  issue(set_a, wa, sa, ba);
+  issue(set_b, wb, sb, bb);
+
+  // ---- stage x once per workgroup (zero beyond K), then one barrier
+  if (vec) {
+#pragma unroll
+    for (int i = 0; i < XS; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (c < chunks) smem[c] = xok[i] ? xv[i] : make_uint4(0, 0, 0, 0);
+    }
+  } else {  // K not a multiple of 8: rows of x are not 16-byte aligned, copy element-wise
+    uint16_t* xs16 = reinterpret_cast<uint16_t*>(smem);
+    for (int i = threadIdx.x; i < NB * kpad; i += 256) {
+      const int b = i / kpad, k = i - b * kpad;
+      xs16[i] = k < p.K ? x[static_cast<int64_t>(b) * p.K + k] : uint16_t(0);
+    }
+  }
+  __syncthreads();
+
+  // ---- this lane's x slice in pair order, and the correction terms
+  uint32_t xr[NB][ITERS][HP];
+  float corr[NB][ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      uint32_t nat[HP];
+#pragma unroll
+      for (int c = 0; c < G / 8; ++c) {
+        uint4 raw = smem[(b * kpad + gidx[it] * G) / 8 + c];
+        if (!gok[it]) raw = make_uint4(0, 0, 0, 0);
+        nat[4 * c + 0] = raw.x; nat[4 * c + 1] = raw.y; nat[4 * c + 2] = raw.z; nat[4 * c + 3] = raw.w;
+      }
+      corr[b][it] = permute_group<BITS>(nat, xr[b][it]);
+    }
+  }
+
+  // ---- persistent walk: reduce one set, then refill its registers with the set two strides on
+  auto reduce = [&](int cur, const uint4 (&wc)[R][ITERS], const uint32_t (&sc)[R][ITERS],
+                    uint32_t bias_bits) {
+    float acc[R][NB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        float a = 0.f;
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          const float sv = gok[it] ? h2f(static_cast<uint16_t>(sc[r][it])) : 0.f;  // lanes past the last group add nothing
+          a = fmaf(sv, group_dot<BITS>(wc[r][it], xr[b][it], corr[b][it]), a);
+        }
+        acc[r][b] = wave_sum_last(a);
+      }
+    const float bias_lane = p.bias != nullptr ? h2f(static_cast<uint16_t>(bias_bits)) : 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float bias = __builtin_bit_cast(
+          float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_lane), r));
+      const int row = cur * R + r;
+      if (lane == 63 && row < p.N) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          const float v = acc[r][b] + bias;
+          const int64_t oi = static_cast<int64_t>(slot + b) * p.N + row;  // slot > 0 only if NB == 1
+          if (p.out_f32) static_cast<float*>(p.y)[oi] = v;
+          else static_cast<uint16_t*>(p.y)[oi] = f2h(v);
+        }
+      }
+    }
+  };
+  while (set_a < nsets) {
+    reduce(set_a, wa, sa, ba);
+    set_a += 2 * nwaves;
+    issue(set_a, wa, sa, ba);
+    reduce(set_b, wb, sb, bb);  // past the end: rows >= N, nothing is stored
+    set_b += 2 * nwaves;
+    issue(set_b, wb, sb, bb);
+  }
+}
+
+template <int BITS, int NB, int R, int ITERS>
+static hipError_t launch_k(const GemvParams& p, int slots, int blocks, int nsets, hipStream_t s) {
+  const int threads = 256;
+  const size_t lds = static_cast<size_t>(NB) * p.ng * GemvTraits<BITS>::G * 2;
+  hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS>), dim3(blocks, slots), dim3(threads), lds,
+                     s, p, nsets);
+  return hipGetLastError();
+}
+
+template <int BITS, int NB, int R>
+static hipError_t launch_iters(const GemvParams& p, int slots, int iters, int blocks, int nsets,
+                               hipStream_t s) {
+  switch (iters) {
+    case 1: return launch_k<BITS, NB, R, 1>(p, slots, blocks, nsets, s);
+    case 2: return launch_k<BITS, NB, R, 2>(p, slots, blocks, nsets, s);
+    case 3: if constexpr (R * NB <= 2) return launch_k<BITS, NB, R, 3>(p, slots, blocks, nsets, s); break;
+    case 4: if constexpr (R * NB <= 2) return launch_k<BITS, NB, R, 4>(p, slots, blocks, nsets, s); break;
+    case 5: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 5>(p, slots, blocks, nsets, s); break;
+    case 6: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 6>(p, slots, blocks, nsets, s); break;
+    case 7: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 7>(p, slots, blocks, nsets, s); break;
+    case 8: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 8>(p, slots, blocks, nsets, s); break;
+    default: break;
+  }
+  return hipErrorNotSupported;
+}
+
+template <int BITS>
+static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_t s) {
+  const int iters = (p.ng + 63) / 64;
+  if (iters < 1 || iters > 8) return hipErrorNotSupported;
+  // register budget: R * ITERS loads in flight, NB * ITERS x slices resident
+  int rmax = iters <= 2 ? 4 : (iters <= 4 ? 2 : 1);
+  if (nb == 2) rmax = iters <= 2 ? 2 : (iters <= 4 ? 1 : 0);
+  if (nb > 2 || rmax == 0) return hipErrorNotSupported;
+  // Measured on MI355X (q4, batch 1): short K wants one row per set until the matrix is large
+  // (fine-grained sets hide the pipeline fill of a 5 us kernel), large matrices want 4 rows per
+  // set; long K is register-bound and runs one wave per SIMD.
+  const int64_t rows_total = static_cast<int64_t>(p.N) * slots;
+  int R = options().gemv_rows_per_wave;
+  if (R != 1 && R != 2 && R != 4) {
+    if (iters <= 2) R = rows_total >= 65536 ? 4 : (rows_total >= 16384 ? 2 : 1);
+    else R = 2;
+  }
+  if (R > rmax) R = rmax;
+  const int nsets = (p.N + R - 1) / R;
+  int waves;
+  if (options().gemv_split > 0) {
+    waves = options().gemv_split;
+  } else if (iters > 2) {
+    waves = 1024;
+  } else {
+    const int64_t half = static_cast<int64_t>(nsets) * slots / 2;  // about two sets per wave
+    waves = half <= 3072 ? static_cast<int>(half) : 2048;
+    if (waves < 1024) waves = 1024;
+  }
+  waves = (waves + slots - 1) / slots;  // grid.y = slots
+  if (waves < 4) waves = 4;
+  const int rounds = (nsets + waves - 1) / waves;
+  const int blocks = ((nsets + rounds - 1) / rounds + 3) / 4;  // even share of sets per wave
+  if (nb == 1) {
+    if (R == 4) return launch_iters<BITS, 1, 4>(p, slots, iters, blocks, nsets, s);
+    if (R == 2) return launch_iters<BITS, 1, 2>(p, slots, iters, blocks, nsets, s);
+    return launch_iters<BITS, 1, 1>(p, slots, iters, blocks, nsets, s);
+  }
+  if (R == 2) return launch_iters<BITS, 2, 2>(p, slots, iters, blocks, nsets, s);
+  return launch_iters<BITS, 2, 1>(p, slots, iters, blocks, nsets, s);
+}
+
+hipError_t launch_gemv_reg(const GemvParams& p, int bits, int nb, int slots, hipStream_t s) {
+  if (p.ng == 0) return hipErrorNotSupported;
+  if (static_cast<int64_t>(nb) * p.ng * (bits == 4 ? 32 : 40) * 2 > 65536) return hipErrorNotSupported;
+  return bits == 4 ? launch_bits<4>(p, nb, slots, s) : launch_bits<3>(p, nb, slots, s);
+}
+
+}  // namespace gq

@@ -11,7 +11,7 @@ struct Options {
   int gemv_rows_per_wave = -1;  // -1: heuristic
   int gemv_variant = -1;        // -1: heuristic, 0: dot2 kernel, 1: mfma kernel
   int gemm_variant = -1;
-  int gemv_split = -1;
+  int gemv_split = -1;        // total waves of the persistent GEMV grid
 };
 Options& options();
 
@@ -44,6 +44,9 @@ struct GemmArgs {
   int bits, group_size, out_f32;
 };
 hipError_t launch_gemm(const GemmArgs& a, hipStream_t s);
+// MFMA kernel for few activation rows per segment (q4 only; hipErrorNotSupported otherwise).
+// rows_max bounds the rows of any one segment.
+hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s);
 
 hipError_t launch_quantize(const uint16_t* w, int64_t rows, int64_t K, int bits, int group_size,
                            int round_mode, uint32_t* qw, uint16_t* qs, hipStream_t s);
