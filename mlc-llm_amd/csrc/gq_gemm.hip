@@ -17,72 +17,12 @@
 //  * each wave feeds v_mfma_f32_32x32x16_f16 from 16-byte LDS fragments, fp32 accumulators;
 //  * global loads of tile t+1 are issued before the MFMAs of tile t, dequantisation and the LDS
 //    stores of t+1 after them (two LDS stages, one barrier per tile).
-#include "gq_common.hpp"
-#include "gq_internal.hpp"
+#include "gq_gemm_common.hpp"
 
 namespace gq {
 
-template <int BITS>
-struct GemmTraits;
-template <>
-struct GemmTraits<4> {
-  static constexpr int G = 32;
-};
-template <>
-struct GemmTraits<3> {
-  static constexpr int G = 40;
-};
-
-struct GemmParams {
-  const uint16_t* x;
-  const uint32_t* qw;
-  const uint16_t* qs;
-  const uint16_t* bias;
-  void* y;
-  const void* indptr;
-  int64_t expert_w_stride, expert_s_stride;
-  int rows, N, K, ng, nw;
-  int num_experts;
-  int out_f32, indptr_i64;
-};
-
-// One group (4 storage words) -> G halves in natural k order, (q - m) * s with fp16 rounding.
-template <int BITS>
-__device__ __forceinline__ void dequant_group(const uint4 w4, const uint16_t scale_bits,
-                                              uint32_t* __restrict__ out /* G/2 half pairs */) {
-  constexpr uint32_t kMagic = 0x64006400u;  // 1024.0 in both halves
-  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
-  const _Float16 s = __builtin_bit_cast(_Float16, scale_bits);
-  const half2_t s2 = {s, s};
-  if (BITS == 4) {
-    const half2_t off = {static_cast<_Float16>(-1031.0f), static_cast<_Float16>(-1031.0f)};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t t1 = w[i] >> 4;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // byte j of w -> low half (field 2j in its low nibble), byte j of w>>4 -> high half
-        const uint32_t sel = 0x0c000c00u | ((4u + j) << 16) | static_cast<uint32_t>(j);
-        const uint32_t r = and_or(__builtin_amdgcn_perm(t1, w[i], sel), 0x000f000fu, kMagic);
-        out[4 * i + j] = as_u32((as_half2(r) + off) * s2);
-      }
-    }
-  } else {
-    const half2_t off = {static_cast<_Float16>(-1027.0f), static_cast<_Float16>(-1027.0f)};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int j = 0; j < 5; ++j) {
-        const uint32_t t = w[i] >> (6 * j);
-        const uint32_t r = and_or(t << 13, 0x00070000u, and_or(t, 0x00000007u, kMagic));
-        out[5 * i + j] = as_u32((as_half2(r) + off) * s2);
-      }
-    }
-  }
-}
-
 template <int BITS, int BM, int BN, int WM, int WN>
-__global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
+__global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_kernel(const GemmParams p) {
   using T = GemmTraits<BITS>;
   constexpr int G = T::G;
   constexpr int BK = 2 * G;            // 64 | 80
@@ -90,11 +30,12 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   constexpr int CPR = BK / 8;          // 16-byte chunks per tile row
   constexpr int LDA = BK + 8;          // padded row, in halves
   constexpr int WAVES_N = BN / WN;
-  static_assert((BM / WM) * (BN / WN) == 4, "4 waves per workgroup");
+  constexpr int NT = 64 * (BM / WM) * (BN / WN);  // threads per workgroup (4 or 8 waves)
+  static_assert(NT == 256 || NT == 512, "4 or 8 waves per workgroup");
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int A_CHUNKS = BM * CPR / 256;  // 16-byte chunks of x per thread per tile
-  constexpr int W_GROUPS = BN * 2 / 256;    // groups of W per thread per tile
-  static_assert(BM * CPR % 256 == 0 && BN * 2 % 256 == 0, "tile / thread mismatch");
+  constexpr int A_CHUNKS = BM * CPR / NT;  // 16-byte chunks of x per thread per tile
+  constexpr int W_GROUPS = BN * 2 / NT;    // groups of W per thread per tile
+  static_assert(BM * CPR % NT == 0 && BN * 2 % NT == 0, "tile / thread mismatch");
 
   extern __shared__ uint4 smem[];
   uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
@@ -107,34 +48,8 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
   const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
 
   // ---- which rows / which expert does this workgroup own
-  int seg_lo = 0, seg_hi = p.rows, mt = blockIdx.y, expert = 0;
-  if (p.indptr != nullptr) {
-    int t = blockIdx.y;
-    bool found = false;
-    for (int e = 0; e < p.num_experts; ++e) {
-      int64_t lo, hi;
-      if (p.indptr_i64) {
-        lo = static_cast<const int64_t*>(p.indptr)[e];
-        hi = static_cast<const int64_t*>(p.indptr)[e + 1];
-      } else {
-        lo = static_cast<const int32_t*>(p.indptr)[e];
-        hi = static_cast<const int32_t*>(p.indptr)[e + 1];
-      }
-      lo = lo < 0 ? 0 : (lo > p.rows ? p.rows : lo);  // a corrupt indptr must not leave the tensors
-      hi = hi < lo ? lo : (hi > p.rows ? p.rows : hi);
-      const int tiles = static_cast<int>((hi - lo + BM - 1) / BM);
-      if (t < tiles) {
-        seg_lo = static_cast<int>(lo);
-        seg_hi = static_cast<int>(hi);
-        mt = t;
-        expert = e;
-        found = true;
-        break;
-      }
-      t -= tiles;
-    }
-    if (!found) return;  // uniform over the workgroup
-  }
+  int seg_lo, seg_hi, mt, expert;
+  if (!locate_tile<BM>(p, blockIdx.y, seg_lo, seg_hi, mt, expert)) return;  // uniform
   const int m0 = seg_lo + mt * BM;
   if (m0 >= seg_hi) return;
   const int n0 = blockIdx.x * BN;
@@ -158,7 +73,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
     const int k_base = kt * BK;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
-      const int idx = tid + 256 * i;
+      const int idx = tid + NT * i;
       const int r = idx / CPR, c = idx - r * CPR;
       const int row = m0 + r, k = k_base + 8 * c;
       uint4 v = make_uint4(0, 0, 0, 0);
@@ -178,7 +93,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
     }
 #pragma unroll
     for (int i = 0; i < W_GROUPS; ++i) {
-      const int idx = tid + 256 * i;
+      const int idx = tid + NT * i;
       const int r = idx >> 1, gsel = idx & 1;
       const int row = min(n0 + r, p.N - 1);
       const int g = 2 * kt + gsel;
@@ -197,13 +112,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
     uint16_t* wt = w_tile(s);
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
-      const int idx = tid + 256 * i;
+      const int idx = tid + NT * i;
       const int r = idx / CPR, c = idx - r * CPR;
       *reinterpret_cast<uint4*>(at + r * LDA + 8 * c) = a_reg[i];
     }
 #pragma unroll
     for (int i = 0; i < W_GROUPS; ++i) {
-      const int idx = tid + 256 * i;
+      const int idx = tid + NT * i;
       const int r = idx >> 1, gsel = idx & 1;
       uint32_t d[G / 2];
       dequant_group<BITS>(w_reg[i], s_reg[i], d);
@@ -280,7 +195,7 @@ static hipError_t launch_cfg(const GemmParams& p, hipStream_t s) {
   }
   const int m_tiles = p.indptr ? (p.rows + BM - 1) / BM + p.num_experts : (p.rows + BM - 1) / BM;
   const dim3 grid((p.N + BN - 1) / BN, m_tiles);
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, p);
+  hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
   return hipGetLastError();
 }
 
@@ -296,7 +211,19 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   p.num_experts = static_cast<int>(a.num_experts);
   p.out_f32 = a.out_f32;
   if (a.rows == 0 || a.N == 0) return hipSuccess;
-  if (a.bits == 4) return launch_cfg<4, 128, 128, 64, 64>(p, s);
+  const int variant = options().gemm_variant;
+  if (variant != 3 && variant != 4 && variant != 5) {
+    const hipError_t e = launch_gemm_pipe(p, a.bits, s);
+    if (e != hipErrorNotSupported) return e;
+  }
+  if (a.bits == 4) {
+    // big tile (256 x 256, 128 x 128 per wave) once there are enough tiles to fill 256 CUs
+    const int64_t big_tiles = ((a.rows + 255) / 256) * ((a.N + 255) / 256);
+    const bool big = variant == 4 ? true : (variant == 3 ? false : (a.indptr == nullptr && big_tiles >= 128));
+    if (variant == 5) return launch_cfg<4, 256, 256, 128, 128>(p, s);
+    if (big) return launch_cfg<4, 256, 256, 128, 64>(p, s);
+    return launch_cfg<4, 128, 128, 64, 64>(p, s);
+  }
   return launch_cfg<3, 128, 128, 64, 64>(p, s);
 }
 

@@ -1,0 +1,118 @@
+// Pieces shared by the MFMA GEMM kernels: scheme traits, kernel parameters, the segment walk of
+// the grouped (MoE) form and the in-register dequantisation of one group.
+#pragma once
+
+#include "gq_common.hpp"
+#include "gq_internal.hpp"
+
+namespace gq {
+
+template <int BITS>
+struct GemmTraits;
+template <>
+struct GemmTraits<4> {
+  static constexpr int G = 32;
+};
+template <>
+struct GemmTraits<3> {
+  static constexpr int G = 40;
+};
+
+struct GemmParams {
+  const uint16_t* x;
+  const uint32_t* qw;
+  const uint16_t* qs;
+  const uint16_t* bias;
+  void* y;
+  const void* indptr;
+  int64_t expert_w_stride, expert_s_stride;
+  int rows, N, K, ng, nw;
+  int num_experts;
+  int out_f32, indptr_i64;
+};
+
+// One group (4 storage words) -> G halves in natural k order, (q - m) * s with fp16 rounding.
+template <int BITS>
+__device__ __forceinline__ void dequant_group(const uint4 w4, const uint16_t scale_bits,
+                                              uint32_t* __restrict__ out /* G/2 half pairs */) {
+  constexpr uint32_t kMagic = 0x64006400u;  // 1024.0 in both halves
+  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+  const _Float16 s = __builtin_bit_cast(_Float16, scale_bits);
+  const half2_t s2 = {s, s};
+  if (BITS == 4) {
+    const half2_t off = {static_cast<_Float16>(-1031.0f), static_cast<_Float16>(-1031.0f)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t t1 = w[i] >> 4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // byte j of w -> low half (field 2j in its low nibble), byte j of w>>4 -> high half
+        const uint32_t sel = 0x0c000c00u | ((4u + j) << 16) | static_cast<uint32_t>(j);
+        const uint32_t r = and_or(__builtin_amdgcn_perm(t1, w[i], sel), 0x000f000fu, kMagic);
+        out[4 * i + j] = as_u32((as_half2(r) + off) * s2);
+      }
+    }
+  } else {
+    const half2_t off = {static_cast<_Float16>(-1027.0f), static_cast<_Float16>(-1027.0f)};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 5; ++j) {
+        const uint32_t t = w[i] >> (6 * j);
+        const uint32_t r = and_or(t << 13, 0x00070000u, and_or(t, 0x00000007u, kMagic));
+        out[5 * i + j] = as_u32((as_half2(r) + off) * s2);
+      }
+    }
+  }
+}
+
+
+// One q4 storage word -> 8 halves in natural k order (4 half pairs), (q - 7) * s.
+__device__ __forceinline__ void dequant_word4(const uint32_t w, const uint16_t scale_bits,
+                                              uint32_t* __restrict__ out) {
+  constexpr uint32_t kMagic = 0x64006400u;
+  const _Float16 s = __builtin_bit_cast(_Float16, scale_bits);
+  const half2_t s2 = {s, s};
+  const half2_t off = {static_cast<_Float16>(-1031.0f), static_cast<_Float16>(-1031.0f)};
+  const uint32_t t1 = w >> 4;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint32_t sel = 0x0c000c00u | ((4u + j) << 16) | static_cast<uint32_t>(j);
+    const uint32_t r = and_or(__builtin_amdgcn_perm(t1, w, sel), 0x000f000fu, kMagic);
+    out[j] = as_u32((as_half2(r) + off) * s2);
+  }
+}
+
+// Which activation rows [seg_lo, seg_hi) and which expert the m-tile `t` of a launch belongs to.
+// Plain linear: one segment.  Grouped: walk indptr (python/mlc_llm/op/moe_matmul.py:653-679 of
+// the reference does the same walk per tile).  Returns false when the tile does not exist.
+template <int BM>
+__device__ __forceinline__ bool locate_tile(const GemmParams& p, int t, int& seg_lo, int& seg_hi,
+                                            int& mt, int& expert) {
+  seg_lo = 0; seg_hi = p.rows; mt = t; expert = 0;
+  if (p.indptr == nullptr) return t * BM < p.rows;
+  for (int e = 0; e < p.num_experts; ++e) {
+    int64_t lo, hi;
+    if (p.indptr_i64) {
+      lo = static_cast<const int64_t*>(p.indptr)[e];
+      hi = static_cast<const int64_t*>(p.indptr)[e + 1];
+    } else {
+      lo = static_cast<const int32_t*>(p.indptr)[e];
+      hi = static_cast<const int32_t*>(p.indptr)[e + 1];
+    }
+    lo = lo < 0 ? 0 : (lo > p.rows ? p.rows : lo);  // a corrupt indptr must not leave the tensors
+    hi = hi < lo ? lo : (hi > p.rows ? p.rows : hi);
+    const int tiles = static_cast<int>((hi - lo + BM - 1) / BM);
+    if (t < tiles) {
+      seg_lo = static_cast<int>(lo); seg_hi = static_cast<int>(hi); mt = t; expert = e;
+      return true;
+    }
+    t -= tiles;
+  }
+  return false;
+}
+
+// software-pipelined kernel family (needs K % 8 == 0); hipErrorNotSupported otherwise
+hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s);
+
+}  // namespace gq

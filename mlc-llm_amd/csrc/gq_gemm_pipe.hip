@@ -1,0 +1,245 @@
+// Prefill GEMM / MoE grouped GEMM, software-pipelined form (the one that normally runs).
+//
+// Same tiling and LDS layout as gq_gemm.hip; what differs is how latency is hidden:
+//  * global loads run TWO K tiles ahead of the MFMAs (register ping-pong), because one tile of
+//    MFMA work (~0.4 us) is shorter than a trip to L2 / HBM;
+//  * every load is branch-free (addresses are clamped, out-of-range data is zeroed when it is
+//    written to LDS) so that the compiler's wait-count insertion can leave the newest loads in
+//    flight instead of draining the queue at every join;
+//  * the MFMA fragments of k-step s+1 are read from LDS before the MFMAs of step s are issued.
+// Requires K % 8 == 0 (16-byte aligned activation rows); other K take the kernel in gq_gemm.hip.
+#include "gq_gemm_common.hpp"
+
+namespace gq {
+
+template <int BITS, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(const GemmParams p) {
+  using T = GemmTraits<BITS>;
+  constexpr int G = T::G;
+  constexpr int BK = 2 * G;        // 64 | 80
+  constexpr int KSTEPS = BK / 16;  // MFMA k = 16
+  constexpr int CPR = BK / 8;      // 16-byte chunks per tile row
+  constexpr int LDA = BK + 8;      // padded row, in halves
+  constexpr int WAVES_N = BN / WN;
+  constexpr int NT = 64 * (BM / WM) * (BN / WN);
+  static_assert(NT == 256 || NT == 512, "4 or 8 waves per workgroup");
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int A_CHUNKS = BM * CPR / NT;
+  constexpr int W_GROUPS = BN * 2 / NT;
+  static_assert(BM * CPR % NT == 0 && BN * 2 % NT == 0, "tile / thread mismatch");
+
+  extern __shared__ uint4 smem[];
+  uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
+  auto a_tile = [&](int s) { return lds + s * (BM + BN) * LDA; };
+  auto w_tile = [&](int s) { return lds + s * (BM + BN) * LDA + BM * LDA; };
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+
+  int seg_lo, seg_hi, mt, expert;
+  if (!locate_tile<BM>(p, blockIdx.y, seg_lo, seg_hi, mt, expert)) return;  // uniform
+  const int m0 = seg_lo + mt * BM;
+  const int n0 = blockIdx.x * BN;
+  const uint32_t* qw = p.qw + expert * p.expert_w_stride;
+  const uint16_t* qs = p.qs + expert * p.expert_s_stride;
+
+  // ---- per-thread load slots: where each 16-byte chunk of x / each group of W comes from
+  const uint16_t* a_src[A_CHUNKS];  // chunk address at K tile 0 (row clamped into the segment)
+  bool a_row_ok[A_CHUNKS];
+  int a_k[A_CHUNKS];                // k offset of the chunk inside a tile
+  int a_dst[A_CHUNKS];              // offset (halves) inside the LDS tile
+#pragma unroll
+  for (int i = 0; i < A_CHUNKS; ++i) {
+    const int idx = tid + NT * i;
+    const int r = idx / CPR, c = idx - r * CPR;
+    a_row_ok[i] = m0 + r < seg_hi;
+    a_k[i] = 8 * c;
+    a_src[i] = p.x + static_cast<int64_t>(a_row_ok[i] ? m0 + r : m0) * p.K + 8 * c;
+    a_dst[i] = r * LDA + 8 * c;
+  }
+  const uint32_t* w_src[W_GROUPS];
+  const uint16_t* s_src[W_GROUPS];
+  int w_g[W_GROUPS];  // group index at K tile 0
+  int w_dst[W_GROUPS];
+#pragma unroll
+  for (int i = 0; i < W_GROUPS; ++i) {
+    const int idx = tid + NT * i;
+    const int r = idx >> 1, gsel = idx & 1;
+    const int row = min(n0 + r, p.N - 1);  // rows past N are computed and dropped
+    w_src[i] = qw + static_cast<int64_t>(row) * p.nw;
+    s_src[i] = qs + static_cast<int64_t>(row) * p.ng;
+    w_g[i] = gsel;
+    w_dst[i] = r * LDA + gsel * G;
+  }
+
+  struct Stage {
+    uint4 a[A_CHUNKS];
+    uint4 w[W_GROUPS];
+    uint32_t s[W_GROUPS];  // fp16 scale bits (32 bits wide on purpose: in flight, never re-packed)
+  };
+  Stage r0, r1;
+
+  // K tile kt into registers.  Always valid addresses; validity is re-derived at store time.
+  auto load_tile = [&](int kt, Stage& st) {
+    const int k_base = kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const bool ok = k_base + a_k[i] < p.K;  // K % 8 == 0: a chunk is entirely inside or outside
+      st.a[i] = *reinterpret_cast<const uint4*>(ok ? a_src[i] + k_base : a_src[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < W_GROUPS; ++i) {
+      const int g = 2 * kt + w_g[i];
+      const int gc = g < p.ng ? g : 0;
+      st.w[i] = *reinterpret_cast<const uint4*>(w_src[i] + 4 * gc);
+      st.s[i] = s_src[i][gc];
+    }
+  };
+  // One of KSTEPS slices of "tile kt: registers -> LDS stage s".  The slices are issued between the
+  // MFMA k-steps of the tile being multiplied, so that dequantisation (VALU) and the LDS stores
+  // run in the shadow of the matrix pipe instead of after it.
+  auto store_part = [&](int kt, const Stage& st, int s, int part) {
+    uint16_t* at = a_tile(s);
+    uint16_t* wt = w_tile(s);
+    const int k_base = kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      if (i % KSTEPS != part) continue;
+      const bool ok = a_row_ok[i] && (k_base + a_k[i] < p.K);
+      *reinterpret_cast<uint4*>(at + a_dst[i]) = ok ? st.a[i] : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < W_GROUPS; ++i) {
+      const bool ok = 2 * kt + w_g[i] < p.ng;
+      // a group past the end gets scale +0.0: every value becomes (q - m) * 0 = +-0
+      const uint16_t sb = ok ? static_cast<uint16_t>(st.s[i]) : uint16_t(0);
+      uint4* dst = reinterpret_cast<uint4*>(wt + w_dst[i]);
+      if (BITS == 4) {
+        // word `part` of the group -> 8 halves = one 16-byte chunk
+        const uint32_t w4[4] = {st.w[i].x, st.w[i].y, st.w[i].z, st.w[i].w};
+        uint32_t d[4];
+        dequant_word4(w4[part], sb, d);
+        dst[part] = make_uint4(d[0], d[1], d[2], d[3]);
+      } else if (part == 0) {
+        uint32_t d[G / 2];
+        dequant_group<BITS>(st.w[i], sb, d);
+#pragma unroll
+        for (int c = 0; c < G / 8; ++c) dst[c] = make_uint4(d[4 * c], d[4 * c + 1], d[4 * c + 2], d[4 * c + 3]);
+      }
+    }
+  };
+  auto store_tile = [&](int kt, const Stage& st, int s) {
+#pragma unroll
+    for (int part = 0; part < KSTEPS; ++part) store_part(kt, st, s, part);
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int frag_row = lane & 31, frag_k = 8 * (lane >> 5);
+  // MFMAs of the tile in stage s; slice ks of the next tile's store is issued after k-step ks
+  auto mfma_tile = [&](int s, int kt_store, const Stage& st_store) {
+    const uint16_t* at = a_tile(s) + (wm0 + frag_row) * LDA + frag_k;
+    const uint16_t* wt = w_tile(s) + (wn0 + frag_row) * LDA + frag_k;
+    half8_t af[2][TM], bf[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < KSTEPS) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          af[nxt][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA + (ks + 1) * 16);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          bf[nxt][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA + (ks + 1) * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+      store_part(kt_store, st_store, s ^ 1, ks);
+      __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
+    }
+  };
+
+  // ---- pipeline: tile t in LDS stage t&1, tile t+1 in registers, tile t+2 in flight
+  const int nk = (p.ng + 1) / 2;
+  load_tile(0, r0);
+  load_tile(1, r1);
+  store_tile(0, r0, 0);
+  load_tile(2, r0);
+  __syncthreads();
+  // (registers of tile t+2 are overwritten only after tile t+1 has left them for LDS, so the
+  //  refill of a register stage is issued right after the MFMA/store block that drains it)
+  for (int kt = 0; kt < nk; kt += 2) {
+    mfma_tile(0, kt + 1, r1);  // a tile past the end is stored as zeros and adds nothing
+    load_tile(kt + 3, r1);
+    __syncthreads();
+    mfma_tile(1, kt + 2, r0);
+    load_tile(kt + 4, r0);
+    __syncthreads();
+  }
+
+  // ---- epilogue: D[i][j] of a 32x32 tile sits in lane (j + 32*((i/4)%2)), register 4*(i/8) + i%4
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn0 + j * 32 + (lane & 31);
+      const float b = (p.bias != nullptr && col < p.N) ? h2f(p.bias[col]) : 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < seg_hi && col < p.N) {
+          const float v = acc[i][j][r] + b;
+          const int64_t o = static_cast<int64_t>(row) * p.N + col;
+          if (p.out_f32) static_cast<float*>(p.y)[o] = v;
+          else static_cast<uint16_t*>(p.y)[o] = f2h(v);
+        }
+      }
+    }
+  }
+}
+
+template <int BITS, int BM, int BN, int WM, int WN>
+static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
+  constexpr int BK = 2 * GemmTraits<BITS>::G;
+  constexpr int LDA = BK + 8;
+  constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
+  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN>;
+  if (lds > 65536) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(lds));
+    if (e != hipSuccess) return e;
+  }
+  const int m_tiles = p.indptr ? (p.rows + BM - 1) / BM + p.num_experts : (p.rows + BM - 1) / BM;
+  const dim3 grid((p.N + BN - 1) / BN, m_tiles);
+  hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
+  if ((p.K & 7) != 0 || p.ng == 0) return hipErrorNotSupported;
+  const int variant = options().gemm_variant;
+  if (bits == 4) {
+    const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
+    const bool big = variant == 7 ? true : (variant == 6 ? false : (p.indptr == nullptr && big_tiles >= 200));
+    if (big) return launch_pipe_cfg<4, 256, 256, 128, 64>(p, s);
+    return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
+  }
+  return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
+}
+
+}  // namespace gq
