@@ -58,6 +58,9 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--skip-extra", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 256 MiB device copy (known bytes) so that a rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE run of this command can scale its counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.stderr.write("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1\n")
@@ -166,8 +169,15 @@ def main() -> int:
     if os.path.exists(tpath):
         with open(tpath, encoding="utf-8") as f:
             traffic = json.load(f).get("hbm_bytes_per_launch")
+    if args.calibrate_copy:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).fill_(7)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     roofline = {
-        "bound": "hbm", "kernel": "gq::gemv_dot2_kernel<4,1,R> on gate_up 28672x4096, batch 1",
+        "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2> (gate_up 28672x4096, batch 1)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
         "bytes_per_launch": gu_bytes, "us_per_launch": round(us_gate_up, 3),
@@ -210,7 +220,82 @@ def main() -> int:
                                     "frac_mfma": round(tf / MFMA_F16_PEAK_TFLOPS, 3)}
             del ym
         extra["prefill_gemm"] = gemm
+        for m2 in (256, 8192):  # the other two prefill sizes, on the largest per-layer shape
+            n, k = SHAPES["gate_up"]
+            xm2 = torch.randn((m2, k), generator=gx, device=dev).half()
+            ym2 = torch.empty((m2, n), dtype=torch.float16, device=dev)
+            qw, qs = layers[0]["gate_up"]
+            ms = timed(lambda: ops.linear(xm2, qw, qs, BITS, G, None, torch.float16, ym2), 5, 2, False)
+            tf = 2.0 * m2 * n * k / (ms * 1e-3) / 1e12
+            gemm[f"gate_up_m{m2}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
+                                      "frac_mfma": round(tf / MFMA_F16_PEAK_TFLOPS, 3)}
+            del xm2, ym2
+        del xm
         extra["decode_tokens_per_s_linear_only"] = round(1e3 / ms_step, 1)
+
+        # what a plain library streaming read reaches on this box (context for the HBM fractions):
+        # torch's int32 sum over four distinct 1 GiB buffers
+        bufs = [torch.ones(256 * 1024 * 1024, dtype=torch.int32, device=dev) for _ in range(4)]
+
+        def read_sweep():
+            for t in bufs:
+                t.sum()
+        ms = timed(read_sweep, 3, 1, False) / len(bufs)
+        extra["stream_read_reference"] = {"what": "torch.sum over 1 GiB int32", "GB/s": round(2**30 / (ms * 1e-3) / 1e9, 1)}
+        del bufs
+
+        # q3f16_1 decode GEMV at Llama-2-7B shapes, batch 1 (BASELINE configs[3])
+        q3 = {}
+        for name, (n, k) in {"qkv": (12288, 4096), "o_proj": (4096, 4096), "gate_up": (22016, 4096),
+                             "down": (4096, 11008)}.items():
+            ng3 = -(-k // 40)
+            copies = max(2, min(32, int(1.2e9 // (n * ng3 * 18))))
+            ws = []
+            for c in range(copies):
+                g = torch.Generator(device=dev).manual_seed(5000 + c)
+                w = (torch.randn((n, k), generator=g, device=dev) * 0.02).half()
+                ws.append(ops.quantize(w, 3, 40))
+                del w
+            x3 = torch.randn((1, k), generator=gx, device=dev).half()
+            y3 = torch.empty((1, n), dtype=torch.float16, device=dev)
+
+            def sweep3():
+                for qw, qs in ws:
+                    ops.linear(x3, qw, qs, 3, 40, None, torch.float16, y3)
+            us = timed(sweep3, 5, 1, use_graph) * 1e3 / copies
+            nbytes = n * 4 * ng3 * 4 + n * ng3 * 2 + k * 2 + n * 2
+            q3[name] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                        "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)}
+            del ws
+        extra["q3f16_1_gemv_b1"] = q3
+
+        # q4f16_1 Mixtral-8x7B MoE layer (BASELINE configs[4]): 8 experts, top-2, T in {1, 16, 512}
+        from mlc_llm_amd import QUANTIZATION
+        from mlc_llm_amd.nn import MixtralMoE
+
+        moe = MixtralMoE(4096, 14336, 8, 2, QUANTIZATION["q4f16_1"], device=dev)
+        for e in range(8):
+            g = torch.Generator(device=dev).manual_seed(7000 + e)
+            w13 = (torch.randn((28672, 4096), generator=g, device=dev) * 0.02).half()
+            moe.e1_e3.q_weight.data[e], moe.e1_e3.q_scale.data[e] = ops.quantize(w13, BITS, G)
+            w2 = (torch.randn((4096, 14336), generator=g, device=dev) * 0.02).half()
+            moe.e2.q_weight.data[e], moe.e2.q_scale.data[e] = ops.quantize(w2, BITS, G)
+            del w13, w2
+        g2 = torch.Generator(device=dev).manual_seed(2)
+        moe_res = {}
+        for t in (1, 16, 512):
+            xt = torch.randn((1, t, 4096), generator=gx, device=dev).half()
+            logits = torch.randn((t, 8), generator=g2, device=dev).half()
+            ms = timed(lambda: moe(xt, logits), 5, 2, False)
+            ids = ops.gating_softmax_topk(logits, 2)[1]
+            distinct = int(torch.unique(ids).numel())
+            wbytes = distinct * 99_090_432
+            flops = 2.0 * t * 2 * (28672 * 4096 + 4096 * 14336)
+            moe_res[f"T{t}"] = {"us": round(ms * 1e3, 1), "experts_touched": distinct,
+                                "weight_GB/s": round(wbytes / (ms * 1e-3) / 1e9, 1),
+                                "TFLOP/s": round(flops / (ms * 1e-3) / 1e12, 2)}
+        extra["mixtral_moe_layer"] = moe_res
+        del moe
 
     # ---------------------------------------------------------------- CPU baseline (bounded sample)
     cpu = None

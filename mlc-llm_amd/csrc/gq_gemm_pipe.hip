@@ -235,7 +235,7 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   const int variant = options().gemm_variant;
   if (bits == 4) {
     const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
-    const bool big = variant == 7 ? true : (variant == 6 ? false : (p.indptr == nullptr && big_tiles >= 200));
+    const bool big = variant == 7 ? true : (variant == 6 ? false : (p.indptr == nullptr && big_tiles >= 160));
     if (big) return launch_pipe_cfg<4, 256, 256, 128, 64>(p, s);
     return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
   }

@@ -1,0 +1,126 @@
+// TVM-FFI adapter: registers the C ABI of include/mi355gq.h as global packed functions, so that
+// a Relax module can reach the kernels through
+//     R.call_dps_packed("mlc.gq.linear", (x, q_weight, q_scale, bits, group_size), out_sinfo=...)
+// the same way the reference reaches "fastertransformer.gemm_fp16_int"
+// (python/mlc_llm/op/ft_gemm.py:72-92) or "cutlass.group_gemm" (op/cutlass.py:71-77).
+// Registration follows the reference's own idiom (cpp/multi_gpu/builtin.cc:89-94).
+//
+// NOT COMPILED IN THIS TREE BY DEFAULT: build.py adds this file only when the `tvm_ffi` Python
+// package (which ships the tvm/ffi headers) is importable.  The container this library was
+// developed in has no TVM, so this file has never been compiled; it is the binding a maintainer
+// adds, kept next to the code it binds.  Everything it calls is the verified C ABI.
+//
+// DPS convention: the destination tensor(s) come last.  Tensors arrive as DLTensor views; ints as
+// int64.  Errors of the C ABI are rethrown as TVM errors carrying mi355gq_last_error().
+#include <tvm/ffi/container/tensor.h>
+#include <tvm/ffi/error.h>
+#include <tvm/ffi/extra/c_env_api.h>
+#include <tvm/ffi/function.h>
+#include <tvm/ffi/optional.h>
+#include <tvm/ffi/reflection/registry.h>
+
+#include "../../include/mi355gq.h"
+
+namespace mlc {
+namespace llm {
+namespace gq {
+
+using tvm::ffi::Optional;
+using tvm::ffi::TensorView;
+
+namespace {
+
+inline void* Ptr(const TensorView& t) {
+  return static_cast<char*>(t.data_ptr()) + t.byte_offset();
+}
+
+inline void* StreamOf(const TensorView& t) {
+  const DLDevice dev = t.device();
+  TVM_FFI_ICHECK(dev.device_type == kDLROCM) << "mlc.gq.*: tensors must live on a ROCm device";
+  return TVMFFIEnvGetStream(dev.device_type, dev.device_id);
+}
+
+inline void Check(int rc, const char* what) {
+  if (rc != MI355GQ_OK) TVM_FFI_THROW(RuntimeError) << what << ": " << mi355gq_last_error();
+}
+
+inline int64_t Rows(const TensorView& t) {  // product of all dims but the last
+  int64_t m = 1;
+  for (int i = 0; i + 1 < t.ndim(); ++i) m *= t.shape()[i];
+  return m;
+}
+
+inline int OutDtype(const TensorView& y) { return y.dtype().bits == 32 ? MI355GQ_F32 : MI355GQ_F16; }
+
+}  // namespace
+
+// y = x . dequantize(q_weight, q_scale)^T (+ bias)
+void Linear(TensorView x, TensorView q_weight, TensorView q_scale, Optional<TensorView> bias,
+            int64_t bits, int64_t group_size, TensorView y) {
+  const int64_t K = x.shape()[x.ndim() - 1], N = q_weight.shape()[0];
+  Check(mi355gq_linear(Ptr(x), Ptr(q_weight), Ptr(q_scale),
+                       bias.has_value() ? Ptr(bias.value()) : nullptr, Rows(x), N, K,
+                       static_cast<int>(bits), static_cast<int>(group_size), OutDtype(y), Ptr(y),
+                       nullptr, 0, StreamOf(x)),
+        "mlc.gq.linear");
+}
+
+void EmbeddingTake(TensorView ids, TensorView q_weight, TensorView q_scale, int64_t bits,
+                   int64_t group_size, TensorView out) {
+  const int64_t K = out.shape()[out.ndim() - 1];
+  Check(mi355gq_embedding_take(Ptr(ids), Rows(out), Ptr(q_weight), Ptr(q_scale),
+                               q_weight.shape()[0], K, static_cast<int>(bits),
+                               static_cast<int>(group_size), Ptr(out), StreamOf(out)),
+        "mlc.gq.embedding_take");
+}
+
+void MoeGemv(TensorView x, TensorView q_weight, TensorView q_scale, TensorView expert_ids,
+             int64_t bits, int64_t group_size, TensorView out) {
+  Check(mi355gq_moe_gemv(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(expert_ids),
+                         expert_ids.shape()[1], q_weight.shape()[0], q_weight.shape()[1],
+                         x.shape()[1], static_cast<int>(bits), static_cast<int>(group_size), Ptr(out),
+                         StreamOf(x)),
+        "mlc.gq.moe_gemv");
+}
+
+void MoeGroupGemm(TensorView x, TensorView q_weight, TensorView q_scale, TensorView indptr,
+                  int64_t bits, int64_t group_size, TensorView out) {
+  Check(mi355gq_moe_group_gemm(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(indptr),
+                               indptr.dtype().bits == 64 ? MI355GQ_I64 : MI355GQ_I32,
+                               q_weight.shape()[0], q_weight.shape()[1], x.shape()[1],
+                               static_cast<int>(bits), static_cast<int>(group_size), Ptr(out),
+                               StreamOf(x)),
+        "mlc.gq.moe_group_gemm");
+}
+
+// quantize has two destinations: (q_weight, q_scale)
+void Quantize(TensorView w, int64_t bits, int64_t group_size, int64_t round_mode,
+              TensorView q_weight, TensorView q_scale) {
+  const int64_t K = w.shape()[w.ndim() - 1];
+  Check(mi355gq_quantize(Ptr(w), Rows(w), K, static_cast<int>(bits), static_cast<int>(group_size),
+                         static_cast<int>(round_mode), Ptr(q_weight), Ptr(q_scale), StreamOf(w)),
+        "mlc.gq.quantize");
+}
+
+void Dequantize(TensorView q_weight, TensorView q_scale, int64_t bits, int64_t group_size,
+                TensorView out) {
+  const int64_t K = out.shape()[out.ndim() - 1];
+  Check(mi355gq_dequantize(Ptr(q_weight), Ptr(q_scale), Rows(out), K, static_cast<int>(bits),
+                           static_cast<int>(group_size), Ptr(out), StreamOf(out)),
+        "mlc.gq.dequantize");
+}
+
+TVM_FFI_STATIC_INIT_BLOCK() {
+  namespace refl = tvm::ffi::reflection;
+  refl::GlobalDef()
+      .def("mlc.gq.linear", Linear)
+      .def("mlc.gq.embedding_take", EmbeddingTake)
+      .def("mlc.gq.moe_gemv", MoeGemv)
+      .def("mlc.gq.moe_group_gemm", MoeGroupGemm)
+      .def("mlc.gq.quantize", Quantize)
+      .def("mlc.gq.dequantize", Dequantize);
+}
+
+}  // namespace gq
+}  // namespace llm
+}  // namespace mlc
