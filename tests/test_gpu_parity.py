@@ -233,6 +233,79 @@ def test_gemv_rows_per_wave_variants(rows_per_wave):
     assert_linear_ok(y, o.linear_fp32(x, qw, qs, s), x, 2048, f"R={rows_per_wave}")
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("m", [1, 2, 5])
+def test_gemv_lds_kernel_forced(name, m):
+    # the LDS-staged fallback kernel must agree too (it normally only sees odd shapes)
+    s = SCHEMES[name]
+    n, k = 777, 2048 if s.bits == 4 else 2000
+    x, qw, qs, b = _linear_case(s, m, n, k, 900 + m, bias=True)
+    gq._lib.set_option("gemv_variant", 0)
+    gq._lib.set_option("gemm_variant", 2)  # keep 3..8 rows on the GEMV path for q4 as well
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+        gq._lib.set_option("gemm_variant", -1)
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"lds gemv {name} m={m}")
+
+
+@pytest.mark.parametrize("mode", [2, 3, 4])  # unpipelined, chunk-pipelined, persistent
+@pytest.mark.parametrize("m", [3, 4, 8, 9, 16])
+@pytest.mark.parametrize("n,k", [(520, 1024), (100, 4096), (2100, 72), (64, 6176)])
+def test_skinny_kernel_forms(mode, m, n, k):
+    s = SCHEMES["q4f16_1"]
+    x, qw, qs, b = _linear_case(s, m, n, k, 31 * m + n + k, bias=True)
+    gq._lib.set_option("gemv_variant", mode)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b))
+        y32 = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, None, torch.float32)
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+    ref = o.linear_fp32(x, qw, qs, s, b)
+    assert_linear_ok(y, ref, x, k, f"skinny mode {mode} {m}x{n}x{k}")
+    assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"skinny mode {mode} fp32 out")
+
+
+@pytest.mark.parametrize("mode", [2, 3, 4])
+def test_skinny_kernel_forms_grouped(mode):
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(61)
+    ne, n, k = 5, 200, 1024
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    ip = np.array([0, 2, 2, 21, 22, 40], np.int32)  # an empty expert and one with 19 rows (2 m-tiles)
+    x = rng.standard_normal((40, k)).astype(np.float16)
+    gq._lib.set_option("gemv_variant", mode)
+    try:
+        out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), 4, 32)
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+    assert_linear_ok(out, o.dequantize_group_gemm_fp32(x, qw, qs, ip, s), x, k, f"grouped skinny mode {mode}")
+
+
+@pytest.mark.parametrize("variant", [3, 4, 6, 7])  # plain 128/256 tiles, pipelined 128/256 tiles
+@pytest.mark.parametrize("m,n,k", [(300, 512, 1024), (17, 260, 4096), (513, 300, 192)])
+def test_gemm_kernel_variants(variant, m, n, k):
+    s = SCHEMES["q4f16_1"]
+    x, qw, qs, b = _linear_case(s, m, n, k, variant * 1000 + m + n + k, bias=True)
+    gq._lib.set_option("gemm_variant", variant)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b))
+    finally:
+        gq._lib.set_option("gemm_variant", -1)
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"gemm variant {variant} {m}x{n}x{k}")
+
+
+def test_gemm_k_not_multiple_of_8_takes_fallback():
+    # K = 100: rows of x are not 16-byte aligned, the pipelined kernel declines and the plain one runs
+    for name in ("q4f16_1", "q3f16_1"):
+        s = SCHEMES[name]
+        x, qw, qs, _ = _linear_case(s, 40, 96, 100, 5)
+        y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size)
+        assert_linear_ok(y, o.linear_fp32(x, qw, qs, s), x, 100, f"gemm K=100 {name}")
+
+
 def test_gemv_config1_golden_shape_fp32_out_and_lm_head():
     # config 1: N = K = 4096, weights N(0, 0.02) seed 0, activation N(0, 1); also the fp32-output
     # path used by GroupQuantizeEmbedding.lm_head_forward
