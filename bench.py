@@ -233,15 +233,16 @@ def main() -> int:
         del xm
         extra["decode_tokens_per_s_linear_only"] = round(1e3 / ms_step, 1)
 
-        # what a plain library streaming read reaches on this box (context for the HBM fractions):
-        # torch's int32 sum over four distinct 1 GiB buffers
-        bufs = [torch.ones(256 * 1024 * 1024, dtype=torch.int32, device=dev) for _ in range(4)]
+        # what the runtime's own device-to-device copy reaches on this box (context for the HBM
+        # fractions): 1 GiB copies between four distinct buffers, bytes = read + written
+        bufs = [torch.ones(1024 * 1024 * 1024, dtype=torch.uint8, device=dev) for _ in range(4)]
 
-        def read_sweep():
-            for t in bufs:
-                t.sum()
-        ms = timed(read_sweep, 3, 1, False) / len(bufs)
-        extra["stream_read_reference"] = {"what": "torch.sum over 1 GiB int32", "GB/s": round(2**30 / (ms * 1e-3) / 1e9, 1)}
+        def copy_sweep():
+            for i in range(4):
+                bufs[(i + 1) % 4].copy_(bufs[i])
+        ms = timed(copy_sweep, 3, 1, False) / 4
+        extra["device_copy_reference"] = {"what": "1 GiB device-to-device copy, read + write bytes",
+                                          "GB/s": round(2 * 2**30 / (ms * 1e-3) / 1e9, 1)}
         del bufs
 
         # q3f16_1 decode GEMV at Llama-2-7B shapes, batch 1 (BASELINE configs[3])
@@ -286,7 +287,7 @@ def main() -> int:
         for t in (1, 16, 512):
             xt = torch.randn((1, t, 4096), generator=gx, device=dev).half()
             logits = torch.randn((t, 8), generator=g2, device=dev).half()
-            ms = timed(lambda: moe(xt, logits), 5, 2, False)
+            ms = timed(lambda: moe(xt, logits), 10, 2, use_graph)
             ids = ops.gating_softmax_topk(logits, 2)[1]
             distinct = int(torch.unique(ids).numel())
             wbytes = distinct * 99_090_432

@@ -192,7 +192,12 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
   g.indptr = nullptr; g.indptr_i64 = 0;
   g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
   g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
+  const int gv = gq::options().gemv_variant;  // 2..5 force a gq_skinny.hip form, 6..8 the quad-row kernel
   if (M <= 16 && bits == 4 && gq::options().gemm_variant != 1) {
+    if ((gv < 0 && M <= 8) || (gv >= 6 && gv <= 8)) {
+      const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
+      if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
+    }
     const hipError_t e = gq::launch_skinny(g, static_cast<int>(M), as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "skinny launch");
   }
@@ -252,7 +257,12 @@ int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, co
   g.rows = rows; g.N = N; g.K = K; g.num_experts = num_experts;
   g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
   // few rows in total: every expert is a skinny problem bound by streaming its weights
+  const int gv = gq::options().gemv_variant;
   if (rows <= 128 && bits == 4 && gq::options().gemm_variant != 1) {
+    if ((gv < 0 && rows <= 32) || (gv >= 6 && gv <= 8)) {
+      const hipError_t q = gq::launch_quadrow(g, static_cast<int>(rows), as_stream(stream));
+      if (q != hipErrorNotSupported) return hip_result(q, "moe quad-row launch");
+    }
     const hipError_t e = gq::launch_skinny(g, static_cast<int>(rows), as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "moe skinny launch");
   }

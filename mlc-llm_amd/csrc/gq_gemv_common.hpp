@@ -70,6 +70,56 @@ __device__ __forceinline__ float group_dot(const uint4 w4, const uint32_t* __res
   }
 }
 
+// x pairs of one group in the order the unpack masks produce them, from the natural-order halves.
+// v_perm_b32 picks the two 16-bit lanes directly: byte selectors 0-3 address S1, 4-7 address S0.
+template <int BITS>
+__device__ __forceinline__ float permute_group(const uint32_t* __restrict__ n /* G/2 natural pairs */,
+                                               uint32_t* __restrict__ xr /* G/2 permuted pairs */) {
+  constexpr uint32_t kLoLo = 0x05040100u;  // (lo16(S1), lo16(S0))
+  constexpr uint32_t kHiHi = 0x07060302u;  // (hi16(S1), hi16(S0))
+  constexpr uint32_t kLoHi = 0x07060100u;  // (lo16(S1), hi16(S0))
+  constexpr uint32_t kHiLo = 0x05040302u;  // (hi16(S1), lo16(S0))
+  float c = 0.f;
+  if (BITS == 4) {
+    // word w holds x[8w..8w+7] as pairs (0,1)(2,3)(4,5)(6,7); wanted (0,4)(1,5)(2,6)(3,7).
+    // Fields 1,3,5,7 come out of the mask times 16: their 1024 shrinks to 64 after rescaling.
+    const uint32_t c_lo = 0x64076407u;  // (1031, 1031)
+    const uint32_t c_hi = 0x54705470u;  // (71, 71)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      xr[4 * w + 0] = __builtin_amdgcn_perm(n[4 * w + 2], n[4 * w + 0], kLoLo);
+      xr[4 * w + 1] = __builtin_amdgcn_perm(n[4 * w + 2], n[4 * w + 0], kHiHi);
+      xr[4 * w + 2] = __builtin_amdgcn_perm(n[4 * w + 3], n[4 * w + 1], kLoLo);
+      xr[4 * w + 3] = __builtin_amdgcn_perm(n[4 * w + 3], n[4 * w + 1], kHiHi);
+      c = dot2(xr[4 * w + 0], c_lo, c);
+      c = dot2(xr[4 * w + 1], c_hi, c);
+      c = dot2(xr[4 * w + 2], c_lo, c);
+      c = dot2(xr[4 * w + 3], c_hi, c);
+    }
+  } else {
+    // word w holds x[10w..10w+9] as 5 natural pairs; wanted (j, j+5); pair j sits at mantissa
+    // bit 3*(j mod 3), so its 1024 becomes 1024, 128 or 16 after rescaling (+ m = 3).
+    const uint32_t c1 = 0x64036403u;   // (1027, 1027)
+    const uint32_t c8 = 0x58185818u;   // (131, 131)
+    const uint32_t c64 = 0x4cc04cc0u;  // (19, 19)
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const uint32_t* r = n + 5 * w;
+      xr[5 * w + 0] = __builtin_amdgcn_perm(r[2], r[0], kLoHi);
+      xr[5 * w + 1] = __builtin_amdgcn_perm(r[3], r[0], kHiLo);
+      xr[5 * w + 2] = __builtin_amdgcn_perm(r[3], r[1], kLoHi);
+      xr[5 * w + 3] = __builtin_amdgcn_perm(r[4], r[1], kHiLo);
+      xr[5 * w + 4] = __builtin_amdgcn_perm(r[4], r[2], kLoHi);
+      c = dot2(xr[5 * w + 0], c1, c);
+      c = dot2(xr[5 * w + 1], c8, c);
+      c = dot2(xr[5 * w + 2], c64, c);
+      c = dot2(xr[5 * w + 3], c1, c);
+      c = dot2(xr[5 * w + 4], c8, c);
+    }
+  }
+  return c;
+}
+
 
 // launchers of the kernel families (each in its own translation unit)
 hipError_t launch_gemv_lds(const GemvParams& p, int bits, int nb, int slots, hipStream_t s);

@@ -47,6 +47,9 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s);
 // MFMA kernel for few activation rows per segment (q4 only; hipErrorNotSupported otherwise).
 // rows_max bounds the rows of any one segment.
 hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s);
+// 4x4x4-MFMA kernel with GEMV-like weight streaming (q4, activations resident in LDS);
+// hipErrorNotSupported when the shape does not fit.
+hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s);
 
 hipError_t launch_quantize(const uint16_t* w, int64_t rows, int64_t K, int bits, int group_size,
                            int round_mode, uint32_t* qw, uint16_t* qs, hipStream_t s);

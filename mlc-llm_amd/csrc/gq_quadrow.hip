@@ -1,0 +1,394 @@
+// Few-row matmul for q4f16_1 on the 16-block 4x4x4 matrix instruction: 3..8 activation rows
+// against streamed weights, with the memory access pattern of the batch-1 GEMV.
+//
+// Covers the same callers as gq_skinny.hip (the low-batch buckets of
+// python/mlc_llm/compiler_pass/low_batch_specialization.py:22-57 and the few-tokens-per-expert
+// case of python/mlc_llm/op/moe_matmul.py:562-768) whenever the activations fit LDS whole.
+//
+// v_mfma_f32_4x4x4_16b_f16 multiplies 16 independent 4x4x4 blocks: in block b (lanes 4b..4b+3)
+// lane 4b+i supplies 4 k of A row i, lane 4b+j supplies the same 4 k of B column j, and lane 4b+j
+// receives D[0..3][j].  Here A rows are 4 consecutive weight rows (a "quad"), B columns are 4
+// activation rows, and the 16 blocks are 16 different quantisation groups of those rows:
+//  * a lane loads ONE 128-bit group of ONE weight row per step, so a wave load covers 4 rows x
+//    256 contiguous bytes (the 16x16x32 layout of gq_skinny.hip touches 16 rows x 64 bytes);
+//  * the four storage words of the group unpack with the (field | 0x6400) trick into eight A
+//    operands (even fields, and odd fields times 16), none of which leaves its lane: no LDS
+//    transpose, no cross-lane move between the load and the matrix core;
+//  * all 8 products of a group land in one accumulator pair, so the group's scale and the
+//    (1024 + m) offset are applied once per group in fp32, as in the GEMV kernels;
+//  * x is staged once per workgroup in LDS, already in operand order ([k step][word][lane] so
+//    that every ds_read_b128 of a wave is one contiguous KiB), with the offset term of every
+//    (activation row, group) beside it;
+//  * waves are persistent and walk (quad, k step) items with the loads of the next two items
+//    in flight, U KiB per item;
+//  * when x does not fit LDS whole (8 rows of a 14336-wide layer), K is walked in phases: each
+//    phase stages its slice of x and visits every quad, partial sums wait in LDS in between, so
+//    the weights are still read exactly once.
+// The 16 blocks are summed across lanes once per quad.
+#include "gq_gemv_common.hpp"
+
+namespace gq {
+
+struct QuadParams {
+  const uint16_t* x;
+  const uint32_t* qw;
+  const uint16_t* qs;
+  const uint16_t* bias;
+  void* y;
+  const void* indptr;  // null: one segment [0, rows)
+  int64_t expert_w_stride, expert_s_stride;
+  int rows, N, K, ng, nw;
+  int nquads;       // N / 4
+  int nsteps;       // k steps per quad and phase; a step is U iterations of 16 groups
+  int steps_total;  // k steps per quad over all phases
+  int nphases;      // passes over K, each with its slice of x in LDS
+  int rounds;       // most quads any wave walks
+  int indptr_i64, out_f32;
+};
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u(uint32_t v) {
+  return static_cast<uint32_t>(
+      __builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ float4_t mfma4(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1,
+                                          float4_t c) {
+  typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+  const u2 a = {a0, a1}, b = {b0, b1};
+  return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, a),
+                                            __builtin_bit_cast(half4_t, b), c, 0, 0, 0);
+}
+
+// NBQ: activation rows / 4 (rows past the segment are zero); U: iterations per item
+template <int NBQ, int U>
+__global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
+  constexpr uint32_t kMagic = 0x64006400u;
+  constexpr int XB = 4;  // (activation row, group) pairs a thread stages per round
+
+  extern __shared__ uint4 smem[];
+
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int lane = tid & 63;
+  const int wpb = nthreads >> 6;
+  const int gw = blockIdx.x * wpb + (tid >> 6);
+  const int nwaves = gridDim.x * wpb;
+  const int li = lane & 3;   // weight row of the quad (A), activation row of the batch quad (B, D)
+  const int ks = lane >> 2;  // block: group 16 * iteration + ks
+
+  // ---- segment of activation rows and the expert they meet
+  int seg_lo = 0, seg_hi = p.rows;
+  const int expert = blockIdx.y;
+  if (p.indptr != nullptr) {
+    int64_t lo, hi;
+    if (p.indptr_i64) {
+      lo = static_cast<const int64_t*>(p.indptr)[expert];
+      hi = static_cast<const int64_t*>(p.indptr)[expert + 1];
+    } else {
+      lo = static_cast<const int32_t*>(p.indptr)[expert];
+      hi = static_cast<const int32_t*>(p.indptr)[expert + 1];
+    }
+    lo = lo < 0 ? 0 : (lo > p.rows ? p.rows : lo);
+    hi = hi < lo ? lo : (hi > p.rows ? p.rows : hi);
+    seg_lo = static_cast<int>(lo);
+    seg_hi = static_cast<int>(hi);
+  }
+  const int m0 = seg_lo + blockIdx.z * (4 * NBQ);
+  if (m0 >= seg_hi) return;  // uniform: this expert has no (more) rows
+  const int m_valid = min(4 * NBQ, seg_hi - m0);
+  const uint32_t* qw = p.qw + expert * p.expert_w_stride;
+  const uint16_t* qs = p.qs + expert * p.expert_s_stride;
+
+  // LDS: x of one phase [NBQ][niter][4 words][64 lanes] uint4, its offset terms [NBQ][niter][64]
+  // floats, then this workgroup's partial sums between phases [wave][quad of the walk][NBQ][16]
+  const int niter = p.nsteps * U;  // staged iterations per phase (groups past ng hold zeros)
+  float* const corr_lds = reinterpret_cast<float*>(smem + static_cast<size_t>(NBQ) * niter * 256);
+  float* const part_lds = corr_lds + NBQ * niter * 64 + (tid >> 6) * (p.rounds * NBQ * 16);
+
+  uint4 wa[U], wb[U];
+  uint32_t sa[U], sb[U];  // fp16 bits, 32 bits wide so that in-flight values are never re-packed
+  uint2 ba, bb;
+  float4_t acc[NBQ];
+
+  // K is walked in phases when x does not fit LDS whole: every phase stages its slice of x and
+  // walks all of this wave's quads; partial sums wait in LDS for the last phase.
+  for (int phase = 0; phase < p.nphases; ++phase) {
+    const int nst = min(p.nsteps, p.steps_total - phase * p.nsteps);  // steps of this phase
+    const int it0 = phase * niter;                                    // first iteration of the phase
+    const bool last_phase = phase == p.nphases - 1;
+#pragma unroll
+    for (int bq = 0; bq < NBQ; ++bq) acc[bq] = float4_t{0.f, 0.f, 0.f, 0.f};  // drops what an item past the end left
+
+    // ---- weight / scale / bias loads of one item.  Branch-free: every path issues the same
+    //      loads, so the wait counts let the other buffer's loads stay in flight across the loop;
+    //      an item past the end reads one cached line instead.
+    auto issue = [&](int quad, int step, uint4 (&wn)[U], uint32_t (&sn)[U], uint2& bn) {
+      const bool live = quad < p.nquads;
+      const int row = min(quad * 4 + li, p.N - 1);
+      const uint32_t* wr = qw + static_cast<int64_t>(row) * p.nw;
+      const uint16_t* sr = qs + static_cast<int64_t>(row) * p.ng;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int g = min((it0 + step * U + u) * 16 + ks, p.ng - 1);
+        wn[u] = *reinterpret_cast<const uint4*>(live ? wr + 4 * g : qw);
+        sn[u] = *(live ? sr + g : qs);
+      }
+      bn = *reinterpret_cast<const uint2*>(
+          (live && p.bias != nullptr) ? p.bias + quad * 4 : reinterpret_cast<const uint16_t*>(qw));
+    };
+    auto advance = [&](int& quad, int& step) {  // two items on
+      step += 2;
+      if (step >= nst) {
+        step -= nst;
+        quad += nwaves;
+        if (step >= nst) {
+          step -= nst;
+          quad += nwaves;
+        }
+      }
+    };
+    int qa = gw, sta = 0, qb = gw, stb = 1;
+    if (stb >= nst) {
+      stb = 0;
+      qb += nwaves;
+    }
+    issue(qa, sta, wa, sa, ba);
+    issue(qb, stb, wb, sb, bb);
+
+    // ---- stage x in operand order.  Pair q = (batch quad, iteration, lane') with lane' = 4 *
+    //      block + activation row; its four 16-byte words go to [q / 64][word][lane'].
+    if (phase > 0) __syncthreads();  // the previous phase's x is still being read
+    {
+      const int npairs = NBQ * niter * 64;
+      for (int q0 = tid; q0 < npairs; q0 += nthreads * XB) {
+        uint4 raw[XB][4];
+        bool ok[XB][4];
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+          const int q = q0 + i * nthreads;
+          const int lp = q & 63, bi = q >> 6;  // bi = bq * niter + it
+          const int bq = bi / niter, it = bi - bq * niter;
+          const int b = 4 * bq + (lp & 3);
+          const int g = 16 * (it0 + it) + (lp >> 2);
+          const uint16_t* src = p.x + static_cast<int64_t>(m0 + min(b, m_valid - 1)) * p.K;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int k = 32 * g + 8 * c;
+            ok[i][c] = q < npairs && b < m_valid && g < p.ng && k + 8 <= p.K;
+            raw[i][c] = *reinterpret_cast<const uint4*>(ok[i][c] ? src + k : p.x);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < XB; ++i) {
+          const int q = q0 + i * nthreads;
+          if (q < npairs) {
+            uint32_t nat[16], xr[16];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              const uint4 r = ok[i][c] ? raw[i][c] : make_uint4(0, 0, 0, 0);
+              nat[4 * c + 0] = r.x; nat[4 * c + 1] = r.y; nat[4 * c + 2] = r.z; nat[4 * c + 3] = r.w;
+            }
+            const float corr = permute_group<4>(nat, xr);
+            const int lp = q & 63, bi = q >> 6;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)  // (even fields: 2 pairs), (odd fields: 2 pairs)
+              smem[(bi * 4 + c) * 64 + lp] =
+                  make_uint4(xr[4 * c + 0], xr[4 * c + 2], xr[4 * c + 1], xr[4 * c + 3]);
+            corr_lds[bi * 64 + lp] = corr;
+          }
+        }
+      }
+    }
+    // Every load above has been consumed by now, but on the path that skips the staging loop the
+    // wait-count bookkeeping cannot see it and would make the walk's first waits conservative.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    // ---- persistent walk
+    int done = 0;  // quads this wave has completed in this phase
+    auto compute = [&](int quad, int step, const uint4 (&wc)[U], const uint32_t (&sc)[U],
+                       uint2 bias_bits) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int it = step * U + u;
+        const uint32_t w[4] = {wc[u].x, wc[u].y, wc[u].z, wc[u].w};
+        uint32_t lo[4][2], hi[4][2];
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint32_t w8 = w[d] >> 8;
+          lo[d][0] = and_or(w[d], 0x000f000fu, kMagic);
+          hi[d][0] = and_or(w[d], 0x00f000f0u, kMagic);
+          lo[d][1] = and_or(w8, 0x000f000fu, kMagic);
+          hi[d][1] = and_or(w8, 0x00f000f0u, kMagic);
+        }
+        // the four rows' scales of this block: lane 4b+i holds row i's
+        float sv[4];
+        sv[0] = h2f(static_cast<uint16_t>(dpp_u<0x00>(sc[u])));
+        sv[1] = h2f(static_cast<uint16_t>(dpp_u<0x55>(sc[u])));
+        sv[2] = h2f(static_cast<uint16_t>(dpp_u<0xAA>(sc[u])));
+        sv[3] = h2f(static_cast<uint16_t>(dpp_u<0xFF>(sc[u])));
+#pragma unroll
+        for (int bq = 0; bq < NBQ; ++bq) {
+          if (bq > 0 && 4 * bq >= m_valid) continue;  // uniform: this segment has no such rows
+          const int bi = bq * niter + it;
+          float4_t tl = {0.f, 0.f, 0.f, 0.f}, th = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const uint4 xv = smem[(bi * 4 + d) * 64 + lane];
+            tl = mfma4(lo[d][0], lo[d][1], xv.x, xv.y, tl);
+            th = mfma4(hi[d][0], hi[d][1], xv.z, xv.w, th);
+          }
+          const float corr = corr_lds[bi * 64 + lane];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[bq][i] = fmaf(sv[i], fmaf(th[i], 0.0625f, tl[i]) - corr, acc[bq][i]);
+        }
+      }
+      if (step == nst - 1) {  // uniform: the quad's share of this phase is complete
+#pragma unroll
+        for (int bq = 0; bq < NBQ; ++bq) {
+          float v[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float t = acc[bq][i];
+            t += dpp_f<0x124>(t);  // row_ror:4
+            t += dpp_f<0x128>(t);  // row_ror:8: every lane holds the sum over its row of 16 lanes
+            t += __shfl_xor(t, 16, kWave);
+            t += __shfl_xor(t, 32, kWave);
+            v[i] = t;
+            acc[bq][i] = 0.f;
+          }
+          const int b = 4 * bq + lane;  // lanes 0..3: one activation row each, 4 weight rows
+          if (lane < 4 && b < m_valid && quad < p.nquads) {
+            float4* part = reinterpret_cast<float4*>(part_lds) + (done * NBQ + bq) * 4 + lane;
+            if (phase > 0) {
+              const float4 pv = *part;
+              v[0] += pv.x; v[1] += pv.y; v[2] += pv.z; v[3] += pv.w;
+            }
+            if (!last_phase) {
+              *part = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+              if (p.bias != nullptr) {
+                v[0] += h2f(static_cast<uint16_t>(bias_bits.x & 0xffffu));
+                v[1] += h2f(static_cast<uint16_t>(bias_bits.x >> 16));
+                v[2] += h2f(static_cast<uint16_t>(bias_bits.y & 0xffffu));
+                v[3] += h2f(static_cast<uint16_t>(bias_bits.y >> 16));
+              }
+              const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
+              if (p.out_f32) {
+                *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) =
+                    make_float4(v[0], v[1], v[2], v[3]);
+              } else {
+                uint2 o;
+                o.x = static_cast<uint32_t>(f2h(v[0])) | (static_cast<uint32_t>(f2h(v[1])) << 16);
+                o.y = static_cast<uint32_t>(f2h(v[2])) | (static_cast<uint32_t>(f2h(v[3])) << 16);
+                *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.y) + oi) = o;
+              }
+            }
+          }
+        }
+        ++done;
+      }
+    };
+
+    while (qa < p.nquads) {
+      compute(qa, sta, wa, sa, ba);
+      advance(qa, sta);
+      issue(qa, sta, wa, sa, ba);
+      __builtin_amdgcn_sched_barrier(0);  // keep the refill ahead of the next item's arithmetic
+      compute(qb, stb, wb, sb, bb);  // past the end: nothing is stored
+      advance(qb, stb);
+      issue(qb, stb, wb, sb, bb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+template <int NBQ, int U>
+static hipError_t launch_quad_cfg(const QuadParams& p, dim3 grid, int threads, size_t lds,
+                                  hipStream_t s) {
+  if (lds > 65536) {
+    const hipError_t e =
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_q4_kernel<NBQ, U>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL((quad_q4_kernel<NBQ, U>), grid, dim3(threads), lds, s, p);
+  return hipGetLastError();
+}
+
+// hipErrorNotSupported when the shape does not fit (the caller falls back to gq_skinny.hip)
+hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
+  if (a.bits != 4 || a.group_size != 32) return hipErrorNotSupported;
+  if (a.rows == 0 || a.N == 0) return hipSuccess;
+  if ((a.N & 3) != 0 || (a.K & 7) != 0) return hipErrorNotSupported;
+  if ((reinterpret_cast<uintptr_t>(a.x) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.y) & 15) != 0 ||
+      (reinterpret_cast<uintptr_t>(a.bias) & 7) != 0 ||
+      (reinterpret_cast<uintptr_t>(a.q_weight) & 15) != 0)
+    return hipErrorNotSupported;
+  QuadParams p;
+  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.y = a.y;
+  p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64;
+  p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
+  p.ng = static_cast<int>((a.K + 31) / 32);
+  p.nw = 4 * p.ng;
+  p.nquads = p.N / 4;
+  p.expert_w_stride = a.N * p.nw;
+  p.expert_s_stride = a.N * p.ng;
+  p.out_f32 = a.out_f32;
+  const int experts = a.indptr ? static_cast<int>(a.num_experts) : 1;
+
+  const int niter = (p.ng + 15) / 16;
+  int U = options().gemv_rows_per_wave;  // tuning override
+  // measured: 4 KiB items pay off only on matrices large enough to run long (gate_up, lm_head)
+  if (U != 2 && U != 4 && U != 8)
+    U = (niter >= 4 && static_cast<int64_t>(a.N) * a.K * experts >= (100ll << 20)) ? 4 : 2;
+  p.steps_total = (niter + U - 1) / U;
+  // More than 4 rows: 8 per pass when their x fits LDS whole.  Otherwise a plain linear runs
+  // two concurrent 4-row passes (the second pass's weight reads hit the last-level cache, and
+  // the grid doubles), a grouped matmul walks K in phases (experts already fill the grid).
+  // Tuning overrides: gemv_variant 7 prefers phases, 8 prefers 4-row passes.
+  const int mode = options().gemv_variant;
+  int nbq = rows_max <= 4 ? 1 : 2;
+  if (nbq == 2) {
+    const size_t whole = static_cast<size_t>(p.steps_total) * U * 2 * (4096 + 256);
+    const bool phases = mode == 7 || (mode != 8 && a.indptr != nullptr);
+    if (mode == 8 || (whole > 150 * 1024 && !phases)) nbq = 1;
+  }
+  const int mtiles = (rows_max + 4 * nbq - 1) / (4 * nbq);
+  if (mtiles > 2 && a.indptr == nullptr) return hipErrorNotSupported;
+
+  // every workgroup stages x for itself, so a small plain matrix wants fewer, longer-lived waves
+  int waves = options().gemv_split > 0 ? options().gemv_split
+                                       : (a.indptr != nullptr || p.nquads >= 6144 ? 2048 : 1024);
+  // workgroups of experts without rows leave at once: share the waves among those that can have rows
+  const int busy = p.rows < experts ? p.rows : experts;
+  waves = (waves + busy - 1) / busy;
+  if (waves > p.nquads) waves = p.nquads;
+  p.rounds = (p.nquads + waves - 1) / waves;
+
+  // LDS per step and batch quad: x (4 rows * 32 halves per group, 16 groups per iteration) and
+  // the offset terms; per wave: the partial sums of its quads.  Phases share K evenly.
+  const size_t lds_cap = 150 * 1024;
+  const size_t lds_step = static_cast<size_t>(U) * nbq * (4096 + 256);
+  const size_t lds_part = static_cast<size_t>(8) * p.rounds * nbq * 64;  // up to 8 waves
+  if (lds_part + lds_step > lds_cap) return hipErrorNotSupported;
+  const int steps_fit = static_cast<int>((lds_cap - lds_part) / lds_step);
+  p.nphases = (p.steps_total + steps_fit - 1) / steps_fit;
+  p.nsteps = (p.steps_total + p.nphases - 1) / p.nphases;
+  const size_t lds_x = lds_step * p.nsteps;
+  // two waves per SIMD: 512-thread workgroups when only one workgroup fits a CU's LDS
+  const int threads = lds_x > 76 * 1024 ? 512 : 256;
+  const int wpb = threads / 64;
+  const size_t lds = lds_x + (p.nphases > 1 ? static_cast<size_t>(wpb) * p.rounds * nbq * 64 : 0);
+  const int blocks = ((p.nquads + p.rounds - 1) / p.rounds + wpb - 1) / wpb;
+  const dim3 grid(blocks, experts, mtiles);
+#define GQ_QUAD_CASE(NBQ_, U_) \
+  if (nbq == NBQ_ && U == U_) return launch_quad_cfg<NBQ_, U_>(p, grid, threads, lds, s);
+  GQ_QUAD_CASE(1, 2) GQ_QUAD_CASE(1, 4) GQ_QUAD_CASE(1, 8)
+  GQ_QUAD_CASE(2, 2) GQ_QUAD_CASE(2, 4) GQ_QUAD_CASE(2, 8)
+#undef GQ_QUAD_CASE
+  return hipErrorNotSupported;
+}
+
+}  // namespace gq
