@@ -230,6 +230,16 @@ def main() -> int:
             gemm[f"gate_up_m{m2}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
                                       "frac_mfma": round(tf / MFMA_F16_PEAK_TFLOPS, 3)}
             del xm2, ym2
+        # context for the MFMA fractions: the vendor library's dense fp16 GEMM (torch's linear) on the
+        # same shapes, weights already dequantised (4x the weight bytes, no unpacking in the loop)
+        lib = {}
+        for name in ("gate_up", "down"):
+            n, k = SHAPES[name]
+            wd = (torch.randn((n, k), generator=gx, device=dev) * 0.02).half()
+            ms = timed(lambda: torch.nn.functional.linear(xm[k], wd), 5, 2, False)
+            lib[f"{name}_m{m}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 1)}
+            del wd
+        extra["library_dense_fp16_gemm_reference"] = lib
         del xm
         extra["decode_tokens_per_s_linear_only"] = round(1e3 / ms_step, 1)
 
