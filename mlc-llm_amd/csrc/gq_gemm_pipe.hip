@@ -236,7 +236,12 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   if (bits == 4) {
     const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
     const bool big = variant == 7 ? true : (variant == 6 ? false : (p.indptr == nullptr && big_tiles >= 160));
+    if (variant == 9) return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     if (big) return launch_pipe_cfg<4, 256, 256, 128, 64>(p, s);
+    // too few 256x256 tiles for 256 CUs (o_proj, down at M = 2048): halve the tile along M
+    const int64_t mid_tiles = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
+    if (variant != 6 && p.indptr == nullptr && mid_tiles >= 192)
+      return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
   }
   return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);

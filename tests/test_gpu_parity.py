@@ -365,7 +365,7 @@ def test_quadrow_kernel_grouped(k):
     assert_linear_ok(out64, ref, x, k, f"grouped quad-row k={k} int64 indptr")
 
 
-@pytest.mark.parametrize("variant", [3, 4, 6, 7])  # plain 128/256 tiles, pipelined 128/256 tiles
+@pytest.mark.parametrize("variant", [3, 4, 6, 7, 9])  # plain 128/256 tiles, pipelined 128/256 tiles, pipelined 128x256
 @pytest.mark.parametrize("m,n,k", [(300, 512, 1024), (17, 260, 4096), (513, 300, 192)])
 def test_gemm_kernel_variants(variant, m, n, k):
     s = SCHEMES["q4f16_1"]
