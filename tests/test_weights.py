@@ -1,0 +1,249 @@
+"""Weight directory format and HuggingFace -> MLC parameter mapping.
+
+No weight directory and no checkpoint ship with the reference, so these tests build tiny synthetic
+checkpoints with the HuggingFace parameter names and check (a) the file format by round trip and
+against its published field list, (b) the mapping against what the reference's loaders do
+(python/mlc_llm/loader/standard_loader.py:89-134, python/mlc_llm/model/mixtral/mixtral_loader.py:44-104),
+(c) on the GPU, that the converted ``q_weight`` / ``q_scale`` equal the oracle's quantisation of the
+concatenated / stacked matrices bit for bit."""
+
+import json
+import os
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+from mlc_llm_amd import loader, tensor_cache
+from oracle import gq_oracle as o
+
+LLAMA = {"model_type": "llama", "hidden_size": 64, "intermediate_size": 160, "num_hidden_layers": 2,
+         "num_attention_heads": 4, "num_key_value_heads": 2, "vocab_size": 96, "tie_word_embeddings": False}
+MIXTRAL = {"model_type": "mixtral", "hidden_size": 64, "intermediate_size": 96, "num_hidden_layers": 1,
+           "num_attention_heads": 4, "num_key_value_heads": 2, "vocab_size": 80, "num_local_experts": 3,
+           "num_experts_per_tok": 2}
+
+
+def _hf_tensors(cfg, seed=0):
+    rng = np.random.default_rng(seed)
+    h, inter, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    kv = h // cfg["num_attention_heads"] * cfg["num_key_value_heads"]
+
+    def w(*shape):
+        return torch.from_numpy((rng.standard_normal(shape) * 0.05).astype(np.float16))
+
+    t = {"model.embed_tokens.weight": w(v, h), "model.norm.weight": w(h), "lm_head.weight": w(v, h)}
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}"
+        t[f"{p}.self_attn.q_proj.weight"] = w(h, h)
+        t[f"{p}.self_attn.k_proj.weight"] = w(kv, h)
+        t[f"{p}.self_attn.v_proj.weight"] = w(kv, h)
+        t[f"{p}.self_attn.o_proj.weight"] = w(h, h)
+        t[f"{p}.input_layernorm.weight"] = w(h)
+        t[f"{p}.post_attention_layernorm.weight"] = w(h)
+        t[f"{p}.self_attn.rotary_emb.inv_freq"] = w(8)
+        if cfg["model_type"] == "mixtral":
+            t[f"{p}.block_sparse_moe.gate.weight"] = w(cfg["num_local_experts"], h)
+            for e in range(cfg["num_local_experts"]):
+                t[f"{p}.block_sparse_moe.experts.{e}.w1.weight"] = w(inter, h)
+                t[f"{p}.block_sparse_moe.experts.{e}.w2.weight"] = w(h, inter)
+                t[f"{p}.block_sparse_moe.experts.{e}.w3.weight"] = w(inter, h)
+        else:
+            t[f"{p}.mlp.gate_proj.weight"] = w(inter, h)
+            t[f"{p}.mlp.up_proj.weight"] = w(inter, h)
+            t[f"{p}.mlp.down_proj.weight"] = w(h, inter)
+    return t
+
+
+def _write_checkpoint(path, cfg, tensors, shards=2):
+    from safetensors.torch import save_file
+
+    os.makedirs(path, exist_ok=True)
+    names = list(tensors)
+    weight_map = {}
+    for s in range(shards):
+        part = {n: tensors[n] for n in names[s::shards]}
+        fn = f"model-{s + 1:05d}-of-{shards:05d}.safetensors"
+        save_file(part, os.path.join(path, fn))
+        weight_map.update({n: fn for n in part})
+    with open(os.path.join(path, "model.safetensors.index.json"), "w") as f:
+        json.dump({"weight_map": weight_map}, f)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+
+
+# ------------------------------------------------------------------------------ file format
+
+def test_bf16_encoding_known_values():
+    # 1.0 -> 0x3F80; ties go to even: 0x3F808000 -> 0x3F80, 0x3F818000 -> 0x3F82; above half rounds up
+    bits = np.array([0x3F800000, 0x3F808000, 0x3F818000, 0x3F808001, 0xBF808001, 0x00000000], np.uint32)
+    enc = tensor_cache.f32_to_bf16(bits.view(np.float32))
+    assert enc.tolist() == [0x3F80, 0x3F80, 0x3F82, 0x3F81, 0xBF81, 0x0000]
+    # the largest float32 must clip to the largest bf16, not round up to infinity
+    big = np.array([np.finfo(np.float32).max, -np.finfo(np.float32).max], np.float32)
+    assert tensor_cache.f32_to_bf16(big).tolist() == [0x7F7F, 0xFF7F]
+    # decode is the exact left shift
+    assert tensor_cache.bf16_to_f32(np.array([0x3F80, 0xC000], np.uint16)).tolist() == [1.0, -2.0]
+    # every bf16-representable float survives a round trip
+    rep = (np.arange(0, 0x7F80, 7, dtype=np.uint32) << 16).view(np.float32)
+    assert np.array_equal(tensor_cache.bf16_to_f32(tensor_cache.f32_to_bf16(rep)), rep)
+
+
+def test_tensor_cache_round_trip_and_schema(tmp_path):
+    rng = np.random.default_rng(3)
+    params = {
+        "a.q_weight": rng.integers(0, 2**32, (40, 16), dtype=np.uint32),
+        "a.q_scale": rng.standard_normal((40, 4)).astype(np.float16),
+        "norm.weight": torch.from_numpy(rng.standard_normal(64).astype(np.float16)),
+        "f32": (np.arange(24, dtype=np.float32) * 0.5).reshape(2, 3, 4),  # exactly representable in bf16
+        "big": rng.integers(0, 2**32, (300, 1024), dtype=np.uint32),      # 1.2 MB > 1 MiB cap: own shard
+        "tail": rng.standard_normal(10).astype(np.float16),
+        "empty": np.zeros((0, 8), np.float16),
+    }
+    doc = tensor_cache.dump_tensor_cache(params, str(tmp_path), meta_data=lambda: {"ParamSize": len(params)},
+                                         shard_cap_mb=1)
+    on_disk = json.load(open(tmp_path / "tensor-cache.json"))
+    assert on_disk == doc and on_disk["metadata"] == {"ParamSize": 7}
+    shards = on_disk["records"]
+    assert [s["dataPath"] for s in shards] == [f"params_shard_{i}.bin" for i in range(len(shards))]
+    for s in shards:
+        assert set(s) == {"dataPath", "format", "nbytes", "records", "md5sum"} and s["format"] == "raw-shard"
+        assert os.path.getsize(tmp_path / s["dataPath"]) == s["nbytes"] <= max(1 << 20, s["records"][0]["nbytes"])
+        end = 0
+        for r in s["records"]:
+            assert set(r) == {"name", "shape", "dtype", "format", "nbytes", "byteOffset"}
+            assert r["byteOffset"] == end  # packed back to back
+            end += r["nbytes"]
+        assert end == s["nbytes"]
+    big = [s for s in shards if s["records"][0]["name"] == "big"][0]
+    assert len(big["records"]) == 1
+    recs = {r["name"]: r for s in shards for r in s["records"]}
+    # a tensor with a shard of its own is written at once, the rest keeps iteration order
+    assert [n for n in recs if n != "big"] == [n for n in params if n != "big"] and "big" in recs
+    assert recs["f32"]["format"] == "f32-to-bf16" and recs["f32"]["nbytes"] == 48 and recs["f32"]["dtype"] == "float32"
+    assert recs["a.q_weight"]["dtype"] == "uint32" and recs["a.q_weight"]["format"] == "raw"
+
+    loaded, meta = tensor_cache.load_tensor_cache(str(tmp_path), verify_md5=True)
+    assert meta == {"ParamSize": 7} and set(loaded) == set(params)
+    assert loaded["a.q_weight"].dtype == torch.int32
+    assert np.array_equal(loaded["a.q_weight"].numpy().view(np.uint32), params["a.q_weight"])
+    assert np.array_equal(loaded["big"].numpy().view(np.uint32), params["big"])
+    assert torch.equal(loaded["norm.weight"], params["norm.weight"])
+    assert np.array_equal(loaded["f32"].numpy(), params["f32"]) and loaded["f32"].dtype == torch.float32
+    assert tuple(loaded["empty"].shape) == (0, 8)
+    only = dict(tensor_cache.iter_tensor_cache(str(tmp_path), names=["tail"]))
+    assert list(only) == ["tail"] and np.array_equal(only["tail"].numpy(), params["tail"])
+
+
+def test_tensor_cache_detects_corruption(tmp_path):
+    tensor_cache.dump_tensor_cache({"x": np.arange(64, dtype=np.int32)}, str(tmp_path))
+    shard = tmp_path / "params_shard_0.bin"
+    data = bytearray(shard.read_bytes())
+    data[5] ^= 0xFF
+    shard.write_bytes(bytes(data))
+    with pytest.raises(ValueError, match="md5"):
+        tensor_cache.load_tensor_cache(str(tmp_path), verify_md5=True)
+    shard.write_bytes(bytes(data[:-4]))
+    with pytest.raises(ValueError, match="bytes on disk"):
+        tensor_cache.load_tensor_cache(str(tmp_path))
+    with pytest.raises(ValueError, match="duplicate"):
+        tensor_cache.dump_tensor_cache([("x", np.zeros(1, np.int32)), ("x", np.zeros(1, np.int32))], str(tmp_path))
+
+
+# ------------------------------------------------------------------------------ mapping
+
+def test_llama_mapping_names_and_concatenation():
+    mapping, quantized = loader.llama_huggingface(LLAMA)
+    t = {k: v.numpy() for k, v in _hf_tensors(LLAMA).items()}
+    assert list(mapping.param_map)[:3] == ["model.embed_tokens.weight", "model.layers.0.self_attn.qkv_proj.weight",
+                                          "model.layers.0.self_attn.o_proj.weight"]
+    qkv = mapping.map_func["model.layers.1.self_attn.qkv_proj.weight"](
+        *[t[n] for n in mapping.param_map["model.layers.1.self_attn.qkv_proj.weight"]])
+    assert qkv.shape == (64 + 32 + 32, 64)
+    assert np.array_equal(qkv[:64], t["model.layers.1.self_attn.q_proj.weight"])
+    assert np.array_equal(qkv[64:96], t["model.layers.1.self_attn.k_proj.weight"])
+    assert np.array_equal(qkv[96:], t["model.layers.1.self_attn.v_proj.weight"])
+    gu = mapping.map_func["model.layers.0.mlp.gate_up_proj.weight"](
+        *[t[n] for n in mapping.param_map["model.layers.0.mlp.gate_up_proj.weight"]])
+    assert np.array_equal(gu[:160], t["model.layers.0.mlp.gate_proj.weight"])
+    assert np.array_equal(gu[160:], t["model.layers.0.mlp.up_proj.weight"])
+    # norms are never quantised; embedding, every projection and the final fc are
+    assert not any("norm" in q for q in quantized)
+    assert {"model.embed_tokens.weight", "lm_head.weight", "model.layers.0.mlp.down_proj.weight"} <= set(quantized)
+    assert len(quantized) == 2 + 4 * LLAMA["num_hidden_layers"]
+    assert loader.check_parameter_usage(mapping, set(t)) == set()  # inv_freq is declared unused
+    tied = dict(LLAMA, tie_word_embeddings=True)
+    m2, q2 = loader.llama_huggingface(tied)
+    assert "lm_head.weight" not in m2.param_map and "lm_head.weight" not in q2
+    with pytest.raises(ValueError, match="do not exist"):
+        loader.check_parameter_usage(mapping, set(t) - {"model.layers.0.mlp.up_proj.weight"})
+
+
+def test_mixtral_mapping_stacks_experts():
+    mapping, quantized = loader.mixtral_huggingface(MIXTRAL)
+    t = {k: v.numpy() for k, v in _hf_tensors(MIXTRAL).items()}
+    e13 = mapping.map_func["model.layers.0.moe.e1_e3.weight"](
+        *[t[n] for n in mapping.param_map["model.layers.0.moe.e1_e3.weight"]])
+    e2 = mapping.map_func["model.layers.0.moe.e2.weight"](
+        *[t[n] for n in mapping.param_map["model.layers.0.moe.e2.weight"]])
+    assert e13.shape == (3, 192, 64) and e2.shape == (3, 64, 96)
+    for e in range(3):
+        assert np.array_equal(e13[e, :96], t[f"model.layers.0.block_sparse_moe.experts.{e}.w1.weight"])
+        assert np.array_equal(e13[e, 96:], t[f"model.layers.0.block_sparse_moe.experts.{e}.w3.weight"])
+        assert np.array_equal(e2[e], t[f"model.layers.0.block_sparse_moe.experts.{e}.w2.weight"])
+    assert mapping.param_map["model.layers.0.moe.gate.weight"] == ["model.layers.0.block_sparse_moe.gate.weight"]
+    assert "model.layers.0.moe.gate.weight" not in quantized  # the router stays in floating point
+    assert {"model.layers.0.moe.e1_e3.weight", "model.layers.0.moe.e2.weight"} <= set(quantized)
+
+
+def test_convert_weight_unquantised_on_cpu(tmp_path):
+    src, dst = str(tmp_path / "hf"), str(tmp_path / "mlc")
+    tensors = _hf_tensors(LLAMA, seed=5)
+    _write_checkpoint(src, LLAMA, tensors)
+    meta = loader.convert_weight(src, dst, quantization="q0f16", device="cpu")
+    params, meta2 = tensor_cache.load_tensor_cache(dst, verify_md5=True)
+    assert meta == meta2 and meta["ParamSize"] == len(params) == 3 + 6 * 2
+    assert meta["BitsPerParam"] == 16.0
+    assert torch.equal(params["model.layers.0.self_attn.qkv_proj.weight"],
+                       torch.cat([tensors[f"model.layers.0.self_attn.{p}_proj.weight"] for p in "qkv"]))
+    assert json.load(open(os.path.join(dst, "mlc-chat-config.json")))["quantization"] == "q0f16"
+
+
+# ------------------------------------------------------------------------------ on the GPU
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("scheme", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("cfg", [LLAMA, MIXTRAL], ids=["llama", "mixtral"])
+def test_convert_weight_quantised_matches_oracle(tmp_path, cfg, scheme):
+    import mlc_llm_amd as gq
+    from mlc_llm_amd import ops
+
+    src, dst = str(tmp_path / "hf"), str(tmp_path / "mlc")
+    tensors = _hf_tensors(cfg, seed=zlib.crc32(scheme.encode()) & 0xFFFF)
+    _write_checkpoint(src, cfg, tensors, shards=3)
+    meta = loader.convert_weight(src, dst, quantization=scheme, device="cuda:0")
+    params, _ = tensor_cache.load_tensor_cache(dst, device="cpu", verify_md5=True)
+    s = o.SCHEMES[scheme]
+    mapping, quantized = loader.MODEL_MAPPINGS[cfg["model_type"]](cfg)
+    assert meta["ParamSize"] == len(params) == len(mapping.param_map) + len(quantized)
+    np_t = {k: v.numpy() for k, v in tensors.items()}
+    for name in mapping.param_map:
+        full = mapping.map_func[name](*[np_t[n] for n in mapping.param_map[name]])
+        if name in quantized:
+            base = name[: -len(".weight")]
+            qw, qs = o.quantize(full, s)
+            assert np.array_equal(params[f"{base}.q_weight"].numpy().view(np.uint32), qw), name
+            assert np.array_equal(params[f"{base}.q_scale"].numpy().view(np.uint16), qs.view(np.uint16)), name
+            assert name not in params
+        else:
+            assert np.array_equal(params[name].numpy(), full), name
+    # the converted directory feeds the kernels: one projection against the oracle
+    name = "model.layers.0.self_attn.qkv_proj"
+    dev = torch.device("cuda:0")
+    x = np.random.default_rng(1).standard_normal((3, cfg["hidden_size"])).astype(np.float16)
+    y = ops.linear(torch.from_numpy(x).to(dev), params[f"{name}.q_weight"].to(dev), params[f"{name}.q_scale"].to(dev),
+                   s.bits, s.group_size)
+    ref = o.linear_fp32(x, params[f"{name}.q_weight"].numpy().view(np.uint32), params[f"{name}.q_scale"].numpy(), s)
+    err, bound, rel = o.check_linear(y.float().cpu().numpy(), ref, x, cfg["hidden_size"])
+    assert err <= bound and rel <= 2e-3  # the linear tolerance of the hot path
