@@ -89,10 +89,12 @@ MI355GQ_API int mi355gq_embedding_take(const void* ids, int64_t T, const void* q
  * (compiler_pass/fuse_dequantize_matmul_ewise.py, fuse_transpose_matmul.py:64-143):
  *   y[M, N] = x[M, K] . dequantize(q_weight, q_scale)[N, K]^T (+ bias[N])
  * x fp16, bias fp16 or NULL, y fp16 (MI355GQ_F16) or fp32 (MI355GQ_F32); fp32 accumulation.
- * M <= 8 runs the decode GEMV, larger M the MFMA GEMM (the regime split of
+ * M <= 8 runs the decode GEMV / few-row kernels, larger M the MFMA GEMM (the regime split of
  * compiler_pass/low_batch_specialization.py:22-57).
- * workspace: device scratch, may be NULL with workspace_bytes = 0 when
- * mi355gq_linear_workspace_bytes() returns 0 for the shape.
+ * workspace: device scratch, 16-byte aligned, of at least mi355gq_linear_workspace_bytes()
+ * bytes for the shape; only the GEMM with 17..256 rows asks for any (fp32 partial sums of its
+ * split along K).  NULL or too small is not an error: the same tiles run unsplit, slower.
+ * Its contents are undefined afterwards; calls that share a workspace must be stream-ordered.
  */
 MI355GQ_API int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size);
 MI355GQ_API int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, const void* bias,

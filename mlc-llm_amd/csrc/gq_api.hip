@@ -150,14 +150,18 @@ int mi355gq_embedding_take(const void* ids, int64_t T, const void* q_weight, con
 }
 
 int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
-  (void)M; (void)N; (void)K; (void)bits; (void)group_size;
-  return 0;  // no kernel of this build needs scratch
+  if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
+      N >= kMaxDim || K >= kMaxDim)
+    return 0;
+  // only the few-row GEMM (more rows than the GEMV / skinny kernels take, at most 256) splits K
+  if (M <= 16 && bits == 4) return 0;
+  if (M <= 8) return 0;
+  return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
 }
 
 int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, const void* bias,
                    int64_t M, int64_t N, int64_t K, int bits, int group_size, int out_dtype,
                    void* y, void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
-  (void)workspace;
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
              "linear: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
@@ -192,6 +196,7 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
   g.indptr = nullptr; g.indptr_i64 = 0;
   g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
   g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
+  g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
   const int gv = gq::options().gemv_variant;  // 2..5 force a gq_skinny.hip form, 6..8 the quad-row kernel
   if (M <= 16 && bits == 4 && gq::options().gemm_variant != 1) {
     if ((gv < 0 && M <= 8) || (gv >= 6 && gv <= 8)) {

@@ -210,10 +210,34 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   p.expert_s_stride = a.N * p.ng;
   p.num_experts = static_cast<int>(a.num_experts);
   p.out_f32 = a.out_f32;
+  p.partial = nullptr;
+  p.kt_per_split = 1 << 28;  // one workgroup walks all of K
+  p.bm_hint = 0;
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int variant = options().gemm_variant;
+  if (variant < 0) {
+    const SplitPlan plan = plan_split_k(a.rows, a.N, a.K, a.bits, a.group_size, a.indptr != nullptr);
+    p.bm_hint = plan.bm;
+    const int64_t need = static_cast<int64_t>(plan.split) * a.rows * a.N * 4;
+    // without (enough) scratch the same tiles run unsplit: slower, never wrong
+    if (plan.bm > 0 && plan.split > 1 && a.workspace != nullptr && a.workspace_bytes >= need &&
+        (reinterpret_cast<uintptr_t>(a.workspace) & 15) == 0) {
+      p.partial = static_cast<float*>(a.workspace);
+      p.kt_per_split = plan.kt_per_split;
+    }
+  }
   if (variant != 3 && variant != 4 && variant != 5) {
     const hipError_t e = launch_gemm_pipe(p, a.bits, s);
+    if (e == hipSuccess && p.partial != nullptr) {
+      const int64_t count = a.rows * a.N;
+      const int nk = (p.ng + 1) / 2;
+      const int split = (nk + p.kt_per_split - 1) / p.kt_per_split;
+      int64_t blocks = (count / 4 + 255) / 256;
+      blocks = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
+      hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
+                         p.partial, split, count, p.N, p.bias, p.y, p.out_f32);
+      return hipGetLastError();
+    }
     if (e != hipErrorNotSupported) return e;
   }
   if (a.bits == 4) {
@@ -225,6 +249,12 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
     return launch_cfg<4, 128, 128, 64, 64>(p, s);
   }
   return launch_cfg<3, 128, 128, 64, 64>(p, s);
+}
+
+int64_t gemm_workspace_bytes(int64_t rows, int64_t N, int64_t K, int bits, int group_size) {
+  if (options().gemm_variant >= 0) return 0;
+  const SplitPlan plan = plan_split_k(rows, N, K, bits, group_size, false);
+  return plan.bm > 0 && plan.split > 1 ? static_cast<int64_t>(plan.split) * rows * N * 4 : 0;
 }
 
 }  // namespace gq

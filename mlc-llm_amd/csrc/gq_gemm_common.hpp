@@ -29,7 +29,23 @@ struct GemmParams {
   int rows, N, K, ng, nw;
   int num_experts;
   int out_f32, indptr_i64;
+  // split-K: workgroup z multiplies K tiles [z * kt_per_split, (z + 1) * kt_per_split) and, when
+  // `partial` is set, leaves its fp32 tile in partial[z][rows][N] for the reduction kernel
+  float* partial;
+  int kt_per_split;
+  int bm_hint;  // rows per tile chosen by plan_split_k (0: regular tiles)
 };
+
+__global__ void splitk_reduce_kernel(const float* partial, int split, int64_t count, int N,
+                                     const uint16_t* bias, void* y, int out_f32);
+
+// How a few-row GEMM is cut so that every CU streams weights: rows per tile and K splits.
+struct SplitPlan {
+  int bm;            // 0: not a few-row problem, use the regular tiles
+  int split;         // workgroups along K (1: no reduction pass)
+  int kt_per_split;  // K tiles (2 groups each) per workgroup
+};
+SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_size, bool grouped);
 
 // One group (4 storage words) -> G halves in natural k order, (q - m) * s with fp16 rounding.
 template <int BITS>

@@ -73,6 +73,13 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     w_dst[i] = r * LDA + gsel * G;
   }
 
+  // this workgroup's share of K (all of it unless the launch splits K)
+  const int nk = (p.ng + 1) / 2;
+  const int kt0 = blockIdx.z * p.kt_per_split;
+  const int kt1 = min(nk, kt0 + p.kt_per_split);
+  const int k_lim = min(p.K, kt1 * BK);  // k and groups from here on contribute nothing
+  const int g_lim = min(p.ng, 2 * kt1);
+
   struct Stage {
     uint4 a[A_CHUNKS];
     uint4 w[W_GROUPS];
@@ -85,7 +92,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     const int k_base = kt * BK;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
-      const bool ok = k_base + a_k[i] < p.K;  // K % 8 == 0: a chunk is entirely inside or outside
+      const bool ok = k_base + a_k[i] < k_lim;  // K % 8 == 0: a chunk is entirely inside or outside
       st.a[i] = *reinterpret_cast<const uint4*>(ok ? a_src[i] + k_base : a_src[i]);
     }
 #pragma unroll
@@ -106,12 +113,12 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       if (i % KSTEPS != part) continue;
-      const bool ok = a_row_ok[i] && (k_base + a_k[i] < p.K);
+      const bool ok = a_row_ok[i] && (k_base + a_k[i] < k_lim);
       *reinterpret_cast<uint4*>(at + a_dst[i]) = ok ? st.a[i] : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < W_GROUPS; ++i) {
-      const bool ok = 2 * kt + w_g[i] < p.ng;
+      const bool ok = 2 * kt + w_g[i] < g_lim;
       // a group past the end gets scale +0.0: every value becomes (q - m) * 0 = +-0
       const uint16_t sb = ok ? static_cast<uint16_t>(st.s[i]) : uint16_t(0);
       uint4* dst = reinterpret_cast<uint4*>(wt + w_dst[i]);
@@ -174,15 +181,14 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   };
 
   // ---- pipeline: tile t in LDS stage t&1, tile t+1 in registers, tile t+2 in flight
-  const int nk = (p.ng + 1) / 2;
-  load_tile(0, r0);
-  load_tile(1, r1);
-  store_tile(0, r0, 0);
-  load_tile(2, r0);
+  load_tile(kt0, r0);
+  load_tile(kt0 + 1, r1);
+  store_tile(kt0, r0, 0);
+  load_tile(kt0 + 2, r0);
   __syncthreads();
   // (registers of tile t+2 are overwritten only after tile t+1 has left them for LDS, so the
   //  refill of a register stage is issued right after the MFMA/store block that drains it)
-  for (int kt = 0; kt < nk; kt += 2) {
+  for (int kt = kt0; kt < kt1; kt += 2) {
     mfma_tile(0, kt + 1, r1);  // a tile past the end is stored as zeros and adds nothing
     load_tile(kt + 3, r1);
     __syncthreads();
@@ -197,11 +203,13 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int col = n0 + wn0 + j * 32 + (lane & 31);
-      const float b = (p.bias != nullptr && col < p.N) ? h2f(p.bias[col]) : 0.f;
+      const float b = (p.bias != nullptr && p.partial == nullptr && col < p.N) ? h2f(p.bias[col]) : 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (row < seg_hi && col < p.N) {
+        if (row < seg_hi && col < p.N && p.partial != nullptr) {
+          p.partial[(static_cast<int64_t>(blockIdx.z) * p.rows + row) * p.N + col] = acc[i][j][r];
+        } else if (row < seg_hi && col < p.N) {
           const float v = acc[i][j][r] + b;
           const int64_t o = static_cast<int64_t>(row) * p.N + col;
           if (p.out_f32) static_cast<float*>(p.y)[o] = v;
@@ -225,14 +233,90 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
     if (e != hipSuccess) return e;
   }
   const int m_tiles = p.indptr ? (p.rows + BM - 1) / BM + p.num_experts : (p.rows + BM - 1) / BM;
-  const dim3 grid((p.N + BN - 1) / BN, m_tiles);
+  const int nk = (p.ng + 1) / 2;
+  const int split = p.partial ? (nk + p.kt_per_split - 1) / p.kt_per_split : 1;
+  const dim3 grid((p.N + BN - 1) / BN, m_tiles, split);
   hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
   return hipGetLastError();
+}
+
+// y = sum over splits of partial[s] + bias, in the output type
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int split,
+                                                            int64_t count /* rows * N */, int N,
+                                                            const uint16_t* __restrict__ bias,
+                                                            void* __restrict__ y, int out_f32) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  if ((N & 3) == 0) {  // rows are 16-byte aligned: four columns per thread
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; 4 * i < count; i += stride) {
+      float4 a = *reinterpret_cast<const float4*>(partial + 4 * i);
+      for (int sidx = 1; sidx < split; ++sidx) {
+        const float4 b = *reinterpret_cast<const float4*>(partial + sidx * count + 4 * i);
+        a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+      }
+      if (bias != nullptr) {
+        const int col = static_cast<int>((4 * i) % N);
+        const uint2 bb = *reinterpret_cast<const uint2*>(bias + col);
+        a.x += h2f(static_cast<uint16_t>(bb.x & 0xffffu)); a.y += h2f(static_cast<uint16_t>(bb.x >> 16));
+        a.z += h2f(static_cast<uint16_t>(bb.y & 0xffffu)); a.w += h2f(static_cast<uint16_t>(bb.y >> 16));
+      }
+      if (out_f32) {
+        *reinterpret_cast<float4*>(static_cast<float*>(y) + 4 * i) = a;
+      } else {
+        uint2 o;
+        o.x = static_cast<uint32_t>(f2h(a.x)) | (static_cast<uint32_t>(f2h(a.y)) << 16);
+        o.y = static_cast<uint32_t>(f2h(a.z)) | (static_cast<uint32_t>(f2h(a.w)) << 16);
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + 4 * i) = o;
+      }
+    }
+  } else {
+    for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < count; i += stride) {
+      float a = partial[i];
+      for (int sidx = 1; sidx < split; ++sidx) a += partial[sidx * count + i];
+      if (bias != nullptr) a += h2f(bias[i % N]);
+      if (out_f32) static_cast<float*>(y)[i] = a;
+      else static_cast<uint16_t*>(y)[i] = f2h(a);
+    }
+  }
+}
+
+SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_size, bool grouped) {
+  SplitPlan plan{0, 1, 1 << 28};
+  if (grouped || rows <= 0 || N <= 0 || K <= 0 || (K & 7) != 0) return plan;
+  // few rows: the GEMM is bound by streaming the weights, and 128-wide column tiles alone leave
+  // most CUs idle (o_proj / down have 32 of them).  Match the tile height to the rows and cut K
+  // until about two workgroups per CU exist.
+  if (rows > 256) return plan;
+  const int bm = bits == 4 ? (rows <= 32 ? 32 : (rows <= 64 ? 64 : 128)) : 128;
+  const int64_t tiles = ((rows + bm - 1) / bm) * ((N + 127) / 128);
+  if (rows > 128 && tiles >= 200) return plan;  // the regular tiles already fill the chip
+  plan.bm = bm;
+  const int ng = static_cast<int>((K + group_size - 1) / group_size);
+  const int nk = (ng + 1) / 2;
+  // Splitting K pays with partial sums (split * rows * N * 8 bytes written and read back): only
+  // when the tiles alone leave CUs idle, and never beyond about twice the weight bytes.
+  int split = 1;
+  if (tiles < 200 || options().gemv_split > 0) {
+    const int64_t want = options().gemv_split > 0 ? options().gemv_split : 512;  // tuning override
+    split = static_cast<int>((want + tiles - 1) / tiles);
+    const int64_t cap = K / (7 * rows);
+    if (options().gemv_split <= 0 && split > cap) split = static_cast<int>(cap);
+    if (split > nk / 4) split = nk / 4;  // at least four K tiles per workgroup
+    if (split < 1) split = 1;
+  }
+  plan.kt_per_split = (nk + split - 1) / split;
+  plan.split = (nk + plan.kt_per_split - 1) / plan.kt_per_split;
+  return plan;
 }
 
 hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   if ((p.K & 7) != 0 || p.ng == 0) return hipErrorNotSupported;
   const int variant = options().gemm_variant;
+  if (p.bm_hint > 0 && variant < 0) {
+    if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32>(p, s);
+    if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64>(p, s);
+    if (bits == 4) return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
+    return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
+  }
   if (bits == 4) {
     const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
     const bool big = variant == 7 ? true : (variant == 6 ? false : (p.indptr == nullptr && big_tiles >= 160));

@@ -42,8 +42,12 @@ struct GemmArgs {
   int indptr_i64;
   int64_t rows, N, K, num_experts;
   int bits, group_size, out_f32;
+  void* workspace = nullptr;       // caller's scratch for split-K partial sums (may be null)
+  int64_t workspace_bytes = 0;
 };
 hipError_t launch_gemm(const GemmArgs& a, hipStream_t s);
+// scratch the split-K form of the GEMM wants for this shape (0 when it does not split)
+int64_t gemm_workspace_bytes(int64_t rows, int64_t N, int64_t K, int bits, int group_size);
 // MFMA kernel for few activation rows per segment (q4 only; hipErrorNotSupported otherwise).
 // rows_max bounds the rows of any one segment.
 hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s);

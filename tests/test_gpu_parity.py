@@ -378,6 +378,46 @@ def test_gemm_kernel_variants(variant, m, n, k):
     assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"gemm variant {variant} {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("m", [17, 32, 33, 64, 100, 129, 256])
+@pytest.mark.parametrize("n,k", [(520, 4096), (130, 14336), (384, 1000)])
+def test_few_row_gemm_split_k(name, m, n, k):
+    # 17..256 rows: tile height follows the rows and K is cut across workgroups, partial sums go
+    # through the workspace and a reduction kernel (bias and the output type are applied there)
+    s = SCHEMES[name]
+    x, qw, qs, b = _linear_case(s, m, n, k, 13 * m + n + k, bias=True)
+    ws = gq._lib.lib().mi355gq_linear_workspace_bytes(m, n, k, s.bits, s.group_size)
+    y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
+    y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
+    ref = o.linear_fp32(x, qw, qs, s, b)
+    assert_linear_ok(y, ref, x, k, f"few-row gemm {name} {m}x{n}x{k} (workspace {ws} B)")
+    assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"few-row gemm {name} fp32 out")
+    if k >= 4096:
+        assert ws > 0 and ws % (m * n * 4) == 0  # these shapes do split
+
+
+@pytest.mark.parametrize("want", [64, 4096])  # few / as many splits as K allows
+def test_few_row_gemm_split_counts_and_missing_workspace(want):
+    s = SCHEMES["q4f16_1"]
+    m, n, k = 40, 260, 8192
+    x, qw, qs, b = _linear_case(s, m, n, k, 99, bias=True)
+    ref = o.linear_fp32(x, qw, qs, s, b)
+    gq._lib.set_option("gemv_split", want)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b))
+        ws = gq._lib.lib().mi355gq_linear_workspace_bytes(m, n, k, 4, 32)
+    finally:
+        gq._lib.set_option("gemv_split", -1)
+    assert ws > 0
+    assert_linear_ok(y, ref, x, k, f"few-row gemm, {want} workgroups wanted")
+    # no workspace handed over: same tiles, no split, same answer
+    xd, qwd, qsd, bd = dev(x), dev(qw), dev(qs), dev(b)
+    out = torch.empty((m, n), dtype=torch.float16, device=xd.device)
+    gq._lib.call("mi355gq_linear", xd.data_ptr(), qwd.data_ptr(), qsd.data_ptr(), bd.data_ptr(), m, n, k, 4, 32,
+                 gq._lib.F16, out.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+    assert_linear_ok(out, ref, x, k, "few-row gemm without workspace")
+
+
 def test_gemm_k_not_multiple_of_8_takes_fallback():
     # K = 100: rows of x are not 16-byte aligned, the pipelined kernel declines and the plain one runs
     for name in ("q4f16_1", "q3f16_1"):
