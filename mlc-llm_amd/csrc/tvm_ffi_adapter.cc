@@ -1,6 +1,6 @@
 // TVM-FFI adapter: registers the C ABI of include/mi355gq.h as global packed functions, so that
 // a Relax module can reach the kernels through
-//     R.call_dps_packed("mlc.gq.linear", (x, q_weight, q_scale, bits, group_size), out_sinfo=...)
+//     R.call_dps_packed("mlc.gq.linear", (x, q_weight, q_scale, bias, bits, group_size, workspace), out_sinfo=...)
 // the same way the reference reaches "fastertransformer.gemm_fp16_int"
 // (python/mlc_llm/op/ft_gemm.py:72-92) or "cutlass.group_gemm" (op/cutlass.py:71-77).
 // Registration follows the reference's own idiom (cpp/multi_gpu/builtin.cc:89-94).
@@ -54,15 +54,27 @@ inline int OutDtype(const TensorView& y) { return y.dtype().bits == 32 ? MI355GQ
 
 }  // namespace
 
-// y = x . dequantize(q_weight, q_scale)^T (+ bias)
+// y = x . dequantize(q_weight, q_scale)^T (+ bias).  `workspace` is an optional uint8 scratch
+// tensor of at least mlc.gq.linear_workspace_bytes(M, N, K, bits, group_size) bytes (the few-row
+// GEMM splits K through it); without it the call is still correct, only slower for 17..256 rows.
 void Linear(TensorView x, TensorView q_weight, TensorView q_scale, Optional<TensorView> bias,
-            int64_t bits, int64_t group_size, TensorView y) {
+            int64_t bits, int64_t group_size, Optional<TensorView> workspace, TensorView y) {
   const int64_t K = x.shape()[x.ndim() - 1], N = q_weight.shape()[0];
+  void* ws = workspace.has_value() ? Ptr(workspace.value()) : nullptr;
+  int64_t ws_bytes = 0;
+  if (workspace.has_value()) {
+    ws_bytes = (workspace.value().dtype().bits + 7) / 8;
+    for (int i = 0; i < workspace.value().ndim(); ++i) ws_bytes *= workspace.value().shape()[i];
+  }
   Check(mi355gq_linear(Ptr(x), Ptr(q_weight), Ptr(q_scale),
                        bias.has_value() ? Ptr(bias.value()) : nullptr, Rows(x), N, K,
                        static_cast<int>(bits), static_cast<int>(group_size), OutDtype(y), Ptr(y),
-                       nullptr, 0, StreamOf(x)),
+                       ws, ws_bytes, StreamOf(x)),
         "mlc.gq.linear");
+}
+
+int64_t LinearWorkspaceBytes(int64_t M, int64_t N, int64_t K, int64_t bits, int64_t group_size) {
+  return mi355gq_linear_workspace_bytes(M, N, K, static_cast<int>(bits), static_cast<int>(group_size));
 }
 
 void EmbeddingTake(TensorView ids, TensorView q_weight, TensorView q_scale, int64_t bits,
@@ -114,6 +126,7 @@ TVM_FFI_STATIC_INIT_BLOCK() {
   namespace refl = tvm::ffi::reflection;
   refl::GlobalDef()
       .def("mlc.gq.linear", Linear)
+      .def("mlc.gq.linear_workspace_bytes", LinearWorkspaceBytes)
       .def("mlc.gq.embedding_take", EmbeddingTake)
       .def("mlc.gq.moe_gemv", MoeGemv)
       .def("mlc.gq.moe_group_gemm", MoeGroupGemm)
