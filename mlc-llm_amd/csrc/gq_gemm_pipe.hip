@@ -12,7 +12,9 @@
 
 namespace gq {
 
-template <int BITS, int BM, int BN, int WM, int WN>
+// DEPTH: K tiles of global loads in flight (register stages); even, 2 for the large tiles, more
+// for few-row tiles whose MFMA work per tile is far shorter than a trip to memory
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(const GemmParams p) {
   using T = GemmTraits<BITS>;
   constexpr int G = T::G;
@@ -85,7 +87,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     uint4 w[W_GROUPS];
     uint32_t s[W_GROUPS];  // fp16 scale bits (32 bits wide on purpose: in flight, never re-packed)
   };
-  Stage r0, r1;
+  static_assert(DEPTH >= 2 && DEPTH % 2 == 0, "register stages pair up with the two LDS stages");
+  Stage r[DEPTH];
 
   // K tile kt into registers.  Always valid addresses; validity is re-derived at store time.
   auto load_tile = [&](int kt, Stage& st) {
@@ -154,47 +157,50 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   auto mfma_tile = [&](int s, int kt_store, const Stage& st_store) {
     const uint16_t* at = a_tile(s) + (wm0 + frag_row) * LDA + frag_k;
     const uint16_t* wt = w_tile(s) + (wn0 + frag_row) * LDA + frag_k;
-    half8_t af[2][TM], bf[2][TN];
+    {  // fragments of k-step s+1 are read while the MFMAs of step s run
+      half8_t af[2][TM], bf[2][TN];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA);
+      for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA);
+      for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA);
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks + 1 < KSTEPS) {
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        if (ks + 1 < KSTEPS) {
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+            af[nxt][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA + (ks + 1) * 16);
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            bf[nxt][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA + (ks + 1) * 16);
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-          af[nxt][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA + (ks + 1) * 16);
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          bf[nxt][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA + (ks + 1) * 16);
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+        store_part(kt_store, st_store, s ^ 1, ks);
+        __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
       }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
-      store_part(kt_store, st_store, s ^ 1, ks);
-      __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
     }
   };
 
   // ---- pipeline: tile t in LDS stage t&1, tile t+1 in registers, tile t+2 in flight
-  load_tile(kt0, r0);
-  load_tile(kt0 + 1, r1);
-  store_tile(kt0, r0, 0);
-  load_tile(kt0 + 2, r0);
+  // ---- pipeline: tile t in LDS stage t&1, tiles t+1 .. t+DEPTH-1 in registers, tile t+DEPTH in flight
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) load_tile(kt0 + d, r[d]);
+  store_tile(kt0, r[0], 0);
+  load_tile(kt0 + DEPTH, r[0]);
   __syncthreads();
-  // (registers of tile t+2 are overwritten only after tile t+1 has left them for LDS, so the
-  //  refill of a register stage is issued right after the MFMA/store block that drains it)
-  for (int kt = kt0; kt < kt1; kt += 2) {
-    mfma_tile(0, kt + 1, r1);  // a tile past the end is stored as zeros and adds nothing
-    load_tile(kt + 3, r1);
-    __syncthreads();
-    mfma_tile(1, kt + 2, r0);
-    load_tile(kt + 4, r0);
-    __syncthreads();
+  // (a register stage is refilled right after the MFMA/store block that drains it; a tile past
+  //  the end is stored as zeros and adds nothing)
+  for (int kt = kt0; kt < kt1; kt += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      mfma_tile(d & 1, kt + d + 1, r[(d + 1) % DEPTH]);
+      load_tile(kt + d + 1 + DEPTH, r[(d + 1) % DEPTH]);
+      __syncthreads();
+    }
   }
 
   // ---- epilogue: D[i][j] of a 32x32 tile sits in lane (j + 32*((i/4)%2)), register 4*(i/8) + i%4
@@ -220,12 +226,12 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   }
 }
 
-template <int BITS, int BM, int BN, int WM, int WN>
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2>
 static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr int BK = 2 * GemmTraits<BITS>::G;
   constexpr int LDA = BK + 8;
   constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
-  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN>;
+  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH>;
   if (lds > 65536) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                              hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -303,7 +309,8 @@ SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_s
     if (split > nk / 4) split = nk / 4;  // at least four K tiles per workgroup
     if (split < 1) split = 1;
   }
-  plan.kt_per_split = (nk + split - 1) / split;
+  // the K loop advances four tiles at a time in the few-row kernels: whole rounds per workgroup
+  plan.kt_per_split = ((nk + split - 1) / split + 3) / 4 * 4;
   plan.split = (nk + plan.kt_per_split - 1) / plan.kt_per_split;
   return plan;
 }
@@ -312,8 +319,8 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   if ((p.K & 7) != 0 || p.ng == 0) return hipErrorNotSupported;
   const int variant = options().gemm_variant;
   if (p.bm_hint > 0 && variant < 0) {
-    if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32>(p, s);
-    if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64>(p, s);
+    if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4>(p, s);
+    if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4>(p, s);
     if (bits == 4) return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
     return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
   }
