@@ -177,7 +177,7 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
     roofline = {
-        "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2> (gate_up 28672x4096, batch 1)",
+        "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2,false> (gate_up 28672x4096, batch 1)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
         "bytes_per_launch": gu_bytes, "us_per_launch": round(us_gate_up, 3),

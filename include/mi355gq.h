@@ -102,6 +102,21 @@ MI355GQ_API int mi355gq_linear(const void* x, const void* q_weight, const void* 
                    void* y, void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream);
 
 /*
+ * The same linear with the element-wise tail the reference folds into the matmul kernel:
+ * FuseDequantizeMatmulEwise (compiler_pass/fuse_dequantize_matmul_ewise.py:19-32) fuses the
+ * dequantize + matmul pair together with up to three element-wise operands that operator fusion
+ * attached to the matmul, which for a decoder layer is the residual addition after o_proj and
+ * after down_proj (model/llama/llama_model.py:204-215):
+ *   y[M, N] = x . W^T (+ bias[N]) + residual[M, N]
+ * residual is fp16; it may be y itself when y is fp16 (hidden += proj(x)): every element is read
+ * before it is written, by the same lane.  Accumulation and both additions are fp32, rounded once.
+ */
+MI355GQ_API int mi355gq_linear_residual(const void* x, const void* q_weight, const void* q_scale,
+                            const void* bias, const void* residual, int64_t M, int64_t N, int64_t K,
+                            int bits, int group_size, int out_dtype, void* y, void* workspace,
+                            int64_t workspace_bytes, mi355gq_stream_t stream);
+
+/*
  * moe_matmul.dequantize_gemv (python/mlc_llm/op/moe_matmul.py:77-176), single-token MoE:
  *   out[e, :] = x[x_rows == 1 ? 0 : e, :] . dequantize(W[expert_ids[e]])^T,  e < top_k
  * x fp16 [x_rows, K] with x_rows in {1, top_k}; expert_ids int32 [1, top_k];

@@ -159,9 +159,10 @@ int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits
   return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
 }
 
-int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, const void* bias,
-                   int64_t M, int64_t N, int64_t K, int bits, int group_size, int out_dtype,
-                   void* y, void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
+static int linear_impl(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                       const void* residual, int64_t M, int64_t N, int64_t K, int bits, int group_size,
+                       int out_dtype, void* y, void* workspace, int64_t workspace_bytes,
+                       mi355gq_stream_t stream) {
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
              "linear: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
@@ -171,8 +172,11 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
   GQ_REQUIRE(y != nullptr, "linear: y is null");
   GQ_REQUIRE(K == 0 || (x && q_weight && q_scale), "linear: null pointer");
   GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned2(q_scale) && aligned4(y) &&
-                 aligned2(bias),
+                 aligned2(bias) && aligned2(residual),
              "linear: x and q_weight must be 16-byte aligned");
+  // y may be the residual buffer itself (same element type), nothing else may overlap it
+  GQ_REQUIRE(residual == nullptr || residual != y || out_dtype == MI355GQ_F16,
+             "linear: in-place residual needs a float16 output");
   // regimes: M <= 2 register GEMV; 3..16 MFMA skinny kernel (q4) or LDS GEMV up to 8 (q3); else GEMM
   const bool use_gemv = M <= 2 || (M <= 8 && (bits != 4 || gq::options().gemm_variant == 2));
   if (use_gemv) {
@@ -181,6 +185,7 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
     a.q_weight = static_cast<const uint32_t*>(q_weight);
     a.q_scale = static_cast<const uint16_t*>(q_scale);
     a.bias = static_cast<const uint16_t*>(bias);
+    a.residual = static_cast<const uint16_t*>(residual);
     a.y = y;
     a.expert_ids = nullptr;
     a.M = M; a.N = N; a.K = K; a.slots = 1; a.x_slot_stride = 0; a.num_experts = 1;
@@ -192,6 +197,7 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
   g.q_weight = static_cast<const uint32_t*>(q_weight);
   g.q_scale = static_cast<const uint16_t*>(q_scale);
   g.bias = static_cast<const uint16_t*>(bias);
+  g.residual = static_cast<const uint16_t*>(residual);
   g.y = y;
   g.indptr = nullptr; g.indptr_i64 = 0;
   g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
@@ -207,6 +213,22 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
     if (e != hipErrorNotSupported) return hip_result(e, "skinny launch");
   }
   return hip_result(gq::launch_gemm(g, as_stream(stream)), "gemm launch");
+}
+
+int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                   int64_t M, int64_t N, int64_t K, int bits, int group_size, int out_dtype,
+                   void* y, void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
+  return linear_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, out_dtype, y,
+                     workspace, workspace_bytes, stream);
+}
+
+int mi355gq_linear_residual(const void* x, const void* q_weight, const void* q_scale,
+                            const void* bias, const void* residual, int64_t M, int64_t N, int64_t K,
+                            int bits, int group_size, int out_dtype, void* y, void* workspace,
+                            int64_t workspace_bytes, mi355gq_stream_t stream) {
+  GQ_REQUIRE(residual != nullptr || M == 0 || N == 0, "linear_residual: residual is null");
+  return linear_impl(x, q_weight, q_scale, bias, residual, M, N, K, bits, group_size, out_dtype, y,
+                     workspace, workspace_bytes, stream);
 }
 
 int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,

@@ -171,8 +171,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_kernel(const 
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (row < seg_hi && col < p.N) {
-          const float v = acc[i][j][r] + b;
           const int64_t o = static_cast<int64_t>(row) * p.N + col;
+          const float v = acc[i][j][r] + b + (p.residual != nullptr ? h2f(p.residual[o]) : 0.f);
           if (p.out_f32) static_cast<float*>(p.y)[o] = v;
           else static_cast<uint16_t*>(p.y)[o] = f2h(v);
         }
@@ -201,7 +201,7 @@ static hipError_t launch_cfg(const GemmParams& p, hipStream_t s) {
 
 hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   GemmParams p;
-  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.y = a.y;
+  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
   p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64;
   p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
   p.ng = static_cast<int>((a.K + a.group_size - 1) / a.group_size);
@@ -235,7 +235,7 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
       int64_t blocks = (count / 4 + 255) / 256;
       blocks = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
       hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
-                         p.partial, split, count, p.N, p.bias, p.y, p.out_f32);
+                         p.partial, split, count, p.N, p.bias, p.residual, p.y, p.out_f32);
       return hipGetLastError();
     }
     if (e != hipErrorNotSupported) return e;

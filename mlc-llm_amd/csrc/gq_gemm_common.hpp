@@ -23,6 +23,7 @@ struct GemmParams {
   const uint32_t* qw;
   const uint16_t* qs;
   const uint16_t* bias;
+  const uint16_t* residual;  // [rows, N] or null
   void* y;
   const void* indptr;
   int64_t expert_w_stride, expert_s_stride;
@@ -37,7 +38,7 @@ struct GemmParams {
 };
 
 __global__ void splitk_reduce_kernel(const float* partial, int split, int64_t count, int N,
-                                     const uint16_t* bias, void* y, int out_f32);
+                                     const uint16_t* bias, const uint16_t* residual, void* y, int out_f32);
 
 // How a few-row GEMM is cut so that every CU streams weights: rows per tile and K splits.
 struct SplitPlan {

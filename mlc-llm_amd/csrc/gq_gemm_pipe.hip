@@ -216,8 +216,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
         if (row < seg_hi && col < p.N && p.partial != nullptr) {
           p.partial[(static_cast<int64_t>(blockIdx.z) * p.rows + row) * p.N + col] = acc[i][j][r];
         } else if (row < seg_hi && col < p.N) {
-          const float v = acc[i][j][r] + b;
           const int64_t o = static_cast<int64_t>(row) * p.N + col;
+          const float v = acc[i][j][r] + b + (p.residual != nullptr ? h2f(p.residual[o]) : 0.f);
           if (p.out_f32) static_cast<float*>(p.y)[o] = v;
           else static_cast<uint16_t*>(p.y)[o] = f2h(v);
         }
@@ -246,11 +246,12 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   return hipGetLastError();
 }
 
-// y = sum over splits of partial[s] + bias, in the output type
+// y = sum over splits of partial[s] + bias + residual, in the output type (y may be the residual
+// buffer itself: every element is read before the same thread writes it)
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int split,
                                                             int64_t count /* rows * N */, int N,
                                                             const uint16_t* __restrict__ bias,
-                                                            void* __restrict__ y, int out_f32) {
+                                                            const uint16_t* residual, void* y, int out_f32) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   if ((N & 3) == 0) {  // rows are 16-byte aligned: four columns per thread
     for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; 4 * i < count; i += stride) {
@@ -264,6 +265,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
         const uint2 bb = *reinterpret_cast<const uint2*>(bias + col);
         a.x += h2f(static_cast<uint16_t>(bb.x & 0xffffu)); a.y += h2f(static_cast<uint16_t>(bb.x >> 16));
         a.z += h2f(static_cast<uint16_t>(bb.y & 0xffffu)); a.w += h2f(static_cast<uint16_t>(bb.y >> 16));
+      }
+      if (residual != nullptr) {
+        const uint2 rr = *reinterpret_cast<const uint2*>(residual + 4 * i);
+        a.x += h2f(static_cast<uint16_t>(rr.x & 0xffffu)); a.y += h2f(static_cast<uint16_t>(rr.x >> 16));
+        a.z += h2f(static_cast<uint16_t>(rr.y & 0xffffu)); a.w += h2f(static_cast<uint16_t>(rr.y >> 16));
       }
       if (out_f32) {
         *reinterpret_cast<float4*>(static_cast<float*>(y) + 4 * i) = a;
@@ -279,6 +285,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
       float a = partial[i];
       for (int sidx = 1; sidx < split; ++sidx) a += partial[sidx * count + i];
       if (bias != nullptr) a += h2f(bias[i % N]);
+      if (residual != nullptr) a += h2f(residual[i]);
       if (out_f32) static_cast<float*>(y)[i] = a;
       else static_cast<uint16_t*>(y)[i] = f2h(a);
     }

@@ -184,8 +184,8 @@ __global__ __launch_bounds__(256) void gemv_dot2_kernel(const GemvParams p) {
       const float v = wave_sum(acc[r][b]);
       const int row = row0 + r;
       if (lane == 0 && row < p.N) {
-        const float o = v + (p.bias ? h2f(p.bias[row]) : 0.f);
         const int64_t oi = static_cast<int64_t>(slot + b) * p.N + row;  // slot > 0 only when NB == 1
+        const float o = v + (p.bias ? h2f(p.bias[row]) : 0.f) + (p.residual ? h2f(p.residual[oi]) : 0.f);
         if (p.out_f32) static_cast<float*>(p.y)[oi] = o;
         else static_cast<uint16_t*>(p.y)[oi] = f2h(o);
       }
@@ -246,7 +246,7 @@ hipError_t launch_gemv_lds(const GemvParams& p_in, int bits, int nb, int slots, 
 
 hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
   GemvParams p;
-  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.y = a.y;
+  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
   p.expert_ids = a.expert_ids;
   p.x_slot_stride = a.x_slot_stride;
   p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);

@@ -25,6 +25,7 @@ struct GemvParams {
   const uint32_t* qw;
   const uint16_t* qs;
   const uint16_t* bias;
+  const uint16_t* residual;  // [M, N] or null
   void* y;
   const int32_t* expert_ids;
   int64_t x_slot_stride;

@@ -16,7 +16,9 @@
 
 namespace gq {
 
-template <int BITS, int NB, int R, int ITERS>
+// EXTRA: a bias or residual operand exists (a template flag rather than a run-time test: their loads are
+// two more memory instructions per set, measured at 4-6 % of the plain GEMV's time).
+template <int BITS, int NB, int R, int ITERS, bool EXTRA>
 __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int nsets) {
   using T = GemvTraits<BITS>;
   constexpr int G = T::G;
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
   //      every path issues the same loads.  A set past the end reads one cached line instead.
   uint4 wa[R][ITERS], wb[R][ITERS];
   uint32_t sa[R][ITERS], sb[R][ITERS];  // fp16 bits, kept 32 bits wide so that the in-flight values are never re-packed
-  uint32_t ba = 0, bb = 0;
+  uint32_t ba = 0, bb = 0;  // low half: bias bits, high half: residual bits (lane r + R * b carries element (b, r))
   auto issue = [&](int set, uint4 (&wn)[R][ITERS], uint32_t (&sn)[R][ITERS], uint32_t& bn) {
     const bool live = set < nsets;
 #pragma unroll
@@ -88,9 +90,17 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
         sn[r][it] = *(live ? sr + gidx[it] : qs);
       }
     }
+    if constexpr (!EXTRA) return;
     // lane r carries the bias of row r of the set (read back with readlane at store time)
     const int brow = min(set * R + min(lane, R - 1), p.N - 1);
     bn = *((live && p.bias != nullptr) ? p.bias + brow : qs);
+    // the residual rides with the set's loads too: fetched at store time it would sit behind the
+    // next sets' weights in the in-order load queue and stall the wave until they all land
+    const int e = min(lane, R * NB - 1);
+    const int rrow = min(set * R + e % R, p.N - 1);
+    const uint32_t rb = *((live && p.residual != nullptr)
+                              ? p.residual + static_cast<int64_t>(slot + e / R) * p.N + rrow : qs);
+    bn |= rb << 16;
   };
   int set_a = gw, set_b = gw + nwaves;
   issue(set_a, wa, sa, ba);
@@ -146,16 +156,24 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
         }
         acc[r][b] = wave_sum_last(a);
       }
-    const float bias_lane = p.bias != nullptr ? h2f(static_cast<uint16_t>(bias_bits)) : 0.f;
+    const float bias_lane = (EXTRA && p.bias != nullptr) ? h2f(static_cast<uint16_t>(bias_bits & 0xffffu)) : 0.f;
+    const float res_lane = (EXTRA && p.residual != nullptr) ? h2f(static_cast<uint16_t>(bias_bits >> 16)) : 0.f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const float bias = __builtin_bit_cast(
           float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, bias_lane), r));
       const int row = cur * R + r;
+      // read the other lanes' values here, with every lane active: inside the branch below only
+      // lane 63 runs, and what a readlane sees of the inactive lanes is not defined
+      float res[NB];
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        res[b] = EXTRA ? __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, res_lane), r + R * b))
+                       : 0.f;
       if (lane == 63 && row < p.N) {
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
-          const float v = acc[r][b] + bias;
+          const float v = acc[r][b] + bias + res[b];
           const int64_t oi = static_cast<int64_t>(slot + b) * p.N + row;  // slot > 0 only if NB == 1
           if (p.out_f32) static_cast<float*>(p.y)[oi] = v;
           else static_cast<uint16_t*>(p.y)[oi] = f2h(v);
@@ -177,8 +195,11 @@ template <int BITS, int NB, int R, int ITERS>
 static hipError_t launch_k(const GemvParams& p, int slots, int blocks, int nsets, hipStream_t s) {
   const int threads = 256;
   const size_t lds = static_cast<size_t>(NB) * p.ng * GemvTraits<BITS>::G * 2;
-  hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS>), dim3(blocks, slots), dim3(threads), lds,
-                     s, p, nsets);
+  const dim3 grid(blocks, slots);
+  if (p.bias != nullptr || p.residual != nullptr)
+    hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, true>), grid, dim3(threads), lds, s, p, nsets);
+  else
+    hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, false>), grid, dim3(threads), lds, s, p, nsets);
   return hipGetLastError();
 }
 

@@ -20,6 +20,7 @@ struct GemvArgs {
   const uint32_t* q_weight; // [experts?, N, nw]
   const uint16_t* q_scale;  // [experts?, N, ng]
   const uint16_t* bias;     // [N] or null
+  const uint16_t* residual = nullptr;  // [M, N] fp16 added to the result, or null (plain linear only)
   void* y;                  // [M or slots, N]
   const int32_t* expert_ids;  // null for a plain linear; else [slots]
   int64_t M;                // batch rows of a plain linear (1..8); 1 for MoE slots
@@ -37,6 +38,7 @@ struct GemmArgs {
   const uint32_t* q_weight; // [experts, N, nw]
   const uint16_t* q_scale;  // [experts, N, ng]
   const uint16_t* bias;     // [N] or null (plain linear only)
+  const uint16_t* residual = nullptr;  // [rows, N] fp16 added to the result, or null (plain linear only)
   void* y;                  // [rows, N]
   const void* indptr;       // null for a plain linear
   int indptr_i64;

@@ -34,6 +34,7 @@ struct QuadParams {
   const uint32_t* qw;
   const uint16_t* qs;
   const uint16_t* bias;
+  const uint16_t* residual;  // [rows, N] or null
   void* y;
   const void* indptr;  // null: one segment [0, rows)
   int64_t expert_w_stride, expert_s_stride;
@@ -61,7 +62,8 @@ __device__ __forceinline__ float4_t mfma4(uint32_t a0, uint32_t a1, uint32_t b0,
 }
 
 // NBQ: activation rows / 4 (rows past the segment are zero); U: iterations per item
-template <int NBQ, int U>
+// RES: a residual operand exists (template flag: its loads are extra memory instructions per item)
+template <int NBQ, int U, bool RES>
 __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
   constexpr uint32_t kMagic = 0x64006400u;
   constexpr int XB = 4;  // (activation row, group) pairs a thread stages per round
@@ -108,6 +110,7 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
   uint4 wa[U], wb[U];
   uint32_t sa[U], sb[U];  // fp16 bits, 32 bits wide so that in-flight values are never re-packed
   uint2 ba, bb;
+  uint2 ra[NBQ], rb[NBQ];  // residual of (activation row 4 * bq + lane, the quad's 4 weight rows), lanes 0..3
   float4_t acc[NBQ];
 
   // K is walked in phases when x does not fit LDS whole: every phase stages its slice of x and
@@ -122,7 +125,7 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
     // ---- weight / scale / bias loads of one item.  Branch-free: every path issues the same
     //      loads, so the wait counts let the other buffer's loads stay in flight across the loop;
     //      an item past the end reads one cached line instead.
-    auto issue = [&](int quad, int step, uint4 (&wn)[U], uint32_t (&sn)[U], uint2& bn) {
+    auto issue = [&](int quad, int step, uint4 (&wn)[U], uint32_t (&sn)[U], uint2& bn, uint2 (&rn)[NBQ]) {
       const bool live = quad < p.nquads;
       const int row = min(quad * 4 + li, p.N - 1);
       const uint32_t* wr = qw + static_cast<int64_t>(row) * p.nw;
@@ -135,6 +138,16 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
       }
       bn = *reinterpret_cast<const uint2*>(
           (live && p.bias != nullptr) ? p.bias + quad * 4 : reinterpret_cast<const uint16_t*>(qw));
+      // the residual rides along (at store time it would wait behind the next items' weights)
+      if constexpr (RES) {
+#pragma unroll
+        for (int bq = 0; bq < NBQ; ++bq) {
+          const int b = min(4 * bq + (lane & 3), m_valid - 1);
+          rn[bq] = *reinterpret_cast<const uint2*>(
+              live ? p.residual + static_cast<int64_t>(m0 + b) * p.N + quad * 4
+                   : reinterpret_cast<const uint16_t*>(qw));
+        }
+      }
     };
     auto advance = [&](int& quad, int& step) {  // two items on
       step += 2;
@@ -152,8 +165,8 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
       stb = 0;
       qb += nwaves;
     }
-    issue(qa, sta, wa, sa, ba);
-    issue(qb, stb, wb, sb, bb);
+    issue(qa, sta, wa, sa, ba, ra);
+    issue(qb, stb, wb, sb, bb, rb);
 
     // ---- stage x in operand order.  Pair q = (batch quad, iteration, lane') with lane' = 4 *
     //      block + activation row; its four 16-byte words go to [q / 64][word][lane'].
@@ -207,7 +220,7 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
     // ---- persistent walk
     int done = 0;  // quads this wave has completed in this phase
     auto compute = [&](int quad, int step, const uint4 (&wc)[U], const uint32_t (&sc)[U],
-                       uint2 bias_bits) {
+                       uint2 bias_bits, const uint2 (&res_bits)[NBQ]) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int it = step * U + u;
@@ -274,6 +287,12 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
                 v[2] += h2f(static_cast<uint16_t>(bias_bits.y & 0xffffu));
                 v[3] += h2f(static_cast<uint16_t>(bias_bits.y >> 16));
               }
+              if constexpr (RES) {
+                v[0] += h2f(static_cast<uint16_t>(res_bits[bq].x & 0xffffu));
+                v[1] += h2f(static_cast<uint16_t>(res_bits[bq].x >> 16));
+                v[2] += h2f(static_cast<uint16_t>(res_bits[bq].y & 0xffffu));
+                v[3] += h2f(static_cast<uint16_t>(res_bits[bq].y >> 16));
+              }
               const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
               if (p.out_f32) {
                 *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) =
@@ -292,29 +311,36 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
     };
 
     while (qa < p.nquads) {
-      compute(qa, sta, wa, sa, ba);
+      compute(qa, sta, wa, sa, ba, ra);
       advance(qa, sta);
-      issue(qa, sta, wa, sa, ba);
+      issue(qa, sta, wa, sa, ba, ra);
       __builtin_amdgcn_sched_barrier(0);  // keep the refill ahead of the next item's arithmetic
-      compute(qb, stb, wb, sb, bb);  // past the end: nothing is stored
+      compute(qb, stb, wb, sb, bb, rb);  // past the end: nothing is stored
       advance(qb, stb);
-      issue(qb, stb, wb, sb, bb);
+      issue(qb, stb, wb, sb, bb, rb);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
 
-template <int NBQ, int U>
-static hipError_t launch_quad_cfg(const QuadParams& p, dim3 grid, int threads, size_t lds,
+template <int NBQ, int U, bool RES>
+static hipError_t launch_quad_res(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                   hipStream_t s) {
   if (lds > 65536) {
     const hipError_t e =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_q4_kernel<NBQ, U>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_q4_kernel<NBQ, U, RES>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL((quad_q4_kernel<NBQ, U>), grid, dim3(threads), lds, s, p);
+  hipLaunchKernelGGL((quad_q4_kernel<NBQ, U, RES>), grid, dim3(threads), lds, s, p);
   return hipGetLastError();
+}
+
+template <int NBQ, int U>
+static hipError_t launch_quad_cfg(const QuadParams& p, dim3 grid, int threads, size_t lds,
+                                  hipStream_t s) {
+  return p.residual != nullptr ? launch_quad_res<NBQ, U, true>(p, grid, threads, lds, s)
+                               : launch_quad_res<NBQ, U, false>(p, grid, threads, lds, s);
 }
 
 // hipErrorNotSupported when the shape does not fit (the caller falls back to gq_skinny.hip)
@@ -323,11 +349,11 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   if ((a.N & 3) != 0 || (a.K & 7) != 0) return hipErrorNotSupported;
   if ((reinterpret_cast<uintptr_t>(a.x) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.y) & 15) != 0 ||
-      (reinterpret_cast<uintptr_t>(a.bias) & 7) != 0 ||
+      (reinterpret_cast<uintptr_t>(a.bias) & 7) != 0 || (reinterpret_cast<uintptr_t>(a.residual) & 7) != 0 ||
       (reinterpret_cast<uintptr_t>(a.q_weight) & 15) != 0)
     return hipErrorNotSupported;
   QuadParams p;
-  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.y = a.y;
+  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
   p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64;
   p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
   p.ng = static_cast<int>((a.K + 31) / 32);

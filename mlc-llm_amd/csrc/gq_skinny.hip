@@ -29,6 +29,7 @@ struct SkinnyParams {
   const uint32_t* qw;
   const uint16_t* qs;
   const uint16_t* bias;
+  const uint16_t* residual;  // [rows, N] or null
   void* y;
   const void* indptr;  // null: one segment [0, rows)
   int64_t expert_w_stride, expert_s_stride;
@@ -191,7 +192,7 @@ __global__ __launch_bounds__(256) void skinny_q4_simple_kernel(const SkinnyParam
         const int b = 4 * j + r;
         if (b < m_valid) {
           const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + col;
-          const float o = v[r] + bias;
+          const float o = v[r] + bias + (p.residual != nullptr ? h2f(p.residual[oi]) : 0.f);
           if (p.out_f32) static_cast<float*>(p.y)[oi] = o;
           else static_cast<uint16_t*>(p.y)[oi] = f2h(o);
         }
@@ -394,7 +395,7 @@ __global__ __launch_bounds__(256) void skinny_q4_kernel(const SkinnyParams p) {
         const int b = 4 * j + r;
         if (b < m_valid) {
           const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + col;
-          const float o = v[r] + bias;
+          const float o = v[r] + bias + (p.residual != nullptr ? h2f(p.residual[oi]) : 0.f);
           if (p.out_f32) static_cast<float*>(p.y)[oi] = o;
           else static_cast<uint16_t*>(p.y)[oi] = f2h(o);
         }
@@ -547,7 +548,7 @@ __global__ __launch_bounds__(512) void skinny_q4_persist_kernel(const SkinnyPara
           const int b = 4 * j + r;
           if (b < m_valid) {
             const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + col;
-            const float o = acc[r] + bias;
+            const float o = acc[r] + bias + (p.residual != nullptr ? h2f(p.residual[oi]) : 0.f);
             if (p.out_f32) static_cast<float*>(p.y)[oi] = o;
             else static_cast<uint16_t*>(p.y)[oi] = f2h(o);
           }
@@ -586,7 +587,7 @@ static hipError_t launch_skinny_cfg(const SkinnyParams& p, int experts, int mtil
 hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
   if (a.bits != 4) return hipErrorNotSupported;
   SkinnyParams p;
-  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.y = a.y;
+  p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
   p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64;
   p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
   p.ng = static_cast<int>((a.K + a.group_size - 1) / a.group_size);

@@ -73,6 +73,24 @@ void Linear(TensorView x, TensorView q_weight, TensorView q_scale, Optional<Tens
         "mlc.gq.linear");
 }
 
+// y = x . dequantize(q_weight, q_scale)^T (+ bias) + residual; residual may be y itself
+void LinearResidual(TensorView x, TensorView q_weight, TensorView q_scale, Optional<TensorView> bias,
+                    TensorView residual, int64_t bits, int64_t group_size, Optional<TensorView> workspace,
+                    TensorView y) {
+  const int64_t K = x.shape()[x.ndim() - 1], N = q_weight.shape()[0];
+  void* ws = workspace.has_value() ? Ptr(workspace.value()) : nullptr;
+  int64_t ws_bytes = 0;
+  if (workspace.has_value()) {
+    ws_bytes = (workspace.value().dtype().bits + 7) / 8;
+    for (int i = 0; i < workspace.value().ndim(); ++i) ws_bytes *= workspace.value().shape()[i];
+  }
+  Check(mi355gq_linear_residual(Ptr(x), Ptr(q_weight), Ptr(q_scale),
+                                bias.has_value() ? Ptr(bias.value()) : nullptr, Ptr(residual), Rows(x),
+                                N, K, static_cast<int>(bits), static_cast<int>(group_size), OutDtype(y),
+                                Ptr(y), ws, ws_bytes, StreamOf(x)),
+        "mlc.gq.linear_residual");
+}
+
 int64_t LinearWorkspaceBytes(int64_t M, int64_t N, int64_t K, int64_t bits, int64_t group_size) {
   return mi355gq_linear_workspace_bytes(M, N, K, static_cast<int>(bits), static_cast<int>(group_size));
 }
@@ -126,6 +144,7 @@ TVM_FFI_STATIC_INIT_BLOCK() {
   namespace refl = tvm::ffi::reflection;
   refl::GlobalDef()
       .def("mlc.gq.linear", Linear)
+      .def("mlc.gq.linear_residual", LinearResidual)
       .def("mlc.gq.linear_workspace_bytes", LinearWorkspaceBytes)
       .def("mlc.gq.embedding_take", EmbeddingTake)
       .def("mlc.gq.moe_gemv", MoeGemv)

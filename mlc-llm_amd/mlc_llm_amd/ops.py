@@ -96,8 +96,11 @@ def embedding_take(ids: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Ten
 
 def linear(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits: int,
            group_size: int, bias: Optional[torch.Tensor] = None, out_dtype=torch.float16,
-           out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """y[..., N] = x[..., K] . dequantize(q_weight, q_scale)^T (+ bias)."""
+           out: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y[..., N] = x[..., K] . dequantize(q_weight, q_scale)^T (+ bias) (+ residual[..., N]).
+
+    `residual` (fp16, the shape of y) is added inside the kernel; passing the same tensor as `out`
+    updates it in place."""
     _chk(x, torch.float16, "x")
     _chk(q_weight, _STORAGE, "q_weight")
     _chk(q_scale, torch.float16, "q_scale")
@@ -117,12 +120,19 @@ def linear(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits:
         out = torch.empty((*x.shape[:-1], n), dtype=out_dtype, device=x.device)
     else:
         _chk(out, out_dtype, "out")
+    if residual is not None:
+        _chk(residual, torch.float16, "residual")
+        if tuple(residual.shape) != tuple(out.shape) or not residual.is_contiguous():
+            raise ValueError(f"residual shape {tuple(residual.shape)}, expected contiguous {tuple(out.shape)}")
     ws_bytes = _lib.lib().mi355gq_linear_workspace_bytes(m, n, k, bits, group_size)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
-    _lib.call("mi355gq_linear", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(),
-              bias.data_ptr() if bias is not None else None, m, n, k, bits, group_size,
-              _lib.F32 if out_dtype == torch.float32 else _lib.F16, out.data_ptr(),
-              ws.data_ptr() if ws is not None else None, ws_bytes, _stream())
+    tail = (m, n, k, bits, group_size, _lib.F32 if out_dtype == torch.float32 else _lib.F16, out.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws_bytes, _stream())
+    head = (x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(), bias.data_ptr() if bias is not None else None)
+    if residual is None:
+        _lib.call("mi355gq_linear", *head, *tail)
+    else:
+        _lib.call("mi355gq_linear_residual", *head, residual.data_ptr(), *tail)
     return out
 
 

@@ -616,6 +616,54 @@ def test_mixtral_moe_layer_golden(golden, case):
     assert rel <= 4e-3 and err <= 0.05, (err, rel)  # two chained matmuls + fp16 glue
 
 
+# ------------------------------------------------------------------ fused residual addition
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 8, 12, 16, 40, 100, 300])  # every regime of the dispatcher
+def test_linear_residual_every_regime(name, m):
+    s = SCHEMES[name]
+    n, k = 264, 4096 if s.bits == 4 else 4000
+    x, qw, qs, b = _linear_case(s, m, n, k, 400 + m, bias=True)
+    res = np.random.default_rng(m).standard_normal((m, n)).astype(np.float16)
+    ref = o.linear_fp32(x, qw, qs, s, b) + res.astype(np.float64)
+    y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b), residual=dev(res))
+    y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32, residual=dev(res))
+    assert_linear_ok(y, ref, x, k, f"linear+residual {name} M={m}")
+    assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"linear+residual {name} M={m} fp32 out")
+    # in place: hidden += proj(x)
+    hidden = dev(res)
+    out = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b), out=hidden, residual=hidden)
+    assert out.data_ptr() == hidden.data_ptr()
+    assert torch.equal(out, y), f"in-place residual differs from out-of-place, {name} M={m}"
+
+
+@pytest.mark.parametrize("variant", [0, 2, 3, 4, 7, 8])  # LDS GEMV, the skinny forms, quad-row phases / 4-row passes
+def test_linear_residual_forced_kernels(variant):
+    s = SCHEMES["q4f16_1"]
+    m, n, k = (5, 520, 14336) if variant in (7, 8) else ((2, 520, 1024) if variant == 0 else (9, 520, 1024))
+    x, qw, qs, b = _linear_case(s, m, n, k, 500 + variant, bias=True)
+    res = np.random.default_rng(variant).standard_normal((m, n)).astype(np.float16)
+    gq._lib.set_option("gemv_variant", variant)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b), residual=dev(res))
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b) + res.astype(np.float64), x, k, f"residual, variant {variant}")
+
+
+def test_linear_residual_argument_checks():
+    s = SCHEMES["q4f16_1"]
+    x, qw, qs, _ = _linear_case(s, 2, 64, 128, 1)
+    xd, qwd, qsd = dev(x), dev(qw), dev(qs)
+    out32 = torch.empty((2, 64), dtype=torch.float32, device=xd.device)
+    rc = gq._lib.lib().mi355gq_linear_residual(xd.data_ptr(), qwd.data_ptr(), qsd.data_ptr(), None, None, 2, 64, 128,
+                                                4, 32, gq._lib.F16, out32.data_ptr(), None, 0, None)
+    assert rc == -1 and "residual is null" in gq._lib.lib().mi355gq_last_error().decode()
+    rc = gq._lib.lib().mi355gq_linear_residual(xd.data_ptr(), qwd.data_ptr(), qsd.data_ptr(), None, out32.data_ptr(),
+                                                2, 64, 128, 4, 32, gq._lib.F32, out32.data_ptr(), None, 0, None)
+    assert rc == -1 and "in-place" in gq._lib.lib().mi355gq_last_error().decode()
+
+
 # ------------------------------------------------------------------ HIP graph capture
 
 def test_linear_and_moe_replay_in_hip_graph():
