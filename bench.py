@@ -176,11 +176,27 @@ def main() -> int:
             dst.copy_(src)  # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
+    # the same tensors through the library's read-only probe (one launch per layer, 128-bit
+    # loads, no arithmetic): what this device delivers for these bytes, measured in this run
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def read_sweep():
+        for lw in layers:
+            qw, qs = lw["gate_up"]
+            gq._lib.call("mi355gq_probe_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
+                      sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+
+    us_read = timed(read_sweep, max(5, args.steps), 2, use_graph) * 1e3 / LAYERS
+    read_bytes = layers[0]["gate_up"][0].numel() * 4 + layers[0]["gate_up"][1].numel() * 2
     roofline = {
         "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2,false> (gate_up 28672x4096, batch 1)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
         "bytes_per_launch": gu_bytes, "us_per_launch": round(us_gate_up, 3),
+        "read_only_probe": {"what": "plain 128-bit streaming read of the same weight and scale tensors, one launch each",
+                            "us_per_launch": round(us_read, 3),
+                            "GB/s": round(read_bytes / (us_read * 1e-6) / 1e9, 1),
+                            "gemv_time_over_probe_time": round(us_gate_up / us_read, 3)},
     }
 
     # ---------------------------------------------------------------- extra: per shape, batch 1/4/8, prefill GEMM

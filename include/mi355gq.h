@@ -54,6 +54,13 @@ MI355GQ_API const char* mi355gq_last_error(void);
 /* 0 when the current HIP device is gfx950, MI355GQ_ERR_UNSUPPORTED otherwise. */
 MI355GQ_API int mi355gq_check_device(void);
 
+/* Measurement aid, no counterpart in the reference: one launch that only reads the byte ranges
+ * a and b (sizes multiples of 16, pointers 16-byte aligned) with 128-bit loads and discards
+ * them; sink is 4 bytes of device memory or NULL.  bench.py times it on a GEMV's weight and
+ * scale tensors to quote what the device delivers for those bytes without any arithmetic. */
+MI355GQ_API int mi355gq_probe_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,
+                              void* sink, mi355gq_stream_t stream);
+
 /* Tuning/diagnostic knob (process-global, not thread-safe against running calls):
  * "gemv_rows_per_wave", "gemv_variant", "gemm_variant" ... ; value < 0 restores the default. */
 MI355GQ_API int mi355gq_set_option(const char* name, int value);

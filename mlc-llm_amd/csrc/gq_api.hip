@@ -99,6 +99,16 @@ int mi355gq_set_option(const char* name, int value) {
   return MI355GQ_OK;
 }
 
+int mi355gq_probe_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,
+                              void* sink, mi355gq_stream_t stream) {
+  GQ_REQUIRE(a_bytes >= 0 && b_bytes >= 0 && (a_bytes % 16) == 0 && (b_bytes % 16) == 0,
+             "probe_stream_read: sizes must be non-negative multiples of 16");
+  GQ_REQUIRE((a_bytes == 0 || a) && (b_bytes == 0 || b), "probe_stream_read: null pointer");
+  GQ_REQUIRE(aligned16(a) && aligned16(b) && aligned4(sink), "probe_stream_read: 16-byte alignment");
+  return hip_result(gq::launch_stream_read(a, a_bytes, b, b_bytes, sink, as_stream(stream)),
+                    "stream read launch");
+}
+
 int mi355gq_quantize(const void* w, int64_t rows, int64_t K, int bits, int group_size,
                      int round_mode, void* q_weight, void* q_scale, mi355gq_stream_t stream) {
   GQ_CHECK(check_scheme(bits, group_size));

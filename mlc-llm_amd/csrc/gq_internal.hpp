@@ -57,6 +57,10 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s);
 // hipErrorNotSupported when the shape does not fit.
 hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s);
 
+// plain streaming read of two byte ranges (multiples of 16 bytes, 16-byte aligned)
+hipError_t launch_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,
+                              void* sink, hipStream_t s);
+
 hipError_t launch_quantize(const uint16_t* w, int64_t rows, int64_t K, int bits, int group_size,
                            int round_mode, uint32_t* qw, uint16_t* qs, hipStream_t s);
 hipError_t launch_dequantize(const int32_t* ids, int64_t out_rows, const uint32_t* qw,

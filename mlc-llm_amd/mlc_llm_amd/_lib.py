@@ -31,6 +31,7 @@ SIGNATURES = {
     "mi355gq_set_option": (_I, [c_char_p, _I]),
     "mi355gq_quantize": (_I, [_P, _L, _L, _I, _I, _I, _P, _P, _P]),
     "mi355gq_dequantize": (_I, [_P, _P, _L, _L, _I, _I, _P, _P]),
+    "mi355gq_probe_stream_read": (_I, [_P, _L, _P, _L, _P, _P]),
     "mi355gq_embedding_take": (_I, [_P, _L, _P, _P, _L, _L, _I, _I, _P, _P]),
     "mi355gq_linear_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
     "mi355gq_linear": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),

@@ -664,6 +664,18 @@ def test_linear_residual_argument_checks():
     assert rc == -1 and "in-place" in gq._lib.lib().mi355gq_last_error().decode()
 
 
+def test_stream_read_probe_runs_and_validates():
+    a = torch.arange(4096 + 8, dtype=torch.int32, device="cuda:0")  # sizes that exercise the tail loop
+    b = torch.ones(64, dtype=torch.int32, device="cuda:0")
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda:0")
+    gq._lib.call("mi355gq_probe_stream_read", a.data_ptr(), a.numel() * 4, b.data_ptr(), b.numel() * 4,
+                 sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    gq._lib.call("mi355gq_probe_stream_read", a.data_ptr(), a.numel() * 4, None, 0, None,
+                 torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert gq._lib.lib().mi355gq_probe_stream_read(a.data_ptr(), 24, None, 0, None, None) == -1  # not a multiple of 16
+
+
 # ------------------------------------------------------------------ HIP graph capture
 
 def test_linear_and_moe_replay_in_hip_graph():
