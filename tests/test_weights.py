@@ -247,3 +247,71 @@ def test_convert_weight_quantised_matches_oracle(tmp_path, cfg, scheme):
     ref = o.linear_fp32(x, params[f"{name}.q_weight"].numpy().view(np.uint32), params[f"{name}.q_scale"].numpy(), s)
     err, bound, rel = o.check_linear(y.float().cpu().numpy(), ref, x, cfg["hidden_size"])
     assert err <= bound and rel <= 2e-3  # the linear tolerance of the hot path
+
+
+@pytest.mark.gpu
+def test_converted_directory_loads_into_quantized_modules(tmp_path):
+    """HF checkpoint -> convert_weight -> load_tensor_cache -> load_state_dict into a module tree
+    rewritten by GroupQuantize.quantize_model -> one decoder MLP + residual on the GPU, against
+    fp64 arithmetic over the dequantised weights."""
+    from torch import nn
+
+    from mlc_llm_amd import ops
+    from mlc_llm_amd.quantization import QUANTIZATION, QuantizeMapping
+
+    cfg = dict(LLAMA, hidden_size=256, intermediate_size=384, num_hidden_layers=1)
+    src, dst = str(tmp_path / "hf"), str(tmp_path / "mlc")
+    tensors = _hf_tensors(cfg, seed=11)
+    _write_checkpoint(src, cfg, tensors, shards=1)
+    loader.convert_weight(src, dst, quantization="q4f16_1", device="cuda:0")
+    params, _ = tensor_cache.load_tensor_cache(dst, device="cuda:0")
+
+    class MLP(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate_up_proj = nn.Linear(256, 2 * 384, bias=False)
+            self.down_proj = nn.Linear(384, 256, bias=False)
+
+    class Layer(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.mlp = MLP()
+
+    class Model(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = nn.ModuleList([Layer()])
+
+    class Top(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.model = Model()
+
+    top = Top().half().to("cuda:0")
+    quant = QUANTIZATION["q4f16_1"]
+    qmap = QuantizeMapping({}, {})
+    top = quant.quantize_model(top, qmap, "")
+    assert qmap.param_map["model.layers.0.mlp.down_proj.weight"] == [
+        "model.layers.0.mlp.down_proj.q_weight", "model.layers.0.mlp.down_proj.q_scale"]
+    wanted = {k: v for k, v in params.items() if ".mlp." in k}
+    top.load_state_dict(wanted, strict=True)  # names and shapes of the directory are the modules'
+    mlp = top.model.layers[0].mlp
+
+    x = np.random.default_rng(4).standard_normal((5, 256)).astype(np.float16)
+    xd = torch.from_numpy(x).to("cuda:0")
+    h = ops.silu_mul(mlp.gate_up_proj(xd))
+    y = ops.linear(h, mlp.down_proj.q_weight, mlp.down_proj.q_scale, 4, 32, residual=xd)  # x + down(act)
+
+    s = o.SCHEMES["q4f16_1"]
+    gu = np.concatenate([tensors["model.layers.0.mlp.gate_proj.weight"].numpy(),
+                         tensors["model.layers.0.mlp.up_proj.weight"].numpy()], axis=0)
+    qw1, qs1 = o.quantize(gu, s)
+    qw2, qs2 = o.quantize(tensors["model.layers.0.mlp.down_proj.weight"].numpy(), s)
+    g_ref = o.linear_fp32(x, qw1, qs1, s).astype(np.float16)   # the fp16 the first kernel hands on
+    act = o.silu_mul_f16(g_ref)
+    ref = o.linear_fp32(h.cpu().numpy(), qw2, qs2, s) + x.astype(np.float64)
+    err, bound, rel = o.check_linear(y.float().cpu().numpy(), ref, h.cpu().numpy(), 384)
+    assert err <= bound and rel <= 2e-3
+    # and the whole block against the oracle end to end (two roundings to fp16 on the way)
+    ref_all = o.linear_fp32(act, qw2, qs2, s) + x.astype(np.float64)
+    assert np.abs(y.float().cpu().numpy() - ref_all).max() <= 2 * bound + 1e-2
