@@ -187,8 +187,27 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // y may be the residual buffer itself (same element type), nothing else may overlap it
   GQ_REQUIRE(residual == nullptr || residual != y || out_dtype == MI355GQ_F16,
              "linear: in-place residual needs a float16 output");
-  // regimes: M <= 2 register GEMV; 3..16 MFMA skinny kernel (q4) or LDS GEMV up to 8 (q3); else GEMM
-  const bool use_gemv = M <= 2 || (M <= 8 && (bits != 4 || gq::options().gemm_variant == 2));
+  // regimes: M <= 2 register GEMV; 3..8 quad-row kernel (LDS GEMV when it declines a q3 shape);
+  // 9..16 MFMA skinny kernel (q4); else GEMM
+  gq::GemmArgs g{};
+  g.x = static_cast<const uint16_t*>(x);
+  g.q_weight = static_cast<const uint32_t*>(q_weight);
+  g.q_scale = static_cast<const uint16_t*>(q_scale);
+  g.bias = static_cast<const uint16_t*>(bias);
+  g.residual = static_cast<const uint16_t*>(residual);
+  g.y = y;
+  g.indptr = nullptr; g.indptr_i64 = 0;
+  g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
+  g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
+  g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
+  const int gv = gq::options().gemv_variant;  // 2..5 force a gq_skinny.hip form, 6..8 the quad-row kernel
+  const int gm = gq::options().gemm_variant;  // 1: GEMM only, 2: GEMV up to 8 rows
+  // (q3 has no 16x16x32 skinny kernel: 9..16 rows run as two concurrent 8-row passes of the quad-row kernel)
+  if (bits == 3 && M >= 3 && M <= 16 && gm != 1 && (M > 8 || gm != 2) && (gv < 0 || (gv >= 6 && gv <= 8))) {
+    const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
+    if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
+  }
+  const bool use_gemv = M <= 2 || (M <= 8 && (bits != 4 || gm == 2));
   if (use_gemv) {
     gq::GemvArgs a{};
     a.x = static_cast<const uint16_t*>(x);
@@ -202,19 +221,7 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     a.bits = bits; a.group_size = group_size; a.out_f32 = out_dtype == MI355GQ_F32;
     return hip_result(gq::launch_gemv(a, as_stream(stream)), "gemv launch");
   }
-  gq::GemmArgs g{};
-  g.x = static_cast<const uint16_t*>(x);
-  g.q_weight = static_cast<const uint32_t*>(q_weight);
-  g.q_scale = static_cast<const uint16_t*>(q_scale);
-  g.bias = static_cast<const uint16_t*>(bias);
-  g.residual = static_cast<const uint16_t*>(residual);
-  g.y = y;
-  g.indptr = nullptr; g.indptr_i64 = 0;
-  g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
-  g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
-  g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
-  const int gv = gq::options().gemv_variant;  // 2..5 force a gq_skinny.hip form, 6..8 the quad-row kernel
-  if (M <= 16 && bits == 4 && gq::options().gemm_variant != 1) {
+  if (M <= 16 && bits == 4 && gm != 1) {
     if ((gv < 0 && M <= 8) || (gv >= 6 && gv <= 8)) {
       const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
       if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
@@ -295,11 +302,11 @@ int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, co
   g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
   // few rows in total: every expert is a skinny problem bound by streaming its weights
   const int gv = gq::options().gemv_variant;
+  if (rows <= 128 && gq::options().gemm_variant != 1 && ((gv < 0 && rows <= 32) || (gv >= 6 && gv <= 8))) {
+    const hipError_t q = gq::launch_quadrow(g, static_cast<int>(rows), as_stream(stream));
+    if (q != hipErrorNotSupported) return hip_result(q, "moe quad-row launch");
+  }
   if (rows <= 128 && bits == 4 && gq::options().gemm_variant != 1) {
-    if ((gv < 0 && rows <= 32) || (gv >= 6 && gv <= 8)) {
-      const hipError_t q = gq::launch_quadrow(g, static_cast<int>(rows), as_stream(stream));
-      if (q != hipErrorNotSupported) return hip_result(q, "moe quad-row launch");
-    }
     const hipError_t e = gq::launch_skinny(g, static_cast<int>(rows), as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "moe skinny launch");
   }

@@ -1,4 +1,4 @@
-// Few-row matmul for q4f16_1 on the 16-block 4x4x4 matrix instruction: 3..8 activation rows
+// Few-row matmul for q4f16_1 / q3f16_1 on the 16-block 4x4x4 matrix instruction: 3..8 activation rows
 // against streamed weights, with the memory access pattern of the batch-1 GEMV.
 //
 // Covers the same callers as gq_skinny.hip (the low-batch buckets of
@@ -15,7 +15,9 @@
 //    operands (even fields, and odd fields times 16), none of which leaves its lane: no LDS
 //    transpose, no cross-lane move between the load and the matrix core;
 //  * all 8 products of a group land in one accumulator pair, so the group's scale and the
-//    (1024 + m) offset are applied once per group in fp32, as in the GEMV kernels;
+//    (1024 + m) offset are applied once per group in fp32, as in the GEMV kernels (q3f16_1: ten
+//    operands per group in three classes - fields that come out of the masks times 1, 8 and 64 -
+//    and three accumulators);
 //  * x is staged once per workgroup in LDS, already in operand order ([k step][word][lane] so
 //    that every ds_read_b128 of a wave is one contiguous KiB), with the offset term of every
 //    (activation row, group) beside it;
@@ -62,11 +64,14 @@ __device__ __forceinline__ float4_t mfma4(uint32_t a0, uint32_t a1, uint32_t b0,
 }
 
 // NBQ: activation rows / 4 (rows past the segment are zero); U: iterations per item
-// RES: a residual operand exists (template flag: its loads are extra memory instructions per item)
-template <int NBQ, int U, bool RES>
-__global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
+// EXTRA: a bias or residual operand exists (template flag: their loads are extra memory
+// instructions per item)
+template <int BITS, int NBQ, int U, bool EXTRA>
+__global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
   constexpr uint32_t kMagic = 0x64006400u;
-  constexpr int XB = 4;  // (activation row, group) pairs a thread stages per round
+  constexpr int G = GemvTraits<BITS>::G;    // values per group: 32 | 40
+  constexpr int CH = GemvTraits<BITS>::CH;  // 16-byte words of x per (activation row, group): 4 | 5
+  constexpr int XB = BITS == 4 ? 4 : 3;     // (activation row, group) pairs a thread stages per round
 
   extern __shared__ uint4 smem[];
 
@@ -101,10 +106,10 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
   const uint32_t* qw = p.qw + expert * p.expert_w_stride;
   const uint16_t* qs = p.qs + expert * p.expert_s_stride;
 
-  // LDS: x of one phase [NBQ][niter][4 words][64 lanes] uint4, its offset terms [NBQ][niter][64]
+  // LDS: x of one phase [NBQ][niter][CH words][64 lanes] uint4, its offset terms [NBQ][niter][64]
   // floats, then this workgroup's partial sums between phases [wave][quad of the walk][NBQ][16]
   const int niter = p.nsteps * U;  // staged iterations per phase (groups past ng hold zeros)
-  float* const corr_lds = reinterpret_cast<float*>(smem + static_cast<size_t>(NBQ) * niter * 256);
+  float* const corr_lds = reinterpret_cast<float*>(smem + static_cast<size_t>(NBQ) * niter * CH * 64);
   float* const part_lds = corr_lds + NBQ * niter * 64 + (tid >> 6) * (p.rounds * NBQ * 16);
 
   uint4 wa[U], wb[U];
@@ -136,16 +141,16 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
         wn[u] = *reinterpret_cast<const uint4*>(live ? wr + 4 * g : qw);
         sn[u] = *(live ? sr + g : qs);
       }
-      bn = *reinterpret_cast<const uint2*>(
-          (live && p.bias != nullptr) ? p.bias + quad * 4 : reinterpret_cast<const uint16_t*>(qw));
-      // the residual rides along (at store time it would wait behind the next items' weights)
-      if constexpr (RES) {
+      // bias and residual ride along (at store time they would wait behind the next items' weights)
+      if constexpr (EXTRA) {
+        bn = *reinterpret_cast<const uint2*>(
+            (live && p.bias != nullptr) ? p.bias + quad * 4 : reinterpret_cast<const uint16_t*>(qw));
 #pragma unroll
         for (int bq = 0; bq < NBQ; ++bq) {
           const int b = min(4 * bq + (lane & 3), m_valid - 1);
           rn[bq] = *reinterpret_cast<const uint2*>(
-              live ? p.residual + static_cast<int64_t>(m0 + b) * p.N + quad * 4
-                   : reinterpret_cast<const uint16_t*>(qw));
+              (live && p.residual != nullptr) ? p.residual + static_cast<int64_t>(m0 + b) * p.N + quad * 4
+                                              : reinterpret_cast<const uint16_t*>(qw));
         }
       }
     };
@@ -169,13 +174,13 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
     issue(qb, stb, wb, sb, bb, rb);
 
     // ---- stage x in operand order.  Pair q = (batch quad, iteration, lane') with lane' = 4 *
-    //      block + activation row; its four 16-byte words go to [q / 64][word][lane'].
+    //      block + activation row; its CH 16-byte words go to [q / 64][word][lane'].
     if (phase > 0) __syncthreads();  // the previous phase's x is still being read
     {
       const int npairs = NBQ * niter * 64;
       for (int q0 = tid; q0 < npairs; q0 += nthreads * XB) {
-        uint4 raw[XB][4];
-        bool ok[XB][4];
+        uint4 raw[XB][CH];
+        bool ok[XB][CH];
 #pragma unroll
         for (int i = 0; i < XB; ++i) {
           const int q = q0 + i * nthreads;
@@ -185,8 +190,8 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
           const int g = 16 * (it0 + it) + (lp >> 2);
           const uint16_t* src = p.x + static_cast<int64_t>(m0 + min(b, m_valid - 1)) * p.K;
 #pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const int k = 32 * g + 8 * c;
+          for (int c = 0; c < CH; ++c) {
+            const int k = G * g + 8 * c;
             ok[i][c] = q < npairs && b < m_valid && g < p.ng && k + 8 <= p.K;
             raw[i][c] = *reinterpret_cast<const uint4*>(ok[i][c] ? src + k : p.x);
           }
@@ -195,18 +200,28 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
         for (int i = 0; i < XB; ++i) {
           const int q = q0 + i * nthreads;
           if (q < npairs) {
-            uint32_t nat[16], xr[16];
+            uint32_t nat[G / 2], xr[G / 2];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+            for (int c = 0; c < CH; ++c) {
               const uint4 r = ok[i][c] ? raw[i][c] : make_uint4(0, 0, 0, 0);
               nat[4 * c + 0] = r.x; nat[4 * c + 1] = r.y; nat[4 * c + 2] = r.z; nat[4 * c + 3] = r.w;
             }
-            const float corr = permute_group<4>(nat, xr);
+            const float corr = permute_group<BITS>(nat, xr);
             const int lp = q & 63, bi = q >> 6;
+            if constexpr (BITS == 4) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c)  // (even fields: 2 pairs), (odd fields: 2 pairs)
-              smem[(bi * 4 + c) * 64 + lp] =
-                  make_uint4(xr[4 * c + 0], xr[4 * c + 2], xr[4 * c + 1], xr[4 * c + 3]);
+              for (int c = 0; c < 4; ++c)  // word c: (even fields: 2 pairs), (odd fields: 2 pairs)
+                smem[(bi * CH + c) * 64 + lp] =
+                    make_uint4(xr[4 * c + 0], xr[4 * c + 2], xr[4 * c + 1], xr[4 * c + 3]);
+            } else {
+              // word c: fields (0,5)(3,8) meet the x1 operands, (1,6)(4,9) the x8 operands;
+              // fields (2,7) of all four words, the x64 class, share the fifth 16-byte word
+#pragma unroll
+              for (int c = 0; c < 4; ++c)
+                smem[(bi * CH + c) * 64 + lp] =
+                    make_uint4(xr[5 * c + 0], xr[5 * c + 3], xr[5 * c + 1], xr[5 * c + 4]);
+              smem[(bi * CH + 4) * 64 + lp] = make_uint4(xr[2], xr[7], xr[12], xr[17]);
+            }
             corr_lds[bi * 64 + lp] = corr;
           }
         }
@@ -225,14 +240,27 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
       for (int u = 0; u < U; ++u) {
         const int it = step * U + u;
         const uint32_t w[4] = {wc[u].x, wc[u].y, wc[u].z, wc[u].w};
-        uint32_t lo[4][2], hi[4][2];
+        // A operands: q4 lo/hi = even / odd fields (x1, x16) of word d; q3 a1/a8 = the x1 / x8
+        // fields of word d, a64 = the x64 field pairs of words (0,1) and (2,3)
+        uint32_t lo[4][2], hi[4][2], a64[2][2];
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          const uint32_t w8 = w[d] >> 8;
-          lo[d][0] = and_or(w[d], 0x000f000fu, kMagic);
-          hi[d][0] = and_or(w[d], 0x00f000f0u, kMagic);
-          lo[d][1] = and_or(w8, 0x000f000fu, kMagic);
-          hi[d][1] = and_or(w8, 0x00f000f0u, kMagic);
+          if constexpr (BITS == 4) {
+            const uint32_t w8 = w[d] >> 8;
+            lo[d][0] = and_or(w[d], 0x000f000fu, kMagic);
+            hi[d][0] = and_or(w[d], 0x00f000f0u, kMagic);
+            lo[d][1] = and_or(w8, 0x000f000fu, kMagic);
+            hi[d][1] = and_or(w8, 0x00f000f0u, kMagic);
+          } else {
+            // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
+            const uint32_t t = (w[d] & 0x0000ffffu) | ((w[d] << 1) & 0xffff0000u);
+            const uint32_t t9 = t >> 9;
+            lo[d][0] = and_or(t, 0x00070007u, kMagic);   // fields (0,5)
+            lo[d][1] = and_or(t9, 0x00070007u, kMagic);  // fields (3,8)
+            hi[d][0] = and_or(t, 0x00380038u, kMagic);   // fields (1,6) x 8
+            hi[d][1] = and_or(t9, 0x00380038u, kMagic);  // fields (4,9) x 8
+            a64[d >> 1][d & 1] = and_or(t, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+          }
         }
         // the four rows' scales of this block: lane 4b+i holds row i's
         float sv[4];
@@ -247,14 +275,24 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
           float4_t tl = {0.f, 0.f, 0.f, 0.f}, th = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
-            const uint4 xv = smem[(bi * 4 + d) * 64 + lane];
+            const uint4 xv = smem[(bi * CH + d) * 64 + lane];
             tl = mfma4(lo[d][0], lo[d][1], xv.x, xv.y, tl);
             th = mfma4(hi[d][0], hi[d][1], xv.z, xv.w, th);
           }
           const float corr = corr_lds[bi * 64 + lane];
+          if constexpr (BITS == 4) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
-            acc[bq][i] = fmaf(sv[i], fmaf(th[i], 0.0625f, tl[i]) - corr, acc[bq][i]);
+            for (int i = 0; i < 4; ++i)
+              acc[bq][i] = fmaf(sv[i], fmaf(th[i], 0.0625f, tl[i]) - corr, acc[bq][i]);
+          } else {
+            const uint4 xv = smem[(bi * CH + 4) * 64 + lane];
+            float4_t t64 = {0.f, 0.f, 0.f, 0.f};
+            t64 = mfma4(a64[0][0], a64[0][1], xv.x, xv.y, t64);
+            t64 = mfma4(a64[1][0], a64[1][1], xv.z, xv.w, t64);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              acc[bq][i] = fmaf(sv[i], fmaf(t64[i], 0.015625f, fmaf(th[i], 0.125f, tl[i])) - corr, acc[bq][i]);
+          }
         }
       }
       if (step == nst - 1) {  // uniform: the quad's share of this phase is complete
@@ -281,13 +319,13 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
             if (!last_phase) {
               *part = make_float4(v[0], v[1], v[2], v[3]);
             } else {
-              if (p.bias != nullptr) {
+              if (EXTRA && p.bias != nullptr) {
                 v[0] += h2f(static_cast<uint16_t>(bias_bits.x & 0xffffu));
                 v[1] += h2f(static_cast<uint16_t>(bias_bits.x >> 16));
                 v[2] += h2f(static_cast<uint16_t>(bias_bits.y & 0xffffu));
                 v[3] += h2f(static_cast<uint16_t>(bias_bits.y >> 16));
               }
-              if constexpr (RES) {
+              if (EXTRA && p.residual != nullptr) {
                 v[0] += h2f(static_cast<uint16_t>(res_bits[bq].x & 0xffffu));
                 v[1] += h2f(static_cast<uint16_t>(res_bits[bq].x >> 16));
                 v[2] += h2f(static_cast<uint16_t>(res_bits[bq].y & 0xffffu));
@@ -323,29 +361,33 @@ __global__ __launch_bounds__(512) void quad_q4_kernel(const QuadParams p) {
   }
 }
 
-template <int NBQ, int U, bool RES>
-static hipError_t launch_quad_res(const QuadParams& p, dim3 grid, int threads, size_t lds,
-                                  hipStream_t s) {
+template <int BITS, int NBQ, int U, bool EXTRA>
+static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads, size_t lds,
+                                    hipStream_t s) {
   if (lds > 65536) {
     const hipError_t e =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_q4_kernel<NBQ, U, RES>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, EXTRA>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL((quad_q4_kernel<NBQ, U, RES>), grid, dim3(threads), lds, s, p);
+  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, EXTRA>), grid, dim3(threads), lds, s, p);
   return hipGetLastError();
 }
 
-template <int NBQ, int U>
+template <int BITS, int NBQ, int U>
 static hipError_t launch_quad_cfg(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                   hipStream_t s) {
-  return p.residual != nullptr ? launch_quad_res<NBQ, U, true>(p, grid, threads, lds, s)
-                               : launch_quad_res<NBQ, U, false>(p, grid, threads, lds, s);
+  return (p.bias != nullptr || p.residual != nullptr)
+             ? launch_quad_extra<BITS, NBQ, U, true>(p, grid, threads, lds, s)
+             : launch_quad_extra<BITS, NBQ, U, false>(p, grid, threads, lds, s);
 }
 
-// hipErrorNotSupported when the shape does not fit (the caller falls back to gq_skinny.hip)
-hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
-  if (a.bits != 4 || a.group_size != 32) return hipErrorNotSupported;
+// hipErrorNotSupported when the shape does not fit (the caller falls back to its other kernels)
+template <int BITS>
+static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream_t s) {
+  constexpr int G = GemvTraits<BITS>::G;
+  constexpr int CH = GemvTraits<BITS>::CH;
+  if (a.group_size != G) return hipErrorNotSupported;
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   if ((a.N & 3) != 0 || (a.K & 7) != 0) return hipErrorNotSupported;
   if ((reinterpret_cast<uintptr_t>(a.x) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.y) & 15) != 0 ||
@@ -356,7 +398,7 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
   p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64;
   p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
-  p.ng = static_cast<int>((a.K + 31) / 32);
+  p.ng = static_cast<int>((a.K + G - 1) / G);
   p.nw = 4 * p.ng;
   p.nquads = p.N / 4;
   p.expert_w_stride = a.N * p.nw;
@@ -364,6 +406,8 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   p.out_f32 = a.out_f32;
   const int experts = a.indptr ? static_cast<int>(a.num_experts) : 1;
 
+  // LDS per iteration (16 groups) and batch quad: x in operand order and the offset terms
+  constexpr size_t kLdsIter = CH * 1024 + 256;
   const int niter = (p.ng + 15) / 16;
   int U = options().gemv_rows_per_wave;  // tuning override
   // measured: 4 KiB items pay off only on matrices large enough to run long (gate_up, lm_head)
@@ -377,12 +421,12 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   const int mode = options().gemv_variant;
   int nbq = rows_max <= 4 ? 1 : 2;
   if (nbq == 2) {
-    const size_t whole = static_cast<size_t>(p.steps_total) * U * 2 * (4096 + 256);
+    const size_t whole = static_cast<size_t>(p.steps_total) * U * 2 * kLdsIter;
     const bool phases = mode == 7 || (mode != 8 && a.indptr != nullptr);
     if (mode == 8 || (whole > 150 * 1024 && !phases)) nbq = 1;
   }
   const int mtiles = (rows_max + 4 * nbq - 1) / (4 * nbq);
-  if (mtiles > 2 && a.indptr == nullptr) return hipErrorNotSupported;
+  if (mtiles > 4 && a.indptr == nullptr) return hipErrorNotSupported;
 
   // every workgroup stages x for itself, so a small plain matrix wants fewer, longer-lived waves
   int waves = options().gemv_split > 0 ? options().gemv_split
@@ -393,10 +437,9 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   if (waves > p.nquads) waves = p.nquads;
   p.rounds = (p.nquads + waves - 1) / waves;
 
-  // LDS per step and batch quad: x (4 rows * 32 halves per group, 16 groups per iteration) and
-  // the offset terms; per wave: the partial sums of its quads.  Phases share K evenly.
+  // per wave: the partial sums of its quads.  Phases share K evenly.
   const size_t lds_cap = 150 * 1024;
-  const size_t lds_step = static_cast<size_t>(U) * nbq * (4096 + 256);
+  const size_t lds_step = static_cast<size_t>(U) * nbq * kLdsIter;
   const size_t lds_part = static_cast<size_t>(8) * p.rounds * nbq * 64;  // up to 8 waves
   if (lds_part + lds_step > lds_cap) return hipErrorNotSupported;
   const int steps_fit = static_cast<int>((lds_cap - lds_part) / lds_step);
@@ -410,10 +453,16 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   const int blocks = ((p.nquads + p.rounds - 1) / p.rounds + wpb - 1) / wpb;
   const dim3 grid(blocks, experts, mtiles);
 #define GQ_QUAD_CASE(NBQ_, U_) \
-  if (nbq == NBQ_ && U == U_) return launch_quad_cfg<NBQ_, U_>(p, grid, threads, lds, s);
+  if (nbq == NBQ_ && U == U_) return launch_quad_cfg<BITS, NBQ_, U_>(p, grid, threads, lds, s);
   GQ_QUAD_CASE(1, 2) GQ_QUAD_CASE(1, 4) GQ_QUAD_CASE(1, 8)
   GQ_QUAD_CASE(2, 2) GQ_QUAD_CASE(2, 4) GQ_QUAD_CASE(2, 8)
 #undef GQ_QUAD_CASE
+  return hipErrorNotSupported;
+}
+
+hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s) {
+  if (a.bits == 4) return launch_quadrow_bits<4>(a, rows_max, s);
+  if (a.bits == 3) return launch_quadrow_bits<3>(a, rows_max, s);
   return hipErrorNotSupported;
 }
 

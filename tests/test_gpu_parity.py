@@ -284,40 +284,56 @@ def test_skinny_kernel_forms_grouped(mode):
     assert_linear_ok(out, o.dequantize_group_gemm_fp32(x, qw, qs, ip, s), x, k, f"grouped skinny mode {mode}")
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("u", [-1, 2, 8])  # iterations per item: heuristic, smallest, largest
 @pytest.mark.parametrize("m", [3, 4, 5, 8])
 @pytest.mark.parametrize("n,k", [(520, 1024), (100, 4096), (2100, 72), (64, 6176)])
-def test_quadrow_kernel(u, m, n, k):
+def test_quadrow_kernel(name, u, m, n, k):
     # the 4x4x4-MFMA kernel, forced; it is also what 3 <= M <= 8 takes by default
-    s = SCHEMES["q4f16_1"]
+    s = SCHEMES[name]
+    if s.bits == 3:
+        k = {1024: 1000, 4096: 4000, 72: 80, 6176: 6200}[k]  # whole, partial and odd group counts of 40
     x, qw, qs, b = _linear_case(s, m, n, k, 77 * m + n + k, bias=True)
     gq._lib.set_option("gemv_variant", 6)
     gq._lib.set_option("gemv_rows_per_wave", u)
     try:
-        y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b))
-        y32 = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, None, torch.float32)
+        y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
+        y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
     finally:
         gq._lib.set_option("gemv_variant", -1)
         gq._lib.set_option("gemv_rows_per_wave", -1)
     ref = o.linear_fp32(x, qw, qs, s, b)
-    assert_linear_ok(y, ref, x, k, f"quad-row u={u} {m}x{n}x{k}")
+    assert_linear_ok(y, ref, x, k, f"quad-row {name} u={u} {m}x{n}x{k}")
     assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"quad-row u={u} fp32 out")
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("waves", [-1, 8])  # 8 waves in all: every wave walks many quads
 @pytest.mark.parametrize("m,n,k", [(8, 64, 14336), (5, 520, 20520), (3, 132, 20480), (8, 520, 8200)])
-def test_quadrow_kernel_k_phases(waves, m, n, k):
+def test_quadrow_kernel_k_phases(name, waves, m, n, k):
     # x does not fit LDS whole: K is walked in 2-3 phases with partial sums parked in LDS
-    s = SCHEMES["q4f16_1"]
+    s = SCHEMES[name]
     x, qw, qs, b = _linear_case(s, m, n, k, 5 * m + n + k, bias=True)
     gq._lib.set_option("gemv_variant", 7)
     gq._lib.set_option("gemv_split", waves)
     try:
-        y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b))
+        y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
     finally:
         gq._lib.set_option("gemv_variant", -1)
         gq._lib.set_option("gemv_split", -1)
-    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"quad-row phases {m}x{n}x{k} waves={waves}")
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"quad-row phases {name} {m}x{n}x{k} waves={waves}")
+
+
+@pytest.mark.parametrize("m", [9, 12, 16])
+@pytest.mark.parametrize("n,k", [(520, 4000), (64, 14320), (132, 80)])
+def test_q3_nine_to_sixteen_rows_as_concurrent_passes(m, n, k):
+    # q3f16_1 has no 16x16x32 kernel: 9..16 rows run as two 8-row passes (four 4-row passes when
+    # 8 rows of x do not fit LDS) of the quad-row kernel, on the default path
+    s = SCHEMES["q3f16_1"]
+    x, qw, qs, b = _linear_case(s, m, n, k, 7 * m + n + k, bias=True)
+    res = np.random.default_rng(m + n).standard_normal((m, n)).astype(np.float16)
+    y = ops.linear(dev(x), dev(qw), dev(qs), 3, 40, dev(b), residual=dev(res))
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b) + res.astype(np.float64), x, k, f"q3 {m}x{n}x{k}")
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 64, 14336), (7, 520, 1024)])
@@ -345,9 +361,12 @@ def test_quadrow_kernel_declines_odd_shapes():
     assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, 256, "quad-row declined")
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("k", [1024, 14336])
-def test_quadrow_kernel_grouped(k):
-    s = SCHEMES["q4f16_1"]
+def test_quadrow_kernel_grouped(name, k):
+    s = SCHEMES[name]
+    if s.bits == 3:
+        k = k // 40 * 40
     rng = np.random.default_rng(62)
     ne, n = 5, 200
     w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
@@ -356,12 +375,12 @@ def test_quadrow_kernel_grouped(k):
     x = rng.standard_normal((40, k)).astype(np.float16)
     gq._lib.set_option("gemv_variant", 6)
     try:
-        out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), 4, 32)
-        out64 = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip.astype(np.int64)), 4, 32)
+        out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
+        out64 = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip.astype(np.int64)), s.bits, s.group_size)
     finally:
         gq._lib.set_option("gemv_variant", -1)
     ref = o.dequantize_group_gemm_fp32(x, qw, qs, ip, s)
-    assert_linear_ok(out, ref, x, k, f"grouped quad-row k={k}")
+    assert_linear_ok(out, ref, x, k, f"grouped quad-row {name} k={k}")
     assert_linear_ok(out64, ref, x, k, f"grouped quad-row k={k} int64 indptr")
 
 
