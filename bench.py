@@ -293,8 +293,24 @@ def main() -> int:
             nbytes = n * 4 * ng3 * 4 + n * ng3 * 2 + k * 2 + n * 2
             q3[name] = {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
                         "frac_hbm": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 3)}
+            if name == "gate_up":  # the same matrix at batch 4 / 8 (quad-row kernel) and as a 2048-row prefill GEMM
+                for m3 in (4, 8, 2048):
+                    xm3 = torch.randn((m3, k), generator=gx, device=dev).half()
+                    ym3 = torch.empty((m3, n), dtype=torch.float16, device=dev)
+
+                    def sweep3m():
+                        for qw, qs in ws[: (2 if m3 > 8 else len(ws))]:
+                            ops.linear(xm3, qw, qs, 3, 40, None, torch.float16, ym3)
+                    cnt3 = 2 if m3 > 8 else len(ws)
+                    us = timed(sweep3m, 3, 1, use_graph and m3 <= 8) * 1e3 / cnt3
+                    q3[f"gate_up_m{m3}"] = {"us": round(us, 2)}
+                    if m3 > 8:
+                        q3[f"gate_up_m{m3}"]["TFLOP/s"] = round(2.0 * m3 * n * k / us / 1e6, 1)
+                    else:
+                        q3[f"gate_up_m{m3}"]["GB/s"] = round(nbytes / us / 1e3, 1)
+                    del xm3, ym3
             del ws
-        extra["q3f16_1_gemv_b1"] = q3
+        extra["q3f16_1"] = q3
 
         # q4f16_1 Mixtral-8x7B MoE layer (BASELINE configs[4]): 8 experts, top-2, T in {1, 16, 512}
         from mlc_llm_amd import QUANTIZATION

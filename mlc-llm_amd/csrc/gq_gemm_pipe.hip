@@ -26,9 +26,10 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   constexpr int NT = 64 * (BM / WM) * (BN / WN);
   static_assert(NT == 256 || NT == 512, "4 or 8 waves per workgroup");
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int A_CHUNKS = BM * CPR / NT;
+  constexpr int A_CHUNKS = (BM * CPR + NT - 1) / NT;  // the last round may cover part of the threads only
+  constexpr bool A_EXACT = BM * CPR % NT == 0;
   constexpr int W_GROUPS = BN * 2 / NT;
-  static_assert(BM * CPR % NT == 0 && BN * 2 % NT == 0, "tile / thread mismatch");
+  static_assert(BN * 2 % NT == 0, "tile / thread mismatch");
 
   extern __shared__ uint4 smem[];
   uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
@@ -49,11 +50,14 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // ---- per-thread load slots: where each 16-byte chunk of x / each group of W comes from
   const uint16_t* a_src[A_CHUNKS];  // chunk address at K tile 0 (row clamped into the segment)
   bool a_row_ok[A_CHUNKS];
+  bool a_in_tile[A_CHUNKS];         // false: this thread has no chunk in round i (loads a valid address, stores nothing)
   int a_k[A_CHUNKS];                // k offset of the chunk inside a tile
   int a_dst[A_CHUNKS];              // offset (halves) inside the LDS tile
 #pragma unroll
   for (int i = 0; i < A_CHUNKS; ++i) {
-    const int idx = tid + NT * i;
+    const int idx_raw = tid + NT * i;
+    a_in_tile[i] = A_EXACT || idx_raw < BM * CPR;
+    const int idx = a_in_tile[i] ? idx_raw : 0;
     const int r = idx / CPR, c = idx - r * CPR;
     a_row_ok[i] = m0 + r < seg_hi;
     a_k[i] = 8 * c;
@@ -117,7 +121,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     for (int i = 0; i < A_CHUNKS; ++i) {
       if (i % KSTEPS != part) continue;
       const bool ok = a_row_ok[i] && (k_base + a_k[i] < k_lim);
-      *reinterpret_cast<uint4*>(at + a_dst[i]) = ok ? st.a[i] : make_uint4(0, 0, 0, 0);
+      if (A_EXACT || a_in_tile[i])
+        *reinterpret_cast<uint4*>(at + a_dst[i]) = ok ? st.a[i] : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < W_GROUPS; ++i) {
@@ -342,6 +347,10 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
       return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
   }
+  // q3: a K tile is 80 wide, so the 256 x 256 tile does not fit LDS; 128 x 256 does
+  const int64_t mid_tiles3 = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
+  if (variant == 9 || (variant != 6 && p.indptr == nullptr && mid_tiles3 >= 192))
+    return launch_pipe_cfg<3, 128, 256, 64, 64>(p, s);
   return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
 }
 

@@ -437,6 +437,19 @@ def test_few_row_gemm_split_counts_and_missing_workspace(want):
     assert_linear_ok(out, ref, x, k, "few-row gemm without workspace")
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 512, 1000), (129, 260, 4000), (513, 300, 200)])
+def test_gemm_q3_wide_tile(m, n, k):
+    # q3f16_1 on the 128 x 256 tile (a round of its activation loads covers only part of the threads)
+    s = SCHEMES["q3f16_1"]
+    x, qw, qs, b = _linear_case(s, m, n, k, 9000 + m + n + k, bias=True)
+    gq._lib.set_option("gemm_variant", 9)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), 3, 40, dev(b))
+    finally:
+        gq._lib.set_option("gemm_variant", -1)
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"q3 128x256 tile {m}x{n}x{k}")
+
+
 def test_gemm_k_not_multiple_of_8_takes_fallback():
     # K = 100: rows of x are not 16-byte aligned, the pipelined kernel declines and the plain one runs
     for name in ("q4f16_1", "q3f16_1"):
