@@ -415,6 +415,19 @@ def test_few_row_gemm_split_k(name, m, n, k):
         assert ws > 0 and ws % (m * n * 4) == 0  # these shapes do split
 
 
+@pytest.mark.parametrize("m", [17, 32, 33, 64, 65, 96, 128])
+@pytest.mark.parametrize("n,k", [(520, 4096), (130, 14336), (384, 1000), (257, 4104)])
+def test_few_row_gemm_q4_with_residual(m, n, k):
+    s = SCHEMES["q4f16_1"]
+    x, qw, qs, b = _linear_case(s, m, n, k, 17 * m + n + k, bias=True)
+    res = np.random.default_rng(m + k).standard_normal((m, n)).astype(np.float16)
+    y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b), residual=dev(res))
+    y32 = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, None, torch.float32)
+    ref = o.linear_fp32(x, qw, qs, s, b)
+    assert_linear_ok(y, ref + res.astype(np.float64), x, k, f"few-row gemm {m}x{n}x{k}")
+    assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"few-row gemm fp32 out {m}x{n}x{k}")
+
+
 @pytest.mark.parametrize("want", [64, 4096])  # few / as many splits as K allows
 def test_few_row_gemm_split_counts_and_missing_workspace(want):
     s = SCHEMES["q4f16_1"]
