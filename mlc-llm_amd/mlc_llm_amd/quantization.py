@@ -89,9 +89,9 @@ class GroupQuantize:
         return _DTYPE_BITS[self.quantize_dtype]
 
     def _require_built(self):
-        if self.model_dtype != "float16" or self.linear_weight_layout != "NK":
+        if self.model_dtype != "float16":
             raise NotImplementedError(
-                f"{self.name}: only float16 / NK-layout group quantization has gfx950 kernels"
+                f"{self.name}: only float16 group quantization has gfx950 kernels"
             )
 
     def quantize_weight(self, weight: torch.Tensor, axis: int = -1, output_transpose: bool = False
@@ -101,10 +101,13 @@ class GroupQuantize:
         axis = axis if axis >= 0 else weight.dim() + axis
         if axis != weight.dim() - 1:
             raise NotImplementedError("quantize_weight: only the last axis is supported (NK layout)")
-        if output_transpose:
-            raise NotImplementedError("quantize_weight: output_transpose belongs to the KN layouts")
         mode = _lib.ROUND_HALF_AWAY if self.round_mode == "half_away" else _lib.ROUND_HALF_EVEN
         qw, qs = ops.quantize(weight.contiguous(), self.bits, self.group_size, mode)
+        if output_transpose:
+            # the KN layouts store the same words and scales transposed (group_quantization.py:299-305)
+            if qw.dim() != 2 or qs.dim() != 2:
+                raise ValueError("Does not support transpose output quantized weight with ndim != 2")
+            qw, qs = qw.t().contiguous(), qs.t().contiguous()
         return [qw, qs]
 
     def dequantize_weight(self, q_weight: torch.Tensor, q_scale: torch.Tensor, in_features: int
@@ -215,17 +218,38 @@ class GroupQuantizeLinear(nn.Module):
             device=src.weight.device,
         )
 
+    def _nk_tensors(self):
+        """(q_weight, q_scale) in the [N, ...] layout the kernels stream.  A KN-layout module
+        (q4f16_0 / q3f16_0: the same words and scales, transposed) keeps a transposed copy, made
+        on the device the first time it is needed and again after load_state_dict or when the
+        parameter tensors are replaced; writing into them in place (`.data.copy_`) needs
+        `invalidate_layout_cache()`."""
+        if self.config.linear_weight_layout == "NK":
+            return self.q_weight, self.q_scale
+        key = (self.q_weight.data_ptr(), self.q_scale.data_ptr())
+        if getattr(self, "_nk_key", None) != key:
+            self._nk = (self.q_weight.detach().t().contiguous(), self.q_scale.detach().t().contiguous())
+            self._nk_key = key
+        return self._nk
+
+    def invalidate_layout_cache(self) -> None:
+        self._nk_key = None
+        self._nk = None
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)
+        self.invalidate_layout_cache()
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         self.config._require_built()
         out_dtype = torch.float16 if self.out_dtype is None else _TORCH_DTYPE[self.out_dtype]
+        q_weight, q_scale = self._nk_tensors()
         bias = self.bias
         if bias is not None and bias.dtype != torch.float16:
             # fp32 bias with fp32 output: added after the kernel, as the reference's `x + bias`
-            y = ops.linear(x, self.q_weight, self.q_scale, self.config.bits,
-                           self.config.group_size, None, out_dtype)
+            y = ops.linear(x, q_weight, q_scale, self.config.bits, self.config.group_size, None, out_dtype)
             return y + bias
-        return ops.linear(x, self.q_weight, self.q_scale, self.config.bits,
-                          self.config.group_size, bias, out_dtype)
+        return ops.linear(x, q_weight, q_scale, self.config.bits, self.config.group_size, bias, out_dtype)
 
 
 class GroupQuantizeEmbedding(nn.Module):
@@ -333,7 +357,7 @@ def _group(name: str, group_size: int, qdtype: str, layout: str, model_dtype: st
 
 
 # The group-quant entries of the reference registry (quantization.py:47-90).  The KN-layout
-# entries are listed so that names resolve; their kernels are not built (NotImplementedError).
+# entries hold the NK tensors transposed; their linears run the NK kernels on a transposed copy.
 QUANTIZATION: Dict[str, GroupQuantize] = {
     "q3f16_0": _group("q3f16_0", 40, "int3", "KN"),
     "q3f16_1": _group("q3f16_1", 40, "int3", "NK"),

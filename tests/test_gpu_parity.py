@@ -548,6 +548,34 @@ def test_linear_module_matches_reference_interface():
             o.dequantize(host_u32(qw), qs.cpu().numpy(), SCHEMES["q4f16_1"], 256).view(np.uint16)).all()
 
 
+@pytest.mark.parametrize("kn_name,nk_name", [("q4f16_0", "q4f16_1"), ("q3f16_0", "q3f16_1")])
+def test_kn_layout_is_the_transposed_nk_tensors(kn_name, nk_name):
+    # q4f16_0 / q3f16_0 (reference quantization.py:47-79, transpose at group_quantization.py:299-305)
+    kn, nk = gq.QUANTIZATION[kn_name], gq.QUANTIZATION[nk_name]
+    s = SCHEMES[nk_name]
+    k = 8 * s.group_size
+    rng = np.random.default_rng(21)
+    w = (rng.standard_normal((96, k)) * 0.05).astype(np.float16)
+    qw_ref, qs_ref = o.quantize(w, s)
+    qw, qs = kn.quantize_weight(dev(w), output_transpose=True)
+    assert tuple(qw.shape) == (qw_ref.shape[1], 96) and tuple(qs.shape) == (qs_ref.shape[1], 96)
+    assert np.array_equal(host_u32(qw), qw_ref.T) and np.array_equal(host_f16_bits(qs), qs_ref.view(np.uint16).T)
+    lin_kn = gq.GroupQuantizeLinear(k, 96, kn, bias=False, device=DEV)
+    lin_nk = gq.GroupQuantizeLinear(k, 96, nk, bias=False, device=DEV)
+    lin_kn.q_weight.data, lin_kn.q_scale.data = qw, qs
+    lin_nk.q_weight.data, lin_nk.q_scale.data = dev(qw_ref), dev(qs_ref)
+    for m in (1, 5, 40):
+        x = dev(rng.standard_normal((m, k)).astype(np.float16))
+        assert torch.equal(lin_kn(x), lin_nk(x))
+    # new parameters are picked up (the transposed copy is remade)
+    w2 = (rng.standard_normal((96, k)) * 0.05).astype(np.float16)
+    qw2, qs2 = kn.quantize_weight(dev(w2), output_transpose=True)
+    lin_kn.load_state_dict({"q_weight": qw2, "q_scale": qs2})
+    x = rng.standard_normal((3, k)).astype(np.float16)
+    q2w, q2s = o.quantize(w2, s)
+    assert_linear_ok(lin_kn(dev(x)), o.linear_fp32(x, q2w, q2s, s), x, k, "KN after update")
+
+
 # ------------------------------------------------------------------ MoE
 
 

@@ -93,8 +93,11 @@ def test_registry_and_derived_fields():
     assert q4.linear_quant_axis == 1 and gq.QUANTIZATION["q4f16_0"].linear_quant_axis == 0
     with pytest.raises(ValueError, match="divisible"):
         gq.GroupQuantize("bad", "group-quant", 36, "int3", "uint32", "float16", "NK")
-    with pytest.raises(NotImplementedError):
-        gq.QUANTIZATION["q4f16_0"].quantize_weight(torch.zeros(4, 32, dtype=torch.float16))
+    # the KN entries describe the same tensors transposed: [nw, N] words, [ng, N] scales
+    kn = gq.GroupQuantizeLinear(64, 24, gq.QUANTIZATION["q4f16_0"], bias=False)
+    assert tuple(kn.q_weight.shape) == (8, 24) and tuple(kn.q_scale.shape) == (2, 24)
+    kn3 = gq.GroupQuantizeLinear(80, 24, gq.QUANTIZATION["q3f16_0"], bias=False)
+    assert tuple(kn3.q_weight.shape) == (8, 24) and tuple(kn3.q_scale.shape) == (2, 24)
 
 
 def test_name_predicates():
