@@ -271,7 +271,7 @@ def main() -> int:
                                           "GB/s": round(2 * 2**30 / (ms * 1e-3) / 1e9, 1)}
         del bufs
 
-        # q3f16_1 decode GEMV at Llama-2-7B shapes, batch 1 (BASELINE configs[3])
+        # q3f16_1 decode GEMV at Llama-2-7B shapes, batch 1 (the q3 configuration of the benchmark definition)
         q3 = {}
         for name, (n, k) in {"qkv": (12288, 4096), "o_proj": (4096, 4096), "gate_up": (22016, 4096),
                              "down": (4096, 11008)}.items():
@@ -312,7 +312,7 @@ def main() -> int:
             del ws
         extra["q3f16_1"] = q3
 
-        # q4f16_1 Mixtral-8x7B MoE layer (BASELINE configs[4]): 8 experts, top-2, T in {1, 16, 512}
+        # q4f16_1 Mixtral-8x7B MoE layer (the MoE configuration of the benchmark definition): 8 experts, top-2, T in {1, 16, 512}
         from mlc_llm_amd import QUANTIZATION
         from mlc_llm_amd.nn import MixtralMoE
 
