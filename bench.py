@@ -340,6 +340,28 @@ def main() -> int:
         extra["mixtral_moe_layer"] = moe_res
         del moe
 
+        # packing, unpacking and the embedding gather: HBM-bound byte work, algorithmic bytes =
+        # fp16 matrix + packed words + scales (each once)
+        pk = {}
+        n, k = SHAPES["gate_up"]
+        wq = (torch.randn((n, k), generator=gx, device=dev) * 0.02).half()
+        for bits_, g_ in ((4, 32), (3, 40)):
+            kq = k if bits_ == 4 else (k // 40) * 40
+            wv = wq[:, :kq].contiguous()
+            qwq, qsq = ops.quantize(wv, bits_, g_)
+            nbytes = wv.numel() * 2 + qwq.numel() * 4 + qsq.numel() * 2
+            ms = timed(lambda: ops.quantize(wv, bits_, g_), 5, 2, False)
+            pk[f"quantize_q{bits_}_gate_up"] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
+            ms = timed(lambda: ops.dequantize(qwq, qsq, kq, bits_, g_), 5, 2, False)
+            pk[f"dequantize_q{bits_}_gate_up"] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
+            del wv, qwq, qsq
+        del wq
+        ids = torch.randint(0, LM_HEAD[0], (8192,), generator=gx, device=dev, dtype=torch.int32)
+        ms = timed(lambda: ops.embedding_take(ids, lm_head[0], lm_head[1], LM_HEAD[1], BITS, G), 5, 2, False)
+        row_bytes = LM_HEAD[1] // G * 18 + LM_HEAD[1] * 2  # packed row + scales read, fp16 row written
+        pk["embedding_take_8192_tokens"] = {"us": round(ms * 1e3, 1), "GB/s": round(8192 * row_bytes / ms / 1e6, 1)}
+        extra["packing"] = pk
+
     # ---------------------------------------------------------------- CPU baseline (bounded sample)
     cpu = None
     if not args.skip_cpu:

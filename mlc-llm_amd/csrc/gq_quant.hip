@@ -74,10 +74,21 @@ __global__ __launch_bounds__(256) void quantize_kernel(const uint16_t* __restric
   const float m = static_cast<float>(S::kMaxInt);
   const uint16_t sh = f2h(amax / m);  // fp16 divide: float divide, one rounding to half
   const float s = h2f(sh);
+  // v / s for the E values of this word.  The fp16 quotient of two halves is the float quotient
+  // rounded once more; a float quotient within half an ulp (plus a hair) rounds to the same half,
+  // because a ratio of two 11-bit significands that is not itself a rounding boundary of fp16
+  // stays more than 2^-23 (relative) away from one.  One Newton step on the hardware reciprocal
+  // gives that accuracy for a third of the instructions of a correctly rounded divide.  s = 0
+  // (an all-zero or denormal-only group) and overflowing quotients keep the first product, which
+  // is the NaN / infinity the plain divide yields.
+  const float rs = __builtin_amdgcn_rcpf(s);
   uint32_t word = 0;
 #pragma unroll
   for (int i = 0; i < E; ++i) {
-    float t = h2f(f2h(v[i] / s));  // fp16 divide
+    const float q0 = v[i] * rs;
+    const float q1 = fmaf(fmaf(-q0, s, v[i]), rs, q0);
+    const float quo = (s == 0.0f || fabsf(q0) == __builtin_inff()) ? q0 : q1;
+    float t = h2f(f2h(quo));  // fp16 divide
     t = h2f(f2h(t + m));           // fp16 add
     float r = half_even ? rintf(t) : roundf(t);
     r = (r > 0.0f) ? r : 0.0f;  // compare+select max: NaN (0/0) becomes 0

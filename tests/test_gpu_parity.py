@@ -95,6 +95,28 @@ def test_quantize_extreme_values():
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_quantize_bit_exact_16m_values_all_magnitudes(name, mode):
+    # 16.7 M values whose group maxima sweep the whole fp16 exponent range (denormal scales
+    # included): the kernel's divide is a reciprocal plus one Newton step, and must still land on
+    # the half the plain fp16 divide gives, every time.  Checked against the C restatement.
+    from oracle import c_oracle
+
+    s = SCHEMES[name]
+    rng = np.random.default_rng(1234 + mode)
+    rows, k = 4096, 4096 if s.bits == 4 else 4080
+    mag = np.exp2(rng.uniform(-24, 15, size=(rows, k // s.group_size, 1))).astype(np.float32)
+    w = (rng.standard_normal((rows, k // s.group_size, s.group_size)).astype(np.float32) * mag)
+    w = np.clip(w, -65504, 65504).astype(np.float16).reshape(rows, k)
+    w[::97, ::5] = 0
+    qw_ref, qs_ref = c_oracle.quantize(w, s.bits, s.group_size, mode)
+    qw, qs = ops.quantize(dev(w), s.bits, s.group_size, mode)
+    assert np.array_equal(host_f16_bits(qs), qs_ref.view(np.uint16))
+    bad = np.nonzero(host_u32(qw) != qw_ref)
+    assert bad[0].size == 0, f"{bad[0].size} words differ, first at {bad[0][0]}, {bad[1][0]}"
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 def test_quantize_full_size_roundtrip_properties(name):
     # full decode shape: codes in range, re-quantizing the dequantized matrix is idempotent on
     # the codes' dequantized values, and a row sample agrees with the oracle bit for bit
