@@ -1,5 +1,6 @@
 // C ABI of libmi355gq.so: argument validation, error reporting, dispatch to the launchers.
 // Declarations (with the reference interface each entry replaces) live in include/mi355gq.h.
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
@@ -66,6 +67,28 @@ int check_scheme(int bits, int group_size) {
 hipStream_t as_stream(mi355gq_stream_t s) { return static_cast<hipStream_t>(s); }
 
 constexpr int64_t kMaxDim = int64_t(1) << 31;
+
+// K = 0: the product is empty, the output is bias + residual (zeros without them).  The matmul
+// kernels all assume at least one group, so this case never reaches them.
+__global__ void empty_k_kernel(const __half* bias, const __half* residual, void* y, int64_t count,
+                               int64_t N, int out_f32) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  float v = bias ? __half2float(bias[i % N]) : 0.f;  // one rounding at the end, as in the matmul epilogues
+  if (residual) v += __half2float(residual[i]);
+  if (out_f32) static_cast<float*>(y)[i] = v;
+  else static_cast<__half*>(y)[i] = __float2half(v);
+}
+
+int launch_empty_k(const void* bias, const void* residual, void* y, int64_t rows, int64_t N, int out_f32,
+                   hipStream_t s) {
+  const int64_t count = rows * N;
+  if (count >= (int64_t(1) << 39)) return fail(MI355GQ_ERR_ARG, "K=0 output of %lld elements", (long long)count);
+  hipLaunchKernelGGL(empty_k_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, s,
+                     static_cast<const __half*>(bias), static_cast<const __half*>(residual), y, count, N,
+                     out_f32);
+  return hip_result(hipGetLastError(), "K=0 fill launch");
+}
 
 }  // namespace
 
@@ -187,6 +210,7 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // y may be the residual buffer itself (same element type), nothing else may overlap it
   GQ_REQUIRE(residual == nullptr || residual != y || out_dtype == MI355GQ_F16,
              "linear: in-place residual needs a float16 output");
+  if (K == 0) return launch_empty_k(bias, residual, y, M, N, out_dtype == MI355GQ_F32, as_stream(stream));
   // regimes: M <= 2 register GEMV; 3..8 quad-row kernel (LDS GEMV when it declines a q3 shape);
   // 9..16 MFMA skinny kernel (q4); else GEMM
   gq::GemmArgs g{};
@@ -258,10 +282,11 @@ int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const 
   GQ_REQUIRE(x_rows == 1 || x_rows == top_k, "moe_gemv: x has %lld rows, expected 1 or top_k=%lld",
              (long long)x_rows, (long long)top_k);
   if (top_k == 0 || N == 0) return MI355GQ_OK;
-  GQ_REQUIRE(x && q_weight && q_scale && expert_ids && out, "moe_gemv: null pointer");
+  GQ_REQUIRE(out && (K == 0 || (x && q_weight && q_scale && expert_ids)), "moe_gemv: null pointer");
   GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned4(expert_ids) && aligned2(out),
              "moe_gemv: x and q_weight must be 16-byte aligned");
   GQ_REQUIRE(x_rows == 1 || (K % 8) == 0, "moe_gemv: K must be a multiple of 8 when x has top_k rows");
+  if (K == 0) return launch_empty_k(nullptr, nullptr, out, top_k, N, 0, as_stream(stream));
   gq::GemvArgs a{};
   a.x = static_cast<const uint16_t*>(x);
   a.q_weight = static_cast<const uint32_t*>(q_weight);
@@ -286,11 +311,12 @@ int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, co
   GQ_REQUIRE(indptr_dtype == MI355GQ_I32 || indptr_dtype == MI355GQ_I64,
              "moe_group_gemm: indptr_dtype=%d", indptr_dtype);
   if (rows == 0 || N == 0) return MI355GQ_OK;
-  GQ_REQUIRE(x && q_weight && q_scale && indptr && out, "moe_group_gemm: null pointer");
+  GQ_REQUIRE(out && (K == 0 || (x && q_weight && q_scale && indptr)), "moe_group_gemm: null pointer");
   GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned16(out) &&
                  (indptr_dtype == MI355GQ_I32 ? aligned4(indptr)
                                               : (reinterpret_cast<uintptr_t>(indptr) & 7u) == 0),
              "moe_group_gemm: x, q_weight and out must be 16-byte aligned");
+  if (K == 0) return launch_empty_k(nullptr, nullptr, out, rows, N, 0, as_stream(stream));
   gq::GemmArgs g{};
   g.x = static_cast<const uint16_t*>(x);
   g.q_weight = static_cast<const uint32_t*>(q_weight);

@@ -389,7 +389,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   constexpr int CH = GemvTraits<BITS>::CH;
   if (a.group_size != G) return hipErrorNotSupported;
   if (a.rows == 0 || a.N == 0) return hipSuccess;
-  if ((a.N & 3) != 0 || (a.K & 7) != 0) return hipErrorNotSupported;
+  if ((a.N & 3) != 0 || (a.K & 7) != 0 || a.K == 0) return hipErrorNotSupported;
   if ((reinterpret_cast<uintptr_t>(a.x) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.y) & 15) != 0 ||
       (reinterpret_cast<uintptr_t>(a.bias) & 7) != 0 || (reinterpret_cast<uintptr_t>(a.residual) & 7) != 0 ||
       (reinterpret_cast<uintptr_t>(a.q_weight) & 15) != 0)

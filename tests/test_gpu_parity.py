@@ -771,6 +771,74 @@ def test_stream_read_probe_runs_and_validates():
     assert gq._lib.lib().mi355gq_probe_stream_read(a.data_ptr(), 24, None, 0, None, None) == -1  # not a multiple of 16
 
 
+# ------------------------------------------------------------------ degenerate and hostile inputs
+
+def test_degenerate_sizes_every_entry_point():
+    s = SCHEMES["q4f16_1"]
+    x, qw, qs, _ = _linear_case(s, 3, 8, 64, 5)
+    xd, qwd, qsd = dev(x), dev(qw), dev(qs)
+    # no rows / no columns: nothing is launched, shapes come back right
+    assert tuple(ops.linear(xd[:0], qwd, qsd, 4, 32).shape) == (0, 8)
+    assert tuple(ops.linear(xd, qwd[:0], qsd[:0], 4, 32).shape) == (3, 0)
+    q0, s0 = ops.quantize(torch.empty((0, 64), dtype=torch.float16, device=DEV), 4, 32)
+    assert tuple(q0.shape) == (0, 8) and tuple(s0.shape) == (0, 2)
+    assert tuple(ops.dequantize(qwd[:0], qsd[:0], 64, 4, 32).shape) == (0, 64)
+    # K = 0: the product is the bias
+    b = dev(np.arange(8, dtype=np.float16))
+    y = ops.linear(torch.empty((3, 0), dtype=torch.float16, device=DEV), qwd[:, :0].contiguous(),
+                   qsd[:, :0].contiguous(), 4, 32, b)
+    assert torch.equal(y, b.expand(3, 8))
+    res = dev(np.random.default_rng(1).standard_normal((3, 8)).astype(np.float16))
+    xe = torch.empty((3, 0), dtype=torch.float16, device=DEV)
+    for m in (1, 3, 12, 40):  # one per kernel regime: each hands K = 0 to the same fill
+        yr = ops.linear(xe[:1].expand(m, 0).contiguous(), qwd[:, :0].contiguous(), qsd[:, :0].contiguous(), 4, 32, b,
+                        out_dtype=torch.float32, residual=res[:1].expand(m, 8).contiguous())
+        assert torch.equal(yr, (b.float() + res[:1].float()).expand(m, 8))
+    ew, es = torch.zeros((4, 8, 0), dtype=torch.int32, device=DEV), torch.zeros((4, 8, 0), dtype=torch.float16, device=DEV)
+    eids = torch.tensor([[0, 3]], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.moe_gemv(xe[:1], ew, es, eids, 4, 32), torch.zeros((2, 8), dtype=torch.float16, device=DEV))
+    ip = torch.tensor([0, 1, 1, 2, 3], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.moe_group_gemm(xe, ew, es, ip, 4, 32), torch.zeros((3, 8), dtype=torch.float16, device=DEV))
+    # routing with no tokens
+    w, ids = ops.gating_softmax_topk(torch.empty((0, 8), dtype=torch.float16, device=DEV), 2)
+    assert tuple(w.shape) == (0, 2) and tuple(ids.shape) == (0, 2)
+    # grouped matmul where every expert is empty
+    eqw = torch.zeros((4, 8, 8), dtype=torch.int32, device=DEV)
+    eqs = torch.zeros((4, 8, 2), dtype=torch.float16, device=DEV)
+    out = ops.moe_group_gemm(torch.empty((0, 64), dtype=torch.float16, device=DEV), eqw, eqs,
+                             torch.zeros(5, dtype=torch.int32, device=DEV), 4, 32)
+    assert tuple(out.shape) == (0, 8)
+
+
+def test_hostile_indices_stay_inside_the_tensors():
+    # ids outside the table, expert ids outside the experts and a scrambled indptr are clamped:
+    # results for the valid entries are right and nothing outside the buffers is touched
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(8)
+    w = (rng.standard_normal((3, 16, 64)) * 0.05).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    table_w, table_s = dev(qw[0]), dev(qs[0])
+    ids = torch.tensor([0, 15, -7, 16, 2**30], dtype=torch.int32, device=DEV)
+    emb = ops.embedding_take(ids, table_w, table_s, 64, 4, 32)
+    ref = o.dequantize(qw[0], qs[0], s, 64)
+    assert np.array_equal(host_f16_bits(emb[:2]), ref[[0, 15]].view(np.uint16))
+    assert np.array_equal(host_f16_bits(emb[2:]), ref[[0, 15, 15]].view(np.uint16))  # clamped into the table
+    x = rng.standard_normal((1, 64)).astype(np.float16)
+    eids = torch.tensor([[1, 9]], dtype=torch.int32, device=DEV)  # 9 is past the 3 experts: clamped to 2
+    y = ops.moe_gemv(dev(x), dev(qw), dev(qs), eids, 4, 32)
+    assert_linear_ok(y[0:1], o.linear_fp32(x, qw[1], qs[1], s), x, 64, "expert 1")
+    assert_linear_ok(y[1:2], o.linear_fp32(x, qw[2], qs[2], s), x, 64, "expert id clamped")
+    xs = rng.standard_normal((6, 64)).astype(np.float16)
+    # decreasing, then past the rows: read as [0,4) [4,4) [2,6), so rows 2..3 belong to two experts
+    # (either may win) and the others to exactly one
+    bad_ip = torch.tensor([0, 4, 2, 99], dtype=torch.int32, device=DEV)
+    out = ops.moe_group_gemm(dev(xs), dev(qw), dev(qs), bad_ip, 4, 32)
+    torch.cuda.synchronize()
+    assert tuple(out.shape) == (6, 16) and torch.isfinite(out.float()).all()
+    assert_linear_ok(out[:2], o.linear_fp32(xs[:2], qw[0], qs[0], s), xs[:2], 64, "rows of the first segment only")
+    assert_linear_ok(out[4:], o.linear_fp32(xs[4:], qw[2], qs[2], s), xs[4:], 64, "rows of the clamped last segment")
+
+
 # ------------------------------------------------------------------ HIP graph capture
 
 def test_linear_and_moe_replay_in_hip_graph():
