@@ -189,7 +189,7 @@ def main() -> int:
     us_read = timed(read_sweep, max(5, args.steps), 2, use_graph) * 1e3 / LAYERS
     read_bytes = layers[0]["gate_up"][0].numel() * 4 + layers[0]["gate_up"][1].numel() * 2
     roofline = {
-        "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2,false> (gate_up 28672x4096, batch 1)",
+        "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2,0> (gate_up 28672x4096, batch 1)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
         "bytes_per_launch": gu_bytes, "us_per_launch": round(us_gate_up, 3),
@@ -256,6 +256,24 @@ def main() -> int:
             lib[f"{name}_m{m}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 1)}
             del wd
         extra["library_dense_fp16_gemm_reference"] = lib
+        # gate_up with silu(x1) * x2 folded into the matmul kernel, against the two calls it replaces
+        fused = {}
+        n, k = SHAPES["gate_up"]
+        for mf in (1, 8, 2048):
+            xf = xm[k][:mf].contiguous()
+            sweep_layers = layers if mf <= 8 else layers[:1]  # one launch per layer's weights, as in the GEMV lines
+
+            def run_fused():
+                for lw in sweep_layers:
+                    ops.linear_silu_mul(xf, lw["gate_up"][0], lw["gate_up"][1], BITS, G)
+
+            def run_two():
+                for lw in sweep_layers:
+                    ops.silu_mul(ops.linear(xf, lw["gate_up"][0], lw["gate_up"][1], BITS, G))
+            us_f = timed(run_fused, 5, 2, use_graph) * 1e3 / len(sweep_layers)
+            us_2 = timed(run_two, 5, 2, use_graph) * 1e3 / len(sweep_layers)
+            fused[f"m{mf}"] = {"fused_us": round(us_f, 1), "linear_then_silu_mul_us": round(us_2, 1)}
+        extra["gate_up_silu_mul"] = fused
         del xm
         extra["decode_tokens_per_s_linear_only"] = round(1e3 / ms_step, 1)
 

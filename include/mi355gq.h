@@ -124,6 +124,27 @@ MI355GQ_API int mi355gq_linear_residual(const void* x, const void* q_weight, con
                             int64_t workspace_bytes, mi355gq_stream_t stream);
 
 /*
+ * gate_up projection with the activation folded in: the sequence
+ *   x1, x2 = split(gate_up_proj(x), 2, axis=-1); silu(x1) * x2
+ * of the MLP (model/llama/llama_model.py:122-125; for the experts model/mixtral/mixtral_model.py:64-68),
+ * the element-wise tail the FasterTransformer precedent folds into its matmul as an `activation`
+ * argument (op/ft_gemm.py:72-92).  q_weight / q_scale are the unchanged [N, ...] tensors whose first
+ * N / 2 rows are the gate and last N / 2 rows the up projection:
+ *   y[M, N / 2] = silu(x . W[j]^T) * (x . W[N / 2 + j]^T),  y fp16
+ * with the rounding points of the unfused sequence (fp16 matmul outputs, silu evaluated in fp32 and
+ * rounded to fp16, fp16 product), so the result equals mi355gq_linear followed by mi355gq_silu_mul
+ * bit for bit while the [M, N] intermediate never reaches memory.  N must be even.
+ * Returns MI355GQ_ERR_UNSUPPORTED for shapes no fused kernel takes (K not a multiple of 8; the
+ * caller then runs the two calls).  workspace as for mi355gq_linear, sized by
+ * mi355gq_linear_silu_mul_workspace_bytes().
+ */
+MI355GQ_API int64_t mi355gq_linear_silu_mul_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits,
+                                                            int group_size);
+MI355GQ_API int mi355gq_linear_silu_mul(const void* x, const void* q_weight, const void* q_scale, int64_t M,
+                            int64_t N, int64_t K, int bits, int group_size, void* y, void* workspace,
+                            int64_t workspace_bytes, mi355gq_stream_t stream);
+
+/*
  * moe_matmul.dequantize_gemv (python/mlc_llm/op/moe_matmul.py:77-176), single-token MoE:
  *   out[e, :] = x[x_rows == 1 ? 0 : e, :] . dequantize(W[expert_ids[e]])^T,  e < top_k
  * x fp16 [x_rows, K] with x_rows in {1, top_k}; expert_ids int32 [1, top_k];
@@ -143,6 +164,23 @@ MI355GQ_API int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* 
                            const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
                            int64_t K, int bits, int group_size, void* out,
                            mi355gq_stream_t stream);
+
+/*
+ * The e1_e3 expert matmul of MixtralMoE with its activation folded in (mixtral_model.py:64-68:
+ * x1, x3 = split(e1_e3(x, indptr), 2, axis=-1); silu(x1) * x3), in both forms of the expert matmul.
+ * Same arguments as mi355gq_moe_gemv / mi355gq_moe_group_gemm; N is the stored row count of an
+ * expert (gate rows then up rows, N even) and out is fp16 [top_k | rows, N / 2]; results equal the
+ * unfused call followed by mi355gq_silu_mul bit for bit.  MI355GQ_ERR_UNSUPPORTED when no fused
+ * kernel takes the shape.
+ */
+MI355GQ_API int mi355gq_moe_gemv_silu_mul(const void* x, int64_t x_rows, const void* q_weight,
+                              const void* q_scale, const void* expert_ids, int64_t top_k,
+                              int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,
+                              void* out, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_moe_group_gemm_silu_mul(const void* x, int64_t rows, const void* q_weight,
+                                    const void* q_scale, const void* indptr, int indptr_dtype,
+                                    int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,
+                                    void* out, mi355gq_stream_t stream);
 
 /* ---- routing glue of the MoE layer (python/mlc_llm/op/moe_misc.py) ---- */
 

@@ -192,10 +192,20 @@ int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits
   return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
 }
 
+int64_t mi355gq_linear_silu_mul_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
+  if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
+      N >= kMaxDim || K >= kMaxDim)
+    return 0;
+  if (M <= 16 || (N % 64) != 0) return 0;  // GEMV / few-row kernels, or a shape that never splits
+  return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+}
+
+// paired: the fused gate/up form (y fp16 [M, N / 2]); a shape no fused kernel takes is an
+// MI355GQ_ERR_UNSUPPORTED, for which the caller runs linear and silu_mul
 static int linear_impl(const void* x, const void* q_weight, const void* q_scale, const void* bias,
                        const void* residual, int64_t M, int64_t N, int64_t K, int bits, int group_size,
                        int out_dtype, void* y, void* workspace, int64_t workspace_bytes,
-                       mi355gq_stream_t stream) {
+                       mi355gq_stream_t stream, bool paired = false) {
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
              "linear: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
@@ -210,6 +220,10 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // y may be the residual buffer itself (same element type), nothing else may overlap it
   GQ_REQUIRE(residual == nullptr || residual != y || out_dtype == MI355GQ_F16,
              "linear: in-place residual needs a float16 output");
+  if (paired) {
+    GQ_REQUIRE((N & 1) == 0, "linear_silu_mul: N=%lld must be even (gate rows, then up rows)", (long long)N);
+    if (K == 0) return launch_empty_k(nullptr, nullptr, y, M, N / 2, 0, as_stream(stream));  // silu(0) * 0
+  }
   if (K == 0) return launch_empty_k(bias, residual, y, M, N, out_dtype == MI355GQ_F32, as_stream(stream));
   // regimes: M <= 2 register GEMV; 3..8 quad-row kernel (LDS GEMV when it declines a q3 shape);
   // 9..16 MFMA skinny kernel (q4); else GEMM
@@ -224,6 +238,28 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
   g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
   g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
+  g.paired = paired;
+  if (paired) {
+    // the regimes of the plain linear: register GEMV up to 2 rows, quad-row kernel up to 8 (q3: 16),
+    // skinny kernel up to 16 (q4), else the pipelined GEMM
+    hipError_t e = hipErrorNotSupported;
+    if (M <= 2) {
+      gq::GemvArgs a{};
+      a.x = g.x; a.q_weight = g.q_weight; a.q_scale = g.q_scale; a.bias = nullptr; a.y = y;
+      a.expert_ids = nullptr;
+      a.M = M; a.N = N; a.K = K; a.slots = 1; a.x_slot_stride = 0; a.num_experts = 1;
+      a.bits = bits; a.group_size = group_size; a.out_f32 = 0; a.paired = 1;
+      e = gq::launch_gemv(a, as_stream(stream));
+    } else if (M <= (bits == 3 ? 16 : 8)) {
+      e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
+    }
+    if (e == hipErrorNotSupported && M <= 16 && bits == 4) e = gq::launch_skinny(g, static_cast<int>(M), as_stream(stream));
+    if (e == hipErrorNotSupported) e = gq::launch_gemm(g, as_stream(stream));
+    if (e == hipErrorNotSupported)
+      return fail(MI355GQ_ERR_UNSUPPORTED, "linear_silu_mul: no fused kernel for M=%lld N=%lld K=%lld (K %% 8 != 0?)",
+                  (long long)M, (long long)N, (long long)K);
+    return hip_result(e, "linear_silu_mul launch");
+  }
   const int gv = gq::options().gemv_variant;  // 2..5 force a gq_skinny.hip form, 6..8 the quad-row kernel
   const int gm = gq::options().gemm_variant;  // 1: GEMM only, 2: GEMV up to 8 rows
   // (q3 has no 16x16x32 skinny kernel: 9..16 rows run as two concurrent 8-row passes of the quad-row kernel)
@@ -272,9 +308,17 @@ int mi355gq_linear_residual(const void* x, const void* q_weight, const void* q_s
                      workspace, workspace_bytes, stream);
 }
 
-int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
-                     const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N,
-                     int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream) {
+int mi355gq_linear_silu_mul(const void* x, const void* q_weight, const void* q_scale, int64_t M, int64_t N,
+                            int64_t K, int bits, int group_size, void* y, void* workspace,
+                            int64_t workspace_bytes, mi355gq_stream_t stream) {
+  return linear_impl(x, q_weight, q_scale, nullptr, nullptr, M, N, K, bits, group_size, MI355GQ_F16, y,
+                     workspace, workspace_bytes, stream, true);
+}
+
+static int moe_gemv_impl(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                         const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N,
+                         int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream,
+                         bool paired) {
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(top_k >= 0 && top_k <= 65535 && N >= 0 && K >= 0 && N < kMaxDim && K < kMaxDim &&
                  num_experts > 0 && num_experts < kMaxDim,
@@ -286,7 +330,8 @@ int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const 
   GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned4(expert_ids) && aligned2(out),
              "moe_gemv: x and q_weight must be 16-byte aligned");
   GQ_REQUIRE(x_rows == 1 || (K % 8) == 0, "moe_gemv: K must be a multiple of 8 when x has top_k rows");
-  if (K == 0) return launch_empty_k(nullptr, nullptr, out, top_k, N, 0, as_stream(stream));
+  GQ_REQUIRE(!paired || (N & 1) == 0, "moe_gemv_silu_mul: N=%lld must be even", (long long)N);
+  if (K == 0) return launch_empty_k(nullptr, nullptr, out, top_k, paired ? N / 2 : N, 0, as_stream(stream));
   gq::GemvArgs a{};
   a.x = static_cast<const uint16_t*>(x);
   a.q_weight = static_cast<const uint32_t*>(q_weight);
@@ -296,14 +341,32 @@ int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const 
   a.expert_ids = static_cast<const int32_t*>(expert_ids);
   a.M = 1; a.N = N; a.K = K; a.slots = top_k; a.x_slot_stride = x_rows == 1 ? 0 : K;
   a.num_experts = num_experts;
-  a.bits = bits; a.group_size = group_size; a.out_f32 = 0;
-  return hip_result(gq::launch_gemv(a, as_stream(stream)), "moe_gemv launch");
+  a.bits = bits; a.group_size = group_size; a.out_f32 = 0; a.paired = paired;
+  const hipError_t e = gq::launch_gemv(a, as_stream(stream));
+  if (paired && e == hipErrorNotSupported)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_gemv_silu_mul: no fused kernel for N=%lld K=%lld", (long long)N,
+                (long long)K);
+  return hip_result(e, "moe_gemv launch");
 }
 
-int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
-                           const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
-                           int64_t K, int bits, int group_size, void* out,
-                           mi355gq_stream_t stream) {
+int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                     const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N,
+                     int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream) {
+  return moe_gemv_impl(x, x_rows, q_weight, q_scale, expert_ids, top_k, num_experts, N, K, bits, group_size,
+                       out, stream, false);
+}
+
+int mi355gq_moe_gemv_silu_mul(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                              const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N,
+                              int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream) {
+  return moe_gemv_impl(x, x_rows, q_weight, q_scale, expert_ids, top_k, num_experts, N, K, bits, group_size,
+                       out, stream, true);
+}
+
+static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                               const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
+                               int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream,
+                               bool paired) {
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(rows >= 0 && N >= 0 && K >= 0 && rows < kMaxDim && N < kMaxDim && K < kMaxDim &&
                  num_experts > 0 && num_experts <= 65536,
@@ -316,7 +379,8 @@ int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, co
                  (indptr_dtype == MI355GQ_I32 ? aligned4(indptr)
                                               : (reinterpret_cast<uintptr_t>(indptr) & 7u) == 0),
              "moe_group_gemm: x, q_weight and out must be 16-byte aligned");
-  if (K == 0) return launch_empty_k(nullptr, nullptr, out, rows, N, 0, as_stream(stream));
+  GQ_REQUIRE(!paired || (N & 1) == 0, "moe_group_gemm_silu_mul: N=%lld must be even", (long long)N);
+  if (K == 0) return launch_empty_k(nullptr, nullptr, out, rows, paired ? N / 2 : N, 0, as_stream(stream));
   gq::GemmArgs g{};
   g.x = static_cast<const uint16_t*>(x);
   g.q_weight = static_cast<const uint32_t*>(q_weight);
@@ -325,7 +389,7 @@ int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, co
   g.y = out;
   g.indptr = indptr; g.indptr_i64 = indptr_dtype == MI355GQ_I64;
   g.rows = rows; g.N = N; g.K = K; g.num_experts = num_experts;
-  g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
+  g.bits = bits; g.group_size = group_size; g.out_f32 = 0; g.paired = paired;
   // few rows in total: every expert is a skinny problem bound by streaming its weights
   const int gv = gq::options().gemv_variant;
   if (rows <= 128 && gq::options().gemm_variant != 1 && ((gv < 0 && rows <= 32) || (gv >= 6 && gv <= 8))) {
@@ -336,7 +400,27 @@ int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, co
     const hipError_t e = gq::launch_skinny(g, static_cast<int>(rows), as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "moe skinny launch");
   }
-  return hip_result(gq::launch_gemm(g, as_stream(stream)), "moe_group_gemm launch");
+  const hipError_t e = gq::launch_gemm(g, as_stream(stream));
+  if (paired && e == hipErrorNotSupported)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul: no fused kernel for N=%lld K=%lld",
+                (long long)N, (long long)K);
+  return hip_result(e, "moe_group_gemm launch");
+}
+
+int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                           const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
+                           int64_t K, int bits, int group_size, void* out,
+                           mi355gq_stream_t stream) {
+  return moe_group_gemm_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
+                             group_size, out, stream, false);
+}
+
+int mi355gq_moe_group_gemm_silu_mul(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                                    const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
+                                    int64_t K, int bits, int group_size, void* out,
+                                    mi355gq_stream_t stream) {
+  return moe_group_gemm_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
+                             group_size, out, stream, true);
 }
 
 int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,

@@ -49,6 +49,18 @@ __device__ __forceinline__ uint16_t f2h(float f) {
   return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
 }
 
+// Fused gate/up form of a linear whose N stored rows are [gate rows; up rows] (N / 2 each): a kernel
+// walks the rows in the interleaved order gate 0, up 0, gate 1, up 1, ... so that both halves of an
+// output element are produced side by side.  Interleaved index -> stored row:
+__device__ __forceinline__ int gate_up_row(int j, int N) { return (j >> 1) + (j & 1) * (N >> 1); }
+// silu(gate) * up with the rounding points of the unfused sequence (fp16 matmul outputs, silu in
+// fp32 rounded to fp16, fp16 product): bit-identical to linear followed by silu_mul
+__device__ __forceinline__ uint16_t silu_mul_h(float gate, float up) {
+  const float g = h2f(f2h(gate)), u = h2f(f2h(up));
+  const float silu = h2f(f2h(g / (1.0f + expf(-g))));
+  return f2h(silu * u);
+}
+
 // Sum over the 64 lanes of a wave; every lane ends up with the total.
 // quad_perm and row-mirror steps are DPP moves, the two widest steps cross rows via bpermute.
 template <int CTRL>

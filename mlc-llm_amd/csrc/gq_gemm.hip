@@ -213,6 +213,7 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   p.partial = nullptr;
   p.kt_per_split = 1 << 28;  // one workgroup walks all of K
   p.bm_hint = 0;
+  p.paired = a.paired;
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int variant = options().gemm_variant;
   if (variant < 0) {
@@ -220,8 +221,10 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
     p.bm_hint = plan.bm;
     const int64_t need = static_cast<int64_t>(plan.split) * a.rows * a.N * 4;
     // without (enough) scratch the same tiles run unsplit: slower, never wrong
+    // (fused gate/up form: the partial sums keep the tile's column order, which only lines up with
+    //  rows of N floats when the gate half is whole 32-row blocks)
     if (plan.bm > 0 && plan.split > 1 && a.workspace != nullptr && a.workspace_bytes >= need &&
-        (reinterpret_cast<uintptr_t>(a.workspace) & 15) == 0) {
+        (reinterpret_cast<uintptr_t>(a.workspace) & 15) == 0 && (!a.paired || (a.N % 64) == 0)) {
       p.partial = static_cast<float*>(a.workspace);
       p.kt_per_split = plan.kt_per_split;
     }
@@ -234,12 +237,19 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
       const int split = (nk + p.kt_per_split - 1) / p.kt_per_split;
       int64_t blocks = (count / 4 + 255) / 256;
       blocks = blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks);
+      if (p.paired) {
+        hipLaunchKernelGGL(splitk_reduce_silu_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
+                           p.partial, split, a.rows, p.N, gemm_pipe_pair_block(p, a.bits),
+                           static_cast<uint16_t*>(p.y));
+        return hipGetLastError();
+      }
       hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
                          p.partial, split, count, p.N, p.bias, p.residual, p.y, p.out_f32);
       return hipGetLastError();
     }
     if (e != hipErrorNotSupported) return e;
   }
+  if (p.paired) return hipErrorNotSupported;  // the fused form exists in the pipelined kernel only
   if (a.bits == 4) {
     // big tile (256 x 256, 128 x 128 per wave) once there are enough tiles to fill 256 CUs
     const int64_t big_tiles = ((a.rows + 255) / 256) * ((a.N + 255) / 256);

@@ -35,10 +35,30 @@ struct GemmParams {
   float* partial;
   int kt_per_split;
   int bm_hint;  // rows per tile chosen by plan_split_k (0: regular tiles)
+  // Fused gate/up form: y[rows, N / 2] = silu(x . W[j]) * (x . W[N / 2 + j]).  A tile's columns walk
+  // the stored rows in blocks of 32 gate rows then the matching 32 up rows, so both halves of an
+  // output element sit in the same lane and register of neighbouring 32 x 32 accumulators (blocks of
+  // 16 + 16 in the one tile whose waves own a single accumulator).
+  int paired;
 };
+
+// column c of the block-interleaved order above -> stored weight row (clamped into its half).
+// PB: gate rows per block; 32 where a wave owns pairs of 32-column accumulators, 16 where it owns a
+// single one (then lanes l and l ^ 16 hold the two halves of an output element).
+template <int PB>
+__device__ __forceinline__ int gate_up_row_blk(int c, int N) {
+  const int half = N >> 1;
+  const int o = min((c / (2 * PB)) * PB + (c % PB), half - 1);
+  return (c & PB) ? half + o : o;
+}
 
 __global__ void splitk_reduce_kernel(const float* partial, int split, int64_t count, int N,
                                      const uint16_t* bias, const uint16_t* residual, void* y, int out_f32);
+// fused gate/up form: partial[split][rows][N] in the block-interleaved column order -> y fp16 [rows, N / 2]
+__global__ void splitk_reduce_silu_kernel(const float* partial, int split, int64_t rows, int N, int pb,
+                                          uint16_t* y);
+// gate rows per column block (32 | 16) of the tile launch_gemm_pipe picks for these parameters
+int gemm_pipe_pair_block(const GemmParams& p, int bits);
 
 // How a few-row GEMM is cut so that every CU streams weights: rows per tile and K splits.
 struct SplitPlan {

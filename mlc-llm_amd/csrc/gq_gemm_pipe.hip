@@ -72,7 +72,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   for (int i = 0; i < W_GROUPS; ++i) {
     const int idx = tid + NT * i;
     const int r = idx >> 1, gsel = idx & 1;
-    const int row = min(n0 + r, p.N - 1);  // rows past N are computed and dropped
+    int row = min(n0 + r, p.N - 1);  // rows past N are computed and dropped
+    if (p.paired) row = gate_up_row_blk<(TN % 2 == 0) ? 32 : 16>(n0 + r, p.N);
     w_src[i] = qw + static_cast<int64_t>(row) * p.nw;
     s_src[i] = qs + static_cast<int64_t>(row) * p.ng;
     w_g[i] = gsel;
@@ -209,6 +210,40 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   }
 
   // ---- epilogue: D[i][j] of a 32x32 tile sits in lane (j + 32*((i/4)%2)), register 4*(i/8) + i%4
+  if (p.paired && p.partial == nullptr) {
+    const int half = p.N >> 1;
+    if constexpr (TN % 2 == 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int jj = 0; jj < TN / 2; ++jj) {
+          const int col = ((n0 + wn0) >> 1) + jj * 32 + (lane & 31);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (row < seg_hi && col < half)
+              static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * half + col] =
+                  silu_mul_h(acc[i][2 * jj][r], acc[i][2 * jj + 1][r]);
+          }
+        }
+      }
+    } else {
+      static_assert(TN % 2 == 0 || TN == 1, "one accumulator per wave, or pairs of them");
+      // columns 0..15 of the accumulator are gate rows, 16..31 the matching up rows
+      const int col = ((n0 + wn0) >> 1) + (lane & 15);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float up = __shfl_xor(acc[i][0][r], 16, 64);  // every lane takes part
+          const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          if ((lane & 16) == 0 && row < seg_hi && col < half)
+            static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * half + col] = silu_mul_h(acc[i][0][r], up);
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -246,7 +281,10 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   const int m_tiles = p.indptr ? (p.rows + BM - 1) / BM + p.num_experts : (p.rows + BM - 1) / BM;
   const int nk = (p.ng + 1) / 2;
   const int split = p.partial ? (nk + p.kt_per_split - 1) / p.kt_per_split : 1;
-  const dim3 grid((p.N + BN - 1) / BN, m_tiles, split);
+  // the fused gate/up form walks whole 64-column blocks (32 gate + 32 up rows)
+  constexpr int PB = ((WN / 32) % 2 == 0) ? 32 : 16;
+  const int n_cols = p.paired ? ((p.N / 2 + PB - 1) / PB) * 2 * PB : p.N;
+  const dim3 grid((n_cols + BN - 1) / BN, m_tiles, split);
   hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
   return hipGetLastError();
 }
@@ -297,6 +335,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
   }
 }
 
+__global__ __launch_bounds__(256) void splitk_reduce_silu_kernel(const float* __restrict__ partial, int split,
+                                                                 int64_t rows, int N, int pb,
+                                                                 uint16_t* __restrict__ y) {
+  const int half = N >> 1;
+  const int64_t count = rows * N, outs = rows * half;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < outs; i += stride) {
+    const int64_t row = i / half;
+    const int oc = static_cast<int>(i - row * half);
+    const int64_t at = row * N + (oc / pb) * 2 * pb + oc % pb;  // pb gate columns, then their pb up columns
+    float g = partial[at], u = partial[at + pb];
+    for (int sidx = 1; sidx < split; ++sidx) {
+      g += partial[sidx * count + at];
+      u += partial[sidx * count + at + pb];
+    }
+    y[i] = silu_mul_h(g, u);
+  }
+}
+
 SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_size, bool grouped) {
   SplitPlan plan{0, 1, 1 << 28};
   if (grouped || rows <= 0 || N <= 0 || K <= 0 || (K & 7) != 0) return plan;
@@ -327,9 +384,14 @@ SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_s
   return plan;
 }
 
+int gemm_pipe_pair_block(const GemmParams& p, int bits) {
+  return (p.bm_hint == 32 && bits == 4 && options().gemm_variant < 0) ? 16 : 32;  // the 32 x 128 tile below
+}
+
 hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   if ((p.K & 7) != 0 || p.ng == 0) return hipErrorNotSupported;
   const int variant = options().gemm_variant;
+  if (p.paired && (p.N & 1)) return hipErrorNotSupported;
   if (p.bm_hint > 0 && variant < 0) {
     if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4>(p, s);
     if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4>(p, s);

@@ -35,6 +35,7 @@ struct GemvParams {
   int num_experts;
   int gc;  // groups staged per LDS chunk (multiple of 64)
   int out_f32;
+  int paired;  // fused gate/up form: y[.., N / 2] = silu(x . W[j]) * (x . W[N / 2 + j]), fp16
 };
 
 // sum_k x_k * (field_k - m) for one group, given the 4 storage words and the staged x pairs

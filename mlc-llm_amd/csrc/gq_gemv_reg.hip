@@ -16,11 +16,14 @@
 
 namespace gq {
 
-// EXTRA: a bias or residual operand exists (a template flag rather than a run-time test: their loads are
+// MODE 1: a bias or residual operand exists (a template flag rather than a run-time test: their loads are
 // two more memory instructions per set, measured at 4-6 % of the plain GEMV's time).
-template <int BITS, int NB, int R, int ITERS, bool EXTRA>
+// MODE 2: fused gate/up form; a set holds R / 2 (gate, up) row pairs and stores R / 2 products.
+template <int BITS, int NB, int R, int ITERS, int MODE>
 __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int nsets) {
   using T = GemvTraits<BITS>;
+  constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;
+  static_assert(!PAIRED || R % 2 == 0, "a set holds whole (gate, up) pairs");
   constexpr int G = T::G;
   constexpr int HP = G / 2;  // half pairs of x per group
   // 16-byte x chunks each of the 256 threads stages: NB * ITERS * 64 groups * G/8 chunks / 256
@@ -81,7 +84,8 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
     const bool live = set < nsets;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int row = min(set * R + r, p.N - 1);  // rows past N are computed and dropped
+      int row = min(set * R + r, p.N - 1);  // rows past N are computed and dropped
+      if (PAIRED) row = gate_up_row(row, p.N);
       const uint32_t* wr = qw + static_cast<int64_t>(row) * p.nw;
       const uint16_t* sr = qs + static_cast<int64_t>(row) * p.ng;
 #pragma unroll
@@ -156,6 +160,21 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
         }
         acc[r][b] = wave_sum_last(a);
       }
+    if constexpr (PAIRED) {
+      if (lane == 63) {
+#pragma unroll
+        for (int r = 0; r < R; r += 2) {
+          const int col = (cur * R + r) >> 1;
+          if (col < (p.N >> 1)) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+              static_cast<uint16_t*>(p.y)[static_cast<int64_t>(slot + b) * (p.N >> 1) + col] =
+                  silu_mul_h(acc[r][b], acc[r + 1][b]);
+          }
+        }
+      }
+      return;
+    }
     const float bias_lane = (EXTRA && p.bias != nullptr) ? h2f(static_cast<uint16_t>(bias_bits & 0xffffu)) : 0.f;
     const float res_lane = (EXTRA && p.residual != nullptr) ? h2f(static_cast<uint16_t>(bias_bits >> 16)) : 0.f;
 #pragma unroll
@@ -196,10 +215,16 @@ static hipError_t launch_k(const GemvParams& p, int slots, int blocks, int nsets
   const int threads = 256;
   const size_t lds = static_cast<size_t>(NB) * p.ng * GemvTraits<BITS>::G * 2;
   const dim3 grid(blocks, slots);
-  if (p.bias != nullptr || p.residual != nullptr)
-    hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, true>), grid, dim3(threads), lds, s, p, nsets);
-  else
-    hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, false>), grid, dim3(threads), lds, s, p, nsets);
+  if (p.paired) {
+    if constexpr (R % 2 == 0)
+      hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 2>), grid, dim3(threads), lds, s, p, nsets);
+    else
+      return hipErrorNotSupported;
+  } else if (p.bias != nullptr || p.residual != nullptr) {
+    hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 1>), grid, dim3(threads), lds, s, p, nsets);
+  } else {
+    hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 0>), grid, dim3(threads), lds, s, p, nsets);
+  }
   return hipGetLastError();
 }
 
@@ -238,6 +263,10 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
     else R = 2;
   }
   if (R > rmax) R = rmax;
+  if (p.paired) {
+    if (rmax < 2) return hipErrorNotSupported;
+    if (R < 2) R = 2;
+  }
   const int nsets = (p.N + R - 1) / R;
   int waves;
   if (options().gemv_split > 0) {

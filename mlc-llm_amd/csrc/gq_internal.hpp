@@ -30,6 +30,7 @@ struct GemvArgs {
   int64_t num_experts;
   int bits, group_size;
   int out_f32;
+  int paired = 0;           // fused gate/up form (see gate_up_row): y is [M or slots, N / 2] fp16; N even, no bias / residual
 };
 hipError_t launch_gemv(const GemvArgs& a, hipStream_t s);
 
@@ -46,6 +47,7 @@ struct GemmArgs {
   int bits, group_size, out_f32;
   void* workspace = nullptr;       // caller's scratch for split-K partial sums (may be null)
   int64_t workspace_bytes = 0;
+  int paired = 0;                  // fused gate/up form: y is [rows, N / 2] fp16; N even, no bias / residual
 };
 hipError_t launch_gemm(const GemmArgs& a, hipStream_t s);
 // scratch the split-K form of the GEMM wants for this shape (0 when it does not split)

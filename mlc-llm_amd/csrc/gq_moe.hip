@@ -183,8 +183,7 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
   const int64_t r = i / I, c = i - r * I;
   const float x1 = h2f(x[r * 2 * I + c]);
   const float x3 = h2f(x[r * 2 * I + I + c]);
-  const float silu = h2f(f2h(x1 / (1.0f + expf(-x1))));
-  out[i] = f2h(silu * x3);
+  out[i] = silu_mul_h(x1, x3);
 }
 
 // out[t, h] = sum_j fp16(y[t, j, h] * w[t, j]), fp16 adds left to right

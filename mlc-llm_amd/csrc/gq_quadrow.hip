@@ -47,6 +47,7 @@ struct QuadParams {
   int nphases;      // passes over K, each with its slice of x in LDS
   int rounds;       // most quads any wave walks
   int indptr_i64, out_f32;
+  int paired;       // fused gate/up form: y is [rows, N / 2] fp16
 };
 
 template <int CTRL>
@@ -64,10 +65,11 @@ __device__ __forceinline__ float4_t mfma4(uint32_t a0, uint32_t a1, uint32_t b0,
 }
 
 // NBQ: activation rows / 4 (rows past the segment are zero); U: iterations per item
-// EXTRA: a bias or residual operand exists (template flag: their loads are extra memory
-// instructions per item)
-template <int BITS, int NBQ, int U, bool EXTRA>
+// MODE 1: a bias or residual operand exists (template flag: their loads are extra memory
+// instructions per item); MODE 2: fused gate/up form
+template <int BITS, int NBQ, int U, int MODE>
 __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
+  constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;  // 2: fused gate/up form, quad = 2 (gate, up) pairs
   constexpr uint32_t kMagic = 0x64006400u;
   constexpr int G = GemvTraits<BITS>::G;    // values per group: 32 | 40
   constexpr int CH = GemvTraits<BITS>::CH;  // 16-byte words of x per (activation row, group): 4 | 5
@@ -132,7 +134,8 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
     //      an item past the end reads one cached line instead.
     auto issue = [&](int quad, int step, uint4 (&wn)[U], uint32_t (&sn)[U], uint2& bn, uint2 (&rn)[NBQ]) {
       const bool live = quad < p.nquads;
-      const int row = min(quad * 4 + li, p.N - 1);
+      int row = min(quad * 4 + li, p.N - 1);
+      if (PAIRED) row = gate_up_row(row, p.N);
       const uint32_t* wr = qw + static_cast<int64_t>(row) * p.nw;
       const uint16_t* sr = qs + static_cast<int64_t>(row) * p.ng;
 #pragma unroll
@@ -332,7 +335,11 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
                 v[3] += h2f(static_cast<uint16_t>(res_bits[bq].y >> 16));
               }
               const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
-              if (p.out_f32) {
+              if constexpr (PAIRED) {
+                *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p.y) + (oi >> 1)) =
+                    static_cast<uint32_t>(silu_mul_h(v[0], v[1])) |
+                    (static_cast<uint32_t>(silu_mul_h(v[2], v[3])) << 16);
+              } else if (p.out_f32) {
                 *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) =
                     make_float4(v[0], v[1], v[2], v[3]);
               } else {
@@ -361,25 +368,26 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
   }
 }
 
-template <int BITS, int NBQ, int U, bool EXTRA>
+template <int BITS, int NBQ, int U, int MODE>
 static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                     hipStream_t s) {
   if (lds > 65536) {
     const hipError_t e =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, EXTRA>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, EXTRA>), grid, dim3(threads), lds, s, p);
+  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE>), grid, dim3(threads), lds, s, p);
   return hipGetLastError();
 }
 
 template <int BITS, int NBQ, int U>
 static hipError_t launch_quad_cfg(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                   hipStream_t s) {
+  if (p.paired) return launch_quad_extra<BITS, NBQ, U, 2>(p, grid, threads, lds, s);
   return (p.bias != nullptr || p.residual != nullptr)
-             ? launch_quad_extra<BITS, NBQ, U, true>(p, grid, threads, lds, s)
-             : launch_quad_extra<BITS, NBQ, U, false>(p, grid, threads, lds, s);
+             ? launch_quad_extra<BITS, NBQ, U, 1>(p, grid, threads, lds, s)
+             : launch_quad_extra<BITS, NBQ, U, 0>(p, grid, threads, lds, s);
 }
 
 // hipErrorNotSupported when the shape does not fit (the caller falls back to its other kernels)
@@ -396,7 +404,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
     return hipErrorNotSupported;
   QuadParams p;
   p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
-  p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64;
+  p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64; p.paired = a.paired;
   p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
   p.ng = static_cast<int>((a.K + G - 1) / G);
   p.nw = 4 * p.ng;

@@ -35,7 +35,28 @@ struct SkinnyParams {
   int64_t expert_w_stride, expert_s_stride;
   int rows, N, K, ng, nw;
   int indptr_i64, out_f32;
+  int paired;  // fused gate/up form: columns walk gate 0, up 0, gate 1, ...; y is [rows, N / 2] fp16
 };
+
+
+// Fused gate/up store of a 16 x 16 result tile: lane c holds column `col` for the batch rows 4j .. 4j+3,
+// and columns col, col + 1 (lanes c, c ^ 1) are the gate and the up projection of output element col / 2.
+// Every lane must arrive here: the neighbour's values come over a DPP swap.
+__device__ __forceinline__ void store_gate_up(const SkinnyParams& p, const float4_t v, int col, int c, int j,
+                                              int m0, int m_valid) {
+  float up[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) up[r] = dpp_f<0xB1>(v[r]);  // quad_perm [1,0,3,2]
+  if ((c & 1) == 0 && col < p.N) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int b = 4 * j + r;
+      if (b < m_valid)
+        static_cast<uint16_t*>(p.y)[static_cast<int64_t>(m0 + b) * (p.N >> 1) + (col >> 1)] =
+            silu_mul_h(v[r], up[r]);
+    }
+  }
+}
 
 // Unpipelined form: one chunk at a time, few registers, many workgroups per CU.  Large N hides
 // latency with occupancy and runs this one; small N has too few workgroups for that and runs the
@@ -87,7 +108,8 @@ __global__ __launch_bounds__(256) void skinny_q4_simple_kernel(const SkinnyParam
   const uint16_t* srow[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int row = min(n0 + rt * 16 + c, p.N - 1);  // clamped rows are computed and dropped
+    int row = min(n0 + rt * 16 + c, p.N - 1);  // clamped rows are computed and dropped
+    if (p.paired) row = gate_up_row(row, p.N);
     wrow[rt] = qw + static_cast<int64_t>(row) * p.nw;
     srow[rt] = qs + static_cast<int64_t>(row) * p.ng;
   }
@@ -185,6 +207,10 @@ __global__ __launch_bounds__(256) void skinny_q4_simple_kernel(const SkinnyParam
       v[0] += o[0]; v[1] += o[1]; v[2] += o[2]; v[3] += o[3];
     }
     const int col = n0 + rt * 16 + c;
+    if (p.paired) {  // uniform
+      store_gate_up(p, v, col, c, j, m0, m_valid);
+      continue;
+    }
     if (col < p.N) {
       const float bias = p.bias != nullptr ? h2f(p.bias[col]) : 0.f;
 #pragma unroll
@@ -248,7 +274,8 @@ __global__ __launch_bounds__(256) void skinny_q4_kernel(const SkinnyParams p) {
   const uint16_t* srow[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const int row = min(n0 + rt * 16 + c, p.N - 1);  // clamped rows are computed and dropped
+    int row = min(n0 + rt * 16 + c, p.N - 1);  // clamped rows are computed and dropped
+    if (p.paired) row = gate_up_row(row, p.N);
     wrow[rt] = qw + static_cast<int64_t>(row) * p.nw;
     srow[rt] = qs + static_cast<int64_t>(row) * p.ng;
   }
@@ -388,6 +415,10 @@ __global__ __launch_bounds__(256) void skinny_q4_kernel(const SkinnyParams p) {
       v[0] += o[0]; v[1] += o[1]; v[2] += o[2]; v[3] += o[3];
     }
     const int col = n0 + rt * 16 + c;
+    if (p.paired) {  // uniform
+      store_gate_up(p, v, col, c, j, m0, m_valid);
+      continue;
+    }
     if (col < p.N) {
       const float bias = p.bias != nullptr ? h2f(p.bias[col]) : 0.f;
 #pragma unroll
@@ -460,7 +491,8 @@ __global__ __launch_bounds__(512) void skinny_q4_persist_kernel(const SkinnyPara
   int i_tile = gw, i_blk = 0, i_seq = 0;
   auto issue = [&](WStage& st) {
     const bool live = i_seq < total;
-    const int row = min(i_tile * 16 + c, p.N - 1);
+    int row = min(i_tile * 16 + c, p.N - 1);
+    if (p.paired) row = gate_up_row(row, p.N);
     const uint32_t* wr = qw + static_cast<int64_t>(row) * p.nw;
     const uint16_t* sr = qs + static_cast<int64_t>(row) * p.ng;
 #pragma unroll
@@ -541,7 +573,9 @@ __global__ __launch_bounds__(512) void skinny_q4_persist_kernel(const SkinnyPara
     // last k-block of a tile: store D[b][n] for b < m_valid, start the next tile
     if (c_blk + 1 == nblk) {
       const int col = c_tile * 16 + c;
-      if (col < p.N) {
+      if (p.paired) {  // uniform
+        store_gate_up(p, acc, col, c, j, m0, m_valid);
+      } else if (col < p.N) {
         const float bias = p.bias != nullptr ? h2f(p.bias[col]) : 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -585,7 +619,7 @@ static hipError_t launch_skinny_cfg(const SkinnyParams& p, int experts, int mtil
 
 // rows_max: largest number of activation rows any segment holds (M for a plain linear)
 hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
-  if (a.bits != 4) return hipErrorNotSupported;
+  if (a.bits != 4 || (a.paired && (a.N & 1))) return hipErrorNotSupported;
   SkinnyParams p;
   p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
   p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64;
@@ -595,6 +629,7 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
   p.expert_w_stride = a.N * p.nw;
   p.expert_s_stride = a.N * p.ng;
   p.out_f32 = a.out_f32;
+  p.paired = a.paired;
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int experts = a.indptr ? static_cast<int>(a.num_experts) : 1;
   const int mtiles = (rows_max + 15) / 16;

@@ -95,6 +95,28 @@ int64_t LinearWorkspaceBytes(int64_t M, int64_t N, int64_t K, int64_t bits, int6
   return mi355gq_linear_workspace_bytes(M, N, K, static_cast<int>(bits), static_cast<int>(group_size));
 }
 
+// y[M, N / 2] = silu(x1) * x2 with x1, x2 = split(x . dequantize(q_weight, q_scale)^T, 2, axis=-1): the
+// gate_up projection of an MLP with its activation folded in.  There is no fused kernel when K is
+// not a multiple of 8 (an error here): the pass that rewrites matmul + split + silu + multiply into
+// this call must leave such layers as they are.
+void LinearSiluMul(TensorView x, TensorView q_weight, TensorView q_scale, int64_t bits, int64_t group_size,
+                   Optional<TensorView> workspace, TensorView y) {
+  const int64_t K = x.shape()[x.ndim() - 1], N = q_weight.shape()[0];
+  void* ws = workspace.has_value() ? Ptr(workspace.value()) : nullptr;
+  int64_t ws_bytes = 0;
+  if (workspace.has_value()) {
+    ws_bytes = (workspace.value().dtype().bits + 7) / 8;
+    for (int i = 0; i < workspace.value().ndim(); ++i) ws_bytes *= workspace.value().shape()[i];
+  }
+  Check(mi355gq_linear_silu_mul(Ptr(x), Ptr(q_weight), Ptr(q_scale), Rows(x), N, K, static_cast<int>(bits),
+                                static_cast<int>(group_size), Ptr(y), ws, ws_bytes, StreamOf(x)),
+        "mlc.gq.linear_silu_mul");
+}
+
+int64_t LinearSiluMulWorkspaceBytes(int64_t M, int64_t N, int64_t K, int64_t bits, int64_t group_size) {
+  return mi355gq_linear_silu_mul_workspace_bytes(M, N, K, static_cast<int>(bits), static_cast<int>(group_size));
+}
+
 void EmbeddingTake(TensorView ids, TensorView q_weight, TensorView q_scale, int64_t bits,
                    int64_t group_size, TensorView out) {
   const int64_t K = out.shape()[out.ndim() - 1];
@@ -123,6 +145,26 @@ void MoeGroupGemm(TensorView x, TensorView q_weight, TensorView q_scale, TensorV
         "mlc.gq.moe_group_gemm");
 }
 
+// the e1_e3 expert matmuls with silu(x1) * x3 folded in: out is [top_k | rows, N / 2]
+void MoeGemvSiluMul(TensorView x, TensorView q_weight, TensorView q_scale, TensorView expert_ids,
+                    int64_t bits, int64_t group_size, TensorView out) {
+  Check(mi355gq_moe_gemv_silu_mul(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(expert_ids),
+                                  expert_ids.shape()[1], q_weight.shape()[0], q_weight.shape()[1],
+                                  x.shape()[1], static_cast<int>(bits), static_cast<int>(group_size),
+                                  Ptr(out), StreamOf(x)),
+        "mlc.gq.moe_gemv_silu_mul");
+}
+
+void MoeGroupGemmSiluMul(TensorView x, TensorView q_weight, TensorView q_scale, TensorView indptr,
+                         int64_t bits, int64_t group_size, TensorView out) {
+  Check(mi355gq_moe_group_gemm_silu_mul(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(indptr),
+                                        indptr.dtype().bits == 64 ? MI355GQ_I64 : MI355GQ_I32,
+                                        q_weight.shape()[0], q_weight.shape()[1], x.shape()[1],
+                                        static_cast<int>(bits), static_cast<int>(group_size), Ptr(out),
+                                        StreamOf(x)),
+        "mlc.gq.moe_group_gemm_silu_mul");
+}
+
 // quantize has two destinations: (q_weight, q_scale)
 void Quantize(TensorView w, int64_t bits, int64_t group_size, int64_t round_mode,
               TensorView q_weight, TensorView q_scale) {
@@ -146,9 +188,13 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.linear", Linear)
       .def("mlc.gq.linear_residual", LinearResidual)
       .def("mlc.gq.linear_workspace_bytes", LinearWorkspaceBytes)
+      .def("mlc.gq.linear_silu_mul", LinearSiluMul)
+      .def("mlc.gq.linear_silu_mul_workspace_bytes", LinearSiluMulWorkspaceBytes)
       .def("mlc.gq.embedding_take", EmbeddingTake)
       .def("mlc.gq.moe_gemv", MoeGemv)
       .def("mlc.gq.moe_group_gemm", MoeGroupGemm)
+      .def("mlc.gq.moe_gemv_silu_mul", MoeGemvSiluMul)
+      .def("mlc.gq.moe_group_gemm_silu_mul", MoeGroupGemmSiluMul)
       .def("mlc.gq.quantize", Quantize)
       .def("mlc.gq.dequantize", Dequantize);
 }

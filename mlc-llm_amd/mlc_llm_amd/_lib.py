@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libmi355gq.so")
 HEADER_PATH = os.path.join(os.path.dirname(os.path.dirname(_HERE)), "include", "mi355gq.h")
 
 OK = 0
+ERR_ARG, ERR_HIP, ERR_UNSUPPORTED, ERR_WORKSPACE = -1, -2, -3, -4
 F16, F32 = 0, 1
 ROUND_HALF_AWAY, ROUND_HALF_EVEN = 0, 1
 I32, I64 = 0, 1
@@ -36,6 +37,10 @@ SIGNATURES = {
     "mi355gq_linear_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
     "mi355gq_linear": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_linear_residual": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
+    "mi355gq_linear_silu_mul_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
+    "mi355gq_linear_silu_mul": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P, _P, _L, _P]),
+    "mi355gq_moe_gemv_silu_mul": (_I, [_P, _L, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
+    "mi355gq_moe_group_gemm_silu_mul": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_moe_gemv": (_I, [_P, _L, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_moe_group_gemm": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_gating_softmax_topk": (_I, [_P, _L, _L, _L, _P, _P, _P]),

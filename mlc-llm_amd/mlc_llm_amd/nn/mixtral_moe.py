@@ -30,8 +30,8 @@ class MixtralMoE(nn.Module):
                                               config, device=device)
 
     def _expert_forward(self, x: torch.Tensor, indptr: torch.Tensor) -> torch.Tensor:
-        x1_x3 = self.e1_e3(x, indptr)
-        return self.e2(ops.silu_mul(x1_x3), indptr)
+        # x1, x3 = split(e1_e3(x)); e2(silu(x1) * x3): the activation rides in the e1_e3 kernel
+        return self.e2(self.e1_e3(x, indptr, silu_mul_halves=True), indptr)
 
     def forward(self, x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
         """x fp16 [batch, seq, hidden]; gate fp16 [batch * seq, num_local_experts] router logits."""

@@ -136,8 +136,44 @@ def linear(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits:
     return out
 
 
+def _unsupported(err: _lib.Mi355gqError) -> bool:
+    return err.code == _lib.ERR_UNSUPPORTED
+
+
+def linear_silu_mul(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits: int,
+                    group_size: int) -> torch.Tensor:
+    """silu(x1) * x2 with x1, x2 = split(linear(x), 2, axis=-1): the gate_up projection of an MLP
+    with its activation folded into the matmul kernel.  Bit-identical to linear then silu_mul;
+    shapes without a fused kernel run exactly those two calls."""
+    _chk(x, torch.float16, "x")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    k = x.shape[-1]
+    n = q_weight.shape[0]
+    _check_qshapes(q_weight, q_scale, (n,), k, bits, group_size)
+    if n % 2:
+        raise ValueError(f"linear_silu_mul: {n} rows cannot be split into gate and up halves")
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    out = torch.empty((*x.shape[:-1], n // 2), dtype=torch.float16, device=x.device)
+    ws_bytes = _lib.lib().mi355gq_linear_silu_mul_workspace_bytes(m, n, k, bits, group_size)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    try:
+        _lib.call("mi355gq_linear_silu_mul", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(), m, n, k,
+                  bits, group_size, out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
+                  _stream())
+    except _lib.Mi355gqError as err:
+        if not _unsupported(err):
+            raise
+        return silu_mul(linear(x.reshape(m, k), q_weight, q_scale, bits, group_size)).reshape(out.shape)
+    return out
+
+
 def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
-             expert_ids: torch.Tensor, bits: int, group_size: int) -> torch.Tensor:
+             expert_ids: torch.Tensor, bits: int, group_size: int, silu_mul_halves: bool = False
+             ) -> torch.Tensor:
+    """silu_mul_halves: the experts' rows are [gate; up] and the result is silu(gate) * up, [k, N / 2]."""
     _chk(x, torch.float16, "x")
     _chk(q_weight, _STORAGE, "q_weight")
     _chk(q_scale, torch.float16, "q_scale")
@@ -148,15 +184,27 @@ def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
     k = x.shape[1]
     _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
     top_k = expert_ids.shape[1]
+    args = (x.data_ptr(), x.shape[0], q_weight.data_ptr(), q_scale.data_ptr(), expert_ids.data_ptr(), top_k, ne,
+            n, k, bits, group_size)
+    if silu_mul_halves:
+        if n % 2:
+            raise ValueError(f"moe_gemv: {n} rows cannot be split into gate and up halves")
+        out = torch.empty((top_k, n // 2), dtype=torch.float16, device=x.device)
+        try:
+            _lib.call("mi355gq_moe_gemv_silu_mul", *args, out.data_ptr(), _stream())
+            return out
+        except _lib.Mi355gqError as err:
+            if not _unsupported(err):
+                raise
+            return silu_mul(moe_gemv(x, q_weight, q_scale, expert_ids, bits, group_size))
     out = torch.empty((top_k, n), dtype=torch.float16, device=x.device)
-    _lib.call("mi355gq_moe_gemv", x.data_ptr(), x.shape[0], q_weight.data_ptr(),
-              q_scale.data_ptr(), expert_ids.data_ptr(), top_k, ne, n, k, bits, group_size,
-              out.data_ptr(), _stream())
+    _lib.call("mi355gq_moe_gemv", *args, out.data_ptr(), _stream())
     return out
 
 
 def moe_group_gemm(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
-                   indptr: torch.Tensor, bits: int, group_size: int) -> torch.Tensor:
+                   indptr: torch.Tensor, bits: int, group_size: int, silu_mul_halves: bool = False
+                   ) -> torch.Tensor:
     _chk(x, torch.float16, "x")
     _chk(q_weight, _STORAGE, "q_weight")
     _chk(q_scale, torch.float16, "q_scale")
@@ -166,11 +214,21 @@ def moe_group_gemm(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tenso
     _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
     if tuple(indptr.shape) != (ne + 1,):
         raise ValueError(f"indptr shape {tuple(indptr.shape)}, expected {(ne + 1,)}")
+    args = (x.data_ptr(), rows, q_weight.data_ptr(), q_scale.data_ptr(), indptr.data_ptr(),
+            _lib.I64 if indptr.dtype == torch.int64 else _lib.I32, ne, n, k, bits, group_size)
+    if silu_mul_halves:
+        if n % 2:
+            raise ValueError(f"moe_group_gemm: {n} rows cannot be split into gate and up halves")
+        out = torch.zeros((rows, n // 2), dtype=torch.float16, device=x.device)
+        try:
+            _lib.call("mi355gq_moe_group_gemm_silu_mul", *args, out.data_ptr(), _stream())
+            return out
+        except _lib.Mi355gqError as err:
+            if not _unsupported(err):
+                raise
+            return silu_mul(moe_group_gemm(x, q_weight, q_scale, indptr, bits, group_size))
     out = torch.zeros((rows, n), dtype=torch.float16, device=x.device)
-    _lib.call("mi355gq_moe_group_gemm", x.data_ptr(), rows, q_weight.data_ptr(),
-              q_scale.data_ptr(), indptr.data_ptr(),
-              _lib.I64 if indptr.dtype == torch.int64 else _lib.I32, ne, n, k, bits, group_size,
-              out.data_ptr(), _stream())
+    _lib.call("mi355gq_moe_group_gemm", *args, out.data_ptr(), _stream())
     return out
 
 

@@ -251,6 +251,15 @@ class GroupQuantizeLinear(nn.Module):
             return y + bias
         return ops.linear(x, q_weight, q_scale, self.config.bits, self.config.group_size, bias, out_dtype)
 
+    def forward_silu_mul(self, x: torch.Tensor) -> torch.Tensor:
+        """For a gate_up projection: `x1, x2 = split(self(x), 2, axis=-1); silu(x1) * x2` of the MLP
+        (model/llama/llama_model.py:122-125) in one kernel; same bits as the two steps."""
+        self.config._require_built()
+        if self.bias is not None or self.out_dtype not in (None, "float16"):
+            return ops.silu_mul(self.forward(x).reshape(-1, self.out_features)).reshape(*x.shape[:-1], -1)
+        q_weight, q_scale = self._nk_tensors()
+        return ops.linear_silu_mul(x, q_weight, q_scale, self.config.bits, self.config.group_size)
+
 
 class GroupQuantizeEmbedding(nn.Module):
     """An nn.Embedding with group-quantized table, usable as tied lm_head."""
@@ -330,16 +339,18 @@ class GroupQuantizeMixtralExperts(nn.Module):
             device=src.weight.device,
         )
 
-    def forward(self, x: torch.Tensor, indptr: torch.Tensor) -> torch.Tensor:
-        """2-D `indptr` [1, k] holds the selected expert ids (single token); 1-D is a true indptr."""
+    def forward(self, x: torch.Tensor, indptr: torch.Tensor, silu_mul_halves: bool = False) -> torch.Tensor:
+        """2-D `indptr` [1, k] holds the selected expert ids (single token); 1-D is a true indptr.
+        silu_mul_halves: return silu(x1) * x3 of the two halves of the output (the e1_e3 stack of
+        mixtral_model.py:64-68) from the same kernel."""
         assert x.dim() == 2
         if indptr.dim() == 2:
             assert indptr.shape[0] == 1
             return ops.moe_gemv(x, self.q_weight, self.q_scale, indptr, self.config.bits,
-                                self.group_size)
+                                self.group_size, silu_mul_halves)
         assert indptr.dim() == 1
         return ops.moe_group_gemm(x, self.q_weight, self.q_scale, indptr, self.config.bits,
-                                  self.group_size)
+                                  self.group_size, silu_mul_halves)
 
 
 def _group(name: str, group_size: int, qdtype: str, layout: str, model_dtype: str = "float16"):

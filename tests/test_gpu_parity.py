@@ -771,6 +771,144 @@ def test_stream_read_probe_runs_and_validates():
     assert gq._lib.lib().mi355gq_probe_stream_read(a.data_ptr(), 24, None, 0, None, None) == -1  # not a multiple of 16
 
 
+# ------------------------------------------------------------------ gate_up with the activation folded in
+
+def assert_silu_mul_ok(y: torch.Tensor, ref64: np.ndarray, x: np.ndarray, k: int, what=""):
+    """y = silu(g) * u against the float64 product of the oracle's matmul: the matmul tolerance,
+    carried through d(silu(g) u) <= |u| 1.1 dg + |silu(g)| du, plus the three fp16 roundings."""
+    half = ref64.shape[-1] // 2
+    g, u = ref64[..., :half], ref64[..., half:]
+    silu = g / (1.0 + np.exp(-g))
+    tol = o.linear_tolerance(x, k)
+    bound = tol * (1.1 * np.abs(u) + np.abs(silu)) + 3 * 2.0 ** -10 * np.abs(silu * u) + 2.0 ** -20
+    err = np.abs(y.double().cpu().numpy() - silu * u)
+    assert (err <= bound).all(), f"{what}: worst excess {(err - bound).max():.3e}"
+
+
+@pytest.mark.parametrize("name,m,n,k", [
+    ("q4f16_1", 1, 512, 4096), ("q4f16_1", 2, 264, 1024), ("q4f16_1", 1, 2048, 8192),   # register GEMV
+    ("q4f16_1", 1, 256, 14336), ("q4f16_1", 2, 128, 8192),                                # long K: declined, GEMM
+    ("q4f16_1", 3, 512, 4096), ("q4f16_1", 8, 1032, 2048), ("q4f16_1", 5, 520, 20520),    # quad-row (+ K phases)
+    ("q4f16_1", 6, 130, 512), ("q4f16_1", 3, 64, 100), ("q4f16_1", 11, 64, 100),                                                            # N % 4 != 0: GEMM
+    ("q4f16_1", 12, 256, 2048), ("q4f16_1", 16, 1032, 4096), ("q4f16_1", 20, 28672, 512), ("q4f16_1", 32, 200, 1024), ("q4f16_1", 32, 192, 1024),
+    ("q4f16_1", 24, 512, 8192), ("q4f16_1", 40, 512, 4096), ("q4f16_1", 100, 1024, 1024), # few-row GEMM, split K
+    ("q4f16_1", 64, 144, 256), ("q4f16_1", 300, 328, 512), ("q4f16_1", 130, 2, 64),       # gate half not whole blocks
+    ("q3f16_1", 1, 512, 4096), ("q3f16_1", 2, 256, 2560), ("q3f16_1", 5, 512, 4080),
+    ("q3f16_1", 12, 264, 2000), ("q3f16_1", 40, 512, 4096), ("q3f16_1", 200, 192, 1040),
+])
+def test_linear_silu_mul_equals_the_two_steps(name, m, n, k):
+    s = SCHEMES[name]
+    x, qw, qs, _ = _linear_case(s, m, n, k, 1000 + m + n, scale=0.05)
+    xd, qwd, qsd = dev(x), dev(qw), dev(qs)
+    y = ops.linear_silu_mul(xd, qwd, qsd, s.bits, s.group_size)
+    assert tuple(y.shape) == (m, n // 2) and y.dtype == torch.float16
+    assert_silu_mul_ok(y, o.linear_fp32(x, qw, qs, s), x, k, f"{name} {m}x{n}x{k}")
+    # The fused call walks the same regimes as the plain linear (register GEMV, quad-row, skinny, GEMM)
+    # with the same kernels, so the two-step result is reproduced bit for bit.  The one exception: K
+    # too long for the register GEMV, where the plain linear has another GEMV and the fused call none;
+    # and 17..256 rows with a gate half that is not whole 32-row blocks, where only the plain linear may
+    # split K (another summation order).
+    ng = -(-k // s.group_size)
+    if (m <= 2 and ng > (256 if m == 1 else 128)) or (16 < m <= 256 and n % 64 != 0):
+        return
+    two = ops.silu_mul(ops.linear(xd, qwd, qsd, s.bits, s.group_size))
+    assert torch.equal(y, two), f"{name} {m}x{n}x{k}: {(y != two).sum().item()} of {y.numel()} differ"
+
+
+@pytest.mark.parametrize("variant,m,n,k", [(6, 200, 384, 512), (7, 300, 640, 384), (9, 200, 768, 256)])
+def test_linear_silu_mul_every_gemm_tile(variant, m, n, k):
+    s = SCHEMES["q4f16_1"]
+    x, qw, qs, _ = _linear_case(s, m, n, k, 77 + variant, scale=0.05)
+    xd, qwd, qsd = dev(x), dev(qw), dev(qs)
+    gq._lib.set_option("gemm_variant", variant)
+    try:
+        y = ops.linear_silu_mul(xd, qwd, qsd, 4, 32)
+        two = ops.silu_mul(ops.linear(xd, qwd, qsd, 4, 32))
+        torch.cuda.synchronize()
+    finally:
+        gq._lib.set_option("gemm_variant", -1)
+    assert_silu_mul_ok(y, o.linear_fp32(x, qw, qs, s), x, k, f"variant {variant}")
+    assert torch.equal(y, two)
+
+
+def test_linear_silu_mul_without_a_fused_kernel_runs_the_two_calls():
+    # q3 with K % 8 != 0: the quad-row kernel and the pipelined GEMM both need 16-byte aligned rows of x
+    s = SCHEMES["q3f16_1"]
+    x, qw, qs, _ = _linear_case(s, 3, 64, 100, 5, scale=0.05)
+    xd, qwd, qsd = dev(x), dev(qw), dev(qs)
+    out = torch.empty((3, 32), dtype=torch.float16, device=DEV)
+    with pytest.raises(gq._lib.Mi355gqError) as e:
+        gq._lib.call("mi355gq_linear_silu_mul", xd.data_ptr(), qwd.data_ptr(), qsd.data_ptr(), 3, 64, 100, 3, 40,
+                     out.data_ptr(), None, 0, None)
+    assert e.value.code == gq._lib.ERR_UNSUPPORTED
+    with pytest.raises(gq._lib.Mi355gqError) as e:  # odd N is an argument error, not a missing kernel
+        gq._lib.call("mi355gq_linear_silu_mul", xd.data_ptr(), qwd.data_ptr(), qsd.data_ptr(), 3, 63, 80, 3, 40,
+                     out.data_ptr(), None, 0, None)
+    assert e.value.code == gq._lib.ERR_ARG
+    y = ops.linear_silu_mul(xd, qwd, qsd, 3, 40)
+    assert torch.equal(y, ops.silu_mul(ops.linear(xd, qwd, qsd, 3, 40)))
+    assert_silu_mul_ok(y, o.linear_fp32(x, qw, qs, s), x, 100, "q3 K=100")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+def test_moe_experts_silu_mul_equals_the_two_steps(name):
+    s = SCHEMES[name]
+    rng = np.random.default_rng(91)
+    ne, n, k = 4, 512, 1280
+    w = (rng.standard_normal((ne, n, k)) * 0.05).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    qwd, qsd = dev(qw), dev(qs)
+    # single token: the selected experts' GEMV
+    x1 = rng.standard_normal((1, k)).astype(np.float16)
+    ids = torch.tensor([[3, 1]], dtype=torch.int32, device=DEV)
+    y = ops.moe_gemv(dev(x1), qwd, qsd, ids, s.bits, s.group_size, silu_mul_halves=True)
+    assert tuple(y.shape) == (2, n // 2)
+    assert torch.equal(y, ops.silu_mul(ops.moe_gemv(dev(x1), qwd, qsd, ids, s.bits, s.group_size)))
+    for e_slot, e in enumerate((3, 1)):
+        assert_silu_mul_ok(y[e_slot:e_slot + 1], o.linear_fp32(x1, qw[e], qs[e], s), x1, k, f"moe_gemv {name}")
+    # grouped: few rows (quad-row kernel), more rows (GEMM)
+    for rows, indptr, gemm_only in ((20, [0, 7, 7, 15, 20], False), (100, [0, 40, 41, 41, 100], False),
+                                    (150, [0, 40, 41, 41, 150], False), (700, [0, 300, 380, 700, 700], False)):
+        x = rng.standard_normal((rows, k)).astype(np.float16)
+        ip = torch.tensor(indptr, dtype=torch.int32, device=DEV)
+        y = ops.moe_group_gemm(dev(x), qwd, qsd, ip, s.bits, s.group_size, silu_mul_halves=True)
+        assert tuple(y.shape) == (rows, n // 2)
+        if gemm_only:
+            gq._lib.set_option("gemm_variant", 1)
+        try:
+            two = ops.silu_mul(ops.moe_group_gemm(dev(x), qwd, qsd, ip, s.bits, s.group_size))
+            torch.cuda.synchronize()
+        finally:
+            gq._lib.set_option("gemm_variant", -1)
+        assert torch.equal(y, two), f"{name} rows={rows}: {(y != two).sum().item()} differ"
+        ref = o.dequantize_group_gemm_fp32(x, qw, qs, np.asarray(indptr, dtype=np.int32), s)
+        assert_silu_mul_ok(y, ref, x, k, f"group gemm {name} rows={rows}")
+
+
+def test_mixtral_moe_layer_uses_the_folded_activation():
+    # the layer's output is unchanged by folding silu * mul into e1_e3 (single token and batch)
+    from mlc_llm_amd.nn.mixtral_moe import MixtralMoE
+    s = gq.QUANTIZATION["q4f16_1"]
+    torch.manual_seed(3)
+    moe = MixtralMoE(256, 384, 4, 2, s, device=DEV)
+    for p_ in (moe.e1_e3, moe.e2):
+        w = (torch.randn(p_.num_local_experts, p_.out_features, p_.in_features, device=DEV) * 0.05).half()
+        qw, qs = ops.quantize(w, 4, 32)
+        p_.q_weight.data.copy_(qw)
+        p_.q_scale.data.copy_(qs)
+    for t in (1, 9):
+        x = torch.randn(1, t, 256, device=DEV).half()
+        gate = torch.randn(t, 4, device=DEV).half()
+        got = moe(x, gate)
+        fused = moe._expert_forward
+        moe._expert_forward = lambda xx, ip: moe.e2(ops.silu_mul(moe.e1_e3(xx, ip)), ip)
+        try:
+            want = moe(x, gate)
+        finally:
+            moe._expert_forward = fused
+        assert torch.equal(got, want)
+
+
 # ------------------------------------------------------------------ degenerate and hostile inputs
 
 def test_degenerate_sizes_every_entry_point():
