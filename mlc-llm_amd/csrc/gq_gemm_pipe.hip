@@ -244,25 +244,36 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     }
     return;
   }
+  // (one loop nest per output form keeps each fully unrolled nest small)
+  auto for_each = [&](auto&& body) {
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wn0 + j * 32 + (lane & 31);
-      const float b = (p.bias != nullptr && p.partial == nullptr && col < p.N) ? h2f(p.bias[col]) : 0.f;
+      for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn0 + j * 32 + (lane & 31);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (row < seg_hi && col < p.N && p.partial != nullptr) {
-          p.partial[(static_cast<int64_t>(blockIdx.z) * p.rows + row) * p.N + col] = acc[i][j][r];
-        } else if (row < seg_hi && col < p.N) {
-          const int64_t o = static_cast<int64_t>(row) * p.N + col;
-          const float v = acc[i][j][r] + b + (p.residual != nullptr ? h2f(p.residual[o]) : 0.f);
-          if (p.out_f32) static_cast<float*>(p.y)[o] = v;
-          else static_cast<uint16_t*>(p.y)[o] = f2h(v);
+        for (int r = 0; r < 16; ++r) {
+          const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          if (row < seg_hi && col < p.N) body(row, col, acc[i][j][r]);
         }
       }
     }
+  };
+  if (p.partial != nullptr) {
+    float* part = p.partial + static_cast<int64_t>(blockIdx.z) * p.rows * p.N;
+    for_each([&](int row, int col, float v) { part[static_cast<int64_t>(row) * p.N + col] = v; });
+  } else if (p.bias == nullptr && p.residual == nullptr) {
+    if (p.out_f32)
+      for_each([&](int row, int col, float v) { static_cast<float*>(p.y)[static_cast<int64_t>(row) * p.N + col] = v; });
+    else
+      for_each([&](int row, int col, float v) { static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * p.N + col] = f2h(v); });
+  } else {
+    for_each([&](int row, int col, float v) {
+      const int64_t o = static_cast<int64_t>(row) * p.N + col;
+      const float t = v + (p.bias != nullptr ? h2f(p.bias[col]) : 0.f) + (p.residual != nullptr ? h2f(p.residual[o]) : 0.f);
+      if (p.out_f32) static_cast<float*>(p.y)[o] = t;
+      else static_cast<uint16_t*>(p.y)[o] = f2h(t);
+    });
   }
 }
 
