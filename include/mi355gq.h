@@ -182,7 +182,37 @@ MI355GQ_API int mi355gq_moe_group_gemm_silu_mul(const void* x, int64_t rows, con
                                     int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,
                                     void* out, mi355gq_stream_t stream);
 
+/*
+ * The grouped expert matmul with the steps MixtralMoE.forward wraps around it folded in
+ * (mixtral_model.py:99-109): the gather `x = take(x, token_indices)` becomes an index on the
+ * activation rows (row r of the expert-sorted order reads x[x_row_index[r]]; x_row_index int32 [rows]
+ * or NULL for x already gathered, x has x_rows rows), and epilogue MI355GQ_EPILOGUE_SILU_MUL gives
+ * silu(x1) * x3 of the two halves as in mi355gq_moe_group_gemm_silu_mul.  Same kernels and bits as
+ * mi355gq_take_rows followed by mi355gq_moe_group_gemm(_silu_mul).
+ */
+#define MI355GQ_EPILOGUE_NONE 0
+#define MI355GQ_EPILOGUE_SILU_MUL 1
+MI355GQ_API int mi355gq_moe_experts(const void* x, int64_t x_rows, const void* x_row_index, int64_t rows,
+                        const void* q_weight, const void* q_scale, const void* indptr, int indptr_dtype,
+                        int64_t num_experts, int64_t N, int64_t K, int bits, int group_size, int epilogue,
+                        void* out, mi355gq_stream_t stream);
+
 /* ---- routing glue of the MoE layer (python/mlc_llm/op/moe_misc.py) ---- */
+
+/*
+ * The routing of one MoE layer in one launch: gating_softmax_topk, moe_cumsum, get_indices and
+ * get_indptr (moe_misc.py:135-235, 371-605; the sequence of mixtral_model.py:77-106) for batches one
+ * workgroup can scan (T <= 8192, num_experts <= 64, num_experts * ceil(T / 1024) <= 64; otherwise
+ * MI355GQ_ERR_UNSUPPORTED and the four calls below do the same work).  Outputs as those calls give
+ * them: weights fp16 [T, top_k], ids int32 [T, top_k], token_indices / reverse_indices int32
+ * [T * top_k], indptr [num_experts + 1] (exclusive form, indptr[0] = 0); plus slot_positions int32
+ * [T * top_k], the inverse of reverse_indices (slot t * top_k + j is row slot_positions[...] of the
+ * expert-sorted order), which lets mi355gq_moe_combine_sorted read the experts' output where it lies.
+ * The [num_experts, T] cumsum table is not materialised.
+ */
+MI355GQ_API int mi355gq_moe_route(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
+                      void* weights, void* ids, void* token_indices, void* reverse_indices,
+                      void* slot_positions, void* indptr, int indptr_dtype, mi355gq_stream_t stream);
 
 /* gating_softmax_topk, norm_topk_prob = True (moe_misc.py:135-235): logits fp16 [T, num_experts]
  * -> weights fp16 [T, top_k] (softmax over the selected logits, fp32 maths), ids int32 [T, top_k].
@@ -222,6 +252,11 @@ MI355GQ_API int mi355gq_silu_mul(const void* x, int64_t R, int64_t I, void* out,
  * fp16 left-to-right sum, as the reference's elementwise ops do. */
 MI355GQ_API int mi355gq_moe_combine(const void* y, const void* weights, int64_t T, int64_t top_k, int64_t H,
                         void* out, mi355gq_stream_t stream);
+
+/* scatter_output (moe_misc.py:608-645) + the combine above in one pass: y fp16 [T * top_k, H] still in
+ * expert-sorted order, slot_positions from mi355gq_moe_route; out[t] = sum_j w[t, j] * y[slot_positions[t * top_k + j]]. */
+MI355GQ_API int mi355gq_moe_combine_sorted(const void* y, const void* slot_positions, const void* weights,
+                               int64_t T, int64_t top_k, int64_t H, void* out, mi355gq_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -366,7 +366,7 @@ int mi355gq_moe_gemv_silu_mul(const void* x, int64_t x_rows, const void* q_weigh
 static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
                                const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
                                int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream,
-                               bool paired) {
+                               bool paired, const void* x_row_index = nullptr, int64_t x_rows = 0) {
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(rows >= 0 && N >= 0 && K >= 0 && rows < kMaxDim && N < kMaxDim && K < kMaxDim &&
                  num_experts > 0 && num_experts <= 65536,
@@ -390,6 +390,12 @@ static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight
   g.indptr = indptr; g.indptr_i64 = indptr_dtype == MI355GQ_I64;
   g.rows = rows; g.N = N; g.K = K; g.num_experts = num_experts;
   g.bits = bits; g.group_size = group_size; g.out_f32 = 0; g.paired = paired;
+  if (x_row_index != nullptr) {
+    GQ_REQUIRE(x_rows >= 1 && x_rows < kMaxDim && aligned4(x_row_index), "moe_experts: x has %lld rows",
+               (long long)x_rows);
+    g.x_rows = static_cast<const int32_t*>(x_row_index);
+    g.x_src_rows = x_rows;
+  }
   // few rows in total: every expert is a skinny problem bound by streaming its weights
   const int gv = gq::options().gemv_variant;
   if (rows <= 128 && gq::options().gemm_variant != 1 && ((gv < 0 && rows <= 32) || (gv >= 6 && gv <= 8))) {
@@ -421,6 +427,19 @@ int mi355gq_moe_group_gemm_silu_mul(const void* x, int64_t rows, const void* q_w
                                     mi355gq_stream_t stream) {
   return moe_group_gemm_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
                              group_size, out, stream, true);
+}
+
+int mi355gq_moe_experts(const void* x, int64_t x_rows, const void* x_row_index, int64_t rows,
+                        const void* q_weight, const void* q_scale, const void* indptr, int indptr_dtype,
+                        int64_t num_experts, int64_t N, int64_t K, int bits, int group_size, int epilogue,
+                        void* out, mi355gq_stream_t stream) {
+  GQ_REQUIRE(epilogue == MI355GQ_EPILOGUE_NONE || epilogue == MI355GQ_EPILOGUE_SILU_MUL,
+             "moe_experts: epilogue=%d", epilogue);
+  GQ_REQUIRE(x_row_index != nullptr || x_rows == rows, "moe_experts: x has %lld rows, expected %lld",
+             (long long)x_rows, (long long)rows);
+  return moe_group_gemm_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
+                             group_size, out, stream, epilogue == MI355GQ_EPILOGUE_SILU_MUL, x_row_index,
+                             x_rows);
 }
 
 int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
@@ -513,17 +532,57 @@ int mi355gq_silu_mul(const void* x, int64_t R, int64_t I, void* out, mi355gq_str
                     "silu_mul launch");
 }
 
-int mi355gq_moe_combine(const void* y, const void* weights, int64_t T, int64_t top_k, int64_t H,
-                        void* out, mi355gq_stream_t stream) {
+static int moe_combine_impl(const void* y, const void* weights, const void* positions, int64_t T,
+                            int64_t top_k, int64_t H, void* out, mi355gq_stream_t stream) {
   GQ_REQUIRE(T >= 0 && H >= 0 && T < kMaxDim && H < kMaxDim && top_k >= 1 && top_k <= 64,
              "moe_combine: bad shape");
   if (T == 0 || H == 0) return MI355GQ_OK;
   GQ_REQUIRE(y && weights && out, "moe_combine: null pointer");
   return hip_result(gq::launch_moe_combine(static_cast<const uint16_t*>(y),
-                                           static_cast<const uint16_t*>(weights), T,
+                                           static_cast<const uint16_t*>(weights),
+                                           static_cast<const int32_t*>(positions), T,
                                            static_cast<int>(top_k), H, static_cast<uint16_t*>(out),
                                            as_stream(stream)),
                     "moe_combine launch");
+}
+
+int mi355gq_moe_combine(const void* y, const void* weights, int64_t T, int64_t top_k, int64_t H,
+                        void* out, mi355gq_stream_t stream) {
+  return moe_combine_impl(y, weights, nullptr, T, top_k, H, out, stream);
+}
+
+int mi355gq_moe_combine_sorted(const void* y, const void* slot_positions, const void* weights, int64_t T,
+                               int64_t top_k, int64_t H, void* out, mi355gq_stream_t stream) {
+  GQ_REQUIRE(slot_positions != nullptr || T == 0, "moe_combine_sorted: slot_positions is null");
+  return moe_combine_impl(y, weights, slot_positions, T, top_k, H, out, stream);
+}
+
+int mi355gq_moe_route(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights,
+                      void* ids, void* token_indices, void* reverse_indices, void* slot_positions,
+                      void* indptr, int indptr_dtype, mi355gq_stream_t stream) {
+  GQ_REQUIRE(T >= 0 && T < kMaxDim, "moe_route: bad T");
+  GQ_REQUIRE(num_experts >= 1 && num_experts <= 256, "moe_route: num_experts=%lld (1..256)",
+             (long long)num_experts);
+  GQ_REQUIRE(top_k >= 1 && top_k <= 8 && top_k <= num_experts, "moe_route: top_k=%lld (1..min(8, num_experts))",
+             (long long)top_k);
+  GQ_REQUIRE(indptr_dtype == MI355GQ_I32 || indptr_dtype == MI355GQ_I64, "moe_route: indptr_dtype=%d",
+             indptr_dtype);
+  GQ_REQUIRE(indptr != nullptr, "moe_route: indptr is null");
+  // one workgroup scans the batch expert by expert: worth it while that is a handful of rounds
+  if (T > 8192 || num_experts > 64 || num_experts * ((T + 1023) / 1024) > 64)
+    return fail(MI355GQ_ERR_UNSUPPORTED,
+                "moe_route: T=%lld with %lld experts is past the single-workgroup form; run "
+                "gating_softmax_topk, moe_cumsum, moe_get_indices and moe_get_indptr",
+                (long long)T, (long long)num_experts);
+  GQ_REQUIRE(T == 0 || (logits && weights && ids && token_indices && reverse_indices && slot_positions),
+             "moe_route: null pointer");
+  return hip_result(gq::launch_moe_route(static_cast<const uint16_t*>(logits), T, static_cast<int>(num_experts),
+                                         static_cast<int>(top_k), static_cast<uint16_t*>(weights),
+                                         static_cast<int32_t*>(ids), static_cast<int32_t*>(token_indices),
+                                         static_cast<int32_t*>(reverse_indices),
+                                         static_cast<int32_t*>(slot_positions), indptr_dtype == MI355GQ_I64,
+                                         indptr, as_stream(stream)),
+                    "moe_route launch");
 }
 
 }  // extern "C"

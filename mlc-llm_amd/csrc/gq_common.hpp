@@ -49,6 +49,14 @@ __device__ __forceinline__ uint16_t f2h(float f) {
   return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f));
 }
 
+// Row of x that the (expert-sorted) activation row r reads: r itself, or x_rows[r] when the MoE
+// layer's gather x[token_indices] is folded into the matmul; clamped into x.
+__device__ __forceinline__ int64_t x_row(const int32_t* __restrict__ x_rows, int x_src_rows, int r) {
+  if (x_rows == nullptr) return r;
+  const int j = x_rows[r];
+  return j < 0 ? 0 : (j >= x_src_rows ? x_src_rows - 1 : j);
+}
+
 // Fused gate/up form of a linear whose N stored rows are [gate rows; up rows] (N / 2 each): a kernel
 // walks the rows in the interleaved order gate 0, up 0, gate 1, up 1, ... so that both halves of an
 // output element are produced side by side.  Interleaved index -> stored row:

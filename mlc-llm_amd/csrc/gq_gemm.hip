@@ -78,7 +78,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_kernel(const 
       const int row = m0 + r, k = k_base + 8 * c;
       uint4 v = make_uint4(0, 0, 0, 0);
       if (row < seg_hi && k < p.K) {
-        const uint16_t* src = p.x + static_cast<int64_t>(row) * p.K + k;
+        const uint16_t* src = p.x + x_row(p.x_rows, p.x_src_rows, row) * p.K + k;
         if (k_vec) {
           v = *reinterpret_cast<const uint4*>(src);
         } else {
@@ -214,6 +214,7 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   p.kt_per_split = 1 << 28;  // one workgroup walks all of K
   p.bm_hint = 0;
   p.paired = a.paired;
+  p.x_rows = a.x_rows; p.x_src_rows = static_cast<int>(a.x_src_rows);
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int variant = options().gemm_variant;
   if (variant < 0) {

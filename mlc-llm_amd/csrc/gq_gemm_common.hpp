@@ -40,6 +40,8 @@ struct GemmParams {
   // output element sit in the same lane and register of neighbouring 32 x 32 accumulators (blocks of
   // 16 + 16 in the one tile whose waves own a single accumulator).
   int paired;
+  const int32_t* x_rows;  // null, or the row of x each activation row reads (int32 [rows])
+  int x_src_rows;         // rows of x when x_rows is set
 };
 
 // column c of the block-interleaved order above -> stored weight row (clamped into its half).

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     const int r = idx / CPR, c = idx - r * CPR;
     a_row_ok[i] = m0 + r < seg_hi;
     a_k[i] = 8 * c;
-    a_src[i] = p.x + static_cast<int64_t>(a_row_ok[i] ? m0 + r : m0) * p.K + 8 * c;
+    a_src[i] = p.x + x_row(p.x_rows, p.x_src_rows, a_row_ok[i] ? m0 + r : m0) * p.K + 8 * c;
     a_dst[i] = r * LDA + 8 * c;
   }
   const uint32_t* w_src[W_GROUPS];

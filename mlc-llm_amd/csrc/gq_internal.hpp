@@ -48,6 +48,8 @@ struct GemmArgs {
   void* workspace = nullptr;       // caller's scratch for split-K partial sums (may be null)
   int64_t workspace_bytes = 0;
   int paired = 0;                  // fused gate/up form: y is [rows, N / 2] fp16; N even, no bias / residual
+  const int32_t* x_rows = nullptr; // the MoE gather folded in: activation row r reads x[x_rows[r]] (x has x_src_rows rows)
+  int64_t x_src_rows = 0;
 };
 hipError_t launch_gemm(const GemmArgs& a, hipStream_t s);
 // scratch the split-K form of the GEMM wants for this shape (0 when it does not split)
@@ -80,7 +82,11 @@ hipError_t launch_get_indptr(const int32_t* cumsum, int64_t ne, int64_t T, int i
 hipError_t launch_take_rows(const uint16_t* x, const int32_t* idx, int64_t R, int64_t H,
                             int64_t x_rows, uint16_t* out, int scatter, hipStream_t s);
 hipError_t launch_silu_mul(const uint16_t* x, int64_t R, int64_t I, uint16_t* out, hipStream_t s);
-hipError_t launch_moe_combine(const uint16_t* y, const uint16_t* w, int64_t T, int k, int64_t H,
-                              uint16_t* out, hipStream_t s);
+hipError_t launch_moe_combine(const uint16_t* y, const uint16_t* w, const int32_t* pos, int64_t T, int k,
+                              int64_t H, uint16_t* out, hipStream_t s);
+// fused routing for batches one workgroup can scan (the caller checks T and the expert count)
+hipError_t launch_moe_route(const uint16_t* logits, int64_t T, int ne, int k, uint16_t* w, int32_t* ids,
+                            int32_t* tok, int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr,
+                            hipStream_t s);
 
 }  // namespace gq

@@ -14,12 +14,12 @@ constexpr int kMaxTopK = 8;
 
 // One thread per token: insertion top-k with strict '>' (ties keep the lower expert index),
 // then softmax over the k selected logits in fp32.
-__global__ __launch_bounds__(256) void topk_softmax_kernel(const uint16_t* __restrict__ logits,
-                                                           int64_t T, int ne, int k,
-                                                           uint16_t* __restrict__ w,
-                                                           int32_t* __restrict__ ids) {
-  const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (t >= T) return;
+// KMAX: slots kept (k <= KMAX); the insertion is a chain of KMAX * KMAX predicated moves per expert,
+// so the common k <= 2 gets its own, 16 times shorter, instance
+template <int KMAX>
+__device__ __forceinline__ void topk_softmax_slots(const uint16_t* __restrict__ row, int ne, int k,
+                                                   uint16_t* __restrict__ w, int32_t* __restrict__ ids) {
+  constexpr int kMaxTopK = KMAX;
   float val[kMaxTopK];
   int idx[kMaxTopK];
 #pragma unroll
@@ -27,7 +27,6 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const uint16_t* __res
     val[i] = -65504.0f;  // min_value(fp16)
     idx[i] = 0;
   }
-  const uint16_t* row = logits + t * ne;
   for (int e = 0; e < ne; ++e) {
     const float v = h2f(row[e]);
     bool placed = false;
@@ -63,8 +62,91 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const uint16_t* __res
 #pragma unroll
   for (int i = 0; i < kMaxTopK; ++i) {
     if (i < k) {
-      w[t * k + i] = f2h(ex[i] / den);
-      ids[t * k + i] = idx[i];
+      w[i] = f2h(ex[i] / den);
+      ids[i] = idx[i];
+    }
+  }
+}
+
+__device__ __forceinline__ void topk_softmax_token(const uint16_t* __restrict__ row, int ne, int k,
+                                                   uint16_t* __restrict__ w, int32_t* __restrict__ ids) {
+  if (k <= 2) topk_softmax_slots<2>(row, ne, k, w, ids);
+  else if (k <= 4) topk_softmax_slots<4>(row, ne, k, w, ids);
+  else topk_softmax_slots<kMaxTopK>(row, ne, k, w, ids);
+}
+
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const uint16_t* __restrict__ logits,
+                                                           int64_t T, int ne, int k,
+                                                           uint16_t* __restrict__ w,
+                                                           int32_t* __restrict__ ids) {
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (t >= T) return;
+  topk_softmax_token(logits + t * ne, ne, k, w + t * k, ids + t * k);
+}
+
+// The whole routing step of a MoE layer in one workgroup, for batches a single workgroup can scan:
+// top-k + softmax per token, then, expert by expert, the token-ordered positions of the (expert,
+// token) pairs: the results of gating_softmax_topk, moe_cumsum, get_indices and get_indptr without
+// the [experts, T] cumsum table in memory and without four launches.  pos_of_slot is the inverse of
+// reverse_indices (where slot t * k + j sits in the expert-sorted order).
+__global__ __launch_bounds__(1024) void moe_route_kernel(const uint16_t* __restrict__ logits, int T, int ne,
+                                                         int k, uint16_t* __restrict__ w,
+                                                         int32_t* __restrict__ ids, int32_t* __restrict__ tok,
+                                                         int32_t* __restrict__ rev,
+                                                         int32_t* __restrict__ pos_of_slot, int out_i64,
+                                                         void* indptr, int ids_in_lds) {
+  __shared__ int wave_tot[2][16];
+  extern __shared__ int32_t ids_lds[];  // [T * k] when the launch gave it room: the scans below read
+                                        // every id once per expert, and a trip to L2 each time is what
+                                        // the kernel would otherwise spend its time on
+  const int tid = threadIdx.x, nthreads = blockDim.x;  // a multiple of 64, sized to the batch
+  const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
+  for (int t = tid; t < T; t += nthreads) {
+    topk_softmax_token(logits + static_cast<int64_t>(t) * ne, ne, k, w + static_cast<int64_t>(t) * k,
+                       ids + static_cast<int64_t>(t) * k);
+    if (ids_in_lds)
+      for (int j = 0; j < k; ++j) ids_lds[t * k + j] = ids[static_cast<int64_t>(t) * k + j];  // own writes
+  }
+  __syncthreads();  // ids written above are read back by other threads below
+  const int32_t* id_src = ids_in_lds ? ids_lds : ids;
+  int base = 0, round = 0;
+  if (tid == 0) {
+    if (out_i64) static_cast<int64_t*>(indptr)[0] = 0;
+    else static_cast<int32_t*>(indptr)[0] = 0;
+  }
+  for (int e = 0; e < ne; ++e) {
+    for (int t0 = 0; t0 < T; t0 += nthreads, ++round) {
+      const int t = t0 + tid;
+      int slot = -1;  // the first j with ids[t, j] == e (the mask is boolean: a repeated id counts once)
+      if (t < T)
+        for (int j = k - 1; j >= 0; --j)
+          if (id_src[static_cast<int64_t>(t) * k + j] == e) slot = t * k + j;
+      // tokens of this expert among the wave's 64, and before this lane
+      const unsigned long long m = __ballot(slot >= 0);
+      const int before = __popcll(m & ((1ull << lane) - 1ull));
+      int pre = 0, tot = __popcll(m);
+      if (nwaves > 1) {  // uniform; the two LDS rows alternate so that one barrier per round is enough
+        int* wt = wave_tot[round & 1];
+        if (lane == 0) wt[wave] = tot;
+        __syncthreads();
+        tot = 0;
+        for (int wv = 0; wv < nwaves; ++wv) {
+          const int c = wt[wv];
+          if (wv < wave) pre += c;
+          tot += c;
+        }
+      }
+      if (slot >= 0) {
+        const int pos = base + pre + before;  // < T * k: every pair counted here is a distinct (t, j)
+        tok[pos] = t;
+        rev[pos] = slot;
+        pos_of_slot[slot] = pos;
+      }
+      base += tot;
+    }
+    if (tid == 0) {
+      if (out_i64) static_cast<int64_t*>(indptr)[e + 1] = base;
+      else static_cast<int32_t*>(indptr)[e + 1] = base;
     }
   }
 }
@@ -187,8 +269,10 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restric
 }
 
 // out[t, h] = sum_j fp16(y[t, j, h] * w[t, j]), fp16 adds left to right
+// pos: where slot t * k + j sits among the rows of y (expert-sorted order), or null for y in slot order
 __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __restrict__ y,
                                                           const uint16_t* __restrict__ w,
+                                                          const int32_t* __restrict__ pos,
                                                           int64_t T, int k, int64_t H,
                                                           uint16_t* __restrict__ out) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
@@ -196,7 +280,12 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __rest
   const int64_t t = i / H, h = i - t * H;
   float acc = 0.f;
   for (int j = 0; j < k; ++j) {
-    const float prod = h2f(f2h(h2f(y[(t * k + j) * H + h]) * h2f(w[t * k + j])));
+    int64_t row = t * k + j;
+    if (pos != nullptr) {
+      row = pos[row];
+      row = row < 0 ? 0 : (row >= T * k ? T * k - 1 : row);
+    }
+    const float prod = h2f(f2h(h2f(y[row * H + h]) * h2f(w[t * k + j])));
     acc = (j == 0) ? prod : h2f(f2h(acc + prod));
   }
   out[i] = f2h(acc);
@@ -256,11 +345,23 @@ hipError_t launch_silu_mul(const uint16_t* x, int64_t R, int64_t I, uint16_t* ou
   return hipGetLastError();
 }
 
-hipError_t launch_moe_combine(const uint16_t* y, const uint16_t* w, int64_t T, int k, int64_t H,
-                              uint16_t* out, hipStream_t s) {
+hipError_t launch_moe_combine(const uint16_t* y, const uint16_t* w, const int32_t* pos, int64_t T, int k,
+                              int64_t H, uint16_t* out, hipStream_t s) {
   if (T * H == 0) return hipSuccess;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(blocks_for(T * H, 256)), dim3(256), 0, s, y, w, T, k,
+  hipLaunchKernelGGL(moe_combine_kernel, dim3(blocks_for(T * H, 256)), dim3(256), 0, s, y, w, pos, T, k,
                      H, out);
+  return hipGetLastError();
+}
+
+hipError_t launch_moe_route(const uint16_t* logits, int64_t T, int ne, int k, uint16_t* w, int32_t* ids,
+                            int32_t* tok, int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr,
+                            hipStream_t s) {
+  int threads = static_cast<int>((T + 63) / 64) * 64;
+  threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
+  const size_t lds = static_cast<size_t>(T) * k * sizeof(int32_t);
+  const int ids_in_lds = lds <= 60 * 1024;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(threads), ids_in_lds ? lds : 0, s, logits,
+                     static_cast<int>(T), ne, k, w, ids, tok, rev, pos_of_slot, out_i64, indptr, ids_in_lds);
   return hipGetLastError();
 }
 

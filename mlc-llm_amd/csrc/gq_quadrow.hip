@@ -48,6 +48,8 @@ struct QuadParams {
   int rounds;       // most quads any wave walks
   int indptr_i64, out_f32;
   int paired;       // fused gate/up form: y is [rows, N / 2] fp16
+  const int32_t* x_rows;  // null, or the row of x each activation row reads (int32 [rows])
+  int x_src_rows;         // rows of x when x_rows is set
 };
 
 template <int CTRL>
@@ -191,7 +193,7 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
           const int bq = bi / niter, it = bi - bq * niter;
           const int b = 4 * bq + (lp & 3);
           const int g = 16 * (it0 + it) + (lp >> 2);
-          const uint16_t* src = p.x + static_cast<int64_t>(m0 + min(b, m_valid - 1)) * p.K;
+          const uint16_t* src = p.x + x_row(p.x_rows, p.x_src_rows, m0 + min(b, m_valid - 1)) * p.K;
 #pragma unroll
           for (int c = 0; c < CH; ++c) {
             const int k = G * g + 8 * c;
@@ -405,6 +407,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   QuadParams p;
   p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
   p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64; p.paired = a.paired;
+  p.x_rows = a.x_rows; p.x_src_rows = static_cast<int>(a.x_src_rows);
   p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
   p.ng = static_cast<int>((a.K + G - 1) / G);
   p.nw = 4 * p.ng;

@@ -36,6 +36,8 @@ struct SkinnyParams {
   int rows, N, K, ng, nw;
   int indptr_i64, out_f32;
   int paired;  // fused gate/up form: columns walk gate 0, up 0, gate 1, ...; y is [rows, N / 2] fp16
+  const int32_t* x_rows;  // null, or the row of x each activation row reads (int32 [rows])
+  int x_src_rows;
 };
 
 
@@ -141,7 +143,7 @@ __global__ __launch_bounds__(256) void skinny_q4_simple_kernel(const SkinnyParam
       const int k = ci * KC + kk;
       uint4 v = make_uint4(0, 0, 0, 0);
       if (b < m_valid && k < p.K) {
-        const uint16_t* src = p.x + static_cast<int64_t>(m0 + b) * p.K + k;
+        const uint16_t* src = p.x + x_row(p.x_rows, p.x_src_rows, m0 + b) * p.K + k;
         if (k_vec) {
           v = *reinterpret_cast<const uint4*>(src);
         } else {
@@ -292,7 +294,7 @@ __global__ __launch_bounds__(256) void skinny_q4_kernel(const SkinnyParams p) {
     const int idx = tid + 256 * i;
     x_b[i] = idx / (KC / 8);
     x_kk[i] = (idx - x_b[i] * (KC / 8)) * 8;
-    x_src[i] = p.x + static_cast<int64_t>(m0 + (x_b[i] < m_valid ? x_b[i] : 0)) * p.K + x_kk[i];
+    x_src[i] = p.x + x_row(p.x_rows, p.x_src_rows, m0 + (x_b[i] < m_valid ? x_b[i] : 0)) * p.K + x_kk[i];
   }
   uint4 xreg[XS];
   // branch-free chunk loads (clamped address; validity is applied when the chunk is stored)
@@ -311,7 +313,7 @@ __global__ __launch_bounds__(256) void skinny_q4_kernel(const SkinnyParams p) {
       uint4 v = xreg[i];
       if (!(k_vec && k + 8 <= p.K && x_b[i] < m_valid)) v = make_uint4(0, 0, 0, 0);
       if (!k_vec && x_b[i] < m_valid && k < p.K) {  // unaligned rows: element-wise, rare
-        const uint16_t* src = p.x + static_cast<int64_t>(m0 + x_b[i]) * p.K + k;
+        const uint16_t* src = p.x + x_row(p.x_rows, p.x_src_rows, m0 + x_b[i]) * p.K + k;
         uint16_t e[8];
 #pragma unroll
         for (int q = 0; q < 8; ++q) e[q] = (k + q < p.K) ? src[q] : uint16_t(0);
@@ -519,7 +521,7 @@ __global__ __launch_bounds__(512) void skinny_q4_persist_kernel(const SkinnyPara
       const int k = (i - b * cpr) * 8;
       uint4 v = make_uint4(0, 0, 0, 0);
       if (b < m_valid && k < p.K) {
-        const uint16_t* src = p.x + static_cast<int64_t>(m0 + b) * p.K + k;
+        const uint16_t* src = p.x + x_row(p.x_rows, p.x_src_rows, m0 + b) * p.K + k;
         if (k_vec) {
           v = *reinterpret_cast<const uint4*>(src);
         } else {
@@ -630,6 +632,7 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
   p.expert_s_stride = a.N * p.ng;
   p.out_f32 = a.out_f32;
   p.paired = a.paired;
+  p.x_rows = a.x_rows; p.x_src_rows = static_cast<int>(a.x_src_rows);
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int experts = a.indptr ? static_cast<int>(a.num_experts) : 1;
   const int mtiles = (rows_max + 15) / 16;

@@ -165,6 +165,34 @@ void MoeGroupGemmSiluMul(TensorView x, TensorView q_weight, TensorView q_scale, 
         "mlc.gq.moe_group_gemm_silu_mul");
 }
 
+// group gemm over x[x_row_index] (x_row_index: the layer's token_indices, or absent for gathered x);
+// silu_mul != 0 folds silu(x1) * x3 of the output halves in
+void MoeExperts(TensorView x, Optional<TensorView> x_row_index, TensorView q_weight, TensorView q_scale,
+                TensorView indptr, int64_t bits, int64_t group_size, int64_t silu_mul, TensorView out) {
+  Check(mi355gq_moe_experts(Ptr(x), x.shape()[0], x_row_index.has_value() ? Ptr(x_row_index.value()) : nullptr,
+                            out.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(indptr),
+                            indptr.dtype().bits == 64 ? MI355GQ_I64 : MI355GQ_I32, q_weight.shape()[0],
+                            q_weight.shape()[1], x.shape()[1], static_cast<int>(bits),
+                            static_cast<int>(group_size),
+                            silu_mul ? MI355GQ_EPILOGUE_SILU_MUL : MI355GQ_EPILOGUE_NONE, Ptr(out), StreamOf(x)),
+        "mlc.gq.moe_experts");
+}
+
+// routing of one MoE layer; six destinations
+void MoeRoute(TensorView logits, int64_t top_k, TensorView weights, TensorView ids, TensorView token_indices,
+              TensorView reverse_indices, TensorView slot_positions, TensorView indptr) {
+  Check(mi355gq_moe_route(Ptr(logits), logits.shape()[0], logits.shape()[1], top_k, Ptr(weights), Ptr(ids),
+                          Ptr(token_indices), Ptr(reverse_indices), Ptr(slot_positions), Ptr(indptr),
+                          indptr.dtype().bits == 64 ? MI355GQ_I64 : MI355GQ_I32, StreamOf(logits)),
+        "mlc.gq.moe_route");
+}
+
+void MoeCombineSorted(TensorView y, TensorView slot_positions, TensorView weights, TensorView out) {
+  Check(mi355gq_moe_combine_sorted(Ptr(y), Ptr(slot_positions), Ptr(weights), weights.shape()[0],
+                                   weights.shape()[1], y.shape()[1], Ptr(out), StreamOf(y)),
+        "mlc.gq.moe_combine_sorted");
+}
+
 // quantize has two destinations: (q_weight, q_scale)
 void Quantize(TensorView w, int64_t bits, int64_t group_size, int64_t round_mode,
               TensorView q_weight, TensorView q_scale) {
@@ -195,6 +223,9 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.moe_group_gemm", MoeGroupGemm)
       .def("mlc.gq.moe_gemv_silu_mul", MoeGemvSiluMul)
       .def("mlc.gq.moe_group_gemm_silu_mul", MoeGroupGemmSiluMul)
+      .def("mlc.gq.moe_experts", MoeExperts)
+      .def("mlc.gq.moe_route", MoeRoute)
+      .def("mlc.gq.moe_combine_sorted", MoeCombineSorted)
       .def("mlc.gq.quantize", Quantize)
       .def("mlc.gq.dequantize", Dequantize);
 }

@@ -21,6 +21,7 @@ ERR_ARG, ERR_HIP, ERR_UNSUPPORTED, ERR_WORKSPACE = -1, -2, -3, -4
 F16, F32 = 0, 1
 ROUND_HALF_AWAY, ROUND_HALF_EVEN = 0, 1
 I32, I64 = 0, 1
+EPILOGUE_NONE, EPILOGUE_SILU_MUL = 0, 1
 
 _P, _I, _L = c_void_p, c_int, c_int64
 
@@ -43,6 +44,9 @@ SIGNATURES = {
     "mi355gq_moe_group_gemm_silu_mul": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_moe_gemv": (_I, [_P, _L, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_moe_group_gemm": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _P, _P]),
+    "mi355gq_moe_experts": (_I, [_P, _L, _P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _I, _P, _P]),
+    "mi355gq_moe_route": (_I, [_P, _L, _L, _L, _P, _P, _P, _P, _P, _P, _I, _P]),
+    "mi355gq_moe_combine_sorted": (_I, [_P, _P, _P, _L, _L, _L, _P, _P]),
     "mi355gq_gating_softmax_topk": (_I, [_P, _L, _L, _L, _P, _P, _P]),
     "mi355gq_moe_cumsum": (_I, [_P, _L, _L, _L, _P, _P]),
     "mi355gq_moe_get_indices": (_I, [_P, _P, _L, _L, _L, _P, _P, _P]),

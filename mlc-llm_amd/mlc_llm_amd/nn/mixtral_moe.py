@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 from torch import nn
 
-from .. import ops
+from .. import _lib, ops
 from ..op import moe_misc
 from ..quantization import GroupQuantize, GroupQuantizeMixtralExperts
 
@@ -40,6 +40,24 @@ class MixtralMoE(nn.Module):
         batch_size, seq_len, hidden_size = x.shape
         num_tokens = batch_size * seq_len
         x = x.reshape(num_tokens, hidden_size).contiguous()
+        if num_tokens > 1:
+            try:
+                # routing in one launch; the gather rides in e1_e3's row addressing, the scatter in the
+                # combine's: four launches where the op-by-op sequence below takes nine
+                weights, _, token_indices, _, slot_positions, indptr = ops.moe_route(gate, experts_per_tok)
+            except _lib.Mi355gqError as err:
+                if err.code != _lib.ERR_UNSUPPORTED:
+                    raise
+            else:
+                cfg = self.e1_e3.config
+                if num_tokens * experts_per_tok > 128:
+                    # the GEMM's workgroups would each start with one more dependent load (index, then
+                    # rows): measured slower than a separate gather once the few-row kernels are left
+                    x, token_indices = ops.take_rows(x, token_indices), None
+                h = ops.moe_experts(x, token_indices, self.e1_e3.q_weight, self.e1_e3.q_scale, indptr, cfg.bits,
+                                    self.e1_e3.group_size, silu_mul_halves=True)
+                y = self.e2(h, indptr)
+                return ops.moe_combine_sorted(y, slot_positions, weights).reshape(batch_size, seq_len, hidden_size)
         expert_weights, expert_indices = moe_misc.gating_softmax_topk(gate, experts_per_tok)
         if num_tokens == 1:
             x = self._expert_forward(x, expert_indices)

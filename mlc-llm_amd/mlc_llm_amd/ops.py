@@ -232,6 +232,67 @@ def moe_group_gemm(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tenso
     return out
 
 
+def moe_experts(x: torch.Tensor, x_row_index: Optional[torch.Tensor], q_weight: torch.Tensor,
+                q_scale: torch.Tensor, indptr: torch.Tensor, bits: int, group_size: int,
+                silu_mul_halves: bool = False) -> torch.Tensor:
+    """moe_group_gemm on x[x_row_index] (the layer's gather folded into the matmul's row addressing);
+    x_row_index None: x is already in expert order."""
+    _chk(x, torch.float16, "x")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    _chk(indptr, (torch.int32, torch.int64), "indptr")
+    ne, n, _ = q_weight.shape
+    x_rows, k = x.shape
+    _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
+    if tuple(indptr.shape) != (ne + 1,):
+        raise ValueError(f"indptr shape {tuple(indptr.shape)}, expected {(ne + 1,)}")
+    rows = x_rows
+    if x_row_index is not None:
+        _chk(x_row_index, torch.int32, "x_row_index")
+        rows = x_row_index.numel()
+    if silu_mul_halves and n % 2:
+        raise ValueError(f"moe_experts: {n} rows cannot be split into gate and up halves")
+    out = torch.zeros((rows, n // 2 if silu_mul_halves else n), dtype=torch.float16, device=x.device)
+    _lib.call("mi355gq_moe_experts", x.data_ptr(), x_rows,
+              x_row_index.data_ptr() if x_row_index is not None else None, rows, q_weight.data_ptr(),
+              q_scale.data_ptr(), indptr.data_ptr(), _lib.I64 if indptr.dtype == torch.int64 else _lib.I32,
+              ne, n, k, bits, group_size, _lib.EPILOGUE_SILU_MUL if silu_mul_halves else _lib.EPILOGUE_NONE,
+              out.data_ptr(), _stream())
+    return out
+
+
+def moe_route(logits: torch.Tensor, top_k: int, indptr_dtype=torch.int32):
+    """The routing of a MoE layer in one launch.  Returns (weights [T, k] fp16, ids [T, k] int32,
+    token_indices [T * k], reverse_indices [T * k], slot_positions [T * k], indptr [experts + 1]).
+    Raises Mi355gqError with code ERR_UNSUPPORTED for batches past the single-workgroup form."""
+    _chk(logits, torch.float16, "logits")
+    t, ne = logits.shape
+    dev = logits.device
+    w = torch.empty((t, top_k), dtype=torch.float16, device=dev)
+    ids = torch.empty((t, top_k), dtype=torch.int32, device=dev)
+    tok, rev, pos = (torch.empty((t * top_k,), dtype=torch.int32, device=dev) for _ in range(3))
+    indptr = torch.empty((ne + 1,), dtype=indptr_dtype, device=dev)
+    _lib.call("mi355gq_moe_route", logits.data_ptr(), t, ne, top_k, w.data_ptr(), ids.data_ptr(), tok.data_ptr(),
+              rev.data_ptr(), pos.data_ptr(), indptr.data_ptr(),
+              _lib.I64 if indptr_dtype == torch.int64 else _lib.I32, _stream())
+    return w, ids, tok, rev, pos, indptr
+
+
+def moe_combine_sorted(y: torch.Tensor, slot_positions: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+    """y fp16 [T * k, H] in expert-sorted order, slot_positions int32 [T * k], weights fp16 [T, k] -> [T, H]."""
+    _chk(y, torch.float16, "y")
+    _chk(slot_positions, torch.int32, "slot_positions")
+    _chk(weights, torch.float16, "weights")
+    t, k = weights.shape
+    if y.shape[0] != t * k or slot_positions.numel() != t * k:
+        raise ValueError("moe_combine_sorted: y and slot_positions must have T * k rows")
+    h = y.shape[1]
+    out = torch.empty((t, h), dtype=torch.float16, device=y.device)
+    _lib.call("mi355gq_moe_combine_sorted", y.data_ptr(), slot_positions.data_ptr(), weights.data_ptr(), t, k, h,
+              out.data_ptr(), _stream())
+    return out
+
+
 def gating_softmax_topk(logits: torch.Tensor, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
     _chk(logits, torch.float16, "logits")
     t, ne = logits.shape

@@ -885,8 +885,27 @@ def test_moe_experts_silu_mul_equals_the_two_steps(name):
         assert_silu_mul_ok(y, ref, x, k, f"group gemm {name} rows={rows}")
 
 
-def test_mixtral_moe_layer_uses_the_folded_activation():
-    # the layer's output is unchanged by folding silu * mul into e1_e3 (single token and batch)
+def _op_by_op_layer(moe, x, gate):
+    """MixtralMoE.forward as the reference writes it (mixtral_model.py:77-117), one call per op."""
+    from mlc_llm_amd.op import moe_misc
+    t = x.shape[0] * x.shape[1]
+    h = x.shape[2]
+    xx = x.reshape(t, h).contiguous()
+    w, ids = moe_misc.gating_softmax_topk(gate, moe.num_experts_per_tok)
+    if t == 1:
+        y = moe.e2(ops.silu_mul(moe.e1_e3(xx, ids)), ids)
+    else:
+        cumsum = moe_misc.moe_cumsum(ids, moe.num_local_experts)
+        rev, tok = moe_misc.get_indices(cumsum, ids)
+        indptr = moe_misc.get_indptr(cumsum, moe.num_local_experts, t, inclusive=False, out_dtype="int32")
+        y = moe.e2(ops.silu_mul(moe.e1_e3(ops.take_rows(xx, tok), indptr)), indptr)
+        y = moe_misc.scatter_output(y, rev)
+    return ops.moe_combine(y.reshape(t, moe.num_experts_per_tok, h), w).reshape(x.shape)
+
+
+def test_mixtral_moe_layer_fused_forms_change_no_bit():
+    # folded activation, fused routing, gather in the matmul, scatter in the combine: same output as the
+    # op-by-op sequence, for a single token, few tokens (quad-row), more (skinny) and many (GEMM)
     from mlc_llm_amd.nn.mixtral_moe import MixtralMoE
     s = gq.QUANTIZATION["q4f16_1"]
     torch.manual_seed(3)
@@ -896,17 +915,69 @@ def test_mixtral_moe_layer_uses_the_folded_activation():
         qw, qs = ops.quantize(w, 4, 32)
         p_.q_weight.data.copy_(qw)
         p_.q_scale.data.copy_(qs)
-    for t in (1, 9):
+    for t in (1, 2, 9, 40, 300, 1500):
         x = torch.randn(1, t, 256, device=DEV).half()
         gate = torch.randn(t, 4, device=DEV).half()
-        got = moe(x, gate)
-        fused = moe._expert_forward
-        moe._expert_forward = lambda xx, ip: moe.e2(ops.silu_mul(moe.e1_e3(xx, ip)), ip)
-        try:
-            want = moe(x, gate)
-        finally:
-            moe._expert_forward = fused
-        assert torch.equal(got, want)
+        assert torch.equal(moe(x, gate), _op_by_op_layer(moe, x, gate)), t
+
+
+@pytest.mark.parametrize("t,ne,k", [(2, 8, 2), (9, 8, 2), (100, 4, 1), (1000, 8, 2), (1500, 8, 4), (5000, 6, 2),
+                                    (64, 64, 8), (3, 3, 3)])
+def test_moe_route_equals_the_four_calls(t, ne, k):
+    torch.manual_seed(t + ne + k)
+    logits = torch.randn(t, ne, device=DEV).half()
+    w, ids, tok, rev, pos, indptr = ops.moe_route(logits, k)
+    w0, ids0 = ops.gating_softmax_topk(logits, k)
+    cumsum = ops.moe_cumsum(ids0, ne)
+    rev0, tok0 = ops.get_indices(cumsum, ids0)
+    indptr0 = ops.get_indptr(cumsum, ne, t, inclusive=False)
+    assert torch.equal(w, w0) and torch.equal(ids, ids0)
+    assert torch.equal(tok, tok0) and torch.equal(rev, rev0) and torch.equal(indptr, indptr0)
+    assert torch.equal(rev[pos.long()], torch.arange(t * k, dtype=torch.int32, device=DEV))  # the inverse permutation
+    assert torch.equal(ops.moe_route(logits, k, torch.int64)[5], indptr0.long())
+
+
+def test_moe_route_past_one_workgroup_is_unsupported():
+    for t, ne in ((9000, 8), (16, 100), (4096, 32)):
+        with pytest.raises(gq._lib.Mi355gqError) as e:
+            ops.moe_route(torch.zeros(t, ne, device=DEV).half(), 2)
+        assert e.value.code == gq._lib.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+def test_moe_experts_with_the_gather_folded_in(name):
+    s = SCHEMES[name]
+    rng = np.random.default_rng(17)
+    ne, n, k, t = 4, 256, 640, 37
+    w = (rng.standard_normal((ne, n, k)) * 0.05).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    qwd, qsd = dev(qw), dev(qs)
+    x = dev(rng.standard_normal((t, k)).astype(np.float16))
+    for rows, indptr in ((20, [0, 7, 7, 15, 20]), (100, [0, 40, 41, 41, 100]), (700, [0, 300, 380, 700, 700])):
+        idx = torch.from_numpy(rng.integers(0, t, rows).astype(np.int32)).to(DEV)
+        ip = torch.tensor(indptr, dtype=torch.int32, device=DEV)
+        gathered = ops.take_rows(x, idx)
+        for silu in (False, True):
+            got = ops.moe_experts(x, idx, qwd, qsd, ip, s.bits, s.group_size, silu)
+            want = ops.moe_group_gemm(gathered, qwd, qsd, ip, s.bits, s.group_size, silu)
+            assert torch.equal(got, want), (name, rows, silu)
+            assert torch.equal(ops.moe_experts(gathered, None, qwd, qsd, ip, s.bits, s.group_size, silu), want)
+    # an index outside x is clamped, never followed
+    bad = torch.tensor([0, -5, 36, 99, 2**30], dtype=torch.int32, device=DEV)
+    ip = torch.tensor([0, 5, 5, 5, 5], dtype=torch.int32, device=DEV)
+    got = ops.moe_experts(x, bad, qwd, qsd, ip, s.bits, s.group_size)
+    ok = torch.tensor([0, 0, 36, 36, 36], dtype=torch.int32, device=DEV)
+    assert torch.equal(got, ops.moe_group_gemm(ops.take_rows(x, ok), qwd, qsd, ip, s.bits, s.group_size))
+
+
+def test_moe_combine_sorted_equals_scatter_then_combine():
+    torch.manual_seed(5)
+    t, k, h = 33, 2, 192
+    logits = torch.randn(t, 8, device=DEV).half()
+    w, ids, tok, rev, pos, indptr = ops.moe_route(logits, k)
+    y = torch.randn(t * k, h, device=DEV).half()
+    want = ops.moe_combine(ops.scatter_output(y, rev).reshape(t, k, h), w)
+    assert torch.equal(ops.moe_combine_sorted(y, pos, w), want)
 
 
 # ------------------------------------------------------------------ degenerate and hostile inputs
