@@ -65,7 +65,10 @@ __device__ __forceinline__ int gate_up_row(int j, int N) { return (j >> 1) + (j 
 // fp32 rounded to fp16, fp16 product): bit-identical to linear followed by silu_mul
 __device__ __forceinline__ uint16_t silu_mul_h(float gate, float up) {
   const float g = h2f(f2h(gate)), u = h2f(f2h(up));
-  const float silu = h2f(f2h(g / (1.0f + expf(-g))));
+  // hardware exp2 and reciprocal (1 ulp each): far inside the fp16 rounding of the result, and short
+  // enough that the one lane that runs it in a GEMV epilogue does not hold its wave back
+  const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896341f);
+  const float silu = h2f(f2h(g * __builtin_amdgcn_rcpf(1.0f + e)));
   return f2h(silu * u);
 }
 
