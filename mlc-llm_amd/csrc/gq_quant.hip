@@ -13,61 +13,105 @@
 
 namespace gq {
 
-template <int BITS>
+// Which (row, storage word) a thread owns: thread n of the grid owns word n of the row-major
+// [rows, nw] array.  n / nw by a per-thread 64-bit division costs more instructions than the rest
+// of a dequantize, so the quotient comes from a multiply-high with a constant made on the host
+// (round-up method with one extra bit: q = (((n - h) >> 1) + h) >> shift, h = mulhi(n, magic),
+// exact for every 32-bit n); arrays of 2^32 words or more keep the plain division.
+struct WordGrid {
+  uint32_t nw, magic, shift;
+  uint32_t mode;  // 0: multiply-high, 1: nw is a power of two (shift only), 2: 64-bit division
+};
+__device__ __forceinline__ void locate_word(const WordGrid gr, int64_t nw, int64_t& row, int64_t& wd) {
+  if (gr.mode == 2) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    row = idx / nw;
+    wd = idx - row * nw;
+    return;
+  }
+  const uint32_t n = blockIdx.x * 256u + threadIdx.x;
+  uint32_t q;
+  if (gr.mode == 1) {
+    q = n >> gr.shift;
+  } else {
+    const uint32_t h = __umulhi(n, gr.magic);
+    q = (((n - h) >> 1) + h) >> gr.shift;
+  }
+  row = q;
+  wd = n - q * gr.nw;
+}
+static WordGrid plan_words(int64_t rows, int64_t nw, unsigned& blocks) {
+  WordGrid gr{static_cast<uint32_t>(nw), 0u, 0u, 0u};
+  const int64_t total = rows * nw;
+  const int64_t b = (total + 255) / 256;
+  blocks = b < (int64_t(1) << 31) ? static_cast<unsigned>(b) : 0u;  // 0: more blocks than a grid holds
+  if (total + 256 >= (int64_t(1) << 32)) {
+    gr.mode = 2;
+    return gr;
+  }
+  uint32_t log2 = 0;
+  while ((int64_t(2) << log2) <= nw) ++log2;  // floor(log2(nw))
+  gr.shift = log2;
+  if ((nw & (nw - 1)) == 0) {
+    gr.mode = 1;
+    return gr;
+  }
+  const uint64_t num = uint64_t(1) << (32 + log2);
+  uint64_t m = num / static_cast<uint64_t>(nw);
+  const uint64_t rem = num % static_cast<uint64_t>(nw);
+  m = 2 * m + (2 * rem >= static_cast<uint64_t>(nw) ? 1 : 0) + 1;
+  gr.magic = static_cast<uint32_t>(m);  // the 33rd bit is the "+ n" of the formula
+  return gr;
+}
+
+// HALF_EVEN: the tie rule of the rounding (0: half away from zero, the llvm / rocm lowering of
+// tirx.round; 1: half to even, what CUDA-converted weights carry).
+template <int BITS, int HALF_EVEN>
 __global__ __launch_bounds__(256) void quantize_kernel(const uint16_t* __restrict__ w,
                                                        int64_t rows, int64_t K, int64_t nw,
-                                                       int64_t ng, int group_size, int half_even,
+                                                       int64_t ng, int group_size, WordGrid gr,
                                                        uint32_t* __restrict__ qw,
                                                        uint16_t* __restrict__ qs) {
   using S = Scheme<BITS>;
   constexpr int E = S::kElem;
-  const int64_t total = rows * nw;
-  int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  // quads never straddle rows (nw % 4 == 0); inactive lanes still take part in the shuffles
-  const bool live = idx < total;
-  if (!live) idx = total - 1;
-  const int64_t row = idx / nw;
-  const int64_t wd = idx - row * nw;
+  constexpr int P = E / 2;  // half pairs per storage word
+  int64_t row, wd;
+  locate_word(gr, nw, row, wd);
+  // inactive lanes (whole quads past the last row) still take part in the shuffles
+  const bool live = row < rows;
+  if (!live) { row = rows - 1; wd = nw - 1; }
   const int64_t g = wd >> 2;
   const int64_t k0 = g * group_size + (wd & 3) * E;
   const uint16_t* wr = w + row * K;
 
-  float v[E];
-  bool ok[E];
+  // ---- the word's E values as half pairs; slots beyond K hold zero and are masked out of the
+  //      maximum (the reference pads with fp16 lowest) and of the packed word
+  uint32_t pr[P];
   const bool full = (k0 + E <= K);
   if (BITS == 4 && full && ((K & 7) == 0)) {
     const uint4 raw = *reinterpret_cast<const uint4*>(wr + k0);
-    const uint32_t r4[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[2 * i] = h2f(static_cast<uint16_t>(r4[i] & 0xffffu));
-      v[2 * i + 1] = h2f(static_cast<uint16_t>(r4[i] >> 16));
-      ok[2 * i] = ok[2 * i + 1] = true;
-    }
-  } else if (BITS == 3 && full && ((K & 1) == 0)) {
+    pr[0] = raw.x; pr[1] = raw.y; pr[2] = raw.z; pr[3] = raw.w;
+  } else if (full && ((K & 1) == 0)) {
     const uint32_t* p = reinterpret_cast<const uint32_t*>(wr + k0);
 #pragma unroll
-    for (int i = 0; i < E / 2; ++i) {
-      const uint32_t r = p[i];
-      v[2 * i] = h2f(static_cast<uint16_t>(r & 0xffffu));
-      v[2 * i + 1] = h2f(static_cast<uint16_t>(r >> 16));
-      ok[2 * i] = ok[2 * i + 1] = true;
-    }
+    for (int i = 0; i < P; ++i) pr[i] = p[i];
   } else {
 #pragma unroll
-    for (int i = 0; i < E; ++i) {
-      ok[i] = (k0 + i) < K;
-      v[i] = ok[i] ? h2f(wr[k0 + i]) : 0.0f;
+    for (int i = 0; i < P; ++i) {
+      const uint32_t lo = (k0 + 2 * i) < K ? wr[k0 + 2 * i] : 0u;
+      const uint32_t hi = (k0 + 2 * i + 1) < K ? wr[k0 + 2 * i + 1] : 0u;
+      pr[i] = lo | (hi << 16);
     }
   }
+  const int valid = full ? E : static_cast<int>(K > k0 ? K - k0 : 0);  // values of this word inside K
 
-  // group max of |w|; lanes beyond K contribute fp16 lowest, as the reference pads
-  float amax = -65504.0f;
+  // ---- group max of |w| (packed fp16 maxima ignore NaN operands, as the reference's
+  //      compare-and-select does); zero padding cannot raise a maximum of absolute values
+  half2_t mx = as_half2(pr[0] & 0x7fff7fffu);
 #pragma unroll
-  for (int i = 0; i < E; ++i) {
-    const float a = fabsf(v[i]);
-    amax = (ok[i] && a > amax) ? a : amax;
-  }
+  for (int i = 1; i < P; ++i) mx = __builtin_elementwise_max(mx, as_half2(pr[i] & 0x7fff7fffu));
+  float amax = fmaxf(static_cast<float>(mx[0]), static_cast<float>(mx[1]));
+  if (valid == 0) amax = -65504.0f;
   amax = fmaxf(amax, dpp_f<0xB1>(amax));
   amax = fmaxf(amax, dpp_f<0x4E>(amax));
 
@@ -78,26 +122,55 @@ __global__ __launch_bounds__(256) void quantize_kernel(const uint16_t* __restric
   // rounded once more; a float quotient within half an ulp (plus a hair) rounds to the same half,
   // because a ratio of two 11-bit significands that is not itself a rounding boundary of fp16
   // stays more than 2^-23 (relative) away from one.  One Newton step on the hardware reciprocal
-  // gives that accuracy for a third of the instructions of a correctly rounded divide.  s = 0
-  // (an all-zero or denormal-only group) and overflowing quotients keep the first product, which
-  // is the NaN / infinity the plain divide yields.
+  // gives that accuracy for a third of the instructions of a correctly rounded divide.  A scale
+  // that is zero (an all-zero group), infinite or NaN keeps the first product, which is then the
+  // NaN / zero / NaN the plain divide yields.
   const float rs = __builtin_amdgcn_rcpf(s);
+  const bool plain = !(s > 0.0f && s < __builtin_inff());
+  // Everything after the divide is fp16 arithmetic on pairs: the add of m (rounded), then the
+  // rounding to an integer.  t = quotient + m lies in [-0.004, 2m], so t + 0.5 is exact and its
+  // truncation is round-half-away; (t + 1024) - 1024 is round-half-even (fp16 spacing is 1 there).
+  // A NaN (0 / 0) becomes 0 in the packed maximum, like the reference's compare-and-select.
+  const _Float16 hm = static_cast<_Float16>(m);
+  const half2_t m2 = {hm, hm};
+  const half2_t zero2 = {static_cast<_Float16>(0.0f), static_cast<_Float16>(0.0f)};
+  const half2_t top2 = {static_cast<_Float16>(2.0f * m + 0.5f), static_cast<_Float16>(2.0f * m + 0.5f)};
   uint32_t word = 0;
+  uint16_t qv[E];
 #pragma unroll
-  for (int i = 0; i < E; ++i) {
-    const float q0 = v[i] * rs;
-    const float q1 = fmaf(fmaf(-q0, s, v[i]), rs, q0);
-    const float quo = (s == 0.0f || fabsf(q0) == __builtin_inff()) ? q0 : q1;
-    float t = h2f(f2h(quo));  // fp16 divide
-    t = h2f(f2h(t + m));           // fp16 add
-    float r = half_even ? rintf(t) : roundf(t);
-    r = (r > 0.0f) ? r : 0.0f;  // compare+select max: NaN (0/0) becomes 0
-    r = (r < 2.0f * m) ? r : 2.0f * m;
-    const uint32_t q = ok[i] ? static_cast<uint32_t>(r) : 0u;
-    word |= q << (i * BITS);
+  for (int i = 0; i < P; ++i) {
+    const half2_t hv = as_half2(pr[i]);
+    float quo[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const float v = static_cast<float>(hv[e]);
+      const float q0 = v * rs;
+      const float q1 = fmaf(fmaf(-q0, s, v), rs, q0);
+      quo[e] = plain ? q0 : q1;
+    }
+    const half2_t qh = {static_cast<_Float16>(quo[0]), static_cast<_Float16>(quo[1])};  // fp16 divide
+    const half2_t t = qh + m2;                                                            // fp16 add
+    half2_t r;
+    if (HALF_EVEN) {
+      const half2_t big = {static_cast<_Float16>(1024.0f), static_cast<_Float16>(1024.0f)};
+      r = (t + big) - big;
+    } else {
+      const half2_t hf = {static_cast<_Float16>(0.5f), static_cast<_Float16>(0.5f)};
+      r = t + hf;  // truncated by the conversion below
+    }
+    r = __builtin_elementwise_min(__builtin_elementwise_max(r, zero2), top2);  // [0, 2m] and no NaN left
+    qv[2 * i] = static_cast<uint16_t>(r[0]);  // truncation; the operand is in [0, 2m + 0.5]
+    qv[2 * i + 1] = static_cast<uint16_t>(r[1]);
+  }
+  if (full) {
+#pragma unroll
+    for (int i = 0; i < E; ++i) word |= static_cast<uint32_t>(qv[i]) << (i * BITS);
+  } else {  // a word that straddles K (the last group of a row): slots beyond K stay zero
+#pragma unroll
+    for (int i = 0; i < E; ++i) word |= (i < valid ? static_cast<uint32_t>(qv[i]) : 0u) << (i * BITS);
   }
   if (live) {
-    qw[idx] = word;
+    qw[row * nw + wd] = word;
     if ((wd & 3) == 0) qs[row * ng + g] = sh;
   }
 }
@@ -109,13 +182,13 @@ __global__ __launch_bounds__(256) void dequantize_kernel(const int32_t* __restri
                                                          const uint32_t* __restrict__ qw,
                                                          const uint16_t* __restrict__ qs,
                                                          int64_t table_rows, int64_t K, int64_t nw,
-                                                         int64_t ng, uint16_t* __restrict__ out) {
+                                                         int64_t ng, WordGrid gr,
+                                                         uint16_t* __restrict__ out) {
   using S = Scheme<BITS>;
   constexpr int E = S::kElem;
-  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (idx >= out_rows * nw) return;
-  const int64_t orow = idx / nw;
-  const int64_t wd = idx - orow * nw;
+  int64_t orow, wd;
+  locate_word(gr, nw, orow, wd);
+  if (orow >= out_rows) return;
   int64_t row = orow;
   if (ids != nullptr) {
     row = ids[orow];
@@ -157,13 +230,18 @@ hipError_t launch_quantize(const uint16_t* w, int64_t rows, int64_t K, int bits,
   const int64_t nw = 4 * ng;
   const int64_t total = rows * nw;
   if (total == 0) return hipSuccess;
-  const dim3 grid(static_cast<unsigned>((total + 255) / 256));
-  if (bits == 4)
-    hipLaunchKernelGGL(quantize_kernel<4>, grid, dim3(256), 0, s, w, rows, K, nw, ng, group_size,
-                       round_mode, qw, qs);
+  unsigned blocks = 0;
+  const WordGrid gr = plan_words(rows, nw, blocks);
+  if (blocks == 0) return hipErrorInvalidValue;
+  const dim3 grid(blocks);
+  if (bits == 4 && round_mode == 0)
+    hipLaunchKernelGGL((quantize_kernel<4, 0>), grid, dim3(256), 0, s, w, rows, K, nw, ng, group_size, gr, qw, qs);
+  else if (bits == 4)
+    hipLaunchKernelGGL((quantize_kernel<4, 1>), grid, dim3(256), 0, s, w, rows, K, nw, ng, group_size, gr, qw, qs);
+  else if (round_mode == 0)
+    hipLaunchKernelGGL((quantize_kernel<3, 0>), grid, dim3(256), 0, s, w, rows, K, nw, ng, group_size, gr, qw, qs);
   else
-    hipLaunchKernelGGL(quantize_kernel<3>, grid, dim3(256), 0, s, w, rows, K, nw, ng, group_size,
-                       round_mode, qw, qs);
+    hipLaunchKernelGGL((quantize_kernel<3, 1>), grid, dim3(256), 0, s, w, rows, K, nw, ng, group_size, gr, qw, qs);
   return hipGetLastError();
 }
 
@@ -174,13 +252,16 @@ hipError_t launch_dequantize(const int32_t* ids, int64_t out_rows, const uint32_
   const int64_t nw = 4 * ng;
   const int64_t total = out_rows * nw;
   if (total == 0) return hipSuccess;
-  const dim3 grid(static_cast<unsigned>((total + 255) / 256));
+  unsigned blocks = 0;
+  const WordGrid gr = plan_words(out_rows, nw, blocks);
+  if (blocks == 0) return hipErrorInvalidValue;
+  const dim3 grid(blocks);
   if (bits == 4)
     hipLaunchKernelGGL(dequantize_kernel<4>, grid, dim3(256), 0, s, ids, out_rows, qw, qs,
-                       table_rows, K, nw, ng, out);
+                       table_rows, K, nw, ng, gr, out);
   else
     hipLaunchKernelGGL(dequantize_kernel<3>, grid, dim3(256), 0, s, ids, out_rows, qw, qs,
-                       table_rows, K, nw, ng, out);
+                       table_rows, K, nw, ng, gr, out);
   return hipGetLastError();
 }
 

@@ -771,6 +771,25 @@ def test_stream_read_probe_runs_and_validates():
     assert gq._lib.lib().mi355gq_probe_stream_read(a.data_ptr(), 24, None, 0, None, None) == -1  # not a multiple of 16
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+def test_quantize_dequantize_every_row_length(name):
+    # the kernels find (row, word) of a thread by a multiply-high with a constant per row length:
+    # walk many lengths (odd, powers of two, just under / over a group) and rows that are not a multiple
+    # of anything
+    s = SCHEMES[name]
+    rng = np.random.default_rng(123)
+    ks = sorted(set(list(range(1, 330, 7)) + [32, 40, 64, 80, 128, 256, 512, 1024, 1000, 2047, 2048, 4100, 9999]))
+    for k in ks:
+        rows = 37 if k < 3000 else 5
+        w = (rng.standard_normal((rows, k)) * 0.1).astype(np.float16)
+        qw_ref, qs_ref = o.quantize(w, s)
+        qw, qs = ops.quantize(dev(w), s.bits, s.group_size)
+        assert np.array_equal(host_u32(qw), qw_ref), k
+        assert np.array_equal(host_f16_bits(qs), qs_ref.view(np.uint16)), k
+        d = ops.dequantize(qw, qs, k, s.bits, s.group_size)
+        assert np.array_equal(host_f16_bits(d), o.dequantize(qw_ref, qs_ref, s, k).view(np.uint16)), k
+
+
 # ------------------------------------------------------------------ gate_up with the activation folded in
 
 def assert_silu_mul_ok(y: torch.Tensor, ref64: np.ndarray, x: np.ndarray, k: int, what=""):
