@@ -42,7 +42,7 @@ enum {
   MI355GQ_ERR_WORKSPACE = -4    /* caller's workspace is too small */
 };
 
-enum { MI355GQ_F16 = 0, MI355GQ_F32 = 1 };             /* output dtype */
+enum { MI355GQ_F16 = 0, MI355GQ_F32 = 1, MI355GQ_BF16 = 2 }; /* output dtype (F16 / F32); model dtype of the *_dt entry points */
 enum { MI355GQ_ROUND_HALF_AWAY = 0, MI355GQ_ROUND_HALF_EVEN = 1 };
 enum { MI355GQ_I32 = 0, MI355GQ_I64 = 1 };             /* indptr dtype */
 
@@ -91,6 +91,25 @@ MI355GQ_API int mi355gq_embedding_take(const void* ids, int64_t T, const void* q
                            mi355gq_stream_t stream);
 
 /*
+ * The three packing entry points above for the other model dtypes of the reference registry
+ * (quantization/quantization.py:91-123: q4bf16_0 / q4bf16_1 with model_dtype bfloat16, q4f32_1 with
+ * float32): `GroupQuantize` carries `model_dtype` through _quantize / _dequantize
+ * (group_quantization.py:235-306, 155-186), so w, q_scale, out and every intermediate have that type.
+ * model_dtype MI355GQ_F16 forwards to the float16 entry points; MI355GQ_F32 is IEEE single arithmetic
+ * op for op; MI355GQ_BF16 does each operation in float32 and rounds the result to nearest-even
+ * bfloat16 (TVM's bf16 legalisation).  q_weight layout is that of the float16 schemes.  Tensors need
+ * only their natural alignment.
+ */
+MI355GQ_API int mi355gq_quantize_dt(const void* w, int64_t rows, int64_t K, int bits, int group_size,
+                        int round_mode, int model_dtype, void* q_weight, void* q_scale,
+                        mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_dequantize_dt(const void* q_weight, const void* q_scale, int64_t rows, int64_t K,
+                          int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_embedding_take_dt(const void* ids, int64_t T, const void* q_weight,
+                              const void* q_scale, int64_t num_rows, int64_t K, int bits, int group_size,
+                              int model_dtype, void* out, mi355gq_stream_t stream);
+
+/*
  * GroupQuantizeLinear.forward / GroupQuantizeEmbedding.lm_head_forward
  * (group_quantization.py:390-437, 524-556), i.e. the fused_dequantize*_NT_matmul kernels
  * (compiler_pass/fuse_dequantize_matmul_ewise.py, fuse_transpose_matmul.py:64-143):
@@ -122,6 +141,17 @@ MI355GQ_API int mi355gq_linear_residual(const void* x, const void* q_weight, con
                             const void* bias, const void* residual, int64_t M, int64_t N, int64_t K,
                             int bits, int group_size, int out_dtype, void* y, void* workspace,
                             int64_t workspace_bytes, mi355gq_stream_t stream);
+
+/*
+ * mi355gq_linear for the other model dtypes (see mi355gq_quantize_dt): x, q_scale and bias carry
+ * model_dtype (MI355GQ_F32 or MI355GQ_BF16; MI355GQ_F16 forwards to mi355gq_linear), y carries
+ * out_dtype = model_dtype or MI355GQ_F32.  Weights are dequantised as GroupQuantize._dequantize does
+ * ((q - m) * scale rounded to the model dtype) and accumulated in fp32.  A first form: a fp32-FMA GEMV
+ * up to 8 rows and a v_mfma_f32_32x32x2_f32 GEMM above; no residual / SiLU epilogues, no MoE forms.
+ */
+MI355GQ_API int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                      int64_t M, int64_t N, int64_t K, int bits, int group_size, int model_dtype,
+                      int out_dtype, void* y, mi355gq_stream_t stream);
 
 /*
  * gate_up projection with the activation folded in: the sequence

@@ -182,6 +182,69 @@ int mi355gq_embedding_take(const void* ids, int64_t T, const void* q_weight, con
       "embedding_take launch");
 }
 
+static int check_model_dtype(int model_dtype, const char* what) {
+  if (model_dtype != MI355GQ_F16 && model_dtype != MI355GQ_F32 && model_dtype != MI355GQ_BF16)
+    return fail(MI355GQ_ERR_ARG, "%s: model_dtype=%d (MI355GQ_F16, MI355GQ_F32 or MI355GQ_BF16)", what, model_dtype);
+  return MI355GQ_OK;
+}
+
+int mi355gq_quantize_dt(const void* w, int64_t rows, int64_t K, int bits, int group_size, int round_mode,
+                        int model_dtype, void* q_weight, void* q_scale, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "quantize_dt"));
+  if (model_dtype == MI355GQ_F16)
+    return mi355gq_quantize(w, rows, K, bits, group_size, round_mode, q_weight, q_scale, stream);
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(rows >= 0 && K >= 0 && rows < kMaxDim && K < kMaxDim, "quantize_dt: bad shape [%lld, %lld]",
+             (long long)rows, (long long)K);
+  GQ_REQUIRE(round_mode == MI355GQ_ROUND_HALF_AWAY || round_mode == MI355GQ_ROUND_HALF_EVEN,
+             "quantize_dt: round_mode=%d", round_mode);
+  if (rows == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(w && q_weight && q_scale, "quantize_dt: null pointer");
+  GQ_REQUIRE(aligned4(w) && aligned4(q_weight) && aligned2(q_scale) &&
+                 (model_dtype != MI355GQ_F32 || aligned4(q_scale)),
+             "quantize_dt: misaligned tensor");
+  return hip_result(gq::launch_quantize_dt(w, rows, K, bits, group_size, round_mode, model_dtype,
+                                           static_cast<uint32_t*>(q_weight), q_scale, as_stream(stream)),
+                    "quantize_dt launch");
+}
+
+int mi355gq_dequantize_dt(const void* q_weight, const void* q_scale, int64_t rows, int64_t K, int bits,
+                          int group_size, int model_dtype, void* out, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "dequantize_dt"));
+  if (model_dtype == MI355GQ_F16)
+    return mi355gq_dequantize(q_weight, q_scale, rows, K, bits, group_size, out, stream);
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(rows >= 0 && K >= 0 && rows < kMaxDim && K < kMaxDim, "dequantize_dt: bad shape");
+  if (rows == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(q_weight && q_scale && out, "dequantize_dt: null pointer");
+  GQ_REQUIRE(aligned4(q_weight) && aligned2(out) && aligned2(q_scale) &&
+                 (model_dtype != MI355GQ_F32 || (aligned4(q_scale) && aligned4(out))),
+             "dequantize_dt: misaligned tensor");
+  return hip_result(gq::launch_dequantize_dt(nullptr, rows, static_cast<const uint32_t*>(q_weight), q_scale, rows,
+                                             K, bits, group_size, model_dtype, out, as_stream(stream)),
+                    "dequantize_dt launch");
+}
+
+int mi355gq_embedding_take_dt(const void* ids, int64_t T, const void* q_weight, const void* q_scale,
+                              int64_t num_rows, int64_t K, int bits, int group_size, int model_dtype,
+                              void* out, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "embedding_take_dt"));
+  if (model_dtype == MI355GQ_F16)
+    return mi355gq_embedding_take(ids, T, q_weight, q_scale, num_rows, K, bits, group_size, out, stream);
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(T >= 0 && K >= 0 && num_rows >= 0 && T < kMaxDim && K < kMaxDim, "embedding_take_dt: bad shape");
+  if (T == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(num_rows > 0, "embedding_take_dt: empty table");
+  GQ_REQUIRE(ids && q_weight && q_scale && out, "embedding_take_dt: null pointer");
+  GQ_REQUIRE(aligned4(ids) && aligned4(q_weight) && aligned2(out) && aligned2(q_scale) &&
+                 (model_dtype != MI355GQ_F32 || (aligned4(q_scale) && aligned4(out))),
+             "embedding_take_dt: misaligned tensor");
+  return hip_result(gq::launch_dequantize_dt(static_cast<const int32_t*>(ids), T,
+                                             static_cast<const uint32_t*>(q_weight), q_scale, num_rows, K, bits,
+                                             group_size, model_dtype, out, as_stream(stream)),
+                    "embedding_take_dt launch");
+}
+
 int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
   if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
       N >= kMaxDim || K >= kMaxDim)
@@ -347,6 +410,30 @@ static int moe_gemv_impl(const void* x, int64_t x_rows, const void* q_weight, co
     return fail(MI355GQ_ERR_UNSUPPORTED, "moe_gemv_silu_mul: no fused kernel for N=%lld K=%lld", (long long)N,
                 (long long)K);
   return hip_result(e, "moe_gemv launch");
+}
+
+int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias, int64_t M,
+                      int64_t N, int64_t K, int bits, int group_size, int model_dtype, int out_dtype, void* y,
+                      mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "linear_dt"));
+  if (model_dtype == MI355GQ_F16)
+    return linear_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, out_dtype, y, nullptr, 0,
+                       stream);
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(M >= 0 && N >= 0 && K >= 1 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
+             "linear_dt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  GQ_REQUIRE(out_dtype == MI355GQ_F32 || out_dtype == model_dtype,
+             "linear_dt: out_dtype=%d (the model dtype or MI355GQ_F32)", out_dtype);
+  if (M == 0 || N == 0) return MI355GQ_OK;
+  GQ_REQUIRE(y && x && q_weight && q_scale, "linear_dt: null pointer");
+  const bool f32 = model_dtype == MI355GQ_F32;
+  GQ_REQUIRE(aligned16(q_weight) && (f32 ? aligned4(x) && aligned4(q_scale) && aligned4(bias)
+                                         : aligned2(x) && aligned2(q_scale) && aligned2(bias)) &&
+                 (out_dtype == MI355GQ_F32 ? aligned4(y) : aligned2(y)),
+             "linear_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
+  return hip_result(gq::launch_linear_dt(x, static_cast<const uint32_t*>(q_weight), q_scale, bias, M, N, K, bits,
+                                         group_size, model_dtype, out_dtype, y, as_stream(stream)),
+                    "linear_dt launch");
 }
 
 int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,

@@ -65,6 +65,17 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s);
 hipError_t launch_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,
                               void* sink, hipStream_t s);
 
+// model dtypes beyond float16 (values of the public enum: MI355GQ_F16 = 0, MI355GQ_F32 = 1, MI355GQ_BF16 = 2)
+constexpr int MODEL_F16 = 0, MODEL_F32 = 1, MODEL_BF16 = 2;
+hipError_t launch_quantize_dt(const void* w, int64_t rows, int64_t K, int bits, int group_size, int round_mode,
+                              int model_dtype, uint32_t* qw, void* qs, hipStream_t s);
+hipError_t launch_dequantize_dt(const int32_t* ids, int64_t out_rows, const uint32_t* qw, const void* qs,
+                                int64_t table_rows, int64_t K, int bits, int group_size, int model_dtype,
+                                void* out, hipStream_t s);
+// out_kind: MODEL_F32 or MODEL_BF16
+hipError_t launch_linear_dt(const void* x, const uint32_t* qw, const void* qs, const void* bias, int64_t M, int64_t N,
+                            int64_t K, int bits, int group_size, int model_dtype, int out_kind, void* y,
+                            hipStream_t s);
 hipError_t launch_quantize(const uint16_t* w, int64_t rows, int64_t K, int bits, int group_size,
                            int round_mode, uint32_t* qw, uint16_t* qs, hipStream_t s);
 hipError_t launch_dequantize(const int32_t* ids, int64_t out_rows, const uint32_t* qw,

@@ -1,0 +1,271 @@
+// Linear for the model dtypes other than float16 (q4f32_1, q4bf16_*): the dequantize-fused matmul
+// of GroupQuantizeLinear.forward / lm_head_forward (group_quantization.py:390-437, 524-556) with
+// x, q_scale and bias in float32 or bfloat16.
+//
+// A first, plain form of the two regimes of the float16 path:
+//  * up to 8 activation rows: a GEMV with x resident in LDS as float32, one weight row per wave and
+//    step, fp32 FMAs (there is no dot-product instruction to lean on for these types);
+//  * more rows: a 128 x 128 tile GEMM on v_mfma_f32_32x32x2_f32 with both operands in LDS as
+//    float32 (bfloat16 operands are widened on the way in; their products are exact either way).
+// Weights are dequantised exactly as GroupQuantize._dequantize does, (q - m) * scale rounded to the
+// model dtype, before they meet x; accumulation is fp32.
+#include "gq_common.hpp"
+#include "gq_internal.hpp"
+
+namespace gq {
+
+namespace {
+
+template <int DT>
+struct LinT;
+template <>
+struct LinT<MODEL_F32> {
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return static_cast<const float*>(p)[i]; }
+  static __device__ __forceinline__ float rnd(float v) { return v; }
+};
+template <>
+struct LinT<MODEL_BF16> {
+  static __device__ __forceinline__ float load(const void* p, int64_t i) {
+    return __builtin_bit_cast(float, static_cast<uint32_t>(static_cast<const uint16_t*>(p)[i]) << 16);
+  }
+  static __device__ __forceinline__ float rnd(float v) {  // nearest-even bfloat16 (finite inputs)
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    return __builtin_bit_cast(float, (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u);
+  }
+};
+
+__device__ __forceinline__ uint16_t bf16_bits(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+  return static_cast<uint16_t>((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+// out_kind: 1 float32, 2 bfloat16
+__device__ __forceinline__ void store_out(void* y, int64_t i, float v, int out_kind) {
+  if (out_kind == MODEL_F32) static_cast<float*>(y)[i] = v;
+  else static_cast<uint16_t*>(y)[i] = bf16_bits(v);
+}
+
+struct LinParams {
+  const void* x;
+  const uint32_t* qw;
+  const void* qs;
+  const void* bias;
+  void* y;
+  int M, N, K, ng, nw;
+  int out_kind;
+};
+
+// ---------------------------------------------------------------- up to 8 rows
+
+// LDS: x as float [NB][kpad] (zero beyond K).  Lane l of a wave owns groups l, l + 64, ... of the
+// wave's current weight row.
+template <int BITS, int DT, int NB>
+__global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p) {
+  using S = Scheme<BITS>;
+  using T = LinT<DT>;
+  constexpr int E = S::kElem;
+  constexpr int G = 4 * E;
+  extern __shared__ float xs[];
+  const int kpad = p.ng * G;
+  for (int i = threadIdx.x; i < NB * kpad; i += 256) {
+    const int b = i / kpad, k = i - b * kpad;
+    xs[i] = (b < p.M && k < p.K) ? T::load(p.x, static_cast<int64_t>(b) * p.K + k) : 0.0f;
+  }
+  __syncthreads();
+
+  const int lane = threadIdx.x & 63;
+  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * 4;
+  const float m = static_cast<float>(S::kMaxInt);
+  for (int row = gw; row < p.N; row += nwaves) {
+    float acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[b] = 0.0f;
+    const uint32_t* wr = p.qw + static_cast<int64_t>(row) * p.nw;
+    for (int g = lane; g < p.ng; g += 64) {
+      const uint4 w4 = *reinterpret_cast<const uint4*>(wr + 4 * g);
+      const float s = T::load(p.qs, static_cast<int64_t>(row) * p.ng + g);
+      const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int i = 0; i < E; ++i) {
+          const float q = static_cast<float>((w[j] >> (i * BITS)) & S::kMask);
+          const float wv = T::rnd((q - m) * s);  // GroupQuantize._dequantize, in the model dtype
+          const int k = g * G + j * E + i;
+#pragma unroll
+          for (int b = 0; b < NB; ++b) acc[b] = fmaf(wv, xs[b * kpad + k], acc[b]);
+        }
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const float t = wave_sum(acc[b]);
+      if (lane == 0 && b < p.M) {
+        const float bias = p.bias != nullptr ? T::load(p.bias, row) : 0.0f;
+        store_out(p.y, static_cast<int64_t>(b) * p.N + row, t + bias, p.out_kind);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- more rows: fp32 MFMA GEMM
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+// 128 x 128 tile, 4 waves of 64 x 64 (2 x 2 accumulators of 32 x 32), K tile = one group.
+// LDS rows are G + 1 floats long: consecutive rows fall into consecutive banks, so the 32 rows a
+// fragment read touches hit 32 different banks.
+template <int BITS, int DT>
+__global__ __launch_bounds__(256) void gemm_dt_kernel(const LinParams p) {
+  using S = Scheme<BITS>;
+  using T = LinT<DT>;
+  constexpr int E = S::kElem;
+  constexpr int G = 4 * E;      // K tile: 32 | 40
+  constexpr int LD = G + 1;
+  constexpr int BM = 128, BN = 128;
+  constexpr int A_PER = BM * G / 256;  // x values per thread and tile: 16 | 20
+  extern __shared__ float lds[];
+  auto a_tile = [&](int s) { return lds + s * (BM + BN) * LD; };
+  auto w_tile = [&](int s) { return lds + s * (BM + BN) * LD + BM * LD; };
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave >> 1) * 64, wn0 = (wave & 1) * 64;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const float m = static_cast<float>(S::kMaxInt);
+
+  // this thread's share of a tile: x values (row ar, k offsets ak .. ak + A_PER) and two storage
+  // words of weight row wrow
+  const int ar = tid >> 1, ak = (tid & 1) * A_PER;
+  const int wrow = min(n0 + (tid >> 1), p.N - 1);  // rows past N are computed and dropped
+  const int whalf = tid & 1;
+  float areg[A_PER];
+  uint32_t wreg[2];
+  float sreg = 0.0f;
+  auto load_tile = [&](int kt) {
+    const int64_t row = m0 + ar;
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) {
+      const int k = kt * G + ak + i;
+      areg[i] = (row < p.M && k < p.K) ? T::load(p.x, row * p.K + k) : 0.0f;
+    }
+    const uint32_t* wr = p.qw + static_cast<int64_t>(wrow) * p.nw + 4 * kt + 2 * whalf;
+    wreg[0] = wr[0];
+    wreg[1] = wr[1];
+    sreg = T::load(p.qs, static_cast<int64_t>(wrow) * p.ng + kt);
+  };
+  auto store_tile = [&](int s) {
+    float* at = a_tile(s) + ar * LD + ak;
+#pragma unroll
+    for (int i = 0; i < A_PER; ++i) at[i] = areg[i];
+    float* wt = w_tile(s) + (tid >> 1) * LD + whalf * 2 * E;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float q = static_cast<float>((wreg[j] >> (i * BITS)) & S::kMask);
+        wt[j * E + i] = T::rnd((q - m) * sreg);
+      }
+  };
+
+  float16v acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int frow = lane & 31, fk = lane >> 5;  // fragment: lane supplies element (row, k = 2 * step + fk)
+  const int nk = p.ng;
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int s = kt & 1;
+    if (kt + 1 < nk) load_tile(kt + 1);
+    const float* at = a_tile(s) + (wm0 + frow) * LD + fk;
+    const float* wt = w_tile(s) + (wn0 + frow) * LD + fk;
+#pragma unroll
+    for (int ks = 0; ks < G / 2; ++ks) {
+      float a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[i] = at[i * 32 * LD + 2 * ks];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) b[j] = wt[j * 32 * LD + 2 * ks];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) store_tile(s ^ 1);  // the other stage: nobody reads it during this tile
+    __syncthreads();
+  }
+
+  // D[r][c] of a 32 x 32 accumulator: lane c + 32 * ((r / 4) % 2), register 4 * (r / 8) + r % 4
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn0 + j * 32 + (lane & 31);
+      const float bias = (p.bias != nullptr && col < p.N) ? T::load(p.bias, col) : 0.0f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (row < p.M && col < p.N) store_out(p.y, static_cast<int64_t>(row) * p.N + col, acc[i][j][r] + bias, p.out_kind);
+      }
+    }
+}
+
+template <int BITS, int DT>
+hipError_t launch_dt(const LinParams& p, hipStream_t s) {
+  constexpr int G = 4 * Scheme<BITS>::kElem;
+  if (p.M <= 8) {
+    const int nb = p.M <= 1 ? 1 : (p.M <= 2 ? 2 : (p.M <= 4 ? 4 : 8));
+    const size_t lds = static_cast<size_t>(nb) * p.ng * G * sizeof(float);
+    if (lds <= 150 * 1024) {
+      // a few waves per SIMD, each walking its share of the rows
+      int blocks = (p.N + 3) / 4;
+      if (blocks > 1024) blocks = 1024;
+      auto go = [&](auto kern) -> hipError_t {
+        if (lds > 65536) {
+          const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+          if (e != hipSuccess) return e;
+        }
+        hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, s, p);
+        return hipGetLastError();
+      };
+      if (nb == 1) return go(gemv_dt_kernel<BITS, DT, 1>);
+      if (nb == 2) return go(gemv_dt_kernel<BITS, DT, 2>);
+      if (nb == 4) return go(gemv_dt_kernel<BITS, DT, 4>);
+      return go(gemv_dt_kernel<BITS, DT, 8>);
+    }
+  }
+  constexpr size_t lds = size_t(2) * 256 * (G + 1) * sizeof(float);
+  auto kern = gemm_dt_kernel<BITS, DT>;
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(kern, dim3((p.N + 127) / 128, (p.M + 127) / 128), dim3(256), lds, s, p);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_linear_dt(const void* x, const uint32_t* qw, const void* qs, const void* bias, int64_t M, int64_t N,
+                            int64_t K, int bits, int group_size, int model_dtype, int out_kind, void* y,
+                            hipStream_t s) {
+  LinParams p;
+  p.x = x; p.qw = qw; p.qs = qs; p.bias = bias; p.y = y;
+  p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(K);
+  p.ng = static_cast<int>((K + group_size - 1) / group_size);
+  p.nw = 4 * p.ng;
+  p.out_kind = out_kind;
+  if (model_dtype == MODEL_F32) return bits == 4 ? launch_dt<4, MODEL_F32>(p, s) : launch_dt<3, MODEL_F32>(p, s);
+  if (model_dtype == MODEL_BF16) return bits == 4 ? launch_dt<4, MODEL_BF16>(p, s) : launch_dt<3, MODEL_BF16>(p, s);
+  return hipErrorInvalidValue;
+}
+
+}  // namespace gq

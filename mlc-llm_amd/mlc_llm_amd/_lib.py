@@ -18,7 +18,7 @@ HEADER_PATH = os.path.join(os.path.dirname(os.path.dirname(_HERE)), "include", "
 
 OK = 0
 ERR_ARG, ERR_HIP, ERR_UNSUPPORTED, ERR_WORKSPACE = -1, -2, -3, -4
-F16, F32 = 0, 1
+F16, F32, BF16 = 0, 1, 2
 ROUND_HALF_AWAY, ROUND_HALF_EVEN = 0, 1
 I32, I64 = 0, 1
 EPILOGUE_NONE, EPILOGUE_SILU_MUL = 0, 1
@@ -33,6 +33,10 @@ SIGNATURES = {
     "mi355gq_set_option": (_I, [c_char_p, _I]),
     "mi355gq_quantize": (_I, [_P, _L, _L, _I, _I, _I, _P, _P, _P]),
     "mi355gq_dequantize": (_I, [_P, _P, _L, _L, _I, _I, _P, _P]),
+    "mi355gq_quantize_dt": (_I, [_P, _L, _L, _I, _I, _I, _I, _P, _P, _P]),
+    "mi355gq_dequantize_dt": (_I, [_P, _P, _L, _L, _I, _I, _I, _P, _P]),
+    "mi355gq_embedding_take_dt": (_I, [_P, _L, _P, _P, _L, _L, _I, _I, _I, _P, _P]),
+    "mi355gq_linear_dt": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _I, _P, _P]),
     "mi355gq_probe_stream_read": (_I, [_P, _L, _P, _L, _P, _P]),
     "mi355gq_embedding_take": (_I, [_P, _L, _P, _P, _L, _L, _I, _I, _P, _P]),
     "mi355gq_linear_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),

@@ -33,6 +33,9 @@ def _chk(t: torch.Tensor, dtype, name: str) -> torch.Tensor:
 
 
 _STORAGE = (torch.int32, torch.uint32)
+# model dtypes of the reference's group-quant registry -> the C ABI's dtype codes
+_MODEL_DTYPES = {torch.float16: _lib.F16, torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}
+_FLOATS = tuple(_MODEL_DTYPES)
 
 
 def num_group(k: int, group_size: int) -> int:
@@ -45,30 +48,40 @@ def num_storage(k: int, bits: int, group_size: int) -> int:
 
 def quantize(w: torch.Tensor, bits: int, group_size: int, round_mode: int = _lib.ROUND_HALF_AWAY
              ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """w fp16 [..., K] -> (q_weight int32-as-uint32 [..., nw], q_scale fp16 [..., ng])."""
-    _chk(w, torch.float16, "w")
+    """w [..., K] in the model dtype (float16, or float32 / bfloat16 for the q4f32 / q4bf16 schemes)
+    -> (q_weight int32-as-uint32 [..., nw], q_scale [..., ng] in the same dtype)."""
+    _chk(w, _FLOATS, "w")
     k = w.shape[-1]
     rows = w.numel() // k if k else 0
     lead = tuple(w.shape[:-1])
     qw = torch.empty((*lead, num_storage(k, bits, group_size)), dtype=torch.int32, device=w.device)
-    qs = torch.empty((*lead, num_group(k, group_size)), dtype=torch.float16, device=w.device)
-    _lib.call("mi355gq_quantize", w.data_ptr(), rows, k, bits, group_size, round_mode,
-              qw.data_ptr(), qs.data_ptr(), _stream())
+    qs = torch.empty((*lead, num_group(k, group_size)), dtype=w.dtype, device=w.device)
+    if w.dtype == torch.float16:
+        _lib.call("mi355gq_quantize", w.data_ptr(), rows, k, bits, group_size, round_mode,
+                  qw.data_ptr(), qs.data_ptr(), _stream())
+    else:
+        _lib.call("mi355gq_quantize_dt", w.data_ptr(), rows, k, bits, group_size, round_mode,
+                  _MODEL_DTYPES[w.dtype], qw.data_ptr(), qs.data_ptr(), _stream())
     return qw, qs
 
 
 def dequantize(q_weight: torch.Tensor, q_scale: torch.Tensor, k: int, bits: int, group_size: int
                ) -> torch.Tensor:
+    """(q_weight, q_scale) -> [..., K] in the dtype of q_scale (the scheme's model dtype)."""
     _chk(q_weight, _STORAGE, "q_weight")
-    _chk(q_scale, torch.float16, "q_scale")
+    _chk(q_scale, _FLOATS, "q_scale")
     lead = tuple(q_weight.shape[:-1])
     _check_qshapes(q_weight, q_scale, lead, k, bits, group_size)
     rows = 1
     for d in lead:
         rows *= d
-    out = torch.empty((*lead, k), dtype=torch.float16, device=q_weight.device)
-    _lib.call("mi355gq_dequantize", q_weight.data_ptr(), q_scale.data_ptr(), rows, k, bits,
-              group_size, out.data_ptr(), _stream())
+    out = torch.empty((*lead, k), dtype=q_scale.dtype, device=q_weight.device)
+    if q_scale.dtype == torch.float16:
+        _lib.call("mi355gq_dequantize", q_weight.data_ptr(), q_scale.data_ptr(), rows, k, bits,
+                  group_size, out.data_ptr(), _stream())
+    else:
+        _lib.call("mi355gq_dequantize_dt", q_weight.data_ptr(), q_scale.data_ptr(), rows, k, bits,
+                  group_size, _MODEL_DTYPES[q_scale.dtype], out.data_ptr(), _stream())
     return out
 
 
@@ -84,13 +97,17 @@ def embedding_take(ids: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Ten
                    bits: int, group_size: int) -> torch.Tensor:
     _chk(ids, torch.int32, "ids")
     _chk(q_weight, _STORAGE, "q_weight")
-    _chk(q_scale, torch.float16, "q_scale")
+    _chk(q_scale, _FLOATS, "q_scale")
     num = q_weight.shape[0]
     _check_qshapes(q_weight, q_scale, (num,), k, bits, group_size)
     t = ids.numel()
-    out = torch.empty((*ids.shape, k), dtype=torch.float16, device=q_weight.device)
-    _lib.call("mi355gq_embedding_take", ids.data_ptr(), t, q_weight.data_ptr(), q_scale.data_ptr(),
-              num, k, bits, group_size, out.data_ptr(), _stream())
+    out = torch.empty((*ids.shape, k), dtype=q_scale.dtype, device=q_weight.device)
+    if q_scale.dtype == torch.float16:
+        _lib.call("mi355gq_embedding_take", ids.data_ptr(), t, q_weight.data_ptr(), q_scale.data_ptr(),
+                  num, k, bits, group_size, out.data_ptr(), _stream())
+    else:
+        _lib.call("mi355gq_embedding_take_dt", ids.data_ptr(), t, q_weight.data_ptr(), q_scale.data_ptr(),
+                  num, k, bits, group_size, _MODEL_DTYPES[q_scale.dtype], out.data_ptr(), _stream())
     return out
 
 
@@ -101,7 +118,9 @@ def linear(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits:
 
     `residual` (fp16, the shape of y) is added inside the kernel; passing the same tensor as `out`
     updates it in place."""
-    _chk(x, torch.float16, "x")
+    _chk(x, _FLOATS, "x")
+    if x.dtype != torch.float16:
+        return _linear_other_dtype(x, q_weight, q_scale, bits, group_size, bias, out_dtype, out, residual)
     _chk(q_weight, _STORAGE, "q_weight")
     _chk(q_scale, torch.float16, "q_scale")
     k = x.shape[-1]
@@ -133,6 +152,38 @@ def linear(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits:
         _lib.call("mi355gq_linear", *head, *tail)
     else:
         _lib.call("mi355gq_linear_residual", *head, residual.data_ptr(), *tail)
+    return out
+
+
+def _linear_other_dtype(x, q_weight, q_scale, bits, group_size, bias, out_dtype, out, residual):
+    """linear() for float32 / bfloat16 models: x, q_scale and bias share the model dtype; the output is
+    that dtype (the default here, whatever `out_dtype` defaults to for float16) or float32."""
+    dt = x.dtype
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, dt, "q_scale")
+    if residual is not None:
+        raise NotImplementedError("linear: the residual epilogue exists for float16 models only")
+    k = x.shape[-1]
+    n = q_weight.shape[0]
+    _check_qshapes(q_weight, q_scale, (n,), k, bits, group_size)
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    if bias is not None:
+        _chk(bias, dt, "bias")
+        if tuple(bias.shape) != (n,):
+            raise ValueError(f"bias shape {tuple(bias.shape)}, expected {(n,)}")
+    if out_dtype == torch.float16:  # the float16 default of the signature
+        out_dtype = dt
+    if out_dtype not in (dt, torch.float32):
+        raise TypeError(f"out_dtype {out_dtype} for a {dt} model")
+    if out is None:
+        out = torch.empty((*x.shape[:-1], n), dtype=out_dtype, device=x.device)
+    else:
+        _chk(out, out_dtype, "out")
+    _lib.call("mi355gq_linear_dt", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(),
+              bias.data_ptr() if bias is not None else None, m, n, k, bits, group_size, _MODEL_DTYPES[dt],
+              _MODEL_DTYPES[out_dtype], out.data_ptr(), _stream())
     return out
 
 

@@ -27,6 +27,8 @@ from . import _lib, ops
 
 _DTYPE_BITS = {"int3": 3, "int4": 4, "int8": 8, "uint32": 32}
 _TORCH_DTYPE = {"float16": torch.float16, "float32": torch.float32, "bfloat16": torch.bfloat16}
+MATMUL_MODEL_DTYPES = ("float16", "float32", "bfloat16")  # model dtypes with a linear kernel
+MOE_MODEL_DTYPES = ("float16",)  # ... and with the expert matmuls
 
 
 @dataclasses.dataclass
@@ -88,16 +90,20 @@ class GroupQuantize:
     def bits(self) -> int:
         return _DTYPE_BITS[self.quantize_dtype]
 
-    def _require_built(self):
-        if self.model_dtype != "float16":
+    def _require_built(self, matmul: bool = True):
+        """Packing (quantize / dequantize / embedding take) exists for every model dtype of the
+        registry; the dequantize-fused matmuls for those in MATMUL_MODEL_DTYPES."""
+        if matmul and self.model_dtype not in MATMUL_MODEL_DTYPES:
             raise NotImplementedError(
-                f"{self.name}: only float16 group quantization has gfx950 kernels"
+                f"{self.name}: no gfx950 matmul kernel for model dtype {self.model_dtype} "
+                f"(built: {', '.join(MATMUL_MODEL_DTYPES)}); quantize / dequantize / embedding are available"
             )
 
     def quantize_weight(self, weight: torch.Tensor, axis: int = -1, output_transpose: bool = False
                         ) -> List[torch.Tensor]:
         """Quantize `weight` along `axis` (must be the last axis): [q_weight, q_scale]."""
-        self._require_built()
+        self._require_built(matmul=False)
+        weight = weight.to(_TORCH_DTYPE[self.model_dtype])
         axis = axis if axis >= 0 else weight.dim() + axis
         if axis != weight.dim() - 1:
             raise NotImplementedError("quantize_weight: only the last axis is supported (NK layout)")
@@ -113,7 +119,7 @@ class GroupQuantize:
     def dequantize_weight(self, q_weight: torch.Tensor, q_scale: torch.Tensor, in_features: int
                           ) -> torch.Tensor:
         """GroupQuantize._dequantize over the last axis, out_shape [..., in_features]."""
-        self._require_built()
+        self._require_built(matmul=False)
         return ops.dequantize(q_weight, q_scale, in_features, self.bits, self.group_size)
 
     def quantize_model(self, model: nn.Module, quant_map: QuantizeMapping, name_prefix: str
@@ -242,10 +248,11 @@ class GroupQuantizeLinear(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         self.config._require_built()
-        out_dtype = torch.float16 if self.out_dtype is None else _TORCH_DTYPE[self.out_dtype]
+        model_dtype = _TORCH_DTYPE[self.config.model_dtype]
+        out_dtype = model_dtype if self.out_dtype is None else _TORCH_DTYPE[self.out_dtype]
         q_weight, q_scale = self._nk_tensors()
         bias = self.bias
-        if bias is not None and bias.dtype != torch.float16:
+        if bias is not None and bias.dtype != model_dtype:
             # fp32 bias with fp32 output: added after the kernel, as the reference's `x + bias`
             y = ops.linear(x, q_weight, q_scale, self.config.bits, self.config.group_size, None, out_dtype)
             return y + bias
@@ -255,6 +262,8 @@ class GroupQuantizeLinear(nn.Module):
         """For a gate_up projection: `x1, x2 = split(self(x), 2, axis=-1); silu(x1) * x2` of the MLP
         (model/llama/llama_model.py:122-125) in one kernel; same bits as the two steps."""
         self.config._require_built()
+        if self.config.model_dtype != "float16":
+            raise NotImplementedError(f"{self.config.name}: silu * mul (folded or not) is built for float16 models")
         if self.bias is not None or self.out_dtype not in (None, "float16"):
             return ops.silu_mul(self.forward(x).reshape(-1, self.out_features)).reshape(*x.shape[:-1], -1)
         q_weight, q_scale = self._nk_tensors()
@@ -279,7 +288,7 @@ class GroupQuantizeEmbedding(nn.Module):
         return GroupQuantizeEmbedding(num, dim, config, device=embedding.weight.device)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        self.config._require_built()
+        self.config._require_built(matmul=False)
         ids = x.reshape(-1).to(torch.int32).contiguous()
         out = ops.embedding_take(ids, self.q_weight, self.q_scale, self.dim, self.config.bits,
                                  self.config.group_size)
@@ -344,6 +353,8 @@ class GroupQuantizeMixtralExperts(nn.Module):
         silu_mul_halves: return silu(x1) * x3 of the two halves of the output (the e1_e3 stack of
         mixtral_model.py:64-68) from the same kernel."""
         assert x.dim() == 2
+        if self.config.model_dtype not in MOE_MODEL_DTYPES:
+            raise NotImplementedError(f"{self.config.name}: the expert matmuls are built for {MOE_MODEL_DTYPES} models")
         if indptr.dim() == 2:
             assert indptr.shape[0] == 1
             return ops.moe_gemv(x, self.q_weight, self.q_scale, indptr, self.config.bits,
@@ -353,7 +364,8 @@ class GroupQuantizeMixtralExperts(nn.Module):
                                   self.group_size, silu_mul_halves)
 
 
-def _group(name: str, group_size: int, qdtype: str, layout: str, model_dtype: str = "float16"):
+def _group(name: str, group_size: int, qdtype: str, layout: str, model_dtype: str = "float16",
+           embedding_and_final_fc: bool = True):
     return GroupQuantize(
         name=name,
         kind="group-quant",
@@ -362,8 +374,8 @@ def _group(name: str, group_size: int, qdtype: str, layout: str, model_dtype: st
         storage_dtype="uint32",
         model_dtype=model_dtype,
         linear_weight_layout=layout,
-        quantize_embedding=True,
-        quantize_final_fc=True,
+        quantize_embedding=embedding_and_final_fc,
+        quantize_final_fc=embedding_and_final_fc,
     )
 
 
@@ -374,4 +386,10 @@ QUANTIZATION: Dict[str, GroupQuantize] = {
     "q3f16_1": _group("q3f16_1", 40, "int3", "NK"),
     "q4f16_0": _group("q4f16_0", 32, "int4", "KN"),
     "q4f16_1": _group("q4f16_1", 32, "int4", "NK"),
+    # q4f16_1 that leaves the embedding and the final fc unquantized (quantization.py:124-134)
+    "q4f16_2": _group("q4f16_2", 32, "int4", "NK", embedding_and_final_fc=False),
+    # other model dtypes (quantization.py:91-123): packing built, matmuls per MATMUL_MODEL_DTYPES
+    "q4bf16_0": _group("q4bf16_0", 32, "int4", "KN", "bfloat16"),
+    "q4bf16_1": _group("q4bf16_1", 32, "int4", "NK", "bfloat16"),
+    "q4f32_1": _group("q4f32_1", 32, "int4", "NK", "float32"),
 }

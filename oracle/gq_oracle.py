@@ -155,6 +155,86 @@ def dequantize(q_weight: np.ndarray, q_scale: np.ndarray, scheme: Scheme, k: int
     return (d * s).astype(F16)
 
 
+# --------------------------------------------------------------------------- other model dtypes
+#
+# GroupQuantize carries `model_dtype` through _quantize / _dequantize (group_quantization.py:155-186,
+# 235-306); the registry holds float32 (q4f32_1) and bfloat16 (q4bf16_0/1) next to float16
+# (quantization/quantization.py:91-123).  Tensors of a model dtype travel here as float32 arrays whose
+# values are representable in that dtype ("carrier"); every operation is done in float32 and rounded
+# to the dtype, which for float16 / bfloat16 equals the correctly rounded operation (the operands have
+# 11 / 8 significant bits) and for float32 is the operation itself.  PARITY UNPINNED like the float16
+# path's tie rule, plus, for bfloat16, the assumption that TVM legalises each bf16 operation to
+# "widen, operate in float32, round to nearest even" (the reference holds no test of these schemes).
+
+MODEL_DTYPES = ("float16", "float32", "bfloat16")
+
+
+def bf16_round(a: np.ndarray) -> np.ndarray:
+    """float32 -> nearest-even bfloat16, returned as float32 (NaN stays NaN, overflow goes to inf)."""
+    a = np.ascontiguousarray(a, dtype=F32)
+    bits = a.view(U32)
+    nan = np.isnan(a)
+    out = ((bits + U32(0x7FFF) + ((bits >> U32(16)) & U32(1))) & U32(0xFFFF0000)).view(F32)
+    return np.where(nan, a, out)
+
+
+def round_to(a: np.ndarray, model_dtype: str) -> np.ndarray:
+    if model_dtype == "float16":
+        with np.errstate(over="ignore"):
+            return np.asarray(a, dtype=F32).astype(F16).astype(F32)
+    if model_dtype == "float32":
+        return np.asarray(a, dtype=F32)
+    if model_dtype == "bfloat16":
+        return bf16_round(a)
+    raise ValueError(f"unknown model dtype {model_dtype!r}")
+
+
+_LOWEST = {"float16": -65504.0, "float32": -3.4028234663852886e38, "bfloat16": -3.3895313892515355e38}
+
+
+def quantize_dt(w: np.ndarray, scheme: Scheme, model_dtype: str, round_mode: str = "half_away"):
+    """quantize() for any model dtype.  w: float32 carrier [..., K]; returns (q_weight uint32, q_scale
+    float32 carrier)."""
+    w = round_to(w, model_dtype)
+    g, m = scheme.group_size, scheme.max_int
+    k = w.shape[-1]
+    ng = scheme.num_group(k)
+    lead = w.shape[:-1]
+    pad = ng * g - k
+    absw = np.abs(w)
+    if pad:
+        absw = np.concatenate([absw, np.full((*lead, pad), _LOWEST[model_dtype], F32)], axis=-1)
+    max_abs = absw.reshape(*lead, ng, g).max(axis=-1)
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        scale = round_to(max_abs / F32(m), model_dtype)
+        s_full = np.repeat(scale, g, axis=-1)[..., :k]
+        t = round_to(w / s_full, model_dtype)
+        t = round_to(t + F32(m), model_dtype)
+        r = _round(t, round_mode)
+        r = np.where(r > 0, r, F32(0))
+        r = np.where(r < 2 * m, r, F32(2 * m))
+    return pack(r.astype(U32), scheme), scale
+
+
+def dequantize_dt(q_weight: np.ndarray, q_scale: np.ndarray, scheme: Scheme, k: int, model_dtype: str) -> np.ndarray:
+    """dequantize() for any model dtype; q_scale and the result are float32 carriers."""
+    u = unpack(q_weight, scheme, k).astype(F32) - F32(scheme.max_int)  # exact in every dtype
+    s = np.asarray(q_scale, dtype=F32)[..., np.arange(k) // scheme.group_size]
+    with np.errstate(over="ignore", invalid="ignore"):
+        return round_to(u * s, model_dtype)
+
+
+def linear_dt_fp64(x, q_weight, q_scale, scheme: Scheme, model_dtype: str, bias=None) -> np.ndarray:
+    """Yardstick of the linear for any model dtype: weights dequantised in the model dtype
+    (dequantize_dt), then an exact float64 matmul.  x, q_scale, bias: float32 carriers."""
+    k = x.shape[-1]
+    w = dequantize_dt(q_weight, q_scale, scheme, k, model_dtype).astype(np.float64)
+    y = np.asarray(x, dtype=np.float64) @ w.T
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=np.float64)
+    return y
+
+
 def linear_fp32(x, q_weight, q_scale, scheme: Scheme, bias=None) -> np.ndarray:
     """fp32 dequant-then-matmul: the yardstick the output tolerance is quoted against.
 

@@ -790,6 +790,126 @@ def test_quantize_dequantize_every_row_length(name):
         assert np.array_equal(host_f16_bits(d), o.dequantize(qw_ref, qs_ref, s, k).view(np.uint16)), k
 
 
+# ------------------------------------------------------------------ other model dtypes (q4f32_1, q4bf16_*)
+
+_TORCH_OF = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def _carrier(t: torch.Tensor) -> np.ndarray:
+    return t.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("bits_name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_packing_other_model_dtypes_bit_exact(model_dtype, bits_name, mode):
+    s = SCHEMES[bits_name]
+    dt = _TORCH_OF[model_dtype]
+    rng = np.random.default_rng(77)
+    for rows, k in ((5, 13), (16, 120), (16, 128), (33, 4096), (7, 1000)):
+        w32 = o.round_to((rng.standard_normal((rows, k)) * 0.07).astype(np.float32), model_dtype)
+        w32[0, : min(k, s.group_size)] = 0          # an all-zero group: 0 / 0
+        w32[1, 0] = float(o.round_to(np.array([3.0e4], dtype=np.float32), model_dtype)[0])  # one large value in a group of small ones
+        w = torch.from_numpy(w32).to(dt).to(DEV)
+        assert np.array_equal(_carrier(w), w32)
+        qw_ref, qs_ref = o.quantize_dt(w32, s, model_dtype, ["half_away", "half_even"][mode])
+        qw, qs = ops.quantize(w, s.bits, s.group_size, mode)
+        assert qs.dtype == dt
+        assert np.array_equal(_carrier(qs), qs_ref), (rows, k)
+        assert np.array_equal(host_u32(qw), qw_ref), (rows, k)
+        d = ops.dequantize(qw, qs, k, s.bits, s.group_size)
+        assert d.dtype == dt
+        d_ref = o.dequantize_dt(qw_ref, qs_ref, s, k, model_dtype)
+        assert np.array_equal(_carrier(d), d_ref), (rows, k)
+        ids = torch.tensor([rows - 1, 0, 2, 2, 99, -1], dtype=torch.int32, device=DEV)
+        emb = ops.embedding_take(ids, qw, qs, k, s.bits, s.group_size)
+        assert np.array_equal(_carrier(emb), d_ref[[rows - 1, 0, 2, 2, rows - 1, 0]])
+
+
+def test_other_model_dtypes_modules():
+    # registry entries: quantize_weight / dequantize_weight / embedding work; the matmul says what is missing
+    for name in ("q4bf16_1", "q4f32_1", "q4bf16_0"):
+        cfg = gq.QUANTIZATION[name]
+        dt = _TORCH_OF[cfg.model_dtype]
+        w = (torch.randn(48, 96, device=DEV) * 0.05)
+        qw, qs = cfg.quantize_weight(w, output_transpose=cfg.linear_weight_layout == "KN")
+        assert qs.dtype == dt
+        if cfg.linear_weight_layout == "KN":
+            assert tuple(qw.shape) == (12, 48) and tuple(qs.shape) == (3, 48)
+            qw, qs = qw.t().contiguous(), qs.t().contiguous()
+        back = cfg.dequantize_weight(qw, qs, 96)
+        # half a step, plus the bf16 roundings of the quotient and of the product
+        assert back.dtype == dt and (back.float() - w.to(dt).float()).abs().max() <= qs.float().abs().max() * (0.51 if dt == torch.float32 else 0.6)
+        emb = gq.GroupQuantizeEmbedding(48, 96, cfg, device=DEV)
+        if cfg.linear_weight_layout == "NK":
+            emb.q_weight.data.copy_(qw)
+            emb.q_scale.data.copy_(qs)
+            out = emb(torch.tensor([[3, 47]], device=DEV))
+            assert torch.equal(out[0], back[[3, 47]])
+        if cfg.linear_weight_layout == "NK":  # (the reference has no KN expert stack either)
+            experts = gq.GroupQuantizeMixtralExperts(2, 96, 48, cfg, device=DEV)
+            with pytest.raises(NotImplementedError):
+                experts(torch.zeros(1, 96, dtype=dt, device=DEV), torch.zeros((1, 2), dtype=torch.int32, device=DEV))
+
+
+@pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("bits_name,m,n,k", [
+    ("q4f16_1", 1, 512, 4096), ("q4f16_1", 2, 100, 1000), ("q4f16_1", 4, 257, 2048), ("q4f16_1", 8, 128, 8192),
+    ("q4f16_1", 3, 64, 13), ("q4f16_1", 1, 40, 40000),                     # ragged K; K past the GEMV's LDS
+    ("q4f16_1", 9, 256, 512), ("q4f16_1", 130, 200, 1024), ("q4f16_1", 300, 384, 360), ("q4f16_1", 64, 130, 100),
+    ("q3f16_1", 1, 256, 4096), ("q3f16_1", 5, 96, 1000), ("q3f16_1", 200, 136, 2000),
+])
+def test_linear_other_model_dtypes(model_dtype, bits_name, m, n, k):
+    s = SCHEMES[bits_name]
+    dt = _TORCH_OF[model_dtype]
+    rng = np.random.default_rng(m * 1000 + n)
+    w32 = o.round_to((rng.standard_normal((n, k)) * 0.05).astype(np.float32), model_dtype)
+    x32 = o.round_to(rng.standard_normal((m, k)).astype(np.float32), model_dtype)
+    b32 = o.round_to(rng.standard_normal(n).astype(np.float32), model_dtype)
+    qw_ref, qs_ref = o.quantize_dt(w32, s, model_dtype)
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).to(dt).to(DEV)
+    x, b = torch.from_numpy(x32).to(dt).to(DEV), torch.from_numpy(b32).to(dt).to(DEV)
+    ref = o.linear_dt_fp64(x32, qw_ref, qs_ref, s, model_dtype, b32)
+    den = np.linalg.norm(ref)
+    # float32 result: only the fp32 accumulation separates it from the exact product of the same operands
+    y32 = ops.linear(x, qw, qs, s.bits, s.group_size, b, out_dtype=torch.float32)
+    assert y32.dtype == torch.float32 and tuple(y32.shape) == (m, n)
+    err = y32.double().cpu().numpy() - ref
+    # (relative error of a float32 sum of k terms grows like sqrt(k) * 2^-24)
+    assert np.linalg.norm(err) / den <= 1e-6 + 4e-8 * np.sqrt(k), np.linalg.norm(err) / den
+    assert np.abs(err).max() <= 1e-2 * np.abs(x32).max() * np.sqrt(k) / 64
+    # output in the model dtype: the same numbers rounded once
+    y = ops.linear(x, qw, qs, s.bits, s.group_size, b)
+    assert y.dtype == dt
+    assert np.array_equal(_carrier(y), o.round_to(y32.cpu().numpy(), model_dtype))
+
+
+def test_linear_other_model_dtypes_through_the_modules():
+    for name in ("q4f32_1", "q4bf16_1", "q4bf16_0"):
+        cfg = gq.QUANTIZATION[name]
+        dt = _TORCH_OF[cfg.model_dtype]
+        torch.manual_seed(4)
+        src = torch.nn.Linear(256, 72, bias=True, device=DEV)
+        lin = gq.GroupQuantizeLinear.from_linear(src, cfg)
+        qw, qs = cfg.quantize_weight(src.weight.data, output_transpose=cfg.linear_weight_layout == "KN")
+        lin.q_weight.data.copy_(qw)
+        lin.q_scale.data.copy_(qs)
+        lin.bias.data.copy_(src.bias.data.to(dt))
+        x = torch.randn(3, 5, 256, device=DEV).to(dt)
+        y = lin(x)
+        assert y.dtype == dt and tuple(y.shape) == (3, 5, 72)
+        nk_w, nk_s = (qw.t().contiguous(), qs.t().contiguous()) if cfg.linear_weight_layout == "KN" else (qw, qs)
+        w_deq = cfg.dequantize_weight(nk_w, nk_s, 256)
+        want = x.double() @ w_deq.double().t() + lin.bias.double()
+        assert (y.double() - want).norm() / want.norm() <= (3e-3 if dt == torch.bfloat16 else 1e-6)
+        emb = gq.GroupQuantizeEmbedding(72, 256, cfg, device=DEV)
+        emb.q_weight.data.copy_(nk_w)
+        emb.q_scale.data.copy_(nk_s)
+        logits = emb.lm_head_forward(x)
+        assert logits.dtype == torch.float32
+        assert (logits.double() - x.double() @ w_deq.double().t()).norm() / want.norm() <= 1e-5
+
+
 # ------------------------------------------------------------------ gate_up with the activation folded in
 
 def assert_silu_mul_ok(y: torch.Tensor, ref64: np.ndarray, x: np.ndarray, k: int, what=""):

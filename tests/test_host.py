@@ -184,3 +184,43 @@ def test_tensor_parallel_group_check():
     with pytest.raises(ValueError, match="cannot be evenly distributed"):
         gq.GroupQuantizeLinear(48, 8, cfg)  # 96 input features = 3 groups over 2 shards
     gq.GroupQuantizeLinear(64, 8, cfg)  # 4 groups over 2 shards
+
+
+def test_registry_holds_every_group_quant_entry_of_the_reference():
+    # quantization/quantization.py:47-134 of the reference
+    want = {"q3f16_0": (40, "int3", "KN", "float16", True), "q3f16_1": (40, "int3", "NK", "float16", True),
+            "q4f16_0": (32, "int4", "KN", "float16", True), "q4f16_1": (32, "int4", "NK", "float16", True),
+            "q4bf16_0": (32, "int4", "KN", "bfloat16", True), "q4bf16_1": (32, "int4", "NK", "bfloat16", True),
+            "q4f32_1": (32, "int4", "NK", "float32", True), "q4f16_2": (32, "int4", "NK", "float16", False)}
+    assert set(gq.QUANTIZATION) == set(want)
+    for name, (g, qd, layout, md, emb) in want.items():
+        c = gq.QUANTIZATION[name]
+        assert (c.group_size, c.quantize_dtype, c.linear_weight_layout, c.model_dtype) == (g, qd, layout, md)
+        assert c.quantize_embedding == emb and c.quantize_final_fc == emb
+
+
+def test_q4f16_2_leaves_embedding_and_final_fc_alone():
+    import torch
+    from torch import nn
+
+    class Tiny(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.embed_tokens = nn.Embedding(16, 64)
+            self.proj = nn.Linear(64, 64, bias=False)
+            self.lm_head = nn.Linear(64, 16, bias=False)
+
+    qmap = gq.QuantizeMapping({}, {})
+    m = gq.QUANTIZATION["q4f16_2"].quantize_model(Tiny(), qmap, "")
+    assert isinstance(m.embed_tokens, nn.Embedding) and isinstance(m.lm_head, nn.Linear)
+    assert isinstance(m.proj, gq.GroupQuantizeLinear)
+    assert set(qmap.param_map) == {"proj.weight"}
+
+
+def test_other_model_dtypes_carry_their_dtype_in_the_parameters():
+    import torch
+    for name, dt in (("q4bf16_1", torch.bfloat16), ("q4f32_1", torch.float32)):
+        lin = gq.GroupQuantizeLinear(64, 24, gq.QUANTIZATION[name], bias=True)
+        assert lin.q_scale.dtype == dt and lin.bias.dtype == dt and lin.q_weight.shape == (24, 8)
+        emb = gq.GroupQuantizeEmbedding(10, 64, gq.QUANTIZATION[name])
+        assert emb.q_scale.dtype == dt

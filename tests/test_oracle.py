@@ -355,3 +355,58 @@ def test_golden_fixtures_reproduce(golden):
         elif name.startswith("moe_"):
             y = o.mixtral_moe(z["x"], z["logits"], z["q13"], z["s13"], z["q2"], z["s2"], Q4, 2)
             assert (y.view(np.uint16) == z["y"].view(np.uint16)).all()
+
+
+# --------------------------------------------------------------------------- other model dtypes
+
+def test_generic_dtype_oracle_reproduces_the_pinned_float16_one():
+    # the float32 / bfloat16 restatement shares its code with a float16 instance; that instance must
+    # be the float16 oracle pinned above, bit for bit (codes, scales, dequantised values)
+    rng = np.random.default_rng(11)
+    for name in ("q4f16_1", "q3f16_1"):
+        s = o.SCHEMES[name]
+        w = (rng.standard_normal((9, 203)) * 0.05).astype(np.float16)
+        w[2, :80] = 0
+        w[3, 5] = 60000.0
+        for mode in ("half_away", "half_even"):
+            qw, qs = o.quantize(w, s, mode)
+            qw2, qs2 = o.quantize_dt(w.astype(np.float32), s, "float16", mode)
+            assert np.array_equal(qw, qw2) and np.array_equal(qs.astype(np.float32), qs2)
+        d = o.dequantize(qw, qs, s, 203)
+        assert np.array_equal(d.astype(np.float32), o.dequantize_dt(qw, qs.astype(np.float32), s, 203, "float16"))
+
+
+def test_bf16_rounding_known_values():
+    x = np.array([1.0, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, 1.0 + 2.0 ** -8 + 2.0 ** -20, -2.5, 3.3895314e38, 3.4e38],
+                 dtype=np.float32)
+    want = np.array([1.0, 1.0, 1.015625, 1.0078125, -2.5, 3.3895314e38, np.inf], dtype=np.float32)
+    assert np.array_equal(o.bf16_round(x), want)  # ties to even, overflow to infinity
+    assert np.isnan(o.bf16_round(np.array([np.nan], dtype=np.float32))[0])
+    # agrees with torch's conversion on random values
+    import torch
+    r = np.random.default_rng(3).standard_normal(20000).astype(np.float32) * 10
+    assert np.array_equal(o.bf16_round(r), torch.from_numpy(r).bfloat16().float().numpy())
+
+
+def test_float32_scheme_closed_forms():
+    # float32 arithmetic: scale = max|w| / 7 exactly as numpy float32 divides; a weight equal to +-max
+    # maps to 14 / 0; an all-zero group gives code 0 and scale 0; dequantize is (q - 7) * scale
+    s = o.SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(5)
+    w = rng.standard_normal((4, 96)).astype(np.float32)
+    w[1, 32:64] = 0
+    qw, qs = o.quantize_dt(w, s, "float32")
+    q = o.unpack(qw, s, 96)
+    assert np.array_equal(qs, (np.abs(w).reshape(4, 3, 32).max(-1) / np.float32(7)).astype(np.float32))
+    g = np.abs(w).reshape(4, 3, 32)
+    am = g.argmax(-1)
+    for r in range(4):
+        for gi in range(3):
+            if r == 1 and gi == 1:
+                assert (q[r, 32:64] == 0).all() and qs[r, gi] == 0
+                continue
+            k = gi * 32 + am[r, gi]
+            assert q[r, k] == (14 if w[r, k] > 0 else 0)
+    d = o.dequantize_dt(qw, qs, s, 96, "float32")
+    assert np.array_equal(d, (q.astype(np.float32) - 7) * np.repeat(qs, 32, -1))
+    assert np.abs(d - w).max() <= np.abs(qs).max() * 0.5000001
