@@ -2,13 +2,15 @@
 // of GroupQuantizeLinear.forward / lm_head_forward (group_quantization.py:390-437, 524-556) with
 // x, q_scale and bias in float32 or bfloat16.
 //
-// A first, plain form of the two regimes of the float16 path:
-//  * up to 8 activation rows: a GEMV with x resident in LDS as float32, one weight row per wave and
-//    step, fp32 FMAs (there is no dot-product instruction to lean on for these types);
+// A first form of the two regimes of the float16 path:
+//  * up to 8 activation rows: a persistent-wave GEMV with x resident in LDS in the model dtype
+//    (fp32 FMAs for float32, v_dot2_f32_bf16 on bf16 pairs for bfloat16);
 //  * more rows: a 128 x 128 tile GEMM on v_mfma_f32_32x32x2_f32 with both operands in LDS as
 //    float32 (bfloat16 operands are widened on the way in; their products are exact either way).
 // Weights are dequantised exactly as GroupQuantize._dequantize does, (q - m) * scale rounded to the
 // model dtype, before they meet x; accumulation is fp32.
+#include <type_traits>
+
 #include "gq_common.hpp"
 #include "gq_internal.hpp"
 
@@ -58,55 +60,141 @@ struct LinParams {
 
 // ---------------------------------------------------------------- up to 8 rows
 
-// LDS: x as float [NB][kpad] (zero beyond K).  Lane l of a wave owns groups l, l + 64, ... of the
-// wave's current weight row.
-template <int BITS, int DT, int NB>
-__global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p) {
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+
+// Persistent waves, two weight rows per step, the loads of the next two steps in flight (the
+// structure of the float16 register GEMV); x lives in LDS in the model dtype, zero beyond K, and is
+// read once per group for both rows.  Lane l owns groups l + 64 * it, it < ITERS.
+//  * float32: w = (q - m) * s as _dequantize rounds it, then one FMA per activation row;
+//  * bfloat16: (q - m) * s is exact in float32 (4 x 8 significant bits), v_cvt_pk_bf16_f32 rounds
+//    two of them to the bf16 pair _dequantize would hold, and v_dot2_f32_bf16 multiplies the pair
+//    with the matching pair of x (exact products, fp32 accumulation).
+template <int BITS, int DT, int NB, int ITERS>
+__global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nsets) {
   using S = Scheme<BITS>;
   using T = LinT<DT>;
   constexpr int E = S::kElem;
   constexpr int G = 4 * E;
-  extern __shared__ float xs[];
+  constexpr bool BF = DT == MODEL_BF16;
+  extern __shared__ uint32_t xs_raw[];
+  float* xs = reinterpret_cast<float*>(xs_raw);         // float32: [NB][kpad]
+  uint16_t* xh = reinterpret_cast<uint16_t*>(xs_raw);   // bfloat16: [NB][kpad]
   const int kpad = p.ng * G;
   for (int i = threadIdx.x; i < NB * kpad; i += 256) {
     const int b = i / kpad, k = i - b * kpad;
-    xs[i] = (b < p.M && k < p.K) ? T::load(p.x, static_cast<int64_t>(b) * p.K + k) : 0.0f;
+    const bool ok = b < p.M && k < p.K;
+    if (BF) xh[i] = ok ? static_cast<const uint16_t*>(p.x)[static_cast<int64_t>(b) * p.K + k] : uint16_t(0);
+    else xs[i] = ok ? static_cast<const float*>(p.x)[static_cast<int64_t>(b) * p.K + k] : 0.0f;
   }
-  __syncthreads();
 
   const int lane = threadIdx.x & 63;
   const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * 4;
-  const float m = static_cast<float>(S::kMaxInt);
-  for (int row = gw; row < p.N; row += nwaves) {
-    float acc[NB];
+  int gidx[ITERS];
+  bool gok[ITERS];
 #pragma unroll
-    for (int b = 0; b < NB; ++b) acc[b] = 0.0f;
-    const uint32_t* wr = p.qw + static_cast<int64_t>(row) * p.nw;
-    for (int g = lane; g < p.ng; g += 64) {
-      const uint4 w4 = *reinterpret_cast<const uint4*>(wr + 4 * g);
-      const float s = T::load(p.qs, static_cast<int64_t>(row) * p.ng + g);
-      const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+  for (int it = 0; it < ITERS; ++it) {
+    gok[it] = it * 64 + lane < p.ng;
+    gidx[it] = gok[it] ? it * 64 + lane : p.ng - 1;
+  }
+  // branch-free loads: a set past the end reads valid addresses and is dropped at the store
+  uint4 wa[2][ITERS], wb[2][ITERS];
+  float sa[2][ITERS], sb[2][ITERS];
+  auto issue = [&](int set, uint4 (&wn)[2][ITERS], float (&sn)[2][ITERS]) {
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int row = min(set * 2 + r, p.N - 1);
+      const uint32_t* wr = p.qw + static_cast<int64_t>(row) * p.nw;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        wn[r][it] = *reinterpret_cast<const uint4*>(wr + 4 * gidx[it]);
+        sn[r][it] = T::load(p.qs, static_cast<int64_t>(row) * p.ng + gidx[it]);
+      }
+    }
+  };
+  int set_a = gw, set_b = gw + nwaves;
+  issue(set_a, wa, sa);
+  issue(set_b, wb, sb);
+  __syncthreads();
+
+  const float m = static_cast<float>(S::kMaxInt);
+  auto reduce = [&](int set, const uint4 (&wc)[2][ITERS], const float (&sc)[2][ITERS]) {
+    float acc[2][NB];
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) acc[r][b] = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      float s[2], ms[2];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        s[r] = gok[it] ? sc[r][it] : 0.0f;  // lanes past the last group add nothing
+        ms[r] = -m * s[r];
+      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
+        // the word's E values of x for every activation row, read once for both weight rows
+        float xf[BF ? 1 : NB][BF ? 1 : E];
+        uint32_t xp[BF ? NB : 1][BF ? E / 2 : 1];
+        const int k0 = gidx[it] * G + j * E;
 #pragma unroll
-        for (int i = 0; i < E; ++i) {
-          const float q = static_cast<float>((w[j] >> (i * BITS)) & S::kMask);
-          const float wv = T::rnd((q - m) * s);  // GroupQuantize._dequantize, in the model dtype
-          const int k = g * G + j * E + i;
+        for (int b = 0; b < NB; ++b) {
+          if constexpr (BF) {
 #pragma unroll
-          for (int b = 0; b < NB; ++b) acc[b] = fmaf(wv, xs[b * kpad + k], acc[b]);
+            for (int i = 0; i < E / 2; ++i) xp[b][i] = reinterpret_cast<const uint32_t*>(xh + b * kpad + k0)[i];
+          } else {
+#pragma unroll
+            for (int i = 0; i < E; ++i) xf[b][i] = xs[b * kpad + k0 + i];
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const uint32_t w = j == 0 ? wc[r][it].x : (j == 1 ? wc[r][it].y : (j == 2 ? wc[r][it].z : wc[r][it].w));
+          float q[E];
+#pragma unroll
+          for (int i = 0; i < E; ++i) q[i] = static_cast<float>((w >> (i * BITS)) & S::kMask);
+          if constexpr (BF) {
+#pragma unroll
+            for (int i = 0; i < E / 2; ++i) {
+              const float2_t pr = {fmaf(q[2 * i], s[r], ms[r]), fmaf(q[2 * i + 1], s[r], ms[r])};  // exact
+              const bf16x2_t wp = __builtin_convertvector(pr, bf16x2_t);                            // _dequantize's rounding
+#pragma unroll
+              for (int b = 0; b < NB; ++b)
+                acc[r][b] = __builtin_amdgcn_fdot2_f32_bf16(wp, __builtin_bit_cast(bf16x2_t, xp[b][i]), acc[r][b], false);
+            }
+          } else {
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+              const float wv = (q[i] - m) * s[r];  // one rounding, as _dequantize
+#pragma unroll
+              for (int b = 0; b < NB; ++b) acc[r][b] = fmaf(wv, xf[b][i], acc[r][b]);
+            }
+          }
         }
       }
     }
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      const float t = wave_sum(acc[b]);
-      if (lane == 0 && b < p.M) {
-        const float bias = p.bias != nullptr ? T::load(p.bias, row) : 0.0f;
-        store_out(p.y, static_cast<int64_t>(b) * p.N + row, t + bias, p.out_kind);
+    for (int r = 0; r < 2; ++r) {
+      const int row = set * 2 + r;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        const float t = wave_sum(acc[r][b]);
+        if (lane == 0 && b < p.M && row < p.N) {
+          const float bias = p.bias != nullptr ? T::load(p.bias, row) : 0.0f;
+          store_out(p.y, static_cast<int64_t>(b) * p.N + row, t + bias, p.out_kind);
+        }
       }
     }
+  };
+  while (set_a < nsets) {
+    reduce(set_a, wa, sa);
+    set_a += 2 * nwaves;
+    issue(set_a, wa, sa);
+    reduce(set_b, wb, sb);  // past the end: rows >= N, nothing is stored
+    set_b += 2 * nwaves;
+    issue(set_b, wb, sb);
   }
 }
 
@@ -221,26 +309,45 @@ __global__ __launch_bounds__(256) void gemm_dt_kernel(const LinParams p) {
 template <int BITS, int DT>
 hipError_t launch_dt(const LinParams& p, hipStream_t s) {
   constexpr int G = 4 * Scheme<BITS>::kElem;
-  if (p.M <= 8) {
-    const int nb = p.M <= 1 ? 1 : (p.M <= 2 ? 2 : (p.M <= 4 ? 4 : 8));
-    const size_t lds = static_cast<size_t>(nb) * p.ng * G * sizeof(float);
+  const int iters = (p.ng + 63) / 64;
+  if (p.M <= 8 && iters <= 4) {
+    // at most 4 activation rows per pass (more rows cost more registers and LDS reads than a second
+    // pass over the weights: measured 5..8 rows as two passes of 4)
+    const int per_pass = p.M <= 4 ? p.M : (p.M + 1) / 2;
+    const int nb = per_pass <= 1 ? 1 : (per_pass <= 2 ? 2 : 4);
+    const size_t lds = static_cast<size_t>(nb) * p.ng * G * (DT == MODEL_BF16 ? 2 : 4);
     if (lds <= 150 * 1024) {
-      // a few waves per SIMD, each walking its share of the rows
-      int blocks = (p.N + 3) / 4;
-      if (blocks > 1024) blocks = 1024;
-      auto go = [&](auto kern) -> hipError_t {
-        if (lds > 65536) {
-          const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-          if (e != hipSuccess) return e;
-        }
-        hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, s, p);
-        return hipGetLastError();
-      };
-      if (nb == 1) return go(gemv_dt_kernel<BITS, DT, 1>);
-      if (nb == 2) return go(gemv_dt_kernel<BITS, DT, 2>);
-      if (nb == 4) return go(gemv_dt_kernel<BITS, DT, 4>);
-      return go(gemv_dt_kernel<BITS, DT, 8>);
+      const int nsets = (p.N + 1) / 2;
+      int waves = nsets / 2;  // about two sets per wave, a few waves per SIMD
+      waves = waves < 4 ? 4 : (waves > 2048 ? 2048 : waves);
+      const int blocks = (waves + 3) / 4;
+      const size_t x_el = DT == MODEL_BF16 ? 2 : 4, y_el = p.out_kind == MODEL_BF16 ? 2 : 4;
+      for (int m0 = 0; m0 < p.M; m0 += per_pass) {
+        LinParams q = p;
+        q.x = static_cast<const char*>(p.x) + static_cast<size_t>(m0) * p.K * x_el;
+        q.y = static_cast<char*>(p.y) + static_cast<size_t>(m0) * p.N * y_el;
+        q.M = p.M - m0 < per_pass ? p.M - m0 : per_pass;
+        auto go = [&](auto kern) -> hipError_t {
+          if (lds > 65536) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            if (e != hipSuccess) return e;
+          }
+          hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds, s, q, nsets);
+          return hipGetLastError();
+        };
+        auto by_iters = [&](auto nbc) -> hipError_t {
+          constexpr int NBC = decltype(nbc)::value;
+          if (iters == 1) return go(gemv_dt_kernel<BITS, DT, NBC, 1>);
+          if (iters == 2) return go(gemv_dt_kernel<BITS, DT, NBC, 2>);
+          return go(gemv_dt_kernel<BITS, DT, NBC, 4>);
+        };
+        const hipError_t e = nb == 1 ? by_iters(std::integral_constant<int, 1>{})
+                                     : (nb == 2 ? by_iters(std::integral_constant<int, 2>{})
+                                                : by_iters(std::integral_constant<int, 4>{}));
+        if (e != hipSuccess) return e;
+      }
+      return hipSuccess;
     }
   }
   constexpr size_t lds = size_t(2) * 256 * (G + 1) * sizeof(float);

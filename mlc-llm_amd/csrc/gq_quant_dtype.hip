@@ -24,6 +24,32 @@ struct ModelT<MODEL_F32> {
   static __device__ __forceinline__ void save(void* p, int64_t i, float v) { static_cast<float*>(p)[i] = v; }
   static __device__ __forceinline__ float rnd(float v) { return v; }
   static constexpr float kLowest = -3.402823466e+38f;  // min_value(float32), the pad of the group maximum
+  // E consecutive values at an even element index (a multiple of 8 when E == 8)
+  template <int E>
+  static __device__ __forceinline__ void load_word(const void* p, int64_t i, float (&v)[E]) {
+    const float* f = static_cast<const float*>(p) + i;
+    if constexpr (E == 8) {
+      const float4 a = *reinterpret_cast<const float4*>(f), b = *reinterpret_cast<const float4*>(f + 4);
+      v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < E / 2; ++j) {
+        const float2 a = *reinterpret_cast<const float2*>(f + 2 * j);
+        v[2 * j] = a.x; v[2 * j + 1] = a.y;
+      }
+    }
+  }
+  template <int E>
+  static __device__ __forceinline__ void save_word(void* p, int64_t i, const float (&v)[E]) {
+    float* f = static_cast<float*>(p) + i;
+    if constexpr (E == 8) {
+      *reinterpret_cast<float4*>(f) = make_float4(v[0], v[1], v[2], v[3]);
+      *reinterpret_cast<float4*>(f + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < E / 2; ++j) *reinterpret_cast<float2*>(f + 2 * j) = make_float2(v[2 * j], v[2 * j + 1]);
+    }
+  }
 };
 
 template <>
@@ -42,6 +68,36 @@ struct ModelT<MODEL_BF16> {
     return __builtin_bit_cast(float, static_cast<uint32_t>(bits(v)) << 16);
   }
   static constexpr float kLowest = -3.38953139e+38f;  // min_value(bfloat16)
+  template <int E>
+  static __device__ __forceinline__ void load_word(const void* p, int64_t i, float (&v)[E]) {
+    const uint16_t* h = static_cast<const uint16_t*>(p) + i;
+    uint32_t pr[E / 2];
+    if constexpr (E == 8) {
+      const uint4 a = *reinterpret_cast<const uint4*>(h);
+      pr[0] = a.x; pr[1] = a.y; pr[2] = a.z; pr[3] = a.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < E / 2; ++j) pr[j] = reinterpret_cast<const uint32_t*>(h)[j];
+    }
+#pragma unroll
+    for (int j = 0; j < E / 2; ++j) {
+      v[2 * j] = __builtin_bit_cast(float, pr[j] << 16);
+      v[2 * j + 1] = __builtin_bit_cast(float, pr[j] & 0xffff0000u);
+    }
+  }
+  template <int E>
+  static __device__ __forceinline__ void save_word(void* p, int64_t i, const float (&v)[E]) {
+    uint16_t* h = static_cast<uint16_t*>(p) + i;
+    uint32_t pr[E / 2];
+#pragma unroll
+    for (int j = 0; j < E / 2; ++j) pr[j] = static_cast<uint32_t>(bits(v[2 * j])) | (static_cast<uint32_t>(bits(v[2 * j + 1])) << 16);
+    if constexpr (E == 8) {
+      *reinterpret_cast<uint4*>(h) = make_uint4(pr[0], pr[1], pr[2], pr[3]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < E / 2; ++j) reinterpret_cast<uint32_t*>(h)[j] = pr[j];
+    }
+  }
 };
 
 // One thread per storage word, a lane quad per group (the layout of gq_quant.hip).
@@ -62,10 +118,20 @@ __global__ __launch_bounds__(256) void quantize_dt_kernel(const void* __restrict
   float v[E];
   bool ok[E];
   float amax = T::kLowest;  // lanes beyond K contribute the type's lowest value, as the reference pads
+  if (k0 + E <= K && (K & 7) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+    // whole word inside the row and rows 16-byte aligned: 8-byte (q3) or 16-byte (q4) loads
+    T::template load_word<E>(w, row * K + k0, v);
+#pragma unroll
+    for (int i = 0; i < E; ++i) ok[i] = true;
+  } else {
+#pragma unroll
+    for (int i = 0; i < E; ++i) {
+      ok[i] = (k0 + i) < K;
+      v[i] = ok[i] ? T::load(w, row * K + k0 + i) : 0.0f;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < E; ++i) {
-    ok[i] = (k0 + i) < K;
-    v[i] = ok[i] ? T::load(w, row * K + k0 + i) : 0.0f;
     const float a = fabsf(v[i]);
     amax = (ok[i] && a > amax) ? a : amax;
   }
@@ -113,11 +179,18 @@ __global__ __launch_bounds__(256) void dequantize_dt_kernel(const int32_t* __res
   if (k0 >= K) return;
   const uint32_t word = qw[row * nw + wd];
   const float s = T::load(qs, row * ng + (wd >> 2));
+  float o[E];
 #pragma unroll
   for (int i = 0; i < E; ++i) {
     const int u = static_cast<int>((word >> (i * BITS)) & S::kMask);
-    // (u - m) is exact in either type; one multiply, one rounding
-    if (k0 + i < K) T::save(out, orow * K + k0 + i, static_cast<float>(u - S::kMaxInt) * s);
+    o[i] = static_cast<float>(u - S::kMaxInt) * s;  // (u - m) is exact in either type; one multiply, rounded at the store
+  }
+  if (k0 + E <= K && (K & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+    T::template save_word<E>(out, orow * K + k0, o);
+  } else {
+#pragma unroll
+    for (int i = 0; i < E; ++i)
+      if (k0 + i < K) T::save(out, orow * K + k0 + i, o[i]);
   }
 }
 

@@ -210,6 +210,44 @@ void Dequantize(TensorView q_weight, TensorView q_scale, int64_t bits, int64_t g
         "mlc.gq.dequantize");
 }
 
+// the same four for the other model dtypes: model_dtype is MI355GQ_F16 / MI355GQ_F32 / MI355GQ_BF16
+void QuantizeDt(TensorView w, int64_t bits, int64_t group_size, int64_t round_mode, int64_t model_dtype,
+                TensorView q_weight, TensorView q_scale) {
+  const int64_t K = w.shape()[w.ndim() - 1];
+  Check(mi355gq_quantize_dt(Ptr(w), Rows(w), K, static_cast<int>(bits), static_cast<int>(group_size),
+                            static_cast<int>(round_mode), static_cast<int>(model_dtype), Ptr(q_weight),
+                            Ptr(q_scale), StreamOf(w)),
+        "mlc.gq.quantize_dt");
+}
+
+void DequantizeDt(TensorView q_weight, TensorView q_scale, int64_t bits, int64_t group_size, int64_t model_dtype,
+                  TensorView out) {
+  const int64_t K = out.shape()[out.ndim() - 1];
+  Check(mi355gq_dequantize_dt(Ptr(q_weight), Ptr(q_scale), Rows(out), K, static_cast<int>(bits),
+                              static_cast<int>(group_size), static_cast<int>(model_dtype), Ptr(out),
+                              StreamOf(out)),
+        "mlc.gq.dequantize_dt");
+}
+
+void EmbeddingTakeDt(TensorView ids, TensorView q_weight, TensorView q_scale, int64_t bits, int64_t group_size,
+                     int64_t model_dtype, TensorView out) {
+  const int64_t K = out.shape()[out.ndim() - 1];
+  Check(mi355gq_embedding_take_dt(Ptr(ids), Rows(out), Ptr(q_weight), Ptr(q_scale), q_weight.shape()[0], K,
+                                  static_cast<int>(bits), static_cast<int>(group_size),
+                                  static_cast<int>(model_dtype), Ptr(out), StreamOf(out)),
+        "mlc.gq.embedding_take_dt");
+}
+
+void LinearDt(TensorView x, TensorView q_weight, TensorView q_scale, Optional<TensorView> bias, int64_t bits,
+              int64_t group_size, int64_t model_dtype, TensorView y) {
+  const int64_t K = x.shape()[x.ndim() - 1], N = q_weight.shape()[0];
+  const int out_dtype = y.dtype().bits == 32 ? MI355GQ_F32 : static_cast<int>(model_dtype);
+  Check(mi355gq_linear_dt(Ptr(x), Ptr(q_weight), Ptr(q_scale), bias.has_value() ? Ptr(bias.value()) : nullptr,
+                          Rows(x), N, K, static_cast<int>(bits), static_cast<int>(group_size),
+                          static_cast<int>(model_dtype), out_dtype, Ptr(y), StreamOf(x)),
+        "mlc.gq.linear_dt");
+}
+
 TVM_FFI_STATIC_INIT_BLOCK() {
   namespace refl = tvm::ffi::reflection;
   refl::GlobalDef()
@@ -227,7 +265,11 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.moe_route", MoeRoute)
       .def("mlc.gq.moe_combine_sorted", MoeCombineSorted)
       .def("mlc.gq.quantize", Quantize)
-      .def("mlc.gq.dequantize", Dequantize);
+      .def("mlc.gq.dequantize", Dequantize)
+      .def("mlc.gq.quantize_dt", QuantizeDt)
+      .def("mlc.gq.dequantize_dt", DequantizeDt)
+      .def("mlc.gq.embedding_take_dt", EmbeddingTakeDt)
+      .def("mlc.gq.linear_dt", LinearDt);
 }
 
 }  // namespace gq
