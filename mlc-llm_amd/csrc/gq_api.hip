@@ -431,6 +431,21 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
                                          : aligned2(x) && aligned2(q_scale) && aligned2(bias)) &&
                  (out_dtype == MI355GQ_F32 ? aligned4(y) : aligned2(y)),
              "linear_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
+  if (model_dtype == MI355GQ_BF16 && M > 2 && (K & 7) == 0 && aligned16(x)) {
+    // the float16 GEMM's tiles on the bf16 matrix instruction (from 3 rows on it already beats the GEMV)
+    gq::GemmArgs g{};
+    g.x = static_cast<const uint16_t*>(x);
+    g.q_weight = static_cast<const uint32_t*>(q_weight);
+    g.q_scale = static_cast<const uint16_t*>(q_scale);
+    g.bias = static_cast<const uint16_t*>(bias);
+    g.y = y;
+    g.indptr = nullptr; g.indptr_i64 = 0;
+    g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
+    g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
+    g.bf16 = 1;
+    const hipError_t e = gq::launch_gemm(g, as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemm launch");
+  }
   return hip_result(gq::launch_linear_dt(x, static_cast<const uint32_t*>(q_weight), q_scale, bias, M, N, K, bits,
                                          group_size, model_dtype, out_dtype, y, as_stream(stream)),
                     "linear_dt launch");

@@ -215,8 +215,13 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   p.bm_hint = 0;
   p.paired = a.paired;
   p.x_rows = a.x_rows; p.x_src_rows = static_cast<int>(a.x_src_rows);
+  p.bf16 = a.bf16;
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int variant = options().gemm_variant;
+  if (a.bf16) {  // bfloat16 models run the pipelined kernel's regular tiles or nothing
+    const hipError_t e = launch_gemm_pipe(p, a.bits, s);
+    return e;
+  }
   if (variant < 0) {
     const SplitPlan plan = plan_split_k(a.rows, a.N, a.K, a.bits, a.group_size, a.indptr != nullptr);
     p.bm_hint = plan.bm;

@@ -42,6 +42,7 @@ struct GemmParams {
   int paired;
   const int32_t* x_rows;  // null, or the row of x each activation row reads (int32 [rows])
   int x_src_rows;         // rows of x when x_rows is set
+  int bf16;               // x, q_scale, bias and a 16-bit y are bfloat16 (q4bf16_* models), not float16
 };
 
 // column c of the block-interleaved order above -> stored weight row (clamped into its half).
@@ -120,6 +121,49 @@ __device__ __forceinline__ void dequant_word4(const uint32_t w, const uint16_t s
     const uint32_t r = and_or(__builtin_amdgcn_perm(t1, w, sel), 0x000f000fu, kMagic);
     out[j] = as_u32((as_half2(r) + off) * s2);
   }
+}
+
+// bfloat16 models (q4bf16_*): the same, with the product (q - m) * s formed exactly in float32
+// (a 4-bit by an 8-bit significand) and rounded to a bf16 pair by v_cvt_pk_bf16_f32, which is the
+// rounding GroupQuantize._dequantize applies in that dtype.  scale_bits are bfloat16 bits.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t bf16_pair(float a, float b) {
+  const float2_t f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+__device__ __forceinline__ uint16_t bf16_bits_of(float v) {
+  return static_cast<uint16_t>(bf16_pair(v, 0.0f) & 0xffffu);
+}
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) {
+  return __builtin_bit_cast(float, static_cast<uint32_t>(b) << 16);
+}
+__device__ __forceinline__ void dequant_word4_bf16(const uint32_t w, const uint16_t scale_bits,
+                                                   uint32_t* __restrict__ out) {
+  const float s = bf16_to_f32(scale_bits), ms = -7.0f * s;
+  const uint32_t t0 = w & 0x0f0f0f0fu, t1 = (w >> 4) & 0x0f0f0f0fu;  // even / odd fields, one per byte
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float lo = static_cast<float>((t0 >> (8 * j)) & 0xffu), hi = static_cast<float>((t1 >> (8 * j)) & 0xffu);
+    out[j] = bf16_pair(fmaf(lo, s, ms), fmaf(hi, s, ms));
+  }
+}
+template <int BITS>
+__device__ __forceinline__ void dequant_group_bf16(const uint4 w4, const uint16_t scale_bits,
+                                                   uint32_t* __restrict__ out /* G/2 bf16 pairs */) {
+  using S = Scheme<BITS>;
+  constexpr int E = S::kElem;
+  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+  const float s = bf16_to_f32(scale_bits), ms = -static_cast<float>(S::kMaxInt) * s;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < E / 2; ++j) {
+      const float lo = static_cast<float>((w[i] >> (2 * j * BITS)) & S::kMask);
+      const float hi = static_cast<float>((w[i] >> ((2 * j + 1) * BITS)) & S::kMask);
+      out[(E / 2) * i + j] = bf16_pair(fmaf(lo, s, ms), fmaf(hi, s, ms));
+    }
 }
 
 // Which activation rows [seg_lo, seg_hi) and which expert the m-tile `t` of a launch belongs to.

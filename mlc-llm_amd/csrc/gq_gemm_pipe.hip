@@ -14,7 +14,8 @@ namespace gq {
 
 // DEPTH: K tiles of global loads in flight (register stages); even, 2 for the large tiles, more
 // for few-row tiles whose MFMA work per tile is far shorter than a trip to memory
-template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2>
+// BF: bfloat16 model (operands and 16-bit outputs are bf16; see dequant_word4_bf16)
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(const GemmParams p) {
   using T = GemmTraits<BITS>;
   constexpr int G = T::G;
@@ -135,11 +136,13 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
         // word `part` of the group -> 8 halves = one 16-byte chunk
         const uint32_t w4[4] = {st.w[i].x, st.w[i].y, st.w[i].z, st.w[i].w};
         uint32_t d[4];
-        dequant_word4(w4[part], sb, d);
+        if constexpr (BF) dequant_word4_bf16(w4[part], sb, d);
+        else dequant_word4(w4[part], sb, d);
         dst[part] = make_uint4(d[0], d[1], d[2], d[3]);
       } else if (part == 0) {
         uint32_t d[G / 2];
-        dequant_group<BITS>(st.w[i], sb, d);
+        if constexpr (BF) dequant_group_bf16<BITS>(st.w[i], sb, d);
+        else dequant_group<BITS>(st.w[i], sb, d);
 #pragma unroll
         for (int c = 0; c < G / 8; ++c) dst[c] = make_uint4(d[4 * c], d[4 * c + 1], d[4 * c + 2], d[4 * c + 3]);
       }
@@ -184,7 +187,12 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
         for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+            if constexpr (BF)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[cur][i]),
+                                                                  __builtin_bit_cast(bf16x8_t, bf[cur][j]), acc[i][j],
+                                                                  0, 0, 0);
+            else
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
         store_part(kt_store, st_store, s ^ 1, ks);
         __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
       }
@@ -266,23 +274,26 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     if (p.out_f32)
       for_each([&](int row, int col, float v) { static_cast<float*>(p.y)[static_cast<int64_t>(row) * p.N + col] = v; });
     else
-      for_each([&](int row, int col, float v) { static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * p.N + col] = f2h(v); });
+      for_each([&](int row, int col, float v) {
+        static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * p.N + col] = BF ? bf16_bits_of(v) : f2h(v);
+      });
   } else {
     for_each([&](int row, int col, float v) {
       const int64_t o = static_cast<int64_t>(row) * p.N + col;
-      const float t = v + (p.bias != nullptr ? h2f(p.bias[col]) : 0.f) + (p.residual != nullptr ? h2f(p.residual[o]) : 0.f);
+      const float t = v + (p.bias != nullptr ? (BF ? bf16_to_f32(p.bias[col]) : h2f(p.bias[col])) : 0.f) +
+                      (p.residual != nullptr ? (BF ? bf16_to_f32(p.residual[o]) : h2f(p.residual[o])) : 0.f);
       if (p.out_f32) static_cast<float*>(p.y)[o] = t;
-      else static_cast<uint16_t*>(p.y)[o] = f2h(t);
+      else static_cast<uint16_t*>(p.y)[o] = BF ? bf16_bits_of(t) : f2h(t);
     });
   }
 }
 
-template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2>
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false>
 static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr int BK = 2 * GemmTraits<BITS>::G;
   constexpr int LDA = BK + 8;
   constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
-  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH>;
+  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH, BF>;
   if (lds > 65536) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                              hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -403,6 +414,19 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   if ((p.K & 7) != 0 || p.ng == 0) return hipErrorNotSupported;
   const int variant = options().gemm_variant;
   if (p.paired && (p.N & 1)) return hipErrorNotSupported;
+  if (p.bf16) {
+    // bfloat16 models: plain linear only, the three regular tiles (no split K, no folded activation)
+    if (p.paired || p.partial != nullptr || p.indptr != nullptr) return hipErrorNotSupported;
+    const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
+    const int64_t mid_tiles = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
+    if (bits == 4) {
+      if (big_tiles >= 160) return launch_pipe_cfg<4, 256, 256, 128, 64, 2, true>(p, s);
+      if (mid_tiles >= 192) return launch_pipe_cfg<4, 128, 256, 64, 64, 2, true>(p, s);
+      return launch_pipe_cfg<4, 128, 128, 64, 64, 2, true>(p, s);
+    }
+    if (mid_tiles >= 192) return launch_pipe_cfg<3, 128, 256, 64, 64, 2, true>(p, s);
+    return launch_pipe_cfg<3, 128, 128, 64, 64, 2, true>(p, s);
+  }
   if (p.bm_hint > 0 && variant < 0) {
     if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4>(p, s);
     if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4>(p, s);

@@ -50,6 +50,7 @@ struct GemmArgs {
   int paired = 0;                  // fused gate/up form: y is [rows, N / 2] fp16; N even, no bias / residual
   const int32_t* x_rows = nullptr; // the MoE gather folded in: activation row r reads x[x_rows[r]] (x has x_src_rows rows)
   int64_t x_src_rows = 0;
+  int bf16 = 0;                    // bfloat16 model: x, q_scale, bias and a 16-bit y are bf16 (plain linear only)
 };
 hipError_t launch_gemm(const GemmArgs& a, hipStream_t s);
 // scratch the split-K form of the GEMM wants for this shape (0 when it does not split)
