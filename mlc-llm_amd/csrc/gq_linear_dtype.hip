@@ -153,8 +153,18 @@ __global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nse
         for (int r = 0; r < 2; ++r) {
           const uint32_t w = j == 0 ? wc[r][it].x : (j == 1 ? wc[r][it].y : (j == 2 ? wc[r][it].z : wc[r][it].w));
           float q[E];
+          if constexpr (BITS == 4) {
+            // even / odd fields spread one per byte: each conversion is then a single v_cvt_f32_ubyteN
+            const uint32_t t0 = w & 0x0f0f0f0fu, t1 = (w >> 4) & 0x0f0f0f0fu;
 #pragma unroll
-          for (int i = 0; i < E; ++i) q[i] = static_cast<float>((w >> (i * BITS)) & S::kMask);
+            for (int i = 0; i < 4; ++i) {
+              q[2 * i] = static_cast<float>((t0 >> (8 * i)) & 0xffu);
+              q[2 * i + 1] = static_cast<float>((t1 >> (8 * i)) & 0xffu);
+            }
+          } else {
+#pragma unroll
+            for (int i = 0; i < E; ++i) q[i] = static_cast<float>((w >> (i * BITS)) & S::kMask);
+          }
           if constexpr (BF) {
 #pragma unroll
             for (int i = 0; i < E / 2; ++i) {
