@@ -380,6 +380,34 @@ def main() -> int:
         pk["embedding_take_8192_tokens"] = {"us": round(ms * 1e3, 1), "GB/s": round(8192 * row_bytes / ms / 1e6, 1)}
         extra["packing"] = pk
 
+        # the other model dtypes of the registry (q4bf16_1, q4f32_1) on the gate_up shape: packing,
+        # batch-1 GEMV (weight bytes per second) and the M = 2048 GEMM
+        other = {}
+        n, k = SHAPES["gate_up"]
+        for label, dt in (("q4bf16_1", torch.bfloat16), ("q4f32_1", torch.float32)):
+            wd = (torch.randn((n, k), generator=gx, device=dev) * 0.02).to(dt)
+            qwd, qsd = ops.quantize(wd, 4, 32)
+            el = wd.element_size()
+            nbytes = wd.numel() * el + qwd.numel() * 4 + qsd.numel() * el
+            res = {}
+            ms = timed(lambda: ops.quantize(wd, 4, 32), 5, 2, False)
+            res["quantize"] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
+            ms = timed(lambda: ops.dequantize(qwd, qsd, k, 4, 32), 5, 2, False)
+            res["dequantize"] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
+            del wd
+            x1 = torch.randn((1, k), generator=gx, device=dev).to(dt)
+            ms = timed(lambda: ops.linear(x1, qwd, qsd, 4, 32), 10, 2, False)
+            res["gemv_b1"] = {"us": round(ms * 1e3, 1),
+                              "GB/s": round((qwd.numel() * 4 + qsd.numel() * el + (k + n) * el) / ms / 1e6, 1)}
+            xm_ = torch.randn((2048, k), generator=gx, device=dev).to(dt)
+            ms = timed(lambda: ops.linear(xm_, qwd, qsd, 4, 32), 3, 1, False)
+            res["gemm_m2048"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(2.0 * 2048 * n * k / ms / 1e9, 1),
+                                 "matrix_instruction": "v_mfma_f32_32x32x16_bf16" if dt == torch.bfloat16
+                                 else "v_mfma_f32_32x32x2_f32 (157 TFLOP/s peak)"}
+            other[label] = res
+            del qwd, qsd, x1, xm_
+        extra["other_model_dtypes"] = other
+
     # ---------------------------------------------------------------- CPU baseline (bounded sample)
     cpu = None
     if not args.skip_cpu:

@@ -431,8 +431,8 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
                                          : aligned2(x) && aligned2(q_scale) && aligned2(bias)) &&
                  (out_dtype == MI355GQ_F32 ? aligned4(y) : aligned2(y)),
              "linear_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
-  if (model_dtype == MI355GQ_BF16 && M > 2 && (K & 7) == 0 && aligned16(x)) {
-    // the float16 GEMM's tiles on the bf16 matrix instruction (from 3 rows on it already beats the GEMV)
+  if (model_dtype == MI355GQ_BF16 && M > 1 && (K & 7) == 0 && aligned16(x)) {
+    // the float16 GEMM's tiles on the bf16 matrix instruction (from 2 rows on it already beats the GEMV)
     gq::GemmArgs g{};
     g.x = static_cast<const uint16_t*>(x);
     g.q_weight = static_cast<const uint32_t*>(q_weight);

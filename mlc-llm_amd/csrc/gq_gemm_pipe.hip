@@ -420,6 +420,9 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
     const int64_t mid_tiles = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
     if (bits == 4) {
+      // few rows: tile height follows the rows (the float16 path's few-row tiles, unsplit)
+      if (p.rows <= 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4, true>(p, s);
+      if (p.rows <= 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4, true>(p, s);
       if (big_tiles >= 160) return launch_pipe_cfg<4, 256, 256, 128, 64, 2, true>(p, s);
       if (mid_tiles >= 192) return launch_pipe_cfg<4, 128, 256, 64, 64, 2, true>(p, s);
       return launch_pipe_cfg<4, 128, 128, 64, 64, 2, true>(p, s);

@@ -140,10 +140,24 @@ __global__ __launch_bounds__(256) void quantize_dt_kernel(const void* __restrict
 
   const float m = static_cast<float>(S::kMaxInt);
   const float s = T::rnd(amax / m);
+  // bfloat16: the quotient only has to round to the right bf16, and a ratio of two 8-bit significands
+  // that is not itself a bf16 rounding boundary stays 2^-17 (relative) away from one, so the hardware
+  // reciprocal with one Newton step (about 1 ulp of float32) rounds like the exact quotient; scales
+  // of zero, infinity or NaN keep the first product (NaN / infinity / zero, as a divide gives).
+  // float32 needs the correctly rounded divide itself.
+  const float rs = __builtin_amdgcn_rcpf(s);
+  const bool plain = !(s > 0.0f && s < __builtin_inff());
   uint32_t word = 0;
 #pragma unroll
   for (int i = 0; i < E; ++i) {
-    float t = T::rnd(v[i] / s);  // IEEE divide (0 / 0 = NaN for an all-zero group)
+    float quo;
+    if constexpr (DT == MODEL_BF16) {
+      const float q0 = v[i] * rs;
+      quo = plain ? q0 : fmaf(fmaf(-q0, s, v[i]), rs, q0);
+    } else {
+      quo = v[i] / s;  // IEEE divide (0 / 0 = NaN for an all-zero group)
+    }
+    float t = T::rnd(quo);
     t = T::rnd(t + m);
     float r = HALF_EVEN ? rintf(t) : roundf(t);
     r = (r > 0.0f) ? r : 0.0f;  // compare-and-select max: NaN becomes 0
