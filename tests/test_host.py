@@ -71,6 +71,42 @@ def test_argument_validation_never_launches():
     assert ei.value.code == -1 and "bogus" in str(ei.value)
 
 
+def test_argument_validation_of_the_later_entry_points():
+    lib = _lib.lib()
+    P = ctypes.c_void_p
+    # folded activation: odd N is an argument error; empty problems succeed
+    assert lib.mi355gq_linear_silu_mul(P(0x1000), P(0x2000), P(0x3000), 2, 63, 64, 4, 32, P(0x4000), None, 0, None) == -1
+    assert "even" in _err()
+    assert lib.mi355gq_linear_silu_mul(None, None, None, 0, 64, 64, 4, 32, None, None, 0, None) == 0
+    assert lib.mi355gq_linear_silu_mul_workspace_bytes(4, 28672, 4096, 4, 32) == 0
+    assert lib.mi355gq_moe_gemv_silu_mul(P(0x1000), 1, P(0x2000), P(0x3000), P(0x4000), 2, 8, 15, 64, 4, 32, P(0x5000), None) == -1
+    # routing: limits of the single-workgroup form are a missing kernel, bad sizes an argument error
+    assert lib.mi355gq_moe_route(P(0x1000), 9000, 8, 2, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
+                                 P(0x7000), 0, None) == -3
+    assert "four" in _err() or "gating_softmax_topk" in _err()
+    assert lib.mi355gq_moe_route(P(0x1000), 16, 100, 2, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
+                                 P(0x7000), 0, None) == -3
+    assert lib.mi355gq_moe_route(P(0x1000), 16, 8, 9, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
+                                 P(0x7000), 0, None) == -1
+    assert lib.mi355gq_moe_route(P(0x1000), 16, 8, 2, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
+                                 None, 0, None) == -1
+    assert lib.mi355gq_moe_experts(P(0x1000), 4, None, 5, P(0x2000), P(0x3000), P(0x4000), 0, 8, 16, 64, 4, 32, 0,
+                                   P(0x5000), None) == -1  # x rows must equal rows without an index
+    assert lib.mi355gq_moe_experts(P(0x1000), 4, None, 4, P(0x2000), P(0x3000), P(0x4000), 0, 8, 16, 64, 4, 32, 7,
+                                   P(0x5000), None) == -1  # unknown epilogue
+    assert lib.mi355gq_moe_combine_sorted(P(0x1000), None, P(0x2000), 4, 2, 64, P(0x3000), None) == -1
+    # model dtypes: unknown code, out dtype that is neither the model's nor float32, K = 0
+    assert lib.mi355gq_quantize_dt(P(0x1000), 4, 32, 4, 32, 0, 5, P(0x2000), P(0x3000), None) == -1
+    assert "model_dtype" in _err()
+    assert lib.mi355gq_dequantize_dt(P(0x1000), P(0x2000), 4, 32, 4, 32, 3, P(0x3000), None) == -1
+    assert lib.mi355gq_linear_dt(P(0x1000), P(0x2000), P(0x3000), None, 2, 8, 64, 4, 32, 2, 0, P(0x4000), None) == -1
+    assert "out_dtype" in _err()
+    assert lib.mi355gq_linear_dt(P(0x1000), P(0x2000), P(0x3000), None, 2, 8, 0, 4, 32, 1, 1, P(0x4000), None) == -1
+    assert lib.mi355gq_linear_dt(P(0x1002), P(0x2000), P(0x3000), None, 2, 8, 64, 4, 32, 1, 1, P(0x4000), None) == -1
+    assert lib.mi355gq_quantize_dt(None, 0, 32, 4, 32, 0, 2, None, None, None) == 0
+    assert lib.mi355gq_embedding_take_dt(None, 0, None, None, 10, 32, 4, 32, 1, None, None) == 0
+
+
 def test_ops_refuse_cpu_tensors():
     x = torch.zeros(1, 32, dtype=torch.float16)
     qw = torch.zeros(8, 4, dtype=torch.int32)
