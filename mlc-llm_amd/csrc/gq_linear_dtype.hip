@@ -70,6 +70,11 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 //  * bfloat16: (q - m) * s is exact in float32 (4 x 8 significant bits), v_cvt_pk_bf16_f32 rounds
 //    two of them to the bf16 pair _dequantize would hold, and v_dot2_f32_bf16 multiplies the pair
 //    with the matching pair of x (exact products, fp32 accumulation).
+constexpr int gemv_dt_group_stride(int bits, int dt) {
+  // float32: 16 bytes of padding (strides of 144 / 176 bytes); bfloat16: 80 / 88 bytes
+  return dt == MODEL_F32 ? (bits == 4 ? 36 : 44) : (bits == 4 ? 40 : 44);
+}
+
 template <int BITS, int DT, int NB, int ITERS>
 __global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nsets) {
   using S = Scheme<BITS>;
@@ -80,12 +85,16 @@ __global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nse
   extern __shared__ uint32_t xs_raw[];
   float* xs = reinterpret_cast<float*>(xs_raw);         // float32: [NB][kpad]
   uint16_t* xh = reinterpret_cast<uint16_t*>(xs_raw);   // bfloat16: [NB][kpad]
-  const int kpad = p.ng * G;
-  for (int i = threadIdx.x; i < NB * kpad; i += 256) {
-    const int b = i / kpad, k = i - b * kpad;
+  // a group of x is padded to GS elements so that the lanes of a wave, one group apart each, read
+  // different LDS banks (unpadded, a group is 64 / 128 / 160 bytes and every lane lands on the same ones)
+  constexpr int GS = gemv_dt_group_stride(BITS, DT);
+  const int kpad = p.ng * GS;
+  for (int i = threadIdx.x; i < NB * p.ng * G; i += 256) {
+    const int b = i / (p.ng * G), k = i - b * (p.ng * G);
     const bool ok = b < p.M && k < p.K;
-    if (BF) xh[i] = ok ? static_cast<const uint16_t*>(p.x)[static_cast<int64_t>(b) * p.K + k] : uint16_t(0);
-    else xs[i] = ok ? static_cast<const float*>(p.x)[static_cast<int64_t>(b) * p.K + k] : 0.0f;
+    const int at = b * kpad + (k / G) * GS + k % G;
+    if (BF) xh[at] = ok ? static_cast<const uint16_t*>(p.x)[static_cast<int64_t>(b) * p.K + k] : uint16_t(0);
+    else xs[at] = ok ? static_cast<const float*>(p.x)[static_cast<int64_t>(b) * p.K + k] : 0.0f;
   }
 
   const int lane = threadIdx.x & 63;
@@ -138,15 +147,28 @@ __global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nse
         // the word's E values of x for every activation row, read once for both weight rows
         float xf[BF ? 1 : NB][BF ? 1 : E];
         uint32_t xp[BF ? NB : 1][BF ? E / 2 : 1];
-        const int k0 = gidx[it] * G + j * E;
+        const int k0 = gidx[it] * GS + j * E;
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
           if constexpr (BF) {
+            if constexpr (E == 8) {  // 8 bf16 = one 16-byte read
+              const uint4 v4 = *reinterpret_cast<const uint4*>(xh + b * kpad + k0);
+              xp[b][0] = v4.x; xp[b][1] = v4.y; xp[b][2] = v4.z; xp[b][3] = v4.w;
+            } else {
 #pragma unroll
-            for (int i = 0; i < E / 2; ++i) xp[b][i] = reinterpret_cast<const uint32_t*>(xh + b * kpad + k0)[i];
-          } else {
+              for (int i = 0; i < E / 2; ++i) xp[b][i] = reinterpret_cast<const uint32_t*>(xh + b * kpad + k0)[i];
+            }
+          } else if constexpr (E == 8) {  // k0 is a multiple of 8 floats: two 16-byte reads
+            const float4 lo = *reinterpret_cast<const float4*>(xs + b * kpad + k0);
+            const float4 hi = *reinterpret_cast<const float4*>(xs + b * kpad + k0 + 4);
+            xf[b][0] = lo.x; xf[b][1] = lo.y; xf[b][2] = lo.z; xf[b][3] = lo.w;
+            xf[b][4] = hi.x; xf[b][5] = hi.y; xf[b][6] = hi.z; xf[b][7] = hi.w;
+          } else {                        // q3: k0 is a multiple of 10 floats: 8-byte reads
 #pragma unroll
-            for (int i = 0; i < E; ++i) xf[b][i] = xs[b * kpad + k0 + i];
+            for (int i = 0; i < E; i += 2) {
+              const float2 v2 = *reinterpret_cast<const float2*>(xs + b * kpad + k0 + i);
+              xf[b][i] = v2.x; xf[b][i + 1] = v2.y;
+            }
           }
         }
 #pragma unroll
@@ -241,12 +263,26 @@ __global__ __launch_bounds__(256) void gemm_dt_kernel(const LinParams p) {
   float areg[A_PER];
   uint32_t wreg[2];
   float sreg = 0.0f;
+  // rows of x that start 16-byte aligned (float32, K % 4 == 0) are read four values at a time
+  const bool a_vec = DT == MODEL_F32 && (p.K & 3) == 0 && (reinterpret_cast<uintptr_t>(p.x) & 15) == 0;
   auto load_tile = [&](int kt) {
     const int64_t row = m0 + ar;
+    if (a_vec) {
+      const int64_t rc = row < p.M ? row : p.M - 1;  // a valid row; its values are dropped below
 #pragma unroll
-    for (int i = 0; i < A_PER; ++i) {
-      const int k = kt * G + ak + i;
-      areg[i] = (row < p.M && k < p.K) ? T::load(p.x, row * p.K + k) : 0.0f;
+      for (int i = 0; i < A_PER; i += 4) {
+        const int k = kt * G + ak + i;  // a multiple of 4, so the four values are inside K together
+        const bool ok = row < p.M && k < p.K;
+        const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(p.x) + rc * p.K + (k < p.K ? k : 0));
+        areg[i] = ok ? v.x : 0.0f; areg[i + 1] = ok ? v.y : 0.0f;
+        areg[i + 2] = ok ? v.z : 0.0f; areg[i + 3] = ok ? v.w : 0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < A_PER; ++i) {
+        const int k = kt * G + ak + i;
+        areg[i] = (row < p.M && k < p.K) ? T::load(p.x, row * p.K + k) : 0.0f;
+      }
     }
     const uint32_t* wr = p.qw + static_cast<int64_t>(wrow) * p.nw + 4 * kt + 2 * whalf;
     wreg[0] = wr[0];
@@ -321,11 +357,14 @@ hipError_t launch_dt(const LinParams& p, hipStream_t s) {
   constexpr int G = 4 * Scheme<BITS>::kElem;
   const int iters = (p.ng + 63) / 64;
   if (p.M <= 8 && iters <= 4) {
-    // at most 4 activation rows per pass (more rows cost more registers and LDS reads than a second
-    // pass over the weights: measured 5..8 rows as two passes of 4)
-    const int per_pass = p.M <= 4 ? p.M : (p.M + 1) / 2;
+    // few activation rows per pass: the kernel's registers grow with rows x groups per lane (374 for
+    // four float32 rows at K = 4096, one wave per SIMD), so more rows run as more passes over the
+    // weights: measured faster from 3 rows (float32) / 5 rows (bfloat16) on
+    const int cap = DT == MODEL_F32 ? 2 : 4;
+    const int passes = (p.M + cap - 1) / cap;
+    const int per_pass = (p.M + passes - 1) / passes;
     const int nb = per_pass <= 1 ? 1 : (per_pass <= 2 ? 2 : 4);
-    const size_t lds = static_cast<size_t>(nb) * p.ng * G * (DT == MODEL_BF16 ? 2 : 4);
+    const size_t lds = static_cast<size_t>(nb) * p.ng * gemv_dt_group_stride(BITS, DT) * (DT == MODEL_BF16 ? 2 : 4);
     if (lds <= 150 * 1024) {
       const int nsets = (p.N + 1) / 2;
       int waves = nsets / 2;  // about two sets per wave, a few waves per SIMD
