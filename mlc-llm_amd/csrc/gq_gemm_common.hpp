@@ -107,6 +107,24 @@ __device__ __forceinline__ void dequant_group(const uint4 w4, const uint16_t sca
 }
 
 
+// 16-byte chunk c (0..4) of a q3 group: halves 8c .. 8c+7 = pairs 4c .. 4c+3 of the group, pair p being
+// fields (2j, 2j+1) of word p / 5 with j = p % 5 (a pair never straddles two words).
+__device__ __forceinline__ void dequant_chunk3(const uint4 w4, const uint16_t scale_bits, const int c,
+                                               uint32_t* __restrict__ out) {
+  constexpr uint32_t kMagic = 0x64006400u;
+  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+  const _Float16 s = __builtin_bit_cast(_Float16, scale_bits);
+  const half2_t s2 = {s, s};
+  const half2_t off = {static_cast<_Float16>(-1027.0f), static_cast<_Float16>(-1027.0f)};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int pr = 4 * c + i;
+    const uint32_t t = w[pr / 5] >> (6 * (pr % 5));
+    const uint32_t r = and_or(t << 13, 0x00070000u, and_or(t, 0x00000007u, kMagic));
+    out[i] = as_u32((as_half2(r) + off) * s2);
+  }
+}
+
 // One q4 storage word -> 8 halves in natural k order (4 half pairs), (q - 7) * s.
 __device__ __forceinline__ void dequant_word4(const uint32_t w, const uint16_t scale_bits,
                                               uint32_t* __restrict__ out) {

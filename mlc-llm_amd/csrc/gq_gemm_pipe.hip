@@ -139,10 +139,14 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
         if constexpr (BF) dequant_word4_bf16(w4[part], sb, d);
         else dequant_word4(w4[part], sb, d);
         dst[part] = make_uint4(d[0], d[1], d[2], d[3]);
+      } else if constexpr (!BF) {
+        // q3: 16-byte chunk `part` of the group (5 chunks, 5 k-steps)
+        uint32_t d[4];
+        dequant_chunk3(st.w[i], sb, part, d);
+        dst[part] = make_uint4(d[0], d[1], d[2], d[3]);
       } else if (part == 0) {
         uint32_t d[G / 2];
-        if constexpr (BF) dequant_group_bf16<BITS>(st.w[i], sb, d);
-        else dequant_group<BITS>(st.w[i], sb, d);
+        dequant_group_bf16<BITS>(st.w[i], sb, d);
 #pragma unroll
         for (int c = 0; c < G / 8; ++c) dst[c] = make_uint4(d[4 * c], d[4 * c + 1], d[4 * c + 2], d[4 * c + 3]);
       }
