@@ -5,6 +5,7 @@ tolerance quoted for this path against an fp32 (here float64-summed) dequantize-
     max|y - ref| <= 1e-2 * max|x| * sqrt(K) / 64   and   ||y - ref||_2 / ||ref||_2 <= 2e-3.
 """
 
+import os
 import zlib
 
 import numpy as np
@@ -1229,3 +1230,15 @@ def test_linear_and_moe_replay_in_hip_graph():
             assert torch.equal(a, b), f"graph replay {rep} differs from eager at M={m}"
         ref = o.linear_fp32(xs[-2].cpu().numpy(), qw, qs, s)
         assert_linear_ok(replayed[-2], ref, xs[-2].cpu().numpy(), k, f"replay {rep}, M=40")
+
+
+# ------------------------------------------------------------------ the C ABI from plain C
+
+def test_c_abi_from_plain_c():
+    # tests/c_abi/c_abi_check.c: no Python, no torch; quantize + linear in three regimes against the C oracle
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c_abi", "c_abi_check")
+    assert os.path.exists(exe), f"{exe} is missing: run __graft_entry__.build() (or make -C tests/c_abi)"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, f"exit {r.returncode}\n{r.stdout}\n{r.stderr}"
+    assert "c_abi_check ok" in r.stdout
