@@ -827,6 +827,23 @@ def test_packing_other_model_dtypes_bit_exact(model_dtype, bits_name, mode):
         assert np.array_equal(_carrier(emb), d_ref[[rows - 1, 0, 2, 2, rows - 1, 0]])
 
 
+@pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
+def test_other_model_dtypes_golden(golden, model_dtype):
+    dt = _TORCH_OF[model_dtype]
+    for shp in ("2x13", "16x128", "5x200"):
+        z = golden(f"dtype_{model_dtype}_{shp}")
+        k = z["w"].shape[1]
+        w = torch.from_numpy(z["w"]).to(dt).to(DEV)
+        for mode, key in ((0, "half_away"), (1, "half_even")):
+            qw, qs = ops.quantize(w, 4, 32, mode)
+            assert np.array_equal(host_u32(qw), z[f"q_weight_{key}"]) and np.array_equal(_carrier(qs), z[f"q_scale_{key}"])
+        qw, qs = dev(z["q_weight_half_away"]), torch.from_numpy(z["q_scale_half_away"]).to(dt).to(DEV)
+        assert np.array_equal(_carrier(ops.dequantize(qw, qs, k, 4, 32)), z["dequant"])
+        y = ops.linear(torch.from_numpy(z["x"]).to(dt).to(DEV), qw, qs, 4, 32, out_dtype=torch.float32)
+        err = np.linalg.norm(y.double().cpu().numpy() - z["y"]) / np.linalg.norm(z["y"])
+        assert err <= 2e-6, err
+
+
 def test_other_model_dtypes_modules():
     # registry entries: quantize_weight / dequantize_weight / embedding work; the matmul says what is missing
     for name in ("q4bf16_1", "q4f32_1", "q4bf16_0"):

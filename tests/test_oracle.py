@@ -337,6 +337,16 @@ def test_golden_fixtures_reproduce(golden):
             d = o.dequantize(z["q_weight_half_away"], z["q_scale_half_away"], s, k)
             assert (d.view(np.uint16) == z["dequant"].view(np.uint16)).all()
             assert np.array_equal(o.linear_fp32(z["x"], z["q_weight_half_away"], z["q_scale_half_away"], s), z["y"])
+        elif name.startswith("dtype_"):
+            md = name.split("_")[1]
+            s = o.SCHEMES["q4f16_1"]
+            k = z["w"].shape[1]
+            for mode in ("half_away", "half_even"):
+                qw, qs = o.quantize_dt(z["w"], s, md, mode)
+                assert (qw == z[f"q_weight_{mode}"]).all() and np.array_equal(qs, z[f"q_scale_{mode}"])
+            d = o.dequantize_dt(z["q_weight_half_away"], z["q_scale_half_away"], s, k, md)
+            assert np.array_equal(d, z["dequant"])
+            assert np.array_equal(o.linear_dt_fp64(z["x"], z["q_weight_half_away"], z["q_scale_half_away"], s, md), z["y"])
         elif name.startswith("dequant_"):
             s = o.SCHEMES[name.split("_")[1] + "_1"]
             k = z["dequant"].shape[1]
