@@ -458,7 +458,13 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   p.nsteps = (p.steps_total + p.nphases - 1) / p.nphases;
   const size_t lds_x = lds_step * p.nsteps;
   // two waves per SIMD: 512-thread workgroups when only one workgroup fits a CU's LDS
-  const int threads = lds_x > 76 * 1024 ? 512 : 256;
+  // ... unless that leaves CUs without a workgroup (down_proj with 4 rows: 1024 quads = 128 workgroups
+  // of 8 waves): then 4 waves per workgroup and twice the workgroups
+  int threads = lds_x > 76 * 1024 ? 512 : 256;
+  if (threads == 512) {
+    const int64_t wgs = static_cast<int64_t>(((p.nquads + p.rounds - 1) / p.rounds + 7) / 8) * busy * mtiles;
+    if (wgs < 256) threads = 256;
+  }
   const int wpb = threads / 64;
   const size_t lds = lds_x + (p.nphases > 1 ? static_cast<size_t>(wpb) * p.rounds * nbq * 64 : 0);
   const int blocks = ((p.nquads + p.rounds - 1) / p.rounds + wpb - 1) / wpb;
