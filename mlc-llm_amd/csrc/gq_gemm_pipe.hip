@@ -449,11 +449,17 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     const int64_t mid_tiles = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
     if (variant != 6 && p.indptr == nullptr && mid_tiles >= 192)
       return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
+    // grouped: the wider tile once the experts' row tiles alone make several rounds of workgroups
+    if (variant != 6 && p.indptr != nullptr && p.rows >= 96 * p.num_experts &&
+        (static_cast<int64_t>(p.rows) / 128 + p.num_experts) * ((p.N + 255) / 256) >= 768)
+      return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
   }
   // q3: a K tile is 80 wide, so the 256 x 256 tile does not fit LDS; 128 x 256 does
   const int64_t mid_tiles3 = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
-  if (variant == 9 || (variant != 6 && p.indptr == nullptr && mid_tiles3 >= 192))
+  const bool grouped_wide = p.indptr != nullptr && p.rows >= 96 * p.num_experts &&
+                            (static_cast<int64_t>(p.rows) / 128 + p.num_experts) * ((p.N + 255) / 256) >= 768;
+  if (variant == 9 || (variant != 6 && ((p.indptr == nullptr && mid_tiles3 >= 192) || grouped_wide)))
     return launch_pipe_cfg<3, 128, 256, 64, 64>(p, s);
   return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
 }

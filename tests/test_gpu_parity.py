@@ -681,6 +681,23 @@ def test_moe_group_gemm(name, indptr):
     assert bool((out64 == out).all())
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+def test_moe_group_gemm_wide_tile(name):
+    """Enough rows per expert and enough column tiles for the 128 x 256 grouped tile; ragged segments."""
+    s = SCHEMES[name]
+    rng = np.random.default_rng(45)
+    ne, n, k = 2, 49152, 256 if s.bits == 4 else 240
+    ip = np.array([0, 131, 262], np.int32)
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    x = rng.standard_normal((262, k)).astype(np.float16)
+    out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
+    ref = o.dequantize_group_gemm_fp32(x, qw, qs, ip, s)
+    assert_linear_ok(out, ref, x, k, f"group_gemm wide {name}")
+    fused = ops.moe_experts(dev(x), None, dev(qw), dev(qs), dev(ip), s.bits, s.group_size, silu_mul_halves=True)
+    assert bool((fused == ops.silu_mul(out)).all())
+
+
 def test_silu_mul_and_combine():
     rng = np.random.default_rng(47)
     x = (rng.standard_normal((5, 192)) * 3).astype(np.float16)
