@@ -146,8 +146,7 @@ MI355GQ_API int mi355gq_linear_residual(const void* x, const void* q_weight, con
  * mi355gq_linear for the other model dtypes (see mi355gq_quantize_dt): x, q_scale and bias carry
  * model_dtype (MI355GQ_F32 or MI355GQ_BF16; MI355GQ_F16 forwards to mi355gq_linear), y carries
  * out_dtype = model_dtype or MI355GQ_F32.  Weights are dequantised as GroupQuantize._dequantize does
- * ((q - m) * scale rounded to the model dtype) and accumulated in fp32.  A first form: a fp32-FMA GEMV
- * up to 8 rows and a v_mfma_f32_32x32x2_f32 GEMM above; no residual / SiLU epilogues, no MoE forms.
+ * ((q - m) * scale rounded to the model dtype) and accumulated in fp32.  No residual / SiLU epilogues.
  */
 MI355GQ_API int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias,
                       int64_t M, int64_t N, int64_t K, int bits, int group_size, int model_dtype,
@@ -194,6 +193,20 @@ MI355GQ_API int mi355gq_moe_group_gemm(const void* x, int64_t rows, const void* 
                            const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
                            int64_t K, int bits, int group_size, void* out,
                            mi355gq_stream_t stream);
+
+/*
+ * mi355gq_moe_gemv / mi355gq_moe_group_gemm for the other model dtypes (GroupQuantizeMixtralExperts.forward,
+ * quantization/group_quantization.py:619-660, under q4f32_1 / q4bf16_*): x, q_scale and out carry model_dtype
+ * (MI355GQ_F32 or MI355GQ_BF16; MI355GQ_F16 forwards to the entries above); weights are dequantised as
+ * GroupQuantize._dequantize does and accumulated in fp32.  K >= 1.
+ */
+MI355GQ_API int mi355gq_moe_gemv_dt(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                        const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N, int64_t K,
+                        int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_moe_group_gemm_dt(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                              const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
+                              int64_t K, int bits, int group_size, int model_dtype, void* out,
+                              mi355gq_stream_t stream);
 
 /*
  * The e1_e3 expert matmul of MixtralMoE with its activation folded in (mixtral_model.py:64-68:

@@ -544,6 +544,74 @@ int mi355gq_moe_experts(const void* x, int64_t x_rows, const void* x_row_index, 
                              x_rows);
 }
 
+int mi355gq_moe_gemv_dt(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                        const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N, int64_t K, int bits,
+                        int group_size, int model_dtype, void* out, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "moe_gemv_dt"));
+  if (model_dtype == MI355GQ_F16)
+    return moe_gemv_impl(x, x_rows, q_weight, q_scale, expert_ids, top_k, num_experts, N, K, bits, group_size, out,
+                         stream, false);
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(top_k >= 0 && top_k <= 65535 && N >= 0 && K >= 1 && N < kMaxDim && K < kMaxDim && num_experts > 0 &&
+                 num_experts < kMaxDim,
+             "moe_gemv_dt: bad shape");
+  GQ_REQUIRE(x_rows == 1 || x_rows == top_k, "moe_gemv_dt: x has %lld rows, expected 1 or top_k=%lld",
+             (long long)x_rows, (long long)top_k);
+  if (top_k == 0 || N == 0) return MI355GQ_OK;
+  GQ_REQUIRE(out && x && q_weight && q_scale && expert_ids, "moe_gemv_dt: null pointer");
+  const bool f32 = model_dtype == MI355GQ_F32;
+  GQ_REQUIRE(aligned16(q_weight) && aligned4(expert_ids) &&
+                 (f32 ? aligned4(x) && aligned4(q_scale) && aligned4(out)
+                      : aligned2(x) && aligned2(q_scale) && aligned2(out)),
+             "moe_gemv_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
+  return hip_result(gq::launch_moe_gemv_dt(x, x_rows == 1, static_cast<const uint32_t*>(q_weight), q_scale,
+                                           static_cast<const int32_t*>(expert_ids), top_k, num_experts, N, K, bits,
+                                           group_size, model_dtype, out, as_stream(stream)),
+                    "moe_gemv_dt launch");
+}
+
+int mi355gq_moe_group_gemm_dt(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                              const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N, int64_t K,
+                              int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "moe_group_gemm_dt"));
+  if (model_dtype == MI355GQ_F16)
+    return moe_group_gemm_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
+                               group_size, out, stream, false);
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(rows >= 0 && N >= 0 && K >= 1 && rows < kMaxDim && N < kMaxDim && K < kMaxDim && num_experts > 0 &&
+                 num_experts <= 65536,
+             "moe_group_gemm_dt: bad shape");
+  GQ_REQUIRE(indptr_dtype == MI355GQ_I32 || indptr_dtype == MI355GQ_I64, "moe_group_gemm_dt: indptr_dtype=%d",
+             indptr_dtype);
+  if (rows == 0 || N == 0) return MI355GQ_OK;
+  GQ_REQUIRE(out && x && q_weight && q_scale && indptr, "moe_group_gemm_dt: null pointer");
+  const bool f32 = model_dtype == MI355GQ_F32;
+  GQ_REQUIRE(aligned16(q_weight) &&
+                 (indptr_dtype == MI355GQ_I32 ? aligned4(indptr) : (reinterpret_cast<uintptr_t>(indptr) & 7u) == 0) &&
+                 (f32 ? aligned4(x) && aligned4(q_scale) && aligned4(out)
+                      : aligned2(x) && aligned2(q_scale) && aligned2(out)),
+             "moe_group_gemm_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
+  if (model_dtype == MI355GQ_BF16 && rows > 1 && (K & 7) == 0 && aligned16(x) && aligned16(out)) {
+    // the float16 grouped GEMM's tiles on the bf16 matrix instruction (as in linear_dt, faster than the
+    // dot-product kernel from two rows on)
+    gq::GemmArgs g{};
+    g.x = static_cast<const uint16_t*>(x);
+    g.q_weight = static_cast<const uint32_t*>(q_weight);
+    g.q_scale = static_cast<const uint16_t*>(q_scale);
+    g.y = out;
+    g.indptr = indptr; g.indptr_i64 = indptr_dtype == MI355GQ_I64;
+    g.rows = rows; g.N = N; g.K = K; g.num_experts = num_experts;
+    g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
+    g.bf16 = 1;
+    const hipError_t e = gq::launch_gemm(g, as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "moe_group_gemm_dt gemm launch");
+  }
+  return hip_result(gq::launch_moe_group_gemm_dt(x, static_cast<const uint32_t*>(q_weight), q_scale, indptr,
+                                                 indptr_dtype == MI355GQ_I64, rows, num_experts, N, K, bits,
+                                                 group_size, model_dtype, out, as_stream(stream)),
+                    "moe_group_gemm_dt launch");
+}
+
 int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
                                 void* weights, void* ids, mi355gq_stream_t stream) {
   GQ_REQUIRE(T >= 0 && T < kMaxDim, "gating_softmax_topk: bad T");

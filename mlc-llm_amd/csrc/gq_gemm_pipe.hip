@@ -419,8 +419,17 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   const int variant = options().gemm_variant;
   if (p.paired && (p.N & 1)) return hipErrorNotSupported;
   if (p.bf16) {
-    // bfloat16 models: plain linear only, the three regular tiles (no split K, no folded activation)
-    if (p.paired || p.partial != nullptr || p.indptr != nullptr) return hipErrorNotSupported;
+    // bfloat16 models: plain and grouped matmul on the regular tiles (no split K, no folded activation)
+    if (p.paired || p.partial != nullptr || p.x_rows != nullptr) return hipErrorNotSupported;
+    if (p.indptr != nullptr) {
+      const bool wide = p.rows >= 96 * p.num_experts &&
+                        (static_cast<int64_t>(p.rows) / 128 + p.num_experts) * ((p.N + 255) / 256) >= 768;
+      if (bits == 4)
+        return wide ? launch_pipe_cfg<4, 128, 256, 64, 64, 2, true>(p, s)
+                    : launch_pipe_cfg<4, 128, 128, 64, 64, 2, true>(p, s);
+      return wide ? launch_pipe_cfg<3, 128, 256, 64, 64, 2, true>(p, s)
+                  : launch_pipe_cfg<3, 128, 128, 64, 64, 2, true>(p, s);
+    }
     const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
     const int64_t mid_tiles = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
     if (bits == 4) {

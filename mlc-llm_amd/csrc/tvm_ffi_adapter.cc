@@ -248,6 +248,25 @@ void LinearDt(TensorView x, TensorView q_weight, TensorView q_scale, Optional<Te
         "mlc.gq.linear_dt");
 }
 
+void MoeGemvDt(TensorView x, TensorView q_weight, TensorView q_scale, TensorView expert_ids, int64_t bits,
+               int64_t group_size, int64_t model_dtype, TensorView out) {
+  Check(mi355gq_moe_gemv_dt(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(expert_ids),
+                            expert_ids.shape()[1], q_weight.shape()[0], q_weight.shape()[1], x.shape()[1],
+                            static_cast<int>(bits), static_cast<int>(group_size), static_cast<int>(model_dtype),
+                            Ptr(out), StreamOf(x)),
+        "mlc.gq.moe_gemv_dt");
+}
+
+void MoeGroupGemmDt(TensorView x, TensorView q_weight, TensorView q_scale, TensorView indptr, int64_t bits,
+                    int64_t group_size, int64_t model_dtype, TensorView out) {
+  Check(mi355gq_moe_group_gemm_dt(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(indptr),
+                                  indptr.dtype().bits == 64 ? MI355GQ_I64 : MI355GQ_I32, q_weight.shape()[0],
+                                  q_weight.shape()[1], x.shape()[1], static_cast<int>(bits),
+                                  static_cast<int>(group_size), static_cast<int>(model_dtype), Ptr(out),
+                                  StreamOf(x)),
+        "mlc.gq.moe_group_gemm_dt");
+}
+
 TVM_FFI_STATIC_INIT_BLOCK() {
   namespace refl = tvm::ffi::reflection;
   refl::GlobalDef()
@@ -269,7 +288,9 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.quantize_dt", QuantizeDt)
       .def("mlc.gq.dequantize_dt", DequantizeDt)
       .def("mlc.gq.embedding_take_dt", EmbeddingTakeDt)
-      .def("mlc.gq.linear_dt", LinearDt);
+      .def("mlc.gq.linear_dt", LinearDt)
+      .def("mlc.gq.moe_gemv_dt", MoeGemvDt)
+      .def("mlc.gq.moe_group_gemm_dt", MoeGroupGemmDt);
 }
 
 }  // namespace gq

@@ -46,6 +46,8 @@ SIGNATURES = {
     "mi355gq_linear_silu_mul": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P, _P, _L, _P]),
     "mi355gq_moe_gemv_silu_mul": (_I, [_P, _L, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_moe_group_gemm_silu_mul": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _P, _P]),
+    "mi355gq_moe_gemv_dt": (_I, [_P, _L, _P, _P, _P, _L, _L, _L, _L, _I, _I, _I, _P, _P]),
+    "mi355gq_moe_group_gemm_dt": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _I, _P, _P]),
     "mi355gq_moe_gemv": (_I, [_P, _L, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_moe_group_gemm": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_moe_experts": (_I, [_P, _L, _P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _I, _P, _P]),

@@ -224,10 +224,11 @@ def linear_silu_mul(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tens
 def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
              expert_ids: torch.Tensor, bits: int, group_size: int, silu_mul_halves: bool = False
              ) -> torch.Tensor:
-    """silu_mul_halves: the experts' rows are [gate; up] and the result is silu(gate) * up, [k, N / 2]."""
-    _chk(x, torch.float16, "x")
+    """silu_mul_halves: the experts' rows are [gate; up] and the result is silu(gate) * up, [k, N / 2].
+    x, q_scale and the result share the model dtype (float16, float32 or bfloat16)."""
+    _chk(x, _FLOATS, "x")
     _chk(q_weight, _STORAGE, "q_weight")
-    _chk(q_scale, torch.float16, "q_scale")
+    _chk(q_scale, x.dtype, "q_scale")
     _chk(expert_ids, torch.int32, "expert_ids")
     if x.dim() != 2 or expert_ids.dim() != 2 or expert_ids.shape[0] != 1:
         raise ValueError("moe_gemv: x must be [1|k, K] and expert_ids [1, k]")
@@ -235,6 +236,14 @@ def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
     k = x.shape[1]
     _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
     top_k = expert_ids.shape[1]
+    if x.dtype != torch.float16:
+        if silu_mul_halves:
+            raise NotImplementedError("moe_gemv: the SiLU epilogue exists for float16 models only")
+        out = torch.empty((top_k, n), dtype=x.dtype, device=x.device)
+        _lib.call("mi355gq_moe_gemv_dt", x.data_ptr(), x.shape[0], q_weight.data_ptr(), q_scale.data_ptr(),
+                  expert_ids.data_ptr(), top_k, ne, n, k, bits, group_size, _MODEL_DTYPES[x.dtype], out.data_ptr(),
+                  _stream())
+        return out
     args = (x.data_ptr(), x.shape[0], q_weight.data_ptr(), q_scale.data_ptr(), expert_ids.data_ptr(), top_k, ne,
             n, k, bits, group_size)
     if silu_mul_halves:
@@ -256,15 +265,24 @@ def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
 def moe_group_gemm(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
                    indptr: torch.Tensor, bits: int, group_size: int, silu_mul_halves: bool = False
                    ) -> torch.Tensor:
-    _chk(x, torch.float16, "x")
+    """x, q_scale and the result share the model dtype (float16, float32 or bfloat16)."""
+    _chk(x, _FLOATS, "x")
     _chk(q_weight, _STORAGE, "q_weight")
-    _chk(q_scale, torch.float16, "q_scale")
+    _chk(q_scale, x.dtype, "q_scale")
     _chk(indptr, (torch.int32, torch.int64), "indptr")
     ne, n, _ = q_weight.shape
     rows, k = x.shape
     _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
     if tuple(indptr.shape) != (ne + 1,):
         raise ValueError(f"indptr shape {tuple(indptr.shape)}, expected {(ne + 1,)}")
+    if x.dtype != torch.float16:
+        if silu_mul_halves:
+            raise NotImplementedError("moe_group_gemm: the SiLU epilogue exists for float16 models only")
+        out = torch.zeros((rows, n), dtype=x.dtype, device=x.device)
+        _lib.call("mi355gq_moe_group_gemm_dt", x.data_ptr(), rows, q_weight.data_ptr(), q_scale.data_ptr(),
+                  indptr.data_ptr(), _lib.I64 if indptr.dtype == torch.int64 else _lib.I32, ne, n, k, bits,
+                  group_size, _MODEL_DTYPES[x.dtype], out.data_ptr(), _stream())
+        return out
     args = (x.data_ptr(), rows, q_weight.data_ptr(), q_scale.data_ptr(), indptr.data_ptr(),
             _lib.I64 if indptr.dtype == torch.int64 else _lib.I32, ne, n, k, bits, group_size)
     if silu_mul_halves:

@@ -28,7 +28,7 @@ from . import _lib, ops
 _DTYPE_BITS = {"int3": 3, "int4": 4, "int8": 8, "uint32": 32}
 _TORCH_DTYPE = {"float16": torch.float16, "float32": torch.float32, "bfloat16": torch.bfloat16}
 MATMUL_MODEL_DTYPES = ("float16", "float32", "bfloat16")  # model dtypes with a linear kernel
-MOE_MODEL_DTYPES = ("float16",)  # ... and with the expert matmuls
+MOE_MODEL_DTYPES = ("float16", "float32", "bfloat16")  # ... and with the expert matmuls
 
 
 @dataclasses.dataclass

@@ -362,6 +362,31 @@ def dequantize_group_gemm_fp32(x, q_weight, q_scale, indptr, scheme: Scheme) -> 
     return out
 
 
+def moe_dequantize_gemv_dt_fp64(x, q_weight, q_scale, expert_ids, scheme: Scheme, model_dtype: str) -> np.ndarray:
+    """moe_dequantize_gemv_fp32 for any model dtype: each selected expert's weights dequantised in the
+    model dtype (dequantize_dt), exact float64 products.  x, q_scale: float32 carriers."""
+    kdim = x.shape[1]
+    outs = []
+    for e in range(expert_ids.shape[1]):
+        ex = int(expert_ids[0, e])
+        w = dequantize_dt(q_weight[ex], q_scale[ex], scheme, kdim, model_dtype).astype(np.float64)
+        outs.append(w @ np.asarray(x[0 if x.shape[0] == 1 else e], dtype=np.float64))
+    return np.stack(outs)
+
+
+def dequantize_group_gemm_dt_fp64(x, q_weight, q_scale, indptr, scheme: Scheme, model_dtype: str) -> np.ndarray:
+    """dequantize_group_gemm_fp32 for any model dtype (see moe_dequantize_gemv_dt_fp64)."""
+    ne, n, _ = q_weight.shape
+    kdim = x.shape[1]
+    out = np.zeros((x.shape[0], n), np.float64)
+    for e in range(ne):
+        lo, hi = int(indptr[e]), int(indptr[e + 1])
+        if hi > lo:
+            w = dequantize_dt(q_weight[e], q_scale[e], scheme, kdim, model_dtype).astype(np.float64)
+            out[lo:hi] = np.asarray(x[lo:hi], dtype=np.float64) @ w.T
+    return out
+
+
 def silu_mul_f16(x1_x3: np.ndarray) -> np.ndarray:
     """mixtral_model.py:66-68: split in two halves, silu(x1) * x3, all in fp16.
 

@@ -883,8 +883,18 @@ def test_other_model_dtypes_modules():
             assert torch.equal(out[0], back[[3, 47]])
         if cfg.linear_weight_layout == "NK":  # (the reference has no KN expert stack either)
             experts = gq.GroupQuantizeMixtralExperts(2, 96, 48, cfg, device=DEV)
-            with pytest.raises(NotImplementedError):
-                experts(torch.zeros(1, 96, dtype=dt, device=DEV), torch.zeros((1, 2), dtype=torch.int32, device=DEV))
+            experts.q_weight.data.copy_(torch.stack([qw, qw.flip(0)]))
+            experts.q_scale.data.copy_(torch.stack([qs, qs.flip(0)]))
+            x = torch.randn(3, 96, device=DEV).to(dt)
+            # single token: the selected experts' rows are the one-row linear over the same weights
+            picked = experts(x[:1], torch.tensor([[1, 0]], dtype=torch.int32, device=DEV))
+            assert picked.dtype == dt and tuple(picked.shape) == (2, 48)
+            assert torch.equal(picked[1], ops.linear(x[:1], qw, qs, cfg.bits, cfg.group_size)[0])
+            assert torch.equal(picked[0], ops.linear(x[:1], qw.flip(0), qs.flip(0), cfg.bits, cfg.group_size)[0])
+            grouped = experts(x, torch.tensor([0, 1, 3], dtype=torch.int32, device=DEV))
+            want = x.double() @ back.double().t()
+            assert (grouped[0].double() - want[0]).norm() / want[0].norm() <= (3e-3 if dt == torch.bfloat16 else 1e-6)
+            assert (grouped[1:].double() - want[1:].flip(1)).norm() / want[1:].norm() <= (3e-3 if dt == torch.bfloat16 else 1e-6)
 
 
 @pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
@@ -917,6 +927,50 @@ def test_linear_other_model_dtypes(model_dtype, bits_name, m, n, k):
     y = ops.linear(x, qw, qs, s.bits, s.group_size, b)
     assert y.dtype == dt
     assert np.array_equal(_carrier(y), o.round_to(y32.cpu().numpy(), model_dtype))
+
+
+def _assert_dt_matmul_ok(y: torch.Tensor, ref: np.ndarray, x32: np.ndarray, k: int, model_dtype: str, what=""):
+    """Output in the model dtype against the exact product of the same operands: the fp32 accumulation
+    (relative error of a sum of k terms grows like sqrt(k) * 2^-24) plus, for bfloat16, the one rounding of
+    the output (2^-9 per element)."""
+    err = y.double().cpu().numpy() - ref
+    den = max(np.linalg.norm(ref), 1e-30)
+    rel = 1e-6 + 4e-8 * np.sqrt(k) + (2.5e-3 if model_dtype == "bfloat16" else 0.0)
+    assert np.linalg.norm(err) / den <= rel, f"{what}: rel-L2 {np.linalg.norm(err) / den:.3e}"
+    slack = 2.0 ** -8 * np.abs(ref).max() if model_dtype == "bfloat16" else 0.0
+    assert np.abs(err).max() <= 1e-2 * np.abs(x32).max() * np.sqrt(k) / 64 + slack, what
+
+
+@pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("bits_name,k", [("q4f16_1", 512), ("q4f16_1", 1000), ("q3f16_1", 520), ("q3f16_1", 75)])
+def test_moe_matmuls_other_model_dtypes(model_dtype, bits_name, k):
+    """GroupQuantizeMixtralExperts.forward's two matmuls with x, q_scale and the result in the model dtype."""
+    s = SCHEMES[bits_name]
+    dt = _TORCH_OF[model_dtype]
+    rng = np.random.default_rng(k)
+    ne, n = 4, 200
+    w32 = o.round_to((rng.standard_normal((ne, n, k)) * 0.05).astype(np.float32), model_dtype)
+    qw_ref, qs_ref = o.quantize_dt(w32, s, model_dtype)
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).to(dt).to(DEV)
+    ids = np.array([[3, 1]], np.int32)
+    for x_rows in (1, 2):
+        x32 = o.round_to(rng.standard_normal((x_rows, k)).astype(np.float32), model_dtype)
+        y = ops.moe_gemv(torch.from_numpy(x32).to(dt).to(DEV), qw, qs, dev(ids), s.bits, s.group_size)
+        assert y.dtype == dt and tuple(y.shape) == (2, n)
+        ref = o.moe_dequantize_gemv_dt_fp64(x32, qw_ref, qs_ref, ids, s, model_dtype)
+        _assert_dt_matmul_ok(y, ref, x32, k, model_dtype, f"moe_gemv x_rows={x_rows}")
+    for indptr in ([0, 3, 3, 40, 41], [0, 1, 2, 3, 4], [0, 0, 0, 0, 9], [0, 0, 0, 0, 130], [0, 140, 140, 150, 300],
+                   [0, 0, 0, 0, 0]):
+        rows = max(indptr[-1], 1)
+        x32 = o.round_to(rng.standard_normal((rows, k)).astype(np.float32), model_dtype)
+        ip = np.array(indptr, np.int32)
+        x = torch.from_numpy(x32).to(dt).to(DEV)
+        y = ops.moe_group_gemm(x, qw, qs, dev(ip), s.bits, s.group_size)
+        assert y.dtype == dt and tuple(y.shape) == (rows, n)
+        ref = o.dequantize_group_gemm_dt_fp64(x32, qw_ref, qs_ref, ip, s, model_dtype)
+        _assert_dt_matmul_ok(y, ref, x32, k, model_dtype, f"group_gemm {indptr}")
+        y64 = ops.moe_group_gemm(x, qw, qs, dev(ip.astype(np.int64)), s.bits, s.group_size)
+        assert torch.equal(y64, y)
 
 
 def test_linear_other_model_dtypes_through_the_modules():
