@@ -424,9 +424,13 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     if (p.indptr != nullptr) {
       const bool wide = p.rows >= 96 * p.num_experts &&
                         (static_cast<int64_t>(p.rows) / 128 + p.num_experts) * ((p.N + 255) / 256) >= 768;
-      if (bits == 4)
+      if (bits == 4) {
+        // few rows per expert: the tile height follows them (there are no bf16 few-row kernels)
+        if (p.rows <= 16 * p.num_experts) return launch_pipe_cfg<4, 32, 128, 32, 32, 4, true>(p, s);
+        if (p.rows <= 48 * p.num_experts) return launch_pipe_cfg<4, 64, 128, 32, 64, 4, true>(p, s);
         return wide ? launch_pipe_cfg<4, 128, 256, 64, 64, 2, true>(p, s)
                     : launch_pipe_cfg<4, 128, 128, 64, 64, 2, true>(p, s);
+      }
       return wide ? launch_pipe_cfg<3, 128, 256, 64, 64, 2, true>(p, s)
                   : launch_pipe_cfg<3, 128, 128, 64, 64, 2, true>(p, s);
     }
