@@ -454,6 +454,12 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
   }
   if (bits == 4) {
+    // grouped, few rows per expert: the tile height follows them (Mixtral layer, 8 experts: 144-384 routed
+    // rows 18-20 % faster than on 128-row tiles; at 512 rows the 128-row tile is ahead again)
+    if (p.indptr != nullptr && (variant < 0 || variant == 1)) {
+      if (p.rows <= 16 * p.num_experts) return launch_pipe_cfg<4, 32, 128, 32, 32, 4>(p, s);
+      if (p.rows <= 48 * p.num_experts) return launch_pipe_cfg<4, 64, 128, 32, 64, 4>(p, s);
+    }
     const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
     const bool big = variant == 7 ? true : (variant == 6 ? false : (p.indptr == nullptr && big_tiles >= 160));
     if (variant == 9) return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);

@@ -664,7 +664,8 @@ def test_moe_gemv(name, x_rows):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
-@pytest.mark.parametrize("indptr", [[0, 3, 3, 40, 41], [0, 0, 0, 0, 130], [0, 1, 2, 3, 4], [0, 0, 0, 0, 0]])
+@pytest.mark.parametrize("indptr", [[0, 3, 3, 40, 41], [0, 0, 0, 0, 130], [0, 1, 2, 3, 4], [0, 0, 0, 0, 0],
+                                    [0, 33, 34, 60, 64], [0, 70, 70, 71, 200]])
 def test_moe_group_gemm(name, indptr):
     s = SCHEMES[name]
     rng = np.random.default_rng(43)
@@ -1095,7 +1096,9 @@ def test_moe_experts_silu_mul_equals_the_two_steps(name):
     for e_slot, e in enumerate((3, 1)):
         assert_silu_mul_ok(y[e_slot:e_slot + 1], o.linear_fp32(x1, qw[e], qs[e], s), x1, k, f"moe_gemv {name}")
     # grouped: few rows (quad-row kernel), more rows (GEMM)
-    for rows, indptr, gemm_only in ((20, [0, 7, 7, 15, 20], False), (100, [0, 40, 41, 41, 100], False),
+    # (50 and 100 rows: the GEMM's 32- and 64-row grouped tiles)
+    for rows, indptr, gemm_only in ((20, [0, 7, 7, 15, 20], False), (50, [0, 20, 21, 21, 50], False),
+                                    (100, [0, 40, 41, 41, 100], False),
                                     (150, [0, 40, 41, 41, 150], False), (700, [0, 300, 380, 700, 700], False)):
         x = rng.standard_normal((rows, k)).astype(np.float16)
         ip = torch.tensor(indptr, dtype=torch.int32, device=DEV)
