@@ -500,7 +500,10 @@ static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight
   }
   // few rows in total: every expert is a skinny problem bound by streaming its weights
   const int gv = gq::options().gemv_variant;
-  if (rows <= 128 && gq::options().gemm_variant != 1 && ((gv < 0 && rows <= 32) || (gv >= 6 && gv <= 8))) {
+  // (up to about six rows per expert: 8 experts, 40-48 rows 255-263 us for the whole layer against 285 with the
+  //  skinny kernel; from 64 rows on the order flips)
+  const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;
+  if (rows <= 128 && gq::options().gemm_variant != 1 && ((gv < 0 && rows <= quad_rows) || (gv >= 6 && gv <= 8))) {
     const hipError_t q = gq::launch_quadrow(g, static_cast<int>(rows), as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "moe quad-row launch");
   }
