@@ -306,7 +306,10 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     // the regimes of the plain linear: register GEMV up to 2 rows, quad-row kernel up to 8 (q3: 16),
     // skinny kernel up to 16 (q4), else the pipelined GEMM
     hipError_t e = hipErrorNotSupported;
-    if (M <= 2) {
+    if (M == 2 && K > 8192 && bits == 4) e = gq::launch_quadrow(g, 2, as_stream(stream));  // as the plain linear
+    if (e != hipErrorNotSupported) {
+      // served above
+    } else if (M <= 2) {
       gq::GemvArgs a{};
       a.x = g.x; a.q_weight = g.q_weight; a.q_scale = g.q_scale; a.bias = nullptr; a.y = y;
       a.expert_ids = nullptr;
@@ -328,6 +331,12 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // (q3 has no 16x16x32 skinny kernel: 9..16 rows run as two concurrent 8-row passes of the quad-row kernel)
   if (bits == 3 && M >= 3 && M <= 16 && gm != 1 && (M > 8 || gm != 2) && (gv < 0 || (gv >= 6 && gv <= 8))) {
     const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
+    if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
+  }
+  // two rows of a long K (down_proj): the register GEMV holds 7 groups per lane there and measured 19.0 us on
+  // 4096 x 14336 against 15.7-16.4 us for the quad-row kernel at 3-4 rows
+  if (M == 2 && K > 8192 && bits == 4 && gm < 0 && gv < 0) {
+    const hipError_t q = gq::launch_quadrow(g, 2, as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
   }
   const bool use_gemv = M <= 2 || (M <= 8 && (bits != 4 || gm == 2));

@@ -385,8 +385,9 @@ SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_s
   if (grouped || rows <= 0 || N <= 0 || K <= 0 || (K & 7) != 0) return plan;
   // few rows: the GEMM is bound by streaming the weights, and 128-wide column tiles alone leave
   // most CUs idle (o_proj / down have 32 of them).  Match the tile height to the rows and cut K
-  // until about two workgroups per CU exist.
-  if (rows > 256) return plan;
+  // until about one workgroup per CU exists.
+  // (up to 1024 rows: down_proj, 32 column tiles and a long K, ran 150 us flat from 257 to 512 rows unsplit)
+  if (rows > 1024) return plan;
   const int bm = bits == 4 ? (rows <= 32 ? 32 : (rows <= 64 ? 64 : 128)) : 128;
   const int64_t tiles = ((rows + bm - 1) / bm) * ((N + 127) / 128);
   if (rows > 128 && tiles >= 200) return plan;  // the regular tiles already fill the chip
@@ -397,7 +398,9 @@ SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_s
   // when the tiles alone leave CUs idle, and never beyond about twice the weight bytes.
   int split = 1;
   if (tiles < 200 || options().gemv_split > 0) {
-    const int64_t want = options().gemv_split > 0 ? options().gemv_split : 512;  // tuning override
+    // one workgroup per CU: measured 8-20 % faster than two (o_proj, qkv, down at 17..128 rows), whose
+    // partial sums cost more than the second workgroup hides
+    const int64_t want = options().gemv_split > 0 ? options().gemv_split : 256;  // (tuning override)
     split = static_cast<int>((want + tiles - 1) / tiles);
     const int64_t cap = K / (7 * rows);
     if (options().gemv_split <= 0 && split > cap) split = static_cast<int>(cap);
