@@ -302,11 +302,14 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
   g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
   g.paired = paired;
+  // q3, 9..16 rows as passes of the quad-row kernel: only on the smaller matrices (see below)
+  const bool q3_passes_lose = bits == 3 && M > 8 && gq::options().gemv_variant < 0 && N * K >= (40ll << 20) &&
+                              (K & 7) == 0;
   if (paired) {
     // the regimes of the plain linear: register GEMV up to 2 rows, quad-row kernel up to 8 (q3: 16),
     // skinny kernel up to 16 (q4), else the pipelined GEMM
     hipError_t e = hipErrorNotSupported;
-    if (M == 2 && K > 8192 && bits == 4) e = gq::launch_quadrow(g, 2, as_stream(stream));  // as the plain linear
+    if (M == 2 && K > 8192) e = gq::launch_quadrow(g, 2, as_stream(stream));  // as the plain linear
     if (e != hipErrorNotSupported) {
       // served above
     } else if (M <= 2) {
@@ -316,7 +319,7 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
       a.M = M; a.N = N; a.K = K; a.slots = 1; a.x_slot_stride = 0; a.num_experts = 1;
       a.bits = bits; a.group_size = group_size; a.out_f32 = 0; a.paired = 1;
       e = gq::launch_gemv(a, as_stream(stream));
-    } else if (M <= (bits == 3 ? 16 : 8)) {
+    } else if (M <= (bits == 3 ? 16 : 8) && !q3_passes_lose) {
       e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     }
     if (e == hipErrorNotSupported && M <= 16 && bits == 4) e = gq::launch_skinny(g, static_cast<int>(M), as_stream(stream));
@@ -329,13 +332,16 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   const int gv = gq::options().gemv_variant;  // 2..5 force a gq_skinny.hip form, 6..8 the quad-row kernel
   const int gm = gq::options().gemm_variant;  // 1: GEMM only, 2: GEMV up to 8 rows
   // (q3 has no 16x16x32 skinny kernel: 9..16 rows run as two concurrent 8-row passes of the quad-row kernel)
-  if (bits == 3 && M >= 3 && M <= 16 && gm != 1 && (M > 8 || gm != 2) && (gv < 0 || (gv >= 6 && gv <= 8))) {
+  // (... on the smaller matrices: from about 40 M weights on, the GEMM's 32-row tile is ahead of them: gate_up 38
+  //  against 42-46 us, down 25.6 against 27-29.5, while qkv stays at 14.7 against 17.1 and o_proj at 10.3 against 15.2)
+  if (bits == 3 && M >= 3 && M <= 16 && gm != 1 && (M > 8 || gm != 2) && (gv < 0 || (gv >= 6 && gv <= 8)) &&
+      !q3_passes_lose) {
     const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
   }
-  // two rows of a long K (down_proj): the register GEMV holds 7 groups per lane there and measured 19.0 us on
-  // 4096 x 14336 against 15.7-16.4 us for the quad-row kernel at 3-4 rows
-  if (M == 2 && K > 8192 && bits == 4 && gm < 0 && gv < 0) {
+  // two rows of a long K (down_proj): the register GEMV holds 6-7 groups per lane there and measured 19.0 us (q4)
+  // / 17.9 us (q3) on 4096 x 14336 against 14.3-16.4 us for the quad-row kernel at 3-4 rows
+  if (M == 2 && K > 8192 && gm < 0 && gv < 0) {
     const hipError_t q = gq::launch_quadrow(g, 2, as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
   }

@@ -388,7 +388,7 @@ SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_s
   // until about one workgroup per CU exists.
   // (up to 1024 rows: down_proj, 32 column tiles and a long K, ran 150 us flat from 257 to 512 rows unsplit)
   if (rows > 1024) return plan;
-  const int bm = bits == 4 ? (rows <= 32 ? 32 : (rows <= 64 ? 64 : 128)) : 128;
+  const int bm = rows <= 32 ? 32 : (rows <= 64 ? 64 : 128);
   const int64_t tiles = ((rows + bm - 1) / bm) * ((N + 127) / 128);
   if (rows > 128 && tiles >= 200) return plan;  // the regular tiles already fill the chip
   plan.bm = bm;
@@ -414,7 +414,7 @@ SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_s
 }
 
 int gemm_pipe_pair_block(const GemmParams& p, int bits) {
-  return (p.bm_hint == 32 && bits == 4 && options().gemm_variant < 0) ? 16 : 32;  // the 32 x 128 tile below
+  return (p.bm_hint == 32 && options().gemm_variant < 0) ? 16 : 32;  // the 32 x 128 tile below
 }
 
 hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
@@ -454,6 +454,8 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4>(p, s);
     if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4>(p, s);
     if (bits == 4) return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
+    if (p.bm_hint == 32) return launch_pipe_cfg<3, 32, 128, 32, 32, 4>(p, s);
+    if (p.bm_hint == 64) return launch_pipe_cfg<3, 64, 128, 32, 64, 4>(p, s);
     return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
   }
   if (bits == 4) {

@@ -463,7 +463,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   int threads = lds_x > 76 * 1024 ? 512 : 256;
   if (threads == 512) {
     const int64_t wgs = static_cast<int64_t>(((p.nquads + p.rounds - 1) / p.rounds + 7) / 8) * busy * mtiles;
-    if (wgs < 256) threads = 256;
+    if (2 * wgs <= 256) threads = 256;  // (the doubled count must still be one round of workgroups)
   }
   const int wpb = threads / 64;
   const size_t lds = lds_x + (p.nphases > 1 ? static_cast<size_t>(wpb) * p.rounds * nbq * 64 : 0);
