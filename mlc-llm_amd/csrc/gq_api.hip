@@ -309,7 +309,8 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     // the regimes of the plain linear: register GEMV up to 2 rows, quad-row kernel up to 8 (q3: 16),
     // skinny kernel up to 16 (q4), else the pipelined GEMM
     hipError_t e = hipErrorNotSupported;
-    if (M == 2 && K > 8192) e = gq::launch_quadrow(g, 2, as_stream(stream));  // as the plain linear
+    if ((M == 2 && K > 8192) || (M <= 2 && K > 16384))  // as the plain linear
+      e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     if (e != hipErrorNotSupported) {
       // served above
     } else if (M <= 2) {
@@ -322,8 +323,11 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     } else if (M <= (bits == 3 ? 16 : 8) && !q3_passes_lose) {
       e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     }
-    if (e == hipErrorNotSupported && M <= 16 && bits == 4) e = gq::launch_skinny(g, static_cast<int>(M), as_stream(stream));
-    if (e == hipErrorNotSupported) e = gq::launch_gemm(g, as_stream(stream));
+    // (one or two rows never reach the matrix-core kernels in the plain linear either: without a fused form
+    //  the caller runs the two steps, and the result stays the same bit for bit)
+    if (e == hipErrorNotSupported && M > 2 && M <= 16 && bits == 4)
+      e = gq::launch_skinny(g, static_cast<int>(M), as_stream(stream));
+    if (e == hipErrorNotSupported && M > 2) e = gq::launch_gemm(g, as_stream(stream));
     if (e == hipErrorNotSupported)
       return fail(MI355GQ_ERR_UNSUPPORTED, "linear_silu_mul: no fused kernel for M=%lld N=%lld K=%lld (K %% 8 != 0?)",
                   (long long)M, (long long)N, (long long)K);
@@ -341,8 +345,10 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   }
   // two rows of a long K (down_proj): the register GEMV holds 6-7 groups per lane there and measured 19.0 us (q4)
   // / 17.9 us (q3) on 4096 x 14336 against 14.3-16.4 us for the quad-row kernel at 3-4 rows
-  if (M == 2 && K > 8192 && gm < 0 && gv < 0) {
-    const hipError_t q = gq::launch_quadrow(g, 2, as_stream(stream));
+  // (beyond K = 16 Ki the register GEMV does not apply at all and the quad-row kernel also takes single rows)
+  const bool long_k = (M == 2 && K > 8192) || K > 16384;
+  if (M <= 2 && gm < 0 && ((gv < 0 && long_k) || (gv >= 6 && gv <= 8))) {
+    const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
   }
   const bool use_gemv = M <= 2 || (M <= 8 && (bits != 4 || gm == 2));

@@ -215,6 +215,24 @@ def _linear_case(s, m, n, k, seed, bias=False, scale=0.02):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 20480), (2, 64, 20480), (1, 36, 28672), (2, 128, 9000), (1, 62, 20481),
+                                   (2, 62, 20004)])
+def test_one_and_two_rows_of_a_long_k(name, m, n, k):
+    # K past what the register GEMV holds per lane: the quad-row kernel takes over (two rows: from K > 8192;
+    # one row: from K > 16384), the LDS GEMV where that one declines the shape (N % 4, K % 8)
+    s = SCHEMES[name]
+    x, qw, qs, b = _linear_case(s, m, n, k, 7 * m + n + k, bias=True)
+    y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
+    ref = o.linear_fp32(x, qw, qs, s, b)
+    assert_linear_ok(y, ref, x, k, f"long K {name} {m}x{n}x{k}")
+    y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b), out_dtype=torch.float32)
+    assert_linear_ok(y32, ref, x, k, f"long K {name} {m}x{n}x{k} fp32 out")
+    if n % 2 == 0:
+        fused = ops.linear_silu_mul(dev(x), dev(qw), dev(qs), s.bits, s.group_size)
+        assert torch.equal(fused, ops.silu_mul(ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size)))
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_gemv_all_batches(name, m):
     s = SCHEMES[name]
