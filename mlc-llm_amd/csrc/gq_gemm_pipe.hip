@@ -444,10 +444,10 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
       if (p.rows <= 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4, true>(p, s);
       if (p.rows <= 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4, true>(p, s);
       if (big_tiles >= 160) return launch_pipe_cfg<4, 256, 256, 128, 64, 2, true>(p, s);
-      if (mid_tiles >= 192) return launch_pipe_cfg<4, 128, 256, 64, 64, 2, true>(p, s);
+      if (mid_tiles >= 160) return launch_pipe_cfg<4, 128, 256, 64, 64, 2, true>(p, s);
       return launch_pipe_cfg<4, 128, 128, 64, 64, 2, true>(p, s);
     }
-    if (mid_tiles >= 192) return launch_pipe_cfg<3, 128, 256, 64, 64, 2, true>(p, s);
+    if (mid_tiles >= 160) return launch_pipe_cfg<3, 128, 256, 64, 64, 2, true>(p, s);
     return launch_pipe_cfg<3, 128, 128, 64, 64, 2, true>(p, s);
   }
   if (p.bm_hint > 0 && variant < 0) {
@@ -470,8 +470,10 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     if (variant == 9) return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     if (big) return launch_pipe_cfg<4, 256, 256, 128, 64>(p, s);
     // too few 256x256 tiles for 256 CUs (o_proj, down at M = 2048): halve the tile along M
+    // (from 160 such tiles on: 5120-wide 13B projections at 1024 rows ran 589-659 TFLOP/s on them against
+    //  517-572 on twice as many 128x128 tiles)
     const int64_t mid_tiles = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
-    if (variant != 6 && p.indptr == nullptr && mid_tiles >= 192)
+    if (variant != 6 && p.indptr == nullptr && mid_tiles >= 160)
       return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     // grouped: the wider tile once the experts' row tiles alone make several rounds of workgroups
     if (variant != 6 && p.indptr != nullptr && p.rows >= 96 * p.num_experts &&
@@ -483,7 +485,7 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   const int64_t mid_tiles3 = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
   const bool grouped_wide = p.indptr != nullptr && p.rows >= 96 * p.num_experts &&
                             (static_cast<int64_t>(p.rows) / 128 + p.num_experts) * ((p.N + 255) / 256) >= 768;
-  if (variant == 9 || (variant != 6 && ((p.indptr == nullptr && mid_tiles3 >= 192) || grouped_wide)))
+  if (variant == 9 || (variant != 6 && ((p.indptr == nullptr && mid_tiles3 >= 160) || grouped_wide)))
     return launch_pipe_cfg<3, 128, 256, 64, 64>(p, s);
   return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
 }
