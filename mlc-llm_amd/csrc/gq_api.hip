@@ -452,8 +452,23 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
                                          : aligned2(x) && aligned2(q_scale) && aligned2(bias)) &&
                  (out_dtype == MI355GQ_F32 ? aligned4(y) : aligned2(y)),
              "linear_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
+  if (model_dtype == MI355GQ_BF16 && M <= 2 && aligned16(x)) {
+    // one or two rows: the float16 path's register-resident GEMV on v_dot2_f32_bf16
+    gq::GemvArgs a{};
+    a.x = static_cast<const uint16_t*>(x);
+    a.q_weight = static_cast<const uint32_t*>(q_weight);
+    a.q_scale = static_cast<const uint16_t*>(q_scale);
+    a.bias = static_cast<const uint16_t*>(bias);
+    a.y = y;
+    a.expert_ids = nullptr;
+    a.M = M; a.N = N; a.K = K; a.slots = 1; a.x_slot_stride = 0; a.num_experts = 1;
+    a.bits = bits; a.group_size = group_size; a.out_f32 = out_dtype == MI355GQ_F32;
+    a.bf16 = 1;
+    const hipError_t e = gq::launch_gemv(a, as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemv launch");
+  }
   if (model_dtype == MI355GQ_BF16 && M > 1 && (K & 7) == 0 && aligned16(x)) {
-    // the float16 GEMM's tiles on the bf16 matrix instruction (from 2 rows on it already beats the GEMV)
+    // the float16 GEMM's tiles on the bf16 matrix instruction (from 3 rows on; before, where the GEMV declines)
     gq::GemmArgs g{};
     g.x = static_cast<const uint16_t*>(x);
     g.q_weight = static_cast<const uint32_t*>(q_weight);
@@ -590,6 +605,21 @@ int mi355gq_moe_gemv_dt(const void* x, int64_t x_rows, const void* q_weight, con
                  (f32 ? aligned4(x) && aligned4(q_scale) && aligned4(out)
                       : aligned2(x) && aligned2(q_scale) && aligned2(out)),
              "moe_gemv_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
+  if (model_dtype == MI355GQ_BF16 && aligned16(x) && (x_rows == 1 || (K % 8) == 0)) {
+    gq::GemvArgs a{};
+    a.x = static_cast<const uint16_t*>(x);
+    a.q_weight = static_cast<const uint32_t*>(q_weight);
+    a.q_scale = static_cast<const uint16_t*>(q_scale);
+    a.bias = nullptr;
+    a.y = out;
+    a.expert_ids = static_cast<const int32_t*>(expert_ids);
+    a.M = 1; a.N = N; a.K = K; a.slots = top_k; a.x_slot_stride = x_rows == 1 ? 0 : K;
+    a.num_experts = num_experts;
+    a.bits = bits; a.group_size = group_size; a.out_f32 = 0;
+    a.bf16 = 1;
+    const hipError_t e = gq::launch_gemv(a, as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "moe_gemv_dt gemv launch");
+  }
   return hip_result(gq::launch_moe_gemv_dt(x, x_rows == 1, static_cast<const uint32_t*>(q_weight), q_scale,
                                            static_cast<const int32_t*>(expert_ids), top_k, num_experts, N, K, bits,
                                            group_size, model_dtype, out, as_stream(stream)),

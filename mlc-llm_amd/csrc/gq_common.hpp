@@ -32,6 +32,22 @@ __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
   return __builtin_amdgcn_fdot2(as_half2(a), as_half2(b), c, false);
 }
 
+// the same for two bfloat16 pairs: v_dot2_f32_bf16 (exact products, fp32 accumulation)
+typedef __bf16 bf16x2_dot_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_dot_t, a), __builtin_bit_cast(bf16x2_dot_t, b), c,
+                                         false);
+}
+__device__ __forceinline__ float bf2f(uint16_t b) {
+  return __builtin_bit_cast(float, static_cast<uint32_t>(b) << 16);
+}
+// round-to-nearest-even float -> bfloat16 (NaN stays NaN)
+__device__ __forceinline__ uint16_t f2bf(float f) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+  return static_cast<uint16_t>((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
 // (a & mask) | bits as ONE v_and_or_b32.  A VOP3 instruction takes a single 32-bit literal, so the
 // compiler splits the two-constant form into v_and + v_or; keeping the mask in a VGPR and the OR
 // bits in an SGPR makes the fused form encodable (both constants are loop invariant).

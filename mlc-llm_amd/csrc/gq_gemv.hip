@@ -258,6 +258,7 @@ hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
   p.out_f32 = a.out_f32;
   p.gc = 0;
   p.paired = a.paired;
+  p.bf16 = a.bf16;
   if (a.N == 0 || a.slots == 0) return hipSuccess;
   const int nb = static_cast<int>(a.M);
   const int slots = static_cast<int>(a.slots);
@@ -266,7 +267,7 @@ hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
     const hipError_t e = launch_gemv_reg(p, a.bits, nb, slots, s);
     if (e != hipErrorNotSupported) return e;
   }
-  if (p.paired) return hipErrorNotSupported;  // only the register kernel has the fused form
+  if (p.paired || p.bf16) return hipErrorNotSupported;  // only the register kernel has these forms
   return launch_gemv_lds(p, a.bits, nb, slots, s);
 }
 

@@ -36,6 +36,7 @@ struct GemvParams {
   int gc;  // groups staged per LDS chunk (multiple of 64)
   int out_f32;
   int paired;  // fused gate/up form: y[.., N / 2] = silu(x . W[j]) * (x . W[N / 2 + j]), fp16
+  int bf16;    // x, q_scale, bias, residual and a 16-bit y are bfloat16 (register kernel only)
 };
 
 // sum_k x_k * (field_k - m) for one group, given the 4 storage words and the staged x pairs
@@ -72,9 +73,41 @@ __device__ __forceinline__ float group_dot(const uint4 w4, const uint32_t* __res
   }
 }
 
+// The same for bfloat16 activations.  0x4300 | q is the bfloat16 128 + q (q < 128: the seven mantissa bits
+// count ones there), so a field must sit at bit 0 of its half: one shift per field pair where the float16
+// form rescales instead.  Pairs come in the same order as above, so permute_group serves both.
+template <int BITS>
+__device__ __forceinline__ float group_dot_bf16(const uint4 w4, const uint32_t* __restrict__ xr, float corr) {
+  const uint32_t w[4] = {w4.x, w4.y, w4.z, w4.w};
+  constexpr uint32_t kMagic = 0x43004300u;
+  float a0 = 0.f, a1 = 0.f;
+  if (BITS == 4) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a0 = dot2_bf16(and_or(w[i], 0x000f000fu, kMagic), xr[4 * i + 0], a0);
+      a1 = dot2_bf16(and_or(w[i] >> 4, 0x000f000fu, kMagic), xr[4 * i + 1], a1);
+      a0 = dot2_bf16(and_or(w[i] >> 8, 0x000f000fu, kMagic), xr[4 * i + 2], a0);
+      a1 = dot2_bf16(and_or(w[i] >> 12, 0x000f000fu, kMagic), xr[4 * i + 3], a1);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
+      const uint32_t t = (w[i] & 0x0000ffffu) | ((w[i] << 1) & 0xffff0000u);
+      a0 = dot2_bf16(and_or(t, 0x00070007u, kMagic), xr[5 * i + 0], a0);
+      a1 = dot2_bf16(and_or(t >> 3, 0x00070007u, kMagic), xr[5 * i + 1], a1);
+      a0 = dot2_bf16(and_or(t >> 6, 0x00070007u, kMagic), xr[5 * i + 2], a0);
+      a1 = dot2_bf16(and_or(t >> 9, 0x00070007u, kMagic), xr[5 * i + 3], a1);
+      a0 = dot2_bf16(and_or(t >> 12, 0x00070007u, kMagic), xr[5 * i + 4], a0);
+    }
+  }
+  return (a0 + a1) - corr;
+}
+
 // x pairs of one group in the order the unpack masks produce them, from the natural-order halves.
 // v_perm_b32 picks the two 16-bit lanes directly: byte selectors 0-3 address S1, 4-7 address S0.
-template <int BITS>
+// BF: bfloat16 activations; every field then carries the same offset 128 + m.
+template <int BITS, bool BF = false>
 __device__ __forceinline__ float permute_group(const uint32_t* __restrict__ n /* G/2 natural pairs */,
                                                uint32_t* __restrict__ xr /* G/2 permuted pairs */) {
   constexpr uint32_t kLoLo = 0x05040100u;  // (lo16(S1), lo16(S0))
@@ -93,10 +126,15 @@ __device__ __forceinline__ float permute_group(const uint32_t* __restrict__ n /*
       xr[4 * w + 1] = __builtin_amdgcn_perm(n[4 * w + 2], n[4 * w + 0], kHiHi);
       xr[4 * w + 2] = __builtin_amdgcn_perm(n[4 * w + 3], n[4 * w + 1], kLoLo);
       xr[4 * w + 3] = __builtin_amdgcn_perm(n[4 * w + 3], n[4 * w + 1], kHiHi);
-      c = dot2(xr[4 * w + 0], c_lo, c);
-      c = dot2(xr[4 * w + 1], c_hi, c);
-      c = dot2(xr[4 * w + 2], c_lo, c);
-      c = dot2(xr[4 * w + 3], c_hi, c);
+      if constexpr (BF) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c = dot2_bf16(xr[4 * w + j], 0x43074307u /* (135, 135) */, c);
+      } else {
+        c = dot2(xr[4 * w + 0], c_lo, c);
+        c = dot2(xr[4 * w + 1], c_hi, c);
+        c = dot2(xr[4 * w + 2], c_lo, c);
+        c = dot2(xr[4 * w + 3], c_hi, c);
+      }
     }
   } else {
     // word w holds x[10w..10w+9] as 5 natural pairs; wanted (j, j+5); pair j sits at mantissa
@@ -112,11 +150,16 @@ __device__ __forceinline__ float permute_group(const uint32_t* __restrict__ n /*
       xr[5 * w + 2] = __builtin_amdgcn_perm(r[3], r[1], kLoHi);
       xr[5 * w + 3] = __builtin_amdgcn_perm(r[4], r[1], kHiLo);
       xr[5 * w + 4] = __builtin_amdgcn_perm(r[4], r[2], kLoHi);
-      c = dot2(xr[5 * w + 0], c1, c);
-      c = dot2(xr[5 * w + 1], c8, c);
-      c = dot2(xr[5 * w + 2], c64, c);
-      c = dot2(xr[5 * w + 3], c1, c);
-      c = dot2(xr[5 * w + 4], c8, c);
+      if constexpr (BF) {
+#pragma unroll
+        for (int j = 0; j < 5; ++j) c = dot2_bf16(xr[5 * w + j], 0x43034303u /* (131, 131) */, c);
+      } else {
+        c = dot2(xr[5 * w + 0], c1, c);
+        c = dot2(xr[5 * w + 1], c8, c);
+        c = dot2(xr[5 * w + 2], c64, c);
+        c = dot2(xr[5 * w + 3], c1, c);
+        c = dot2(xr[5 * w + 4], c8, c);
+      }
     }
   }
   return c;

@@ -19,10 +19,15 @@ namespace gq {
 // MODE 1: a bias or residual operand exists (a template flag rather than a run-time test: their loads are
 // two more memory instructions per set, measured at 4-6 % of the plain GEMV's time).
 // MODE 2: fused gate/up form; a set holds R / 2 (gate, up) row pairs and stores R / 2 products.
-template <int BITS, int NB, int R, int ITERS, int MODE>
+// BF: bfloat16 model (x, scales, bias, residual and a 16-bit result are bfloat16); the same walk with
+// group_dot_bf16.  Like the float16 form it multiplies x with the integer fields and applies the scale
+// to the group sum in fp32, so the dequantised weight is never rounded to the model dtype on its own.
+template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false>
 __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int nsets) {
   using T = GemvTraits<BITS>;
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;
+  static_assert(!(BF && PAIRED), "the fused gate/up form is float16 only");
+  auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
   static_assert(!PAIRED || R % 2 == 0, "a set holds whole (gate, up) pairs");
   constexpr int G = T::G;
   constexpr int HP = G / 2;  // half pairs of x per group
@@ -140,7 +145,7 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
         if (!gok[it]) raw = make_uint4(0, 0, 0, 0);
         nat[4 * c + 0] = raw.x; nat[4 * c + 1] = raw.y; nat[4 * c + 2] = raw.z; nat[4 * c + 3] = raw.w;
       }
-      corr[b][it] = permute_group<BITS>(nat, xr[b][it]);
+      corr[b][it] = permute_group<BITS, BF>(nat, xr[b][it]);
     }
   }
 
@@ -155,8 +160,10 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
         float a = 0.f;
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
-          const float sv = gok[it] ? h2f(static_cast<uint16_t>(sc[r][it])) : 0.f;  // lanes past the last group add nothing
-          a = fmaf(sv, group_dot<BITS>(wc[r][it], xr[b][it], corr[b][it]), a);
+          const float sv = gok[it] ? to_f32(static_cast<uint16_t>(sc[r][it])) : 0.f;  // lanes past the last group add nothing
+          const float gd = BF ? group_dot_bf16<BITS>(wc[r][it], xr[b][it], corr[b][it])
+                              : group_dot<BITS>(wc[r][it], xr[b][it], corr[b][it]);
+          a = fmaf(sv, gd, a);
         }
         acc[r][b] = wave_sum_last(a);
       }
@@ -175,8 +182,8 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
       }
       return;
     }
-    const float bias_lane = (EXTRA && p.bias != nullptr) ? h2f(static_cast<uint16_t>(bias_bits & 0xffffu)) : 0.f;
-    const float res_lane = (EXTRA && p.residual != nullptr) ? h2f(static_cast<uint16_t>(bias_bits >> 16)) : 0.f;
+    const float bias_lane = (EXTRA && p.bias != nullptr) ? to_f32(static_cast<uint16_t>(bias_bits & 0xffffu)) : 0.f;
+    const float res_lane = (EXTRA && p.residual != nullptr) ? to_f32(static_cast<uint16_t>(bias_bits >> 16)) : 0.f;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const float bias = __builtin_bit_cast(
@@ -195,7 +202,7 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
           const float v = acc[r][b] + bias + res[b];
           const int64_t oi = static_cast<int64_t>(slot + b) * p.N + row;  // slot > 0 only if NB == 1
           if (p.out_f32) static_cast<float*>(p.y)[oi] = v;
-          else static_cast<uint16_t*>(p.y)[oi] = f2h(v);
+          else static_cast<uint16_t*>(p.y)[oi] = BF ? f2bf(v) : f2h(v);
         }
       }
     }
@@ -215,6 +222,14 @@ static hipError_t launch_k(const GemvParams& p, int slots, int blocks, int nsets
   const int threads = 256;
   const size_t lds = static_cast<size_t>(NB) * p.ng * GemvTraits<BITS>::G * 2;
   const dim3 grid(blocks, slots);
+  if (p.bf16) {
+    if (p.paired) return hipErrorNotSupported;
+    if (p.bias != nullptr || p.residual != nullptr)
+      hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 1, true>), grid, dim3(threads), lds, s, p, nsets);
+    else
+      hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 0, true>), grid, dim3(threads), lds, s, p, nsets);
+    return hipGetLastError();
+  }
   if (p.paired) {
     if constexpr (R % 2 == 0)
       hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 2>), grid, dim3(threads), lds, s, p, nsets);

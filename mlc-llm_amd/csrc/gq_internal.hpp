@@ -31,6 +31,7 @@ struct GemvArgs {
   int bits, group_size;
   int out_f32;
   int paired = 0;           // fused gate/up form (see gate_up_row): y is [M or slots, N / 2] fp16; N even, no bias / residual
+  int bf16 = 0;             // bfloat16 model: x, q_scale, bias, residual and a 16-bit y are bf16 (M <= 2, no fused form)
 };
 hipError_t launch_gemv(const GemvArgs& a, hipStream_t s);
 

@@ -224,11 +224,24 @@ def dequantize_dt(q_weight: np.ndarray, q_scale: np.ndarray, scheme: Scheme, k: 
         return round_to(u * s, model_dtype)
 
 
-def linear_dt_fp64(x, q_weight, q_scale, scheme: Scheme, model_dtype: str, bias=None) -> np.ndarray:
+def dequantize_unrounded(q_weight: np.ndarray, q_scale: np.ndarray, scheme: Scheme, k: int) -> np.ndarray:
+    """(q - m) * scale in float64, without the rounding to the model dtype that _dequantize
+    (group_quantization.py:273-305) applies to each weight: what a kernel computes that scales the
+    group's integer dot product instead of materialising weights."""
+    u = unpack(q_weight, scheme, k).astype(np.float64) - float(scheme.max_int)
+    return u * np.asarray(q_scale, dtype=np.float64)[..., np.arange(k) // scheme.group_size]
+
+
+def linear_dt_fp64(x, q_weight, q_scale, scheme: Scheme, model_dtype: str, bias=None,
+                   unrounded_weights: bool = False) -> np.ndarray:
     """Yardstick of the linear for any model dtype: weights dequantised in the model dtype
-    (dequantize_dt), then an exact float64 matmul.  x, q_scale, bias: float32 carriers."""
+    (dequantize_dt; unrounded_weights: dequantize_unrounded), then an exact float64 matmul.
+    x, q_scale, bias: float32 carriers."""
     k = x.shape[-1]
-    w = dequantize_dt(q_weight, q_scale, scheme, k, model_dtype).astype(np.float64)
+    if unrounded_weights:
+        w = dequantize_unrounded(q_weight, q_scale, scheme, k)
+    else:
+        w = dequantize_dt(q_weight, q_scale, scheme, k, model_dtype).astype(np.float64)
     y = np.asarray(x, dtype=np.float64) @ w.T
     if bias is not None:
         y = y + np.asarray(bias, dtype=np.float64)

@@ -921,6 +921,7 @@ def test_other_model_dtypes_modules():
 @pytest.mark.parametrize("bits_name,m,n,k", [
     ("q4f16_1", 1, 512, 4096), ("q4f16_1", 2, 100, 1000), ("q4f16_1", 4, 257, 2048), ("q4f16_1", 8, 128, 8192),
     ("q4f16_1", 3, 64, 13), ("q4f16_1", 1, 40, 40000),                     # ragged K; K past the GEMV's LDS
+    ("q4f16_1", 1, 130, 14336), ("q4f16_1", 2, 96, 8192), ("q4f16_1", 2, 33, 1001), ("q3f16_1", 2, 64, 2000),
     ("q4f16_1", 9, 256, 512), ("q4f16_1", 130, 200, 1024), ("q4f16_1", 300, 384, 360), ("q4f16_1", 64, 130, 100),
     ("q3f16_1", 1, 256, 4096), ("q3f16_1", 5, 96, 1000), ("q3f16_1", 200, 136, 2000),
 ])
@@ -940,8 +941,17 @@ def test_linear_other_model_dtypes(model_dtype, bits_name, m, n, k):
     y32 = ops.linear(x, qw, qs, s.bits, s.group_size, b, out_dtype=torch.float32)
     assert y32.dtype == torch.float32 and tuple(y32.shape) == (m, n)
     err = y32.double().cpu().numpy() - ref
-    # (relative error of a float32 sum of k terms grows like sqrt(k) * 2^-24)
-    assert np.linalg.norm(err) / den <= 1e-6 + 4e-8 * np.sqrt(k), np.linalg.norm(err) / den
+    if model_dtype == "bfloat16" and m <= 2 and -(-k // s.group_size) <= 512:  # (8 groups per lane at most)
+        # the register GEMV scales each group's integer dot product, so its operands are the weights before
+        # _dequantize's rounding to bfloat16: exact against those, and within the matmul tolerance (2^-9 per
+        # weight, random in sign) of the product with the rounded ones
+        exact = y32.double().cpu().numpy() - o.linear_dt_fp64(x32, qw_ref, qs_ref, s, model_dtype, b32, unrounded_weights=True)
+        # (its fp32 sums run over x * (128 + q), some 40 times the size of x * (q - m): that much more rounding)
+        assert np.linalg.norm(exact) / den <= 5e-6 + 1e-7 * np.sqrt(k), np.linalg.norm(exact) / den
+        assert np.linalg.norm(err) / den <= 2e-3, np.linalg.norm(err) / den
+    else:
+        # (relative error of a float32 sum of k terms grows like sqrt(k) * 2^-24)
+        assert np.linalg.norm(err) / den <= 1e-6 + 4e-8 * np.sqrt(k), np.linalg.norm(err) / den
     assert np.abs(err).max() <= 1e-2 * np.abs(x32).max() * np.sqrt(k) / 64
     # output in the model dtype: the same numbers rounded once
     y = ops.linear(x, qw, qs, s.bits, s.group_size, b)
