@@ -189,7 +189,7 @@ def main() -> int:
     us_read = timed(read_sweep, max(5, args.steps), 2, use_graph) * 1e3 / LAYERS
     read_bytes = layers[0]["gate_up"][0].numel() * 4 + layers[0]["gate_up"][1].numel() * 2
     roofline = {
-        "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2,0> (gate_up 28672x4096, batch 1)",
+        "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2,0,false> (gate_up 28672x4096, batch 1)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
         "bytes_per_launch": gu_bytes, "us_per_launch": round(us_gate_up, 3),
