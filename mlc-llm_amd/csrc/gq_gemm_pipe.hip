@@ -481,6 +481,10 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
       return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     return launch_pipe_cfg<4, 128, 128, 64, 64>(p, s);
   }
+  if (p.indptr != nullptr && (variant < 0 || variant == 1)) {  // grouped, few rows per expert: as q4 above
+    if (p.rows <= 16 * p.num_experts) return launch_pipe_cfg<3, 32, 128, 32, 32, 4>(p, s);
+    if (p.rows <= 48 * p.num_experts) return launch_pipe_cfg<3, 64, 128, 32, 64, 4>(p, s);
+  }
   // q3: a K tile is 80 wide, so the 256 x 256 tile does not fit LDS; 128 x 256 does
   const int64_t mid_tiles3 = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
   const bool grouped_wide = p.indptr != nullptr && p.rows >= 96 * p.num_experts &&
