@@ -149,10 +149,15 @@ MI355GQ_API int mi355gq_linear_residual(const void* x, const void* q_weight, con
  * ((q - m) * scale rounded to the model dtype) and accumulated in fp32.  Exception: one or two bfloat16 rows
  * (K <= 16384) run the float16 path's register GEMV, which scales each group's integer dot product in fp32 and so
  * skips that per-weight rounding (as mi355gq_linear does for float16).  No residual / SiLU epilogues.
+ * workspace: device scratch of at least mi355gq_linear_dt_workspace_bytes(M, N, K, ...) bytes, 16-byte aligned,
+ * or null (then few-row bfloat16 matmuls run unsplit: slower, same result up to summation order).
  */
+MI355GQ_API int64_t mi355gq_linear_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size,
+                                          int model_dtype);
 MI355GQ_API int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias,
                       int64_t M, int64_t N, int64_t K, int bits, int group_size, int model_dtype,
-                      int out_dtype, void* y, mi355gq_stream_t stream);
+                      int out_dtype, void* y, void* workspace, int64_t workspace_bytes,
+                      mi355gq_stream_t stream);
 
 /*
  * gate_up projection with the activation folded in: the sequence

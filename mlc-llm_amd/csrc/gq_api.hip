@@ -255,6 +255,16 @@ int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits
   return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
 }
 
+int64_t mi355gq_linear_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size,
+                                          int model_dtype) {
+  if (model_dtype == MI355GQ_F16) return mi355gq_linear_workspace_bytes(M, N, K, bits, group_size);
+  if (model_dtype != MI355GQ_BF16 || check_scheme(bits, group_size) != MI355GQ_OK || M < 2 || N < 0 || K < 0 ||
+      M >= kMaxDim || N >= kMaxDim || K >= kMaxDim)
+    return 0;
+  // bfloat16: every batch from two rows on may run the few-row GEMM (there are no bf16 skinny kernels)
+  return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+}
+
 int64_t mi355gq_linear_silu_mul_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
   if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
       N >= kMaxDim || K >= kMaxDim)
@@ -435,11 +445,11 @@ static int moe_gemv_impl(const void* x, int64_t x_rows, const void* q_weight, co
 
 int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias, int64_t M,
                       int64_t N, int64_t K, int bits, int group_size, int model_dtype, int out_dtype, void* y,
-                      mi355gq_stream_t stream) {
+                      void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
   GQ_CHECK(check_model_dtype(model_dtype, "linear_dt"));
   if (model_dtype == MI355GQ_F16)
-    return linear_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, out_dtype, y, nullptr, 0,
-                       stream);
+    return linear_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, out_dtype, y, workspace,
+                       workspace_bytes, stream);
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(M >= 0 && N >= 0 && K >= 1 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
              "linear_dt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
@@ -478,6 +488,7 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
     g.indptr = nullptr; g.indptr_i64 = 0;
     g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
     g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
+    g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
     g.bf16 = 1;
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemm launch");

@@ -218,11 +218,7 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   p.bf16 = a.bf16;
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int variant = options().gemm_variant;
-  if (a.bf16) {  // bfloat16 models run the pipelined kernel's regular tiles or nothing
-    const hipError_t e = launch_gemm_pipe(p, a.bits, s);
-    return e;
-  }
-  if (variant < 0) {
+  if (variant < 0 || a.bf16) {
     const SplitPlan plan = plan_split_k(a.rows, a.N, a.K, a.bits, a.group_size, a.indptr != nullptr);
     p.bm_hint = plan.bm;
     const int64_t need = static_cast<int64_t>(plan.split) * a.rows * a.N * 4;
@@ -235,7 +231,7 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
       p.kt_per_split = plan.kt_per_split;
     }
   }
-  if (variant != 3 && variant != 4 && variant != 5) {
+  if (a.bf16 || (variant != 3 && variant != 4 && variant != 5)) {
     const hipError_t e = launch_gemm_pipe(p, a.bits, s);
     if (e == hipSuccess && p.partial != nullptr) {
       const int64_t count = a.rows * a.N;
@@ -250,10 +246,10 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
         return hipGetLastError();
       }
       hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
-                         p.partial, split, count, p.N, p.bias, p.residual, p.y, p.out_f32);
+                         p.partial, split, count, p.N, p.bias, p.residual, p.y, p.out_f32, p.bf16);
       return hipGetLastError();
     }
-    if (e != hipErrorNotSupported) return e;
+    if (e != hipErrorNotSupported || a.bf16) return e;  // (bfloat16 models: the pipelined kernel or nothing)
   }
   if (p.paired) return hipErrorNotSupported;  // the fused form exists in the pipelined kernel only
   if (a.bits == 4) {

@@ -56,7 +56,7 @@ __device__ __forceinline__ int gate_up_row_blk(int c, int N) {
 }
 
 __global__ void splitk_reduce_kernel(const float* partial, int split, int64_t count, int N,
-                                     const uint16_t* bias, const uint16_t* residual, void* y, int out_f32);
+                                     const uint16_t* bias, const uint16_t* residual, void* y, int out_f32, int bf16);
 // fused gate/up form: partial[split][rows][N] in the block-interleaved column order -> y fp16 [rows, N / 2]
 __global__ void splitk_reduce_silu_kernel(const float* partial, int split, int64_t rows, int N, int pb,
                                           uint16_t* y);

@@ -320,7 +320,10 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, int split,
                                                             int64_t count /* rows * N */, int N,
                                                             const uint16_t* __restrict__ bias,
-                                                            const uint16_t* residual, void* y, int out_f32) {
+                                                            const uint16_t* residual, void* y, int out_f32, int bf16) {
+  // bias, residual and a 16-bit y carry the model dtype: float16, or bfloat16 when bf16 is set
+  auto in = [bf16](uint16_t bits) { return bf16 ? bf2f(bits) : h2f(bits); };
+  auto out = [bf16](float v) { return bf16 ? f2bf(v) : f2h(v); };
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   if ((N & 3) == 0) {  // rows are 16-byte aligned: four columns per thread
     for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; 4 * i < count; i += stride) {
@@ -332,20 +335,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
       if (bias != nullptr) {
         const int col = static_cast<int>((4 * i) % N);
         const uint2 bb = *reinterpret_cast<const uint2*>(bias + col);
-        a.x += h2f(static_cast<uint16_t>(bb.x & 0xffffu)); a.y += h2f(static_cast<uint16_t>(bb.x >> 16));
-        a.z += h2f(static_cast<uint16_t>(bb.y & 0xffffu)); a.w += h2f(static_cast<uint16_t>(bb.y >> 16));
+        a.x += in(static_cast<uint16_t>(bb.x & 0xffffu)); a.y += in(static_cast<uint16_t>(bb.x >> 16));
+        a.z += in(static_cast<uint16_t>(bb.y & 0xffffu)); a.w += in(static_cast<uint16_t>(bb.y >> 16));
       }
       if (residual != nullptr) {
         const uint2 rr = *reinterpret_cast<const uint2*>(residual + 4 * i);
-        a.x += h2f(static_cast<uint16_t>(rr.x & 0xffffu)); a.y += h2f(static_cast<uint16_t>(rr.x >> 16));
-        a.z += h2f(static_cast<uint16_t>(rr.y & 0xffffu)); a.w += h2f(static_cast<uint16_t>(rr.y >> 16));
+        a.x += in(static_cast<uint16_t>(rr.x & 0xffffu)); a.y += in(static_cast<uint16_t>(rr.x >> 16));
+        a.z += in(static_cast<uint16_t>(rr.y & 0xffffu)); a.w += in(static_cast<uint16_t>(rr.y >> 16));
       }
       if (out_f32) {
         *reinterpret_cast<float4*>(static_cast<float*>(y) + 4 * i) = a;
       } else {
         uint2 o;
-        o.x = static_cast<uint32_t>(f2h(a.x)) | (static_cast<uint32_t>(f2h(a.y)) << 16);
-        o.y = static_cast<uint32_t>(f2h(a.z)) | (static_cast<uint32_t>(f2h(a.w)) << 16);
+        o.x = static_cast<uint32_t>(out(a.x)) | (static_cast<uint32_t>(out(a.y)) << 16);
+        o.y = static_cast<uint32_t>(out(a.z)) | (static_cast<uint32_t>(out(a.w)) << 16);
         *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + 4 * i) = o;
       }
     }
@@ -353,10 +356,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
     for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < count; i += stride) {
       float a = partial[i];
       for (int sidx = 1; sidx < split; ++sidx) a += partial[sidx * count + i];
-      if (bias != nullptr) a += h2f(bias[i % N]);
-      if (residual != nullptr) a += h2f(residual[i]);
+      if (bias != nullptr) a += in(bias[i % N]);
+      if (residual != nullptr) a += in(residual[i]);
       if (out_f32) static_cast<float*>(y)[i] = a;
-      else static_cast<uint16_t*>(y)[i] = f2h(a);
+      else static_cast<uint16_t*>(y)[i] = out(a);
     }
   }
 }
@@ -422,8 +425,15 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   const int variant = options().gemm_variant;
   if (p.paired && (p.N & 1)) return hipErrorNotSupported;
   if (p.bf16) {
-    // bfloat16 models: plain and grouped matmul on the regular tiles (no split K, no folded activation)
-    if (p.paired || p.partial != nullptr || p.x_rows != nullptr) return hipErrorNotSupported;
+    // bfloat16 models: plain and grouped matmul (no folded activation)
+    if (p.paired || p.x_rows != nullptr) return hipErrorNotSupported;
+    if (p.bm_hint > 0 && p.indptr == nullptr) {  // few rows, K possibly split (see plan_split_k)
+      if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4, true>(p, s);
+      if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4, true>(p, s);
+      if (bits == 4) return launch_pipe_cfg<4, 128, 128, 64, 64, 2, true>(p, s);
+      return launch_pipe_cfg<3, 128, 128, 64, 64, 2, true>(p, s);
+    }
+    if (p.partial != nullptr) return hipErrorNotSupported;
     if (p.indptr != nullptr) {
       const bool wide = p.rows >= 96 * p.num_experts &&
                         (static_cast<int64_t>(p.rows) / 128 + p.num_experts) * ((p.N + 255) / 256) >= 768;

@@ -238,13 +238,25 @@ void EmbeddingTakeDt(TensorView ids, TensorView q_weight, TensorView q_scale, in
         "mlc.gq.embedding_take_dt");
 }
 
+int64_t LinearDtWorkspaceBytes(int64_t M, int64_t N, int64_t K, int64_t bits, int64_t group_size,
+                               int64_t model_dtype) {
+  return mi355gq_linear_dt_workspace_bytes(M, N, K, static_cast<int>(bits), static_cast<int>(group_size),
+                                           static_cast<int>(model_dtype));
+}
+
 void LinearDt(TensorView x, TensorView q_weight, TensorView q_scale, Optional<TensorView> bias, int64_t bits,
-              int64_t group_size, int64_t model_dtype, TensorView y) {
+              int64_t group_size, int64_t model_dtype, Optional<TensorView> workspace, TensorView y) {
   const int64_t K = x.shape()[x.ndim() - 1], N = q_weight.shape()[0];
   const int out_dtype = y.dtype().bits == 32 ? MI355GQ_F32 : static_cast<int>(model_dtype);
+  void* ws = workspace.has_value() ? Ptr(workspace.value()) : nullptr;
+  int64_t ws_bytes = 0;
+  if (workspace.has_value()) {
+    ws_bytes = (workspace.value().dtype().bits + 7) / 8;
+    for (int i = 0; i < workspace.value().ndim(); ++i) ws_bytes *= workspace.value().shape()[i];
+  }
   Check(mi355gq_linear_dt(Ptr(x), Ptr(q_weight), Ptr(q_scale), bias.has_value() ? Ptr(bias.value()) : nullptr,
                           Rows(x), N, K, static_cast<int>(bits), static_cast<int>(group_size),
-                          static_cast<int>(model_dtype), out_dtype, Ptr(y), StreamOf(x)),
+                          static_cast<int>(model_dtype), out_dtype, Ptr(y), ws, ws_bytes, StreamOf(x)),
         "mlc.gq.linear_dt");
 }
 
@@ -289,6 +301,7 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.dequantize_dt", DequantizeDt)
       .def("mlc.gq.embedding_take_dt", EmbeddingTakeDt)
       .def("mlc.gq.linear_dt", LinearDt)
+      .def("mlc.gq.linear_dt_workspace_bytes", LinearDtWorkspaceBytes)
       .def("mlc.gq.moe_gemv_dt", MoeGemvDt)
       .def("mlc.gq.moe_group_gemm_dt", MoeGroupGemmDt);
 }

@@ -181,9 +181,12 @@ def _linear_other_dtype(x, q_weight, q_scale, bits, group_size, bias, out_dtype,
         out = torch.empty((*x.shape[:-1], n), dtype=out_dtype, device=x.device)
     else:
         _chk(out, out_dtype, "out")
+    ws_bytes = _lib.lib().mi355gq_linear_dt_workspace_bytes(m, n, k, bits, group_size, _MODEL_DTYPES[dt])
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     _lib.call("mi355gq_linear_dt", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(),
               bias.data_ptr() if bias is not None else None, m, n, k, bits, group_size, _MODEL_DTYPES[dt],
-              _MODEL_DTYPES[out_dtype], out.data_ptr(), _stream())
+              _MODEL_DTYPES[out_dtype], out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
+              _stream())
     return out
 
 

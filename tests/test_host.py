@@ -99,10 +99,10 @@ def test_argument_validation_of_the_later_entry_points():
     assert lib.mi355gq_quantize_dt(P(0x1000), 4, 32, 4, 32, 0, 5, P(0x2000), P(0x3000), None) == -1
     assert "model_dtype" in _err()
     assert lib.mi355gq_dequantize_dt(P(0x1000), P(0x2000), 4, 32, 4, 32, 3, P(0x3000), None) == -1
-    assert lib.mi355gq_linear_dt(P(0x1000), P(0x2000), P(0x3000), None, 2, 8, 64, 4, 32, 2, 0, P(0x4000), None) == -1
+    assert lib.mi355gq_linear_dt(P(0x1000), P(0x2000), P(0x3000), None, 2, 8, 64, 4, 32, 2, 0, P(0x4000), None, 0, None) == -1
     assert "out_dtype" in _err()
-    assert lib.mi355gq_linear_dt(P(0x1000), P(0x2000), P(0x3000), None, 2, 8, 0, 4, 32, 1, 1, P(0x4000), None) == -1
-    assert lib.mi355gq_linear_dt(P(0x1002), P(0x2000), P(0x3000), None, 2, 8, 64, 4, 32, 1, 1, P(0x4000), None) == -1
+    assert lib.mi355gq_linear_dt(P(0x1000), P(0x2000), P(0x3000), None, 2, 8, 0, 4, 32, 1, 1, P(0x4000), None, 0, None) == -1
+    assert lib.mi355gq_linear_dt(P(0x1002), P(0x2000), P(0x3000), None, 2, 8, 64, 4, 32, 1, 1, P(0x4000), None, 0, None) == -1
     # the expert matmuls in the other model dtypes
     assert lib.mi355gq_moe_gemv_dt(P(0x1000), 3, P(0x2000), P(0x3000), P(0x4000), 2, 8, 16, 32, 4, 32, 1, P(0x5000), None) == -1
     assert "expected 1 or top_k" in _err()
