@@ -1308,6 +1308,31 @@ def test_hostile_indices_stay_inside_the_tensors():
     assert_linear_ok(out[4:], o.linear_fp32(xs[4:], qw[2], qs[2], s), xs[4:], 64, "rows of the clamped last segment")
 
 
+@pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
+def test_hostile_indices_other_model_dtypes(model_dtype):
+    # the same clamping in the expert matmuls of the float32 / bfloat16 models
+    s = SCHEMES["q4f16_1"]
+    dt = _TORCH_OF[model_dtype]
+    rng = np.random.default_rng(9)
+    w32 = o.round_to((rng.standard_normal((3, 16, 64)) * 0.05).astype(np.float32), model_dtype)
+    qw_ref, qs_ref = o.quantize_dt(w32, s, model_dtype)
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).to(dt).to(DEV)
+    x32 = o.round_to(rng.standard_normal((1, 64)).astype(np.float32), model_dtype)
+    eids = torch.tensor([[-4, 9]], dtype=torch.int32, device=DEV)  # clamped to experts 0 and 2
+    y = ops.moe_gemv(torch.from_numpy(x32).to(dt).to(DEV), qw, qs, eids, 4, 32)
+    ref = o.moe_dequantize_gemv_dt_fp64(x32, qw_ref, qs_ref, np.array([[0, 2]], np.int32), s, model_dtype)
+    _assert_dt_matmul_ok(y, ref, x32, 64, model_dtype, "expert ids clamped")
+    for rows in (6, 70):  # the dot-product kernel's segments and the tiled kernels' row tiles
+        xs32 = o.round_to(rng.standard_normal((rows, 64)).astype(np.float32), model_dtype)
+        bad_ip = torch.tensor([0, 4, 2, 9999], dtype=torch.int32, device=DEV)  # read as [0,4) [4,4) [2,rows)
+        out = ops.moe_group_gemm(torch.from_numpy(xs32).to(dt).to(DEV), qw, qs, bad_ip, 4, 32)
+        torch.cuda.synchronize()
+        assert tuple(out.shape) == (rows, 16) and torch.isfinite(out.float()).all()
+        full = o.dequantize_group_gemm_dt_fp64(xs32, qw_ref, qs_ref, np.array([0, 2, 2, rows], np.int32), s, model_dtype)
+        _assert_dt_matmul_ok(out[:2], full[:2], xs32[:2], 64, model_dtype, "rows of the first segment only")
+        _assert_dt_matmul_ok(out[4:], full[4:], xs32[4:], 64, model_dtype, "rows of the clamped last segment")
+
+
 # ------------------------------------------------------------------ HIP graph capture
 
 def test_linear_and_moe_replay_in_hip_graph():
