@@ -146,9 +146,9 @@ MI355GQ_API int mi355gq_linear_residual(const void* x, const void* q_weight, con
  * mi355gq_linear for the other model dtypes (see mi355gq_quantize_dt): x, q_scale and bias carry
  * model_dtype (MI355GQ_F32 or MI355GQ_BF16; MI355GQ_F16 forwards to mi355gq_linear), y carries
  * out_dtype = model_dtype or MI355GQ_F32.  Weights are dequantised as GroupQuantize._dequantize does
- * ((q - m) * scale rounded to the model dtype) and accumulated in fp32.  Exception: one or two bfloat16 rows
- * (K <= 16384) run the float16 path's register GEMV, which scales each group's integer dot product in fp32 and so
- * skips that per-weight rounding (as mi355gq_linear does for float16).  No residual / SiLU epilogues.
+ * ((q - m) * scale rounded to the model dtype) and accumulated in fp32.  Exception: up to 8 bfloat16 rows run the
+ * float16 path's register GEMV / quad-row kernel, which scale each group's integer dot product in fp32 and so skip
+ * that per-weight rounding (as mi355gq_linear does for float16).  No residual / SiLU epilogues.
  * workspace: device scratch of at least mi355gq_linear_dt_workspace_bytes(M, N, K, ...) bytes, 16-byte aligned,
  * or null (then few-row bfloat16 matmuls run unsplit: slower, same result up to summation order).
  */

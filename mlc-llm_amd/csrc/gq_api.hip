@@ -480,7 +480,6 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
     if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemv launch");
   }
   if (model_dtype == MI355GQ_BF16 && M > 1 && (K & 7) == 0 && aligned16(x)) {
-    // the float16 GEMM's tiles on the bf16 matrix instruction (from 3 rows on; before, where the GEMV declines)
     gq::GemmArgs g{};
     g.x = static_cast<const uint16_t*>(x);
     g.q_weight = static_cast<const uint32_t*>(q_weight);
@@ -492,6 +491,12 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
     g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
     g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
     g.bf16 = 1;
+    // up to 8 rows: the float16 path's quad-row kernel on the bf16 4x4x4 matrix instruction
+    if (M <= 8) {
+      const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
+      if (q != hipErrorNotSupported) return hip_result(q, "linear_dt quad-row launch");
+    }
+    // the float16 GEMM's tiles on the bf16 matrix instruction
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemm launch");
   }
@@ -672,6 +677,12 @@ int mi355gq_moe_group_gemm_dt(const void* x, int64_t rows, const void* q_weight,
     g.rows = rows; g.N = N; g.K = K; g.num_experts = num_experts;
     g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
     g.bf16 = 1;
+    // few rows in total: every expert streams its weights for a handful of rows (as in float16)
+    const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;
+    if (rows <= quad_rows && rows <= 128) {
+      const hipError_t q = gq::launch_quadrow(g, static_cast<int>(rows), as_stream(stream));
+      if (q != hipErrorNotSupported) return hip_result(q, "moe_group_gemm_dt quad-row launch");
+    }
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "moe_group_gemm_dt gemm launch");
   }

@@ -50,6 +50,7 @@ struct QuadParams {
   int paired;       // fused gate/up form: y is [rows, N / 2] fp16
   const int32_t* x_rows;  // null, or the row of x each activation row reads (int32 [rows])
   int x_src_rows;         // rows of x when x_rows is set
+  int bf16;               // x, scales, bias, residual and a 16-bit y are bfloat16
 };
 
 template <int CTRL>
@@ -66,13 +67,31 @@ __device__ __forceinline__ float4_t mfma4(uint32_t a0, uint32_t a1, uint32_t b0,
                                             __builtin_bit_cast(half4_t, b), c, 0, 0, 0);
 }
 
+// the same blocks on bfloat16 operands (v_mfma_f32_4x4x4_16b_bf16)
+__device__ __forceinline__ float4_t mfma4_bf16(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
+  typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+  typedef short short4_t __attribute__((ext_vector_type(4)));
+  const u2 a = {a0, a1}, b = {b0, b1};
+  return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(short4_t, a), __builtin_bit_cast(short4_t, b), c, 0,
+                                                0, 0);
+}
+
 // NBQ: activation rows / 4 (rows past the segment are zero); U: iterations per item
 // MODE 1: a bias or residual operand exists (template flag: their loads are extra memory
 // instructions per item); MODE 2: fused gate/up form
-template <int BITS, int NBQ, int U, int MODE>
+// BF: bfloat16 model (x, scales, bias, residual and a 16-bit result are bfloat16).  0x4300 | q is the bfloat16
+// 128 + q, so every field is shifted down to bit 0 of its half instead of being rescaled afterwards, and all
+// operand classes share the offset 128 + m.
+template <int BITS, int NBQ, int U, int MODE, bool BF = false>
 __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;  // 2: fused gate/up form, quad = 2 (gate, up) pairs
-  constexpr uint32_t kMagic = 0x64006400u;
+  static_assert(!(BF && PAIRED), "the fused gate/up form is float16 only");
+  constexpr uint32_t kMagic = BF ? 0x43004300u : 0x64006400u;
+  auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
+  auto to_out = [](float v) { return BF ? f2bf(v) : f2h(v); };
+  auto mm = [](uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
+    return BF ? mfma4_bf16(a0, a1, b0, b1, c) : mfma4(a0, a1, b0, b1, c);
+  };
   constexpr int G = GemvTraits<BITS>::G;    // values per group: 32 | 40
   constexpr int CH = GemvTraits<BITS>::CH;  // 16-byte words of x per (activation row, group): 4 | 5
   constexpr int XB = BITS == 4 ? 4 : 3;     // (activation row, group) pairs a thread stages per round
@@ -211,7 +230,7 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
               const uint4 r = ok[i][c] ? raw[i][c] : make_uint4(0, 0, 0, 0);
               nat[4 * c + 0] = r.x; nat[4 * c + 1] = r.y; nat[4 * c + 2] = r.z; nat[4 * c + 3] = r.w;
             }
-            const float corr = permute_group<BITS>(nat, xr);
+            const float corr = permute_group<BITS, BF>(nat, xr);
             const int lp = q & 63, bi = q >> 6;
             if constexpr (BITS == 4) {
 #pragma unroll
@@ -253,26 +272,37 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
           if constexpr (BITS == 4) {
             const uint32_t w8 = w[d] >> 8;
             lo[d][0] = and_or(w[d], 0x000f000fu, kMagic);
-            hi[d][0] = and_or(w[d], 0x00f000f0u, kMagic);
             lo[d][1] = and_or(w8, 0x000f000fu, kMagic);
-            hi[d][1] = and_or(w8, 0x00f000f0u, kMagic);
+            if constexpr (BF) {
+              hi[d][0] = and_or(w[d] >> 4, 0x000f000fu, kMagic);
+              hi[d][1] = and_or(w[d] >> 12, 0x000f000fu, kMagic);
+            } else {
+              hi[d][0] = and_or(w[d], 0x00f000f0u, kMagic);
+              hi[d][1] = and_or(w8, 0x00f000f0u, kMagic);
+            }
           } else {
             // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
             const uint32_t t = (w[d] & 0x0000ffffu) | ((w[d] << 1) & 0xffff0000u);
             const uint32_t t9 = t >> 9;
             lo[d][0] = and_or(t, 0x00070007u, kMagic);   // fields (0,5)
             lo[d][1] = and_or(t9, 0x00070007u, kMagic);  // fields (3,8)
-            hi[d][0] = and_or(t, 0x00380038u, kMagic);   // fields (1,6) x 8
-            hi[d][1] = and_or(t9, 0x00380038u, kMagic);  // fields (4,9) x 8
-            a64[d >> 1][d & 1] = and_or(t, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+            if constexpr (BF) {
+              hi[d][0] = and_or(t >> 3, 0x00070007u, kMagic);   // fields (1,6)
+              hi[d][1] = and_or(t >> 12, 0x00070007u, kMagic);  // fields (4,9)
+              a64[d >> 1][d & 1] = and_or(t >> 6, 0x00070007u, kMagic);  // fields (2,7)
+            } else {
+              hi[d][0] = and_or(t, 0x00380038u, kMagic);   // fields (1,6) x 8
+              hi[d][1] = and_or(t9, 0x00380038u, kMagic);  // fields (4,9) x 8
+              a64[d >> 1][d & 1] = and_or(t, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+            }
           }
         }
         // the four rows' scales of this block: lane 4b+i holds row i's
         float sv[4];
-        sv[0] = h2f(static_cast<uint16_t>(dpp_u<0x00>(sc[u])));
-        sv[1] = h2f(static_cast<uint16_t>(dpp_u<0x55>(sc[u])));
-        sv[2] = h2f(static_cast<uint16_t>(dpp_u<0xAA>(sc[u])));
-        sv[3] = h2f(static_cast<uint16_t>(dpp_u<0xFF>(sc[u])));
+        sv[0] = to_f32(static_cast<uint16_t>(dpp_u<0x00>(sc[u])));
+        sv[1] = to_f32(static_cast<uint16_t>(dpp_u<0x55>(sc[u])));
+        sv[2] = to_f32(static_cast<uint16_t>(dpp_u<0xAA>(sc[u])));
+        sv[3] = to_f32(static_cast<uint16_t>(dpp_u<0xFF>(sc[u])));
 #pragma unroll
         for (int bq = 0; bq < NBQ; ++bq) {
           if (bq > 0 && 4 * bq >= m_valid) continue;  // uniform: this segment has no such rows
@@ -281,22 +311,24 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             const uint4 xv = smem[(bi * CH + d) * 64 + lane];
-            tl = mfma4(lo[d][0], lo[d][1], xv.x, xv.y, tl);
-            th = mfma4(hi[d][0], hi[d][1], xv.z, xv.w, th);
+            tl = mm(lo[d][0], lo[d][1], xv.x, xv.y, tl);
+            th = mm(hi[d][0], hi[d][1], xv.z, xv.w, th);
           }
           const float corr = corr_lds[bi * 64 + lane];
+          // (bfloat16: the classes were shifted, not scaled)
+          constexpr float kHi = BF ? 1.0f : (BITS == 4 ? 0.0625f : 0.125f), k64 = BF ? 1.0f : 0.015625f;
           if constexpr (BITS == 4) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              acc[bq][i] = fmaf(sv[i], fmaf(th[i], 0.0625f, tl[i]) - corr, acc[bq][i]);
+              acc[bq][i] = fmaf(sv[i], fmaf(th[i], kHi, tl[i]) - corr, acc[bq][i]);
           } else {
             const uint4 xv = smem[(bi * CH + 4) * 64 + lane];
             float4_t t64 = {0.f, 0.f, 0.f, 0.f};
-            t64 = mfma4(a64[0][0], a64[0][1], xv.x, xv.y, t64);
-            t64 = mfma4(a64[1][0], a64[1][1], xv.z, xv.w, t64);
+            t64 = mm(a64[0][0], a64[0][1], xv.x, xv.y, t64);
+            t64 = mm(a64[1][0], a64[1][1], xv.z, xv.w, t64);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              acc[bq][i] = fmaf(sv[i], fmaf(t64[i], 0.015625f, fmaf(th[i], 0.125f, tl[i])) - corr, acc[bq][i]);
+              acc[bq][i] = fmaf(sv[i], fmaf(t64[i], k64, fmaf(th[i], kHi, tl[i])) - corr, acc[bq][i]);
           }
         }
       }
@@ -325,16 +357,16 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
               *part = make_float4(v[0], v[1], v[2], v[3]);
             } else {
               if (EXTRA && p.bias != nullptr) {
-                v[0] += h2f(static_cast<uint16_t>(bias_bits.x & 0xffffu));
-                v[1] += h2f(static_cast<uint16_t>(bias_bits.x >> 16));
-                v[2] += h2f(static_cast<uint16_t>(bias_bits.y & 0xffffu));
-                v[3] += h2f(static_cast<uint16_t>(bias_bits.y >> 16));
+                v[0] += to_f32(static_cast<uint16_t>(bias_bits.x & 0xffffu));
+                v[1] += to_f32(static_cast<uint16_t>(bias_bits.x >> 16));
+                v[2] += to_f32(static_cast<uint16_t>(bias_bits.y & 0xffffu));
+                v[3] += to_f32(static_cast<uint16_t>(bias_bits.y >> 16));
               }
               if (EXTRA && p.residual != nullptr) {
-                v[0] += h2f(static_cast<uint16_t>(res_bits[bq].x & 0xffffu));
-                v[1] += h2f(static_cast<uint16_t>(res_bits[bq].x >> 16));
-                v[2] += h2f(static_cast<uint16_t>(res_bits[bq].y & 0xffffu));
-                v[3] += h2f(static_cast<uint16_t>(res_bits[bq].y >> 16));
+                v[0] += to_f32(static_cast<uint16_t>(res_bits[bq].x & 0xffffu));
+                v[1] += to_f32(static_cast<uint16_t>(res_bits[bq].x >> 16));
+                v[2] += to_f32(static_cast<uint16_t>(res_bits[bq].y & 0xffffu));
+                v[3] += to_f32(static_cast<uint16_t>(res_bits[bq].y >> 16));
               }
               const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
               if constexpr (PAIRED) {
@@ -346,8 +378,8 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
                     make_float4(v[0], v[1], v[2], v[3]);
               } else {
                 uint2 o;
-                o.x = static_cast<uint32_t>(f2h(v[0])) | (static_cast<uint32_t>(f2h(v[1])) << 16);
-                o.y = static_cast<uint32_t>(f2h(v[2])) | (static_cast<uint32_t>(f2h(v[3])) << 16);
+                o.x = static_cast<uint32_t>(to_out(v[0])) | (static_cast<uint32_t>(to_out(v[1])) << 16);
+                o.y = static_cast<uint32_t>(to_out(v[2])) | (static_cast<uint32_t>(to_out(v[3])) << 16);
                 *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.y) + oi) = o;
               }
             }
@@ -370,22 +402,28 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
   }
 }
 
-template <int BITS, int NBQ, int U, int MODE>
+template <int BITS, int NBQ, int U, int MODE, bool BF = false>
 static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                     hipStream_t s) {
   if (lds > 65536) {
     const hipError_t e =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE>), grid, dim3(threads), lds, s, p);
+  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF>), grid, dim3(threads), lds, s, p);
   return hipGetLastError();
 }
 
 template <int BITS, int NBQ, int U>
 static hipError_t launch_quad_cfg(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                   hipStream_t s) {
+  if (p.bf16) {
+    if (p.paired) return hipErrorNotSupported;
+    return (p.bias != nullptr || p.residual != nullptr)
+               ? launch_quad_extra<BITS, NBQ, U, 1, true>(p, grid, threads, lds, s)
+               : launch_quad_extra<BITS, NBQ, U, 0, true>(p, grid, threads, lds, s);
+  }
   if (p.paired) return launch_quad_extra<BITS, NBQ, U, 2>(p, grid, threads, lds, s);
   return (p.bias != nullptr || p.residual != nullptr)
              ? launch_quad_extra<BITS, NBQ, U, 1>(p, grid, threads, lds, s)
@@ -408,6 +446,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   p.x = a.x; p.qw = a.q_weight; p.qs = a.q_scale; p.bias = a.bias; p.residual = a.residual; p.y = a.y;
   p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64; p.paired = a.paired;
   p.x_rows = a.x_rows; p.x_src_rows = static_cast<int>(a.x_src_rows);
+  p.bf16 = a.bf16;
   p.rows = static_cast<int>(a.rows); p.N = static_cast<int>(a.N); p.K = static_cast<int>(a.K);
   p.ng = static_cast<int>((a.K + G - 1) / G);
   p.nw = 4 * p.ng;

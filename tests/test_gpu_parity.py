@@ -878,7 +878,9 @@ def test_other_model_dtypes_golden(golden, model_dtype):
         assert np.array_equal(_carrier(ops.dequantize(qw, qs, k, 4, 32)), z["dequant"])
         y = ops.linear(torch.from_numpy(z["x"]).to(dt).to(DEV), qw, qs, 4, 32, out_dtype=torch.float32)
         err = np.linalg.norm(y.double().cpu().numpy() - z["y"]) / np.linalg.norm(z["y"])
-        assert err <= 2e-6, err
+        # (bfloat16, few rows: the kernels that scale group sums skip _dequantize's per-weight rounding, which
+        #  the fixture's product includes: the matmul tolerance applies, not the fp32-accumulation one)
+        assert err <= (2e-3 if model_dtype == "bfloat16" else 2e-6), err
 
 
 def test_other_model_dtypes_modules():
@@ -922,6 +924,8 @@ def test_other_model_dtypes_modules():
     ("q4f16_1", 1, 512, 4096), ("q4f16_1", 2, 100, 1000), ("q4f16_1", 4, 257, 2048), ("q4f16_1", 8, 128, 8192),
     ("q4f16_1", 3, 64, 13), ("q4f16_1", 1, 40, 40000),                     # ragged K; K past the GEMV's LDS
     ("q4f16_1", 1, 130, 14336), ("q4f16_1", 2, 96, 8192), ("q4f16_1", 2, 33, 1001), ("q3f16_1", 2, 64, 2000),
+    ("q4f16_1", 2, 64, 14336), ("q4f16_1", 3, 1024, 4096), ("q4f16_1", 5, 64, 14336), ("q4f16_1", 7, 132, 1000),
+    ("q3f16_1", 4, 96, 4096), ("q3f16_1", 8, 64, 10000),
     ("q4f16_1", 9, 256, 512), ("q4f16_1", 130, 200, 1024), ("q4f16_1", 300, 384, 360), ("q4f16_1", 64, 130, 100),
     ("q3f16_1", 1, 256, 4096), ("q3f16_1", 5, 96, 1000), ("q3f16_1", 200, 136, 2000),
 ])
@@ -941,8 +945,11 @@ def test_linear_other_model_dtypes(model_dtype, bits_name, m, n, k):
     y32 = ops.linear(x, qw, qs, s.bits, s.group_size, b, out_dtype=torch.float32)
     assert y32.dtype == torch.float32 and tuple(y32.shape) == (m, n)
     err = y32.double().cpu().numpy() - ref
-    if model_dtype == "bfloat16" and m <= 2 and -(-k // s.group_size) <= 512:  # (8 groups per lane at most)
-        # the register GEMV scales each group's integer dot product, so its operands are the weights before
+    ng = -(-k // s.group_size)
+    # one row up to 8 groups per lane, two rows up to 4: the register GEMV; 2..8 rows the quad-row kernel
+    unrounded = (m == 1 and ng <= 512) or (m == 2 and ng <= 256) or (2 <= m <= 8 and k % 8 == 0 and n % 4 == 0)
+    if model_dtype == "bfloat16" and unrounded:
+        # these kernels scale each group's integer dot product, so their operands are the weights before
         # _dequantize's rounding to bfloat16: exact against those, and within the matmul tolerance (2^-9 per
         # weight, random in sign) of the product with the rounded ones
         exact = y32.double().cpu().numpy() - o.linear_dt_fp64(x32, qw_ref, qs_ref, s, model_dtype, b32, unrounded_weights=True)
