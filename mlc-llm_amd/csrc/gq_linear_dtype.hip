@@ -106,7 +106,8 @@ typedef float float2_t __attribute__((ext_vector_type(2)));
 // Persistent waves, two weight rows per step, the loads of the next two steps in flight (the
 // structure of the float16 register GEMV); x lives in LDS in the model dtype, zero beyond K, and is
 // read once per group for both rows.  Lane l owns groups l + 64 * it, it < ITERS.
-//  * float32: w = (q - m) * s as _dequantize rounds it, then one FMA per activation row;
+//  * float32: one FMA per weight and activation row on the integer field itself; the group's sum is scaled
+//    and offset once (s * (sum x q - m sum x)), as the float16 kernels do;
 //  * bfloat16: (q - m) * s is exact in float32 (4 x 8 significant bits), v_cvt_pk_bf16_f32 rounds
 //    two of them to the bf16 pair _dequantize would hold, and v_dot2_f32_bf16 multiplies the pair
 //    with the matching pair of x (exact products, fp32 accumulation).
@@ -176,6 +177,19 @@ __global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nse
     __syncthreads();
 
     const float m = static_cast<float>(S::kMaxInt);
+    // float32: sum of x over each of this lane's groups, for the offset term of the scaled group sums below
+    float xsum[BF ? 1 : NB][BF ? 1 : ITERS];
+    if constexpr (!BF) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          float t = 0.0f;
+#pragma unroll
+          for (int i = 0; i < G; ++i) t += xs[b * kpad + gidx[it] * GS + i];
+          xsum[b][it] = t;
+        }
+    }
     auto reduce = [&](int set, const uint4 (&wc)[2][ITERS], const float (&sc)[2][ITERS]) {
       float acc[2][NB];
 #pragma unroll
@@ -190,6 +204,11 @@ __global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nse
           s[r] = gok[it] ? sc[r][it] : 0.0f;  // lanes past the last group add nothing
           ms[r] = -m * s[r];
         }
+        float gacc[2][NB];  // float32: sum of x * q over the group, scaled once below
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+          for (int b = 0; b < NB; ++b) gacc[r][b] = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           // the word's E values of x for every activation row, read once for both weight rows
@@ -246,13 +265,19 @@ __global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nse
               }
             } else {
 #pragma unroll
-              for (int i = 0; i < E; ++i) {
-                const float wv = (q[i] - m) * s[r];  // one rounding, as _dequantize
+              for (int i = 0; i < E; ++i)
 #pragma unroll
-                for (int b = 0; b < NB; ++b) acc[r][b] = fmaf(wv, xf[b][i], acc[r][b]);
-              }
+                for (int b = 0; b < NB; ++b) gacc[r][b] = fmaf(q[i], xf[b][i], gacc[r][b]);
             }
           }
+        }
+        if constexpr (!BF) {
+          // s * sum x (q - m): differs from the sum of x * round((q - m) * s) by 2^-24 per weight, the size of the
+          // fp32 accumulation's own rounding
+#pragma unroll
+          for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) acc[r][b] = fmaf(s[r], fmaf(-m, xsum[b][it], gacc[r][b]), acc[r][b]);
         }
       }
 #pragma unroll
