@@ -148,10 +148,16 @@ MI355GQ_API int mi355gq_linear_residual(const void* x, const void* q_weight, con
  * out_dtype = model_dtype or MI355GQ_F32.  Weights are dequantised as GroupQuantize._dequantize does
  * ((q - m) * scale rounded to the model dtype) and accumulated in fp32.  Exception: up to 8 bfloat16 rows run the
  * float16 path's register GEMV / quad-row kernel, which scale each group's integer dot product in fp32 and so skip
- * that per-weight rounding (as mi355gq_linear does for float16).  No residual / SiLU epilogues.
+ * that per-weight rounding (as mi355gq_linear does for float16).  No SiLU epilogue.
  * workspace: device scratch of at least mi355gq_linear_dt_workspace_bytes(M, N, K, ...) bytes, 16-byte aligned,
  * or null (then few-row bfloat16 matmuls run unsplit: slower, same result up to summation order).
  */
+/* mi355gq_linear_residual for the other model dtypes: residual [M, N] carries model_dtype (it may be y itself when
+ * out_dtype == model_dtype). */
+MI355GQ_API int mi355gq_linear_residual_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                               const void* residual, int64_t M, int64_t N, int64_t K, int bits,
+                               int group_size, int model_dtype, int out_dtype, void* y, void* workspace,
+                               int64_t workspace_bytes, mi355gq_stream_t stream);
 MI355GQ_API int64_t mi355gq_linear_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size,
                                           int model_dtype);
 MI355GQ_API int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias,

@@ -445,12 +445,13 @@ static int moe_gemv_impl(const void* x, int64_t x_rows, const void* q_weight, co
   return hip_result(e, "moe_gemv launch");
 }
 
-int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias, int64_t M,
-                      int64_t N, int64_t K, int bits, int group_size, int model_dtype, int out_dtype, void* y,
-                      void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
+static int linear_dt_impl(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                          const void* residual, int64_t M, int64_t N, int64_t K, int bits, int group_size,
+                          int model_dtype, int out_dtype, void* y, void* workspace, int64_t workspace_bytes,
+                          mi355gq_stream_t stream) {
   GQ_CHECK(check_model_dtype(model_dtype, "linear_dt"));
   if (model_dtype == MI355GQ_F16)
-    return linear_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, out_dtype, y, workspace,
+    return linear_impl(x, q_weight, q_scale, bias, residual, M, N, K, bits, group_size, out_dtype, y, workspace,
                        workspace_bytes, stream);
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(M >= 0 && N >= 0 && K >= 1 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
@@ -460,8 +461,8 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
   if (M == 0 || N == 0) return MI355GQ_OK;
   GQ_REQUIRE(y && x && q_weight && q_scale, "linear_dt: null pointer");
   const bool f32 = model_dtype == MI355GQ_F32;
-  GQ_REQUIRE(aligned16(q_weight) && (f32 ? aligned4(x) && aligned4(q_scale) && aligned4(bias)
-                                         : aligned2(x) && aligned2(q_scale) && aligned2(bias)) &&
+  GQ_REQUIRE(aligned16(q_weight) && (f32 ? aligned4(x) && aligned4(q_scale) && aligned4(bias) && aligned4(residual)
+                                         : aligned2(x) && aligned2(q_scale) && aligned2(bias) && aligned2(residual)) &&
                  (out_dtype == MI355GQ_F32 ? aligned4(y) : aligned2(y)),
              "linear_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
   if (model_dtype == MI355GQ_BF16 && M <= 2 && aligned16(x)) {
@@ -471,6 +472,7 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
     a.q_weight = static_cast<const uint32_t*>(q_weight);
     a.q_scale = static_cast<const uint16_t*>(q_scale);
     a.bias = static_cast<const uint16_t*>(bias);
+    a.residual = static_cast<const uint16_t*>(residual);
     a.y = y;
     a.expert_ids = nullptr;
     a.M = M; a.N = N; a.K = K; a.slots = 1; a.x_slot_stride = 0; a.num_experts = 1;
@@ -485,6 +487,7 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
     g.q_weight = static_cast<const uint32_t*>(q_weight);
     g.q_scale = static_cast<const uint16_t*>(q_scale);
     g.bias = static_cast<const uint16_t*>(bias);
+    g.residual = static_cast<const uint16_t*>(residual);
     g.y = y;
     g.indptr = nullptr; g.indptr_i64 = 0;
     g.rows = M; g.N = N; g.K = K; g.num_experts = 1;
@@ -500,9 +503,25 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemm launch");
   }
-  return hip_result(gq::launch_linear_dt(x, static_cast<const uint32_t*>(q_weight), q_scale, bias, M, N, K, bits,
-                                         group_size, model_dtype, out_dtype, y, as_stream(stream)),
+  return hip_result(gq::launch_linear_dt(x, static_cast<const uint32_t*>(q_weight), q_scale, bias, residual, M, N, K,
+                                         bits, group_size, model_dtype, out_dtype, y, as_stream(stream)),
                     "linear_dt launch");
+}
+
+int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias, int64_t M,
+                      int64_t N, int64_t K, int bits, int group_size, int model_dtype, int out_dtype, void* y,
+                      void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
+  return linear_dt_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, model_dtype, out_dtype, y,
+                        workspace, workspace_bytes, stream);
+}
+
+int mi355gq_linear_residual_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                               const void* residual, int64_t M, int64_t N, int64_t K, int bits, int group_size,
+                               int model_dtype, int out_dtype, void* y, void* workspace, int64_t workspace_bytes,
+                               mi355gq_stream_t stream) {
+  GQ_REQUIRE(residual != nullptr || M == 0 || N == 0, "linear_residual_dt: residual is null");
+  return linear_dt_impl(x, q_weight, q_scale, bias, residual, M, N, K, bits, group_size, model_dtype, out_dtype, y,
+                        workspace, workspace_bytes, stream);
 }
 
 int mi355gq_moe_gemv(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,

@@ -75,9 +75,9 @@ hipError_t launch_dequantize_dt(const int32_t* ids, int64_t out_rows, const uint
                                 int64_t table_rows, int64_t K, int bits, int group_size, int model_dtype,
                                 void* out, hipStream_t s);
 // out_kind: MODEL_F32 or MODEL_BF16
-hipError_t launch_linear_dt(const void* x, const uint32_t* qw, const void* qs, const void* bias, int64_t M, int64_t N,
-                            int64_t K, int bits, int group_size, int model_dtype, int out_kind, void* y,
-                            hipStream_t s);
+hipError_t launch_linear_dt(const void* x, const uint32_t* qw, const void* qs, const void* bias, const void* residual,
+                            int64_t M, int64_t N, int64_t K, int bits, int group_size, int model_dtype, int out_kind,
+                            void* y, hipStream_t s);
 // the two expert matmuls over stacked q_weight / q_scale, everything else in model_dtype
 hipError_t launch_moe_gemv_dt(const void* x, bool x_one_row, const uint32_t* qw, const void* qs, const int32_t* ids,
                               int64_t slots, int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,

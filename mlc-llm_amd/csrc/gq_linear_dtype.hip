@@ -55,6 +55,7 @@ struct LinParams {
   const uint32_t* qw;
   const void* qs;
   const void* bias;
+  const void* residual;  // [M, N] in the model dtype, added to the result, or null (may be y itself)
   void* y;
   int M, N, K, ng, nw;
   int out_kind;
@@ -288,7 +289,9 @@ __global__ __launch_bounds__(256) void gemv_dt_kernel(const LinParams p, int nse
           const float t = wave_sum(acc[r][b]);
           if (lane == 0 && m0 + b < sg.rows && row < p.N) {
             const float bias = p.bias != nullptr ? T::load(p.bias, row) : 0.0f;
-            store_out(p.y, (sg.y_row0 + m0 + b) * p.N + row, t + bias, p.out_kind);
+            const int64_t oi = (sg.y_row0 + m0 + b) * p.N + row;
+            const float res = p.residual != nullptr ? T::load(p.residual, oi) : 0.0f;
+            store_out(p.y, oi, t + bias + res, p.out_kind);
           }
         }
       }
@@ -440,7 +443,11 @@ __global__ __launch_bounds__(256) void gemm_dt_kernel(const LinParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (row < sg.rows && col < p.N) store_out(p.y, (sg.y_row0 + row) * p.N + col, acc[i][j][r] + bias, p.out_kind);
+        if (row < sg.rows && col < p.N) {
+          const int64_t oi = (sg.y_row0 + row) * p.N + col;
+          const float res = p.residual != nullptr ? T::load(p.residual, oi) : 0.0f;
+          store_out(p.y, oi, acc[i][j][r] + bias + res, p.out_kind);
+        }
       }
     }
 }
@@ -478,6 +485,8 @@ hipError_t launch_dt(const LinParams& p, hipStream_t s) {
         if (!stacks) {
           q.x = static_cast<const char*>(p.x) + static_cast<size_t>(m0) * p.K * x_el;
           q.y = static_cast<char*>(p.y) + static_cast<size_t>(m0) * p.N * y_el;
+          if (p.residual != nullptr)
+            q.residual = static_cast<const char*>(p.residual) + static_cast<size_t>(m0) * p.N * x_el;
           q.M = p.M - m0 < per_pass ? p.M - m0 : per_pass;
         }
         auto go = [&](auto kern) -> hipError_t {
@@ -536,11 +545,11 @@ static hipError_t launch_dt_any(int64_t M, int64_t N, int64_t K, int bits, int g
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_linear_dt(const void* x, const uint32_t* qw, const void* qs, const void* bias, int64_t M, int64_t N,
-                            int64_t K, int bits, int group_size, int model_dtype, int out_kind, void* y,
-                            hipStream_t s) {
+hipError_t launch_linear_dt(const void* x, const uint32_t* qw, const void* qs, const void* bias, const void* residual,
+                            int64_t M, int64_t N, int64_t K, int bits, int group_size, int model_dtype, int out_kind,
+                            void* y, hipStream_t s) {
   return launch_dt_any(M, N, K, bits, group_size, model_dtype, out_kind, s, [&](LinParams& p) {
-    p.x = x; p.qw = qw; p.qs = qs; p.bias = bias; p.y = y;
+    p.x = x; p.qw = qw; p.qs = qs; p.bias = bias; p.residual = residual; p.y = y;
   });
 }
 

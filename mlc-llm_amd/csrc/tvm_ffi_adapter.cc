@@ -260,6 +260,24 @@ void LinearDt(TensorView x, TensorView q_weight, TensorView q_scale, Optional<Te
         "mlc.gq.linear_dt");
 }
 
+void LinearResidualDt(TensorView x, TensorView q_weight, TensorView q_scale, Optional<TensorView> bias,
+                      TensorView residual, int64_t bits, int64_t group_size, int64_t model_dtype,
+                      Optional<TensorView> workspace, TensorView y) {
+  const int64_t K = x.shape()[x.ndim() - 1], N = q_weight.shape()[0];
+  const int out_dtype = y.dtype().bits == 32 ? MI355GQ_F32 : static_cast<int>(model_dtype);
+  void* ws = workspace.has_value() ? Ptr(workspace.value()) : nullptr;
+  int64_t ws_bytes = 0;
+  if (workspace.has_value()) {
+    ws_bytes = (workspace.value().dtype().bits + 7) / 8;
+    for (int i = 0; i < workspace.value().ndim(); ++i) ws_bytes *= workspace.value().shape()[i];
+  }
+  Check(mi355gq_linear_residual_dt(Ptr(x), Ptr(q_weight), Ptr(q_scale),
+                                   bias.has_value() ? Ptr(bias.value()) : nullptr, Ptr(residual), Rows(x), N, K,
+                                   static_cast<int>(bits), static_cast<int>(group_size),
+                                   static_cast<int>(model_dtype), out_dtype, Ptr(y), ws, ws_bytes, StreamOf(x)),
+        "mlc.gq.linear_residual_dt");
+}
+
 void MoeGemvDt(TensorView x, TensorView q_weight, TensorView q_scale, TensorView expert_ids, int64_t bits,
                int64_t group_size, int64_t model_dtype, TensorView out) {
   Check(mi355gq_moe_gemv_dt(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(expert_ids),
@@ -302,6 +320,7 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.embedding_take_dt", EmbeddingTakeDt)
       .def("mlc.gq.linear_dt", LinearDt)
       .def("mlc.gq.linear_dt_workspace_bytes", LinearDtWorkspaceBytes)
+      .def("mlc.gq.linear_residual_dt", LinearResidualDt)
       .def("mlc.gq.moe_gemv_dt", MoeGemvDt)
       .def("mlc.gq.moe_group_gemm_dt", MoeGroupGemmDt);
 }

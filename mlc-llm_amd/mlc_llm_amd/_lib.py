@@ -36,6 +36,7 @@ SIGNATURES = {
     "mi355gq_quantize_dt": (_I, [_P, _L, _L, _I, _I, _I, _I, _P, _P, _P]),
     "mi355gq_dequantize_dt": (_I, [_P, _P, _L, _L, _I, _I, _I, _P, _P]),
     "mi355gq_embedding_take_dt": (_I, [_P, _L, _P, _P, _L, _L, _I, _I, _I, _P, _P]),
+    "mi355gq_linear_residual_dt": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_linear_dt_workspace_bytes": (_L, [_L, _L, _L, _I, _I, _I]),
     "mi355gq_linear_dt": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_probe_stream_read": (_I, [_P, _L, _P, _L, _P, _P]),

@@ -161,8 +161,6 @@ def _linear_other_dtype(x, q_weight, q_scale, bits, group_size, bias, out_dtype,
     dt = x.dtype
     _chk(q_weight, _STORAGE, "q_weight")
     _chk(q_scale, dt, "q_scale")
-    if residual is not None:
-        raise NotImplementedError("linear: the residual epilogue exists for float16 models only")
     k = x.shape[-1]
     n = q_weight.shape[0]
     _check_qshapes(q_weight, q_scale, (n,), k, bits, group_size)
@@ -181,12 +179,19 @@ def _linear_other_dtype(x, q_weight, q_scale, bits, group_size, bias, out_dtype,
         out = torch.empty((*x.shape[:-1], n), dtype=out_dtype, device=x.device)
     else:
         _chk(out, out_dtype, "out")
+    if residual is not None:
+        _chk(residual, dt, "residual")
+        if tuple(residual.shape) != tuple(out.shape) or not residual.is_contiguous():
+            raise ValueError(f"residual shape {tuple(residual.shape)}, expected contiguous {tuple(out.shape)}")
     ws_bytes = _lib.lib().mi355gq_linear_dt_workspace_bytes(m, n, k, bits, group_size, _MODEL_DTYPES[dt])
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
-    _lib.call("mi355gq_linear_dt", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(),
-              bias.data_ptr() if bias is not None else None, m, n, k, bits, group_size, _MODEL_DTYPES[dt],
-              _MODEL_DTYPES[out_dtype], out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
-              _stream())
+    head = (x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(), bias.data_ptr() if bias is not None else None)
+    tail = (m, n, k, bits, group_size, _MODEL_DTYPES[dt], _MODEL_DTYPES[out_dtype], out.data_ptr(),
+            ws.data_ptr() if ws is not None else None, ws_bytes, _stream())
+    if residual is None:
+        _lib.call("mi355gq_linear_dt", *head, *tail)
+    else:
+        _lib.call("mi355gq_linear_residual_dt", *head, residual.data_ptr(), *tail)
     return out
 
 

@@ -1010,6 +1010,33 @@ def test_moe_matmuls_other_model_dtypes(model_dtype, bits_name, k):
         assert torch.equal(y64, y)
 
 
+@pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("m,n,k", [(1, 256, 4096), (2, 64, 14336), (4, 132, 2048), (8, 64, 1000), (3, 64, 13),
+                                   (16, 128, 8192), (40, 200, 4096), (130, 264, 1024), (600, 384, 512)])
+def test_linear_residual_other_model_dtypes(model_dtype, m, n, k):
+    """The residual operand in every kernel family of the float32 / bfloat16 linear: the result equals the plain
+    linear's float32 output plus the residual, rounded once (same operations in the same order)."""
+    s = SCHEMES["q4f16_1"]
+    dt = _TORCH_OF[model_dtype]
+    rng = np.random.default_rng(m + n + k)
+    w32 = o.round_to((rng.standard_normal((n, k)) * 0.05).astype(np.float32), model_dtype)
+    qw_ref, qs_ref = o.quantize_dt(w32, s, model_dtype)
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).to(dt).to(DEV)
+    x = torch.from_numpy(o.round_to(rng.standard_normal((m, k)).astype(np.float32), model_dtype)).to(dt).to(DEV)
+    b = torch.from_numpy(o.round_to(rng.standard_normal(n).astype(np.float32), model_dtype)).to(dt).to(DEV)
+    res = torch.from_numpy(o.round_to(rng.standard_normal((m, n)).astype(np.float32), model_dtype)).to(dt).to(DEV)
+    y32 = ops.linear(x, qw, qs, 4, 32, b, out_dtype=torch.float32)
+    y = ops.linear(x, qw, qs, 4, 32, b, residual=res)
+    assert y.dtype == dt
+    assert torch.equal(y, (y32 + res.float()).to(dt))
+    y_f32 = ops.linear(x, qw, qs, 4, 32, b, out_dtype=torch.float32, residual=res)
+    assert torch.equal(y_f32, y32 + res.float())
+    # in place: the residual buffer is the output
+    acc = res.clone()
+    ops.linear(x, qw, qs, 4, 32, b, out=acc, residual=acc)
+    assert torch.equal(acc, y)
+
+
 def test_linear_other_model_dtypes_through_the_modules():
     for name in ("q4f32_1", "q4bf16_1", "q4bf16_0"):
         cfg = gq.QUANTIZATION[name]
