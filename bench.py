@@ -396,16 +396,20 @@ def main() -> int:
             res["dequantize"] = {"us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1)}
             del wd
             x1 = torch.randn((1, k), generator=gx, device=dev).to(dt)
-            ms = timed(lambda: ops.linear(x1, qwd, qsd, 4, 32), 10, 2, False)
+            ms = timed(lambda: ops.linear(x1, qwd, qsd, 4, 32), 20, 3, use_graph)
             res["gemv_b1"] = {"us": round(ms * 1e3, 1),
                               "GB/s": round((qwd.numel() * 4 + qsd.numel() * el + (k + n) * el) / ms / 1e6, 1)}
+            x4 = torch.randn((4, k), generator=gx, device=dev).to(dt)
+            ms = timed(lambda: ops.linear(x4, qwd, qsd, 4, 32), 20, 3, use_graph)
+            res["gemv_b4"] = {"us": round(ms * 1e3, 1),
+                              "GB/s": round((qwd.numel() * 4 + qsd.numel() * el + 4 * (k + n) * el) / ms / 1e6, 1)}
             xm_ = torch.randn((2048, k), generator=gx, device=dev).to(dt)
-            ms = timed(lambda: ops.linear(xm_, qwd, qsd, 4, 32), 3, 1, False)
+            ms = timed(lambda: ops.linear(xm_, qwd, qsd, 4, 32), 6 if dt == torch.bfloat16 else 3, 2, False)
             res["gemm_m2048"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(2.0 * 2048 * n * k / ms / 1e9, 1),
                                  "matrix_instruction": "v_mfma_f32_32x32x16_bf16" if dt == torch.bfloat16
                                  else "v_mfma_f32_32x32x2_f32 (157 TFLOP/s peak)"}
             other[label] = res
-            del qwd, qsd, x1, xm_
+            del qwd, qsd, x1, x4, xm_
         extra["other_model_dtypes"] = other
 
     # ---------------------------------------------------------------- CPU baseline (bounded sample)
