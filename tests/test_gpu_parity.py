@@ -572,6 +572,30 @@ def test_gemm_prefill_shape_and_gemv_agreement():
     assert_linear_ok(y32, o.linear_fp32(x, qw, qs, s), x, 4096, "gemm fp32 out")
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("n,k", [(28672, 4096), (4096, 14336)])
+def test_every_row_regime_agrees_at_full_size(name, n, k):
+    """gate_up and down_proj at their real sizes: the same activation row through every regime of the dispatcher
+    (1 .. 2048 rows) must give the product with the dequantised matrix (itself bit-exact against the oracle in
+    the tests above), within the matmul tolerance."""
+    s = SCHEMES[name]
+    g = torch.Generator(device=DEV).manual_seed(n + k)
+    w = (torch.randn((n, k), generator=g, device=DEV) * 0.02).half()
+    qw, qs = ops.quantize(w, s.bits, s.group_size)
+    del w
+    wd = ops.dequantize(qw, qs, k, s.bits, s.group_size).double()
+    x = torch.randn((2048, k), generator=g, device=DEV).half()
+    ref = x[:3].double() @ wd.t()  # rows 0, 1 and 2 of every batch below
+    del wd
+    tol = 1e-2 * float(x[:3].float().abs().max()) * np.sqrt(k) / 64
+    for m in (1, 2, 3, 4, 8, 9, 16, 17, 32, 64, 128, 256, 300, 1024, 2048):
+        y = ops.linear(x[:m].contiguous(), qw, qs, s.bits, s.group_size)
+        rows = min(m, 3)
+        err = (y[:rows].double() - ref[:rows]).abs().max().item()
+        rel = ((y[:rows].double() - ref[:rows]).norm() / ref[:rows].norm()).item()
+        assert err <= tol and rel <= 2e-3, f"{name} {n}x{k} M={m}: max err {err:.3e} (tol {tol:.3e}), rel-L2 {rel:.2e}"
+
+
 def test_linear_module_matches_reference_interface():
     cfg = gq.QUANTIZATION["q4f16_1"]
     lin = gq.GroupQuantizeLinear(256, 96, cfg, bias=True, device=DEV)
