@@ -596,6 +596,28 @@ def test_every_row_regime_agrees_at_full_size(name, n, k):
         assert err <= tol and rel <= 2e-3, f"{name} {n}x{k} M={m}: max err {err:.3e} (tol {tol:.3e}), rel-L2 {rel:.2e}"
 
 
+@pytest.mark.parametrize("n,k", [(28672, 4096), (4096, 14336)])
+def test_every_row_regime_agrees_at_full_size_bfloat16(n, k):
+    """The same for a q4bf16_1 model (register GEMV, quad-row kernel, few-row and large GEMM tiles in bf16).
+    Tolerance: the matmul one plus the rounding of the output to bfloat16 (2^-9 per element)."""
+    g = torch.Generator(device=DEV).manual_seed(n + k + 1)
+    w = (torch.randn((n, k), generator=g, device=DEV) * 0.02).bfloat16()
+    qw, qs = ops.quantize(w, 4, 32)
+    del w
+    wd = ops.dequantize(qw, qs, k, 4, 32).double()
+    x = torch.randn((2048, k), generator=g, device=DEV).bfloat16()
+    ref = x[:3].double() @ wd.t()
+    del wd
+    tol = 1e-2 * float(x[:3].float().abs().max()) * np.sqrt(k) / 64 + 2.0 ** -8 * float(ref.abs().max())
+    for m in (1, 2, 3, 4, 8, 9, 16, 32, 64, 128, 256, 300, 1024, 2048):
+        y = ops.linear(x[:m].contiguous(), qw, qs, 4, 32)
+        assert y.dtype == torch.bfloat16
+        rows = min(m, 3)
+        err = (y[:rows].double() - ref[:rows]).abs().max().item()
+        rel = ((y[:rows].double() - ref[:rows]).norm() / ref[:rows].norm()).item()
+        assert err <= tol and rel <= 3e-3, f"bf16 {n}x{k} M={m}: max err {err:.3e} (tol {tol:.3e}), rel-L2 {rel:.2e}"
+
+
 def test_linear_module_matches_reference_interface():
     cfg = gq.QUANTIZATION["q4f16_1"]
     lin = gq.GroupQuantizeLinear(256, 96, cfg, bias=True, device=DEV)
