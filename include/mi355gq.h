@@ -314,6 +314,28 @@ MI355GQ_API int mi355gq_moe_combine(const void* y, const void* weights, int64_t 
 MI355GQ_API int mi355gq_moe_combine_sorted(const void* y, const void* slot_positions, const void* weights,
                                int64_t T, int64_t top_k, int64_t H, void* out, mi355gq_stream_t stream);
 
+/*
+ * The routing glue for the other model dtypes (logits, weights, activations and results in model_dtype =
+ * MI355GQ_F32 or MI355GQ_BF16; MI355GQ_F16 is the entries above): the same operations with every
+ * intermediate the reference stores rounded to that dtype (softmax in fp32 as in moe_misc.py:205-219; silu in
+ * fp32, rounded, then the product rounded; the combine's product and left-to-right sums rounded).  take_rows /
+ * moe_scatter_output move rows of the dtype's element size.  mi355gq_moe_combine_dt: slot_positions null for y in
+ * slot order (mi355gq_moe_combine), else the expert-sorted order (mi355gq_moe_combine_sorted).
+ */
+MI355GQ_API int mi355gq_gating_softmax_topk_dt(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
+                                   void* weights, void* ids, int model_dtype, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_moe_route_dt(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights,
+                         void* ids, void* token_indices, void* reverse_indices, void* slot_positions,
+                         void* indptr, int indptr_dtype, int model_dtype, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_take_rows_dt(const void* x, const void* indices, int64_t R, int64_t H, int64_t x_rows,
+                         void* out, int model_dtype, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_moe_scatter_output_dt(const void* x, const void* indices, int64_t R, int64_t H, void* out,
+                                  int model_dtype, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_silu_mul_dt(const void* x, int64_t R, int64_t I, void* out, int model_dtype,
+                        mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_moe_combine_dt(const void* y, const void* slot_positions, const void* weights, int64_t T,
+                           int64_t top_k, int64_t H, void* out, int model_dtype, mi355gq_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

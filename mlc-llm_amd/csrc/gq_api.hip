@@ -711,8 +711,9 @@ int mi355gq_moe_group_gemm_dt(const void* x, int64_t rows, const void* q_weight,
                     "moe_group_gemm_dt launch");
 }
 
-int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
-                                void* weights, void* ids, mi355gq_stream_t stream) {
+static int gating_impl(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights, void* ids,
+                       int model_dtype, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "gating_softmax_topk"));
   GQ_REQUIRE(T >= 0 && T < kMaxDim, "gating_softmax_topk: bad T");
   GQ_REQUIRE(num_experts >= 1 && num_experts <= 256, "gating_softmax_topk: num_experts=%lld (1..256)",
              (long long)num_experts);
@@ -720,11 +721,19 @@ int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_exper
              "gating_softmax_topk: top_k=%lld (1..min(8, num_experts))", (long long)top_k);
   if (T == 0) return MI355GQ_OK;
   GQ_REQUIRE(logits && weights && ids, "gating_softmax_topk: null pointer");
-  return hip_result(gq::launch_topk_softmax(static_cast<const uint16_t*>(logits), T,
-                                            static_cast<int>(num_experts), static_cast<int>(top_k),
-                                            static_cast<uint16_t*>(weights),
-                                            static_cast<int32_t*>(ids), as_stream(stream)),
+  return hip_result(gq::launch_topk_softmax(logits, T, static_cast<int>(num_experts), static_cast<int>(top_k), weights,
+                                            static_cast<int32_t*>(ids), model_dtype, as_stream(stream)),
                     "gating_softmax_topk launch");
+}
+
+int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
+                                void* weights, void* ids, mi355gq_stream_t stream) {
+  return gating_impl(logits, T, num_experts, top_k, weights, ids, MI355GQ_F16, stream);
+}
+
+int mi355gq_gating_softmax_topk_dt(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights,
+                                   void* ids, int model_dtype, mi355gq_stream_t stream) {
+  return gating_impl(logits, T, num_experts, top_k, weights, ids, model_dtype, stream);
 }
 
 int mi355gq_moe_cumsum(const void* ids, int64_t T, int64_t top_k, int64_t num_experts,
@@ -770,65 +779,89 @@ int mi355gq_moe_get_indptr(const void* cumsum, int64_t num_experts, int64_t T, i
                     "moe_get_indptr launch");
 }
 
+// rows of 2-byte elements are moved as they are; float32 rows as twice as many 2-byte units
+static int move_rows_impl(const void* x, const void* indices, int64_t R, int64_t H, int64_t x_rows, void* out,
+                          int scatter, int model_dtype, mi355gq_stream_t stream, const char* what) {
+  GQ_CHECK(check_model_dtype(model_dtype, what));
+  GQ_REQUIRE(R >= 0 && H >= 0 && x_rows >= 0 && R < kMaxDim && H < kMaxDim, "%s: bad shape", what);
+  if (R == 0 || H == 0) return MI355GQ_OK;
+  GQ_REQUIRE(x && indices && out, "%s: null pointer", what);
+  const int64_t units = model_dtype == MI355GQ_F32 ? 2 * H : H;
+  GQ_REQUIRE(model_dtype != MI355GQ_F32 || (aligned4(x) && aligned4(out)), "%s: misaligned float32 tensor", what);
+  return hip_result(gq::launch_take_rows(static_cast<const uint16_t*>(x), static_cast<const int32_t*>(indices), R,
+                                         units, x_rows, static_cast<uint16_t*>(out), scatter, as_stream(stream)),
+                    what);
+}
+
 int mi355gq_take_rows(const void* x, const void* indices, int64_t R, int64_t H, int64_t x_rows,
                       void* out, mi355gq_stream_t stream) {
-  GQ_REQUIRE(R >= 0 && H >= 0 && x_rows >= 0 && R < kMaxDim && H < kMaxDim, "take_rows: bad shape");
-  if (R == 0 || H == 0) return MI355GQ_OK;
-  GQ_REQUIRE(x && indices && out, "take_rows: null pointer");
-  return hip_result(gq::launch_take_rows(static_cast<const uint16_t*>(x),
-                                         static_cast<const int32_t*>(indices), R, H, x_rows,
-                                         static_cast<uint16_t*>(out), 0, as_stream(stream)),
-                    "take_rows launch");
+  return move_rows_impl(x, indices, R, H, x_rows, out, 0, MI355GQ_F16, stream, "take_rows");
+}
+
+int mi355gq_take_rows_dt(const void* x, const void* indices, int64_t R, int64_t H, int64_t x_rows, void* out,
+                         int model_dtype, mi355gq_stream_t stream) {
+  return move_rows_impl(x, indices, R, H, x_rows, out, 0, model_dtype, stream, "take_rows");
 }
 
 int mi355gq_moe_scatter_output(const void* x, const void* indices, int64_t R, int64_t H, void* out,
                                mi355gq_stream_t stream) {
-  GQ_REQUIRE(R >= 0 && H >= 0 && R < kMaxDim && H < kMaxDim, "moe_scatter_output: bad shape");
-  if (R == 0 || H == 0) return MI355GQ_OK;
-  GQ_REQUIRE(x && indices && out, "moe_scatter_output: null pointer");
-  return hip_result(gq::launch_take_rows(static_cast<const uint16_t*>(x),
-                                         static_cast<const int32_t*>(indices), R, H, R,
-                                         static_cast<uint16_t*>(out), 1, as_stream(stream)),
-                    "moe_scatter_output launch");
+  return move_rows_impl(x, indices, R, H, R, out, 1, MI355GQ_F16, stream, "moe_scatter_output");
 }
 
-int mi355gq_silu_mul(const void* x, int64_t R, int64_t I, void* out, mi355gq_stream_t stream) {
+int mi355gq_moe_scatter_output_dt(const void* x, const void* indices, int64_t R, int64_t H, void* out,
+                                  int model_dtype, mi355gq_stream_t stream) {
+  return move_rows_impl(x, indices, R, H, R, out, 1, model_dtype, stream, "moe_scatter_output");
+}
+
+static int silu_mul_impl(const void* x, int64_t R, int64_t I, void* out, int model_dtype, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "silu_mul"));
   GQ_REQUIRE(R >= 0 && I >= 0 && R < kMaxDim && I < kMaxDim, "silu_mul: bad shape");
   if (R == 0 || I == 0) return MI355GQ_OK;
   GQ_REQUIRE(x && out, "silu_mul: null pointer");
-  return hip_result(gq::launch_silu_mul(static_cast<const uint16_t*>(x), R, I,
-                                        static_cast<uint16_t*>(out), as_stream(stream)),
-                    "silu_mul launch");
+  return hip_result(gq::launch_silu_mul(x, R, I, out, model_dtype, as_stream(stream)), "silu_mul launch");
+}
+
+int mi355gq_silu_mul(const void* x, int64_t R, int64_t I, void* out, mi355gq_stream_t stream) {
+  return silu_mul_impl(x, R, I, out, MI355GQ_F16, stream);
+}
+
+int mi355gq_silu_mul_dt(const void* x, int64_t R, int64_t I, void* out, int model_dtype, mi355gq_stream_t stream) {
+  return silu_mul_impl(x, R, I, out, model_dtype, stream);
 }
 
 static int moe_combine_impl(const void* y, const void* weights, const void* positions, int64_t T,
-                            int64_t top_k, int64_t H, void* out, mi355gq_stream_t stream) {
+                            int64_t top_k, int64_t H, void* out, int model_dtype, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "moe_combine"));
   GQ_REQUIRE(T >= 0 && H >= 0 && T < kMaxDim && H < kMaxDim && top_k >= 1 && top_k <= 64,
              "moe_combine: bad shape");
   if (T == 0 || H == 0) return MI355GQ_OK;
   GQ_REQUIRE(y && weights && out, "moe_combine: null pointer");
-  return hip_result(gq::launch_moe_combine(static_cast<const uint16_t*>(y),
-                                           static_cast<const uint16_t*>(weights),
-                                           static_cast<const int32_t*>(positions), T,
-                                           static_cast<int>(top_k), H, static_cast<uint16_t*>(out),
-                                           as_stream(stream)),
+  return hip_result(gq::launch_moe_combine(y, weights, static_cast<const int32_t*>(positions), T,
+                                           static_cast<int>(top_k), H, out, model_dtype, as_stream(stream)),
                     "moe_combine launch");
 }
 
 int mi355gq_moe_combine(const void* y, const void* weights, int64_t T, int64_t top_k, int64_t H,
                         void* out, mi355gq_stream_t stream) {
-  return moe_combine_impl(y, weights, nullptr, T, top_k, H, out, stream);
+  return moe_combine_impl(y, weights, nullptr, T, top_k, H, out, MI355GQ_F16, stream);
 }
 
 int mi355gq_moe_combine_sorted(const void* y, const void* slot_positions, const void* weights, int64_t T,
                                int64_t top_k, int64_t H, void* out, mi355gq_stream_t stream) {
   GQ_REQUIRE(slot_positions != nullptr || T == 0, "moe_combine_sorted: slot_positions is null");
-  return moe_combine_impl(y, weights, slot_positions, T, top_k, H, out, stream);
+  return moe_combine_impl(y, weights, slot_positions, T, top_k, H, out, MI355GQ_F16, stream);
 }
 
-int mi355gq_moe_route(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights,
-                      void* ids, void* token_indices, void* reverse_indices, void* slot_positions,
-                      void* indptr, int indptr_dtype, mi355gq_stream_t stream) {
+/* slot_positions null: y is in slot order (moe_combine); else the expert-sorted order (moe_combine_sorted) */
+int mi355gq_moe_combine_dt(const void* y, const void* slot_positions, const void* weights, int64_t T, int64_t top_k,
+                           int64_t H, void* out, int model_dtype, mi355gq_stream_t stream) {
+  return moe_combine_impl(y, weights, slot_positions, T, top_k, H, out, model_dtype, stream);
+}
+
+static int moe_route_impl(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights,
+                          void* ids, void* token_indices, void* reverse_indices, void* slot_positions,
+                          void* indptr, int indptr_dtype, int model_dtype, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "moe_route"));
   GQ_REQUIRE(T >= 0 && T < kMaxDim, "moe_route: bad T");
   GQ_REQUIRE(num_experts >= 1 && num_experts <= 256, "moe_route: num_experts=%lld (1..256)",
              (long long)num_experts);
@@ -845,13 +878,26 @@ int mi355gq_moe_route(const void* logits, int64_t T, int64_t num_experts, int64_
                 (long long)T, (long long)num_experts);
   GQ_REQUIRE(T == 0 || (logits && weights && ids && token_indices && reverse_indices && slot_positions),
              "moe_route: null pointer");
-  return hip_result(gq::launch_moe_route(static_cast<const uint16_t*>(logits), T, static_cast<int>(num_experts),
-                                         static_cast<int>(top_k), static_cast<uint16_t*>(weights),
+  return hip_result(gq::launch_moe_route(logits, T, static_cast<int>(num_experts), static_cast<int>(top_k), weights,
                                          static_cast<int32_t*>(ids), static_cast<int32_t*>(token_indices),
                                          static_cast<int32_t*>(reverse_indices),
                                          static_cast<int32_t*>(slot_positions), indptr_dtype == MI355GQ_I64,
-                                         indptr, as_stream(stream)),
+                                         indptr, model_dtype, as_stream(stream)),
                     "moe_route launch");
+}
+
+int mi355gq_moe_route(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights,
+                      void* ids, void* token_indices, void* reverse_indices, void* slot_positions,
+                      void* indptr, int indptr_dtype, mi355gq_stream_t stream) {
+  return moe_route_impl(logits, T, num_experts, top_k, weights, ids, token_indices, reverse_indices, slot_positions,
+                        indptr, indptr_dtype, MI355GQ_F16, stream);
+}
+
+int mi355gq_moe_route_dt(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights, void* ids,
+                         void* token_indices, void* reverse_indices, void* slot_positions, void* indptr,
+                         int indptr_dtype, int model_dtype, mi355gq_stream_t stream) {
+  return moe_route_impl(logits, T, num_experts, top_k, weights, ids, token_indices, reverse_indices, slot_positions,
+                        indptr, indptr_dtype, model_dtype, stream);
 }
 
 }  // extern "C"

@@ -91,8 +91,9 @@ hipError_t launch_dequantize(const int32_t* ids, int64_t out_rows, const uint32_
                              const uint16_t* qs, int64_t table_rows, int64_t K, int bits,
                              int group_size, uint16_t* out, hipStream_t s);
 
-hipError_t launch_topk_softmax(const uint16_t* logits, int64_t T, int ne, int k, uint16_t* w,
-                               int32_t* ids, hipStream_t s);
+// (logits, weights, activations of the routing glue carry model_dtype: MODEL_F16 | MODEL_F32 | MODEL_BF16)
+hipError_t launch_topk_softmax(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int model_dtype,
+                               hipStream_t s);
 hipError_t launch_moe_cumsum(const int32_t* ids, int64_t T, int k, int ne, int32_t* cumsum,
                              hipStream_t s);
 hipError_t launch_get_indices(const int32_t* cumsum, const int32_t* ids, int64_t T, int k, int ne,
@@ -101,12 +102,12 @@ hipError_t launch_get_indptr(const int32_t* cumsum, int64_t ne, int64_t T, int i
                              int out_i64, void* indptr, hipStream_t s);
 hipError_t launch_take_rows(const uint16_t* x, const int32_t* idx, int64_t R, int64_t H,
                             int64_t x_rows, uint16_t* out, int scatter, hipStream_t s);
-hipError_t launch_silu_mul(const uint16_t* x, int64_t R, int64_t I, uint16_t* out, hipStream_t s);
-hipError_t launch_moe_combine(const uint16_t* y, const uint16_t* w, const int32_t* pos, int64_t T, int k,
-                              int64_t H, uint16_t* out, hipStream_t s);
+hipError_t launch_silu_mul(const void* x, int64_t R, int64_t I, void* out, int model_dtype, hipStream_t s);
+hipError_t launch_moe_combine(const void* y, const void* w, const int32_t* pos, int64_t T, int k, int64_t H,
+                              void* out, int model_dtype, hipStream_t s);
 // fused routing for batches one workgroup can scan (the caller checks T and the expert count)
-hipError_t launch_moe_route(const uint16_t* logits, int64_t T, int ne, int k, uint16_t* w, int32_t* ids,
-                            int32_t* tok, int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr,
+hipError_t launch_moe_route(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int32_t* tok,
+                            int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr, int model_dtype,
                             hipStream_t s);
 
 }  // namespace gq

@@ -5,6 +5,8 @@
 // (:135-235), moe_cumsum (:371-450), get_indices (:453-525), get_indptr (:528-605),
 // scatter_output (:608-645), moe_sum (:14-32), and the elementwise glue of
 // model/mixtral/mixtral_model.py:64-117.  All of it is integer / tiny fp16 work.
+#include <type_traits>
+
 #include "gq_common.hpp"
 #include "gq_internal.hpp"
 
@@ -12,23 +14,50 @@ namespace gq {
 
 constexpr int kMaxTopK = 8;
 
+// Elements of the model dtype (MODEL_F16 | MODEL_F32 | MODEL_BF16): load as float, round a float to
+// the dtype, store.  The float16 forms are the original kernels; the others follow the same rounding
+// points with their own rounding (every op in fp32, its result rounded to the dtype).
+template <int DT>
+struct Elem;
+template <>
+struct Elem<MODEL_F16> {
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return h2f(static_cast<const uint16_t*>(p)[i]); }
+  static __device__ __forceinline__ float rnd(float v) { return h2f(f2h(v)); }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { static_cast<uint16_t*>(p)[i] = f2h(v); }
+  static constexpr float kLowest = -65504.0f;
+};
+template <>
+struct Elem<MODEL_F32> {
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return static_cast<const float*>(p)[i]; }
+  static __device__ __forceinline__ float rnd(float v) { return v; }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { static_cast<float*>(p)[i] = v; }
+  static constexpr float kLowest = -3.402823466e38f;
+};
+template <>
+struct Elem<MODEL_BF16> {
+  static __device__ __forceinline__ float load(const void* p, int64_t i) { return bf2f(static_cast<const uint16_t*>(p)[i]); }
+  static __device__ __forceinline__ float rnd(float v) { return bf2f(f2bf(v)); }
+  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { static_cast<uint16_t*>(p)[i] = f2bf(v); }
+  static constexpr float kLowest = -3.3895313892515355e38f;  // min_value(bfloat16)
+};
+
 // One thread per token: insertion top-k with strict '>' (ties keep the lower expert index),
 // then softmax over the k selected logits in fp32.
 // KMAX: slots kept (k <= KMAX); the insertion is a chain of KMAX * KMAX predicated moves per expert,
 // so the common k <= 2 gets its own, 16 times shorter, instance
-template <int KMAX>
-__device__ __forceinline__ void topk_softmax_slots(const uint16_t* __restrict__ row, int ne, int k,
-                                                   uint16_t* __restrict__ w, int32_t* __restrict__ ids) {
+template <int KMAX, int DT>
+__device__ __forceinline__ void topk_softmax_slots(const void* __restrict__ logits, int64_t row0, int ne, int k,
+                                                   void* __restrict__ w, int64_t w0, int32_t* __restrict__ ids) {
   constexpr int kMaxTopK = KMAX;
   float val[kMaxTopK];
   int idx[kMaxTopK];
 #pragma unroll
   for (int i = 0; i < kMaxTopK; ++i) {
-    val[i] = -65504.0f;  // min_value(fp16)
+    val[i] = Elem<DT>::kLowest;  // min_value(dtype)
     idx[i] = 0;
   }
   for (int e = 0; e < ne; ++e) {
-    const float v = h2f(row[e]);
+    const float v = Elem<DT>::load(logits, row0 + e);
     bool placed = false;
 #pragma unroll
     for (int i = 0; i < kMaxTopK; ++i) {
@@ -62,26 +91,27 @@ __device__ __forceinline__ void topk_softmax_slots(const uint16_t* __restrict__ 
 #pragma unroll
   for (int i = 0; i < kMaxTopK; ++i) {
     if (i < k) {
-      w[i] = f2h(ex[i] / den);
+      Elem<DT>::store(w, w0 + i, ex[i] / den);
       ids[i] = idx[i];
     }
   }
 }
 
-__device__ __forceinline__ void topk_softmax_token(const uint16_t* __restrict__ row, int ne, int k,
-                                                   uint16_t* __restrict__ w, int32_t* __restrict__ ids) {
-  if (k <= 2) topk_softmax_slots<2>(row, ne, k, w, ids);
-  else if (k <= 4) topk_softmax_slots<4>(row, ne, k, w, ids);
-  else topk_softmax_slots<kMaxTopK>(row, ne, k, w, ids);
+// token t: logits[t, :] -> w[t, :k], ids[t, :k]
+template <int DT>
+__device__ __forceinline__ void topk_softmax_token(const void* __restrict__ logits, int64_t t, int ne, int k,
+                                                   void* __restrict__ w, int32_t* __restrict__ ids) {
+  if (k <= 2) topk_softmax_slots<2, DT>(logits, t * ne, ne, k, w, t * k, ids + t * k);
+  else if (k <= 4) topk_softmax_slots<4, DT>(logits, t * ne, ne, k, w, t * k, ids + t * k);
+  else topk_softmax_slots<kMaxTopK, DT>(logits, t * ne, ne, k, w, t * k, ids + t * k);
 }
 
-__global__ __launch_bounds__(256) void topk_softmax_kernel(const uint16_t* __restrict__ logits,
-                                                           int64_t T, int ne, int k,
-                                                           uint16_t* __restrict__ w,
-                                                           int32_t* __restrict__ ids) {
+template <int DT>
+__global__ __launch_bounds__(256) void topk_softmax_kernel(const void* __restrict__ logits, int64_t T, int ne, int k,
+                                                           void* __restrict__ w, int32_t* __restrict__ ids) {
   const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (t >= T) return;
-  topk_softmax_token(logits + t * ne, ne, k, w + t * k, ids + t * k);
+  topk_softmax_token<DT>(logits, t, ne, k, w, ids);
 }
 
 // The whole routing step of a MoE layer in one workgroup, for batches a single workgroup can scan:
@@ -89,8 +119,9 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const uint16_t* __res
 // token) pairs: the results of gating_softmax_topk, moe_cumsum, get_indices and get_indptr without
 // the [experts, T] cumsum table in memory and without four launches.  pos_of_slot is the inverse of
 // reverse_indices (where slot t * k + j sits in the expert-sorted order).
-__global__ __launch_bounds__(1024) void moe_route_kernel(const uint16_t* __restrict__ logits, int T, int ne,
-                                                         int k, uint16_t* __restrict__ w,
+template <int DT>
+__global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict__ logits, int T, int ne,
+                                                         int k, void* __restrict__ w,
                                                          int32_t* __restrict__ ids, int32_t* __restrict__ tok,
                                                          int32_t* __restrict__ rev,
                                                          int32_t* __restrict__ pos_of_slot, int out_i64,
@@ -102,8 +133,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const uint16_t* __restr
   const int tid = threadIdx.x, nthreads = blockDim.x;  // a multiple of 64, sized to the batch
   const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
   for (int t = tid; t < T; t += nthreads) {
-    topk_softmax_token(logits + static_cast<int64_t>(t) * ne, ne, k, w + static_cast<int64_t>(t) * k,
-                       ids + static_cast<int64_t>(t) * k);
+    topk_softmax_token<DT>(logits, t, ne, k, w, ids);
     if (ids_in_lds)
       for (int j = 0; j < k; ++j) ids_lds[t * k + j] = ids[static_cast<int64_t>(t) * k + j];  // own writes
   }
@@ -258,23 +288,29 @@ __global__ __launch_bounds__(256) void move_rows_kernel(const uint16_t* __restri
 }
 
 // out[r, i] = fp16(silu(x[r, i])) * x[r, I + i]; silu in fp32, one rounding, then an fp16 product
-__global__ __launch_bounds__(256) void silu_mul_kernel(const uint16_t* __restrict__ x, int64_t R,
-                                                       int64_t I, uint16_t* __restrict__ out) {
+// (other model dtypes: the same two roundings in that dtype; float32 evaluates silu with expf and a true divide)
+template <int DT>
+__global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ x, int64_t R, int64_t I,
+                                                       void* __restrict__ out) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (i >= R * I) return;
   const int64_t r = i / I, c = i - r * I;
-  const float x1 = h2f(x[r * 2 * I + c]);
-  const float x3 = h2f(x[r * 2 * I + I + c]);
-  out[i] = silu_mul_h(x1, x3);
+  const float x1 = Elem<DT>::load(x, r * 2 * I + c);
+  const float x3 = Elem<DT>::load(x, r * 2 * I + I + c);
+  if constexpr (DT == MODEL_F16) {
+    static_cast<uint16_t*>(out)[i] = silu_mul_h(x1, x3);
+  } else {
+    const float silu = Elem<DT>::rnd(x1 / (1.0f + expf(-x1)));
+    Elem<DT>::store(out, i, silu * x3);
+  }
 }
 
 // out[t, h] = sum_j fp16(y[t, j, h] * w[t, j]), fp16 adds left to right
 // pos: where slot t * k + j sits among the rows of y (expert-sorted order), or null for y in slot order
-__global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __restrict__ y,
-                                                          const uint16_t* __restrict__ w,
-                                                          const int32_t* __restrict__ pos,
-                                                          int64_t T, int k, int64_t H,
-                                                          uint16_t* __restrict__ out) {
+template <int DT>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict__ y, const void* __restrict__ w,
+                                                          const int32_t* __restrict__ pos, int64_t T, int k,
+                                                          int64_t H, void* __restrict__ out) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (i >= T * H) return;
   const int64_t t = i / H, h = i - t * H;
@@ -285,20 +321,31 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __rest
       row = pos[row];
       row = row < 0 ? 0 : (row >= T * k ? T * k - 1 : row);
     }
-    const float prod = h2f(f2h(h2f(y[row * H + h]) * h2f(w[t * k + j])));
-    acc = (j == 0) ? prod : h2f(f2h(acc + prod));
+    const float prod = Elem<DT>::rnd(Elem<DT>::load(y, row * H + h) * Elem<DT>::load(w, t * k + j));
+    acc = (j == 0) ? prod : Elem<DT>::rnd(acc + prod);
   }
-  out[i] = f2h(acc);
+  Elem<DT>::store(out, i, acc);
 }
 
 static inline unsigned blocks_for(int64_t n, int per) { return static_cast<unsigned>((n + per - 1) / per); }
 
-hipError_t launch_topk_softmax(const uint16_t* logits, int64_t T, int ne, int k, uint16_t* w,
-                               int32_t* ids, hipStream_t s) {
-  if (T == 0) return hipSuccess;
-  hipLaunchKernelGGL(topk_softmax_kernel, dim3(blocks_for(T, 256)), dim3(256), 0, s, logits, T, ne,
-                     k, w, ids);
+// dispatch on the model dtype: fn(std::integral_constant<int, DT>)
+template <typename Fn>
+static hipError_t by_dtype(int model_dtype, Fn fn) {
+  if (model_dtype == MODEL_F16) fn(std::integral_constant<int, MODEL_F16>{});
+  else if (model_dtype == MODEL_F32) fn(std::integral_constant<int, MODEL_F32>{});
+  else if (model_dtype == MODEL_BF16) fn(std::integral_constant<int, MODEL_BF16>{});
+  else return hipErrorInvalidValue;
   return hipGetLastError();
+}
+
+hipError_t launch_topk_softmax(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int model_dtype,
+                               hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  return by_dtype(model_dtype, [&](auto dt) {
+    hipLaunchKernelGGL(topk_softmax_kernel<decltype(dt)::value>, dim3(blocks_for(T, 256)), dim3(256), 0, s, logits, T,
+                       ne, k, w, ids);
+  });
 }
 
 hipError_t launch_moe_cumsum(const int32_t* ids, int64_t T, int k, int ne, int32_t* cumsum,
@@ -339,30 +386,34 @@ hipError_t launch_take_rows(const uint16_t* x, const int32_t* idx, int64_t R, in
   return hipGetLastError();
 }
 
-hipError_t launch_silu_mul(const uint16_t* x, int64_t R, int64_t I, uint16_t* out, hipStream_t s) {
+hipError_t launch_silu_mul(const void* x, int64_t R, int64_t I, void* out, int model_dtype, hipStream_t s) {
   if (R * I == 0) return hipSuccess;
-  hipLaunchKernelGGL(silu_mul_kernel, dim3(blocks_for(R * I, 256)), dim3(256), 0, s, x, R, I, out);
-  return hipGetLastError();
+  return by_dtype(model_dtype, [&](auto dt) {
+    hipLaunchKernelGGL(silu_mul_kernel<decltype(dt)::value>, dim3(blocks_for(R * I, 256)), dim3(256), 0, s, x, R, I,
+                       out);
+  });
 }
 
-hipError_t launch_moe_combine(const uint16_t* y, const uint16_t* w, const int32_t* pos, int64_t T, int k,
-                              int64_t H, uint16_t* out, hipStream_t s) {
+hipError_t launch_moe_combine(const void* y, const void* w, const int32_t* pos, int64_t T, int k, int64_t H,
+                              void* out, int model_dtype, hipStream_t s) {
   if (T * H == 0) return hipSuccess;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3(blocks_for(T * H, 256)), dim3(256), 0, s, y, w, pos, T, k,
-                     H, out);
-  return hipGetLastError();
+  return by_dtype(model_dtype, [&](auto dt) {
+    hipLaunchKernelGGL(moe_combine_kernel<decltype(dt)::value>, dim3(blocks_for(T * H, 256)), dim3(256), 0, s, y, w,
+                       pos, T, k, H, out);
+  });
 }
 
-hipError_t launch_moe_route(const uint16_t* logits, int64_t T, int ne, int k, uint16_t* w, int32_t* ids,
-                            int32_t* tok, int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr,
+hipError_t launch_moe_route(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int32_t* tok,
+                            int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr, int model_dtype,
                             hipStream_t s) {
   int threads = static_cast<int>((T + 63) / 64) * 64;
   threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
   const size_t lds = static_cast<size_t>(T) * k * sizeof(int32_t);
   const int ids_in_lds = lds <= 60 * 1024;
-  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(threads), ids_in_lds ? lds : 0, s, logits,
-                     static_cast<int>(T), ne, k, w, ids, tok, rev, pos_of_slot, out_i64, indptr, ids_in_lds);
-  return hipGetLastError();
+  return by_dtype(model_dtype, [&](auto dt) {
+    hipLaunchKernelGGL(moe_route_kernel<decltype(dt)::value>, dim3(1), dim3(threads), ids_in_lds ? lds : 0, s, logits,
+                       static_cast<int>(T), ne, k, w, ids, tok, rev, pos_of_slot, out_i64, indptr, ids_in_lds);
+  });
 }
 
 }  // namespace gq

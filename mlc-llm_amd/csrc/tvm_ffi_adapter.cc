@@ -297,6 +297,39 @@ void MoeGroupGemmDt(TensorView x, TensorView q_weight, TensorView q_scale, Tenso
         "mlc.gq.moe_group_gemm_dt");
 }
 
+// routing glue with logits, weights and activations in model_dtype
+void GatingSoftmaxTopkDt(TensorView logits, int64_t top_k, int64_t model_dtype, TensorView weights, TensorView ids) {
+  Check(mi355gq_gating_softmax_topk_dt(Ptr(logits), logits.shape()[0], logits.shape()[1], top_k, Ptr(weights),
+                                       Ptr(ids), static_cast<int>(model_dtype), StreamOf(logits)),
+        "mlc.gq.gating_softmax_topk_dt");
+}
+
+void TakeRowsDt(TensorView x, TensorView indices, int64_t model_dtype, TensorView out) {
+  Check(mi355gq_take_rows_dt(Ptr(x), Ptr(indices), out.shape()[0], x.shape()[1], x.shape()[0], Ptr(out),
+                             static_cast<int>(model_dtype), StreamOf(x)),
+        "mlc.gq.take_rows_dt");
+}
+
+void ScatterOutputDt(TensorView x, TensorView indices, int64_t model_dtype, TensorView out) {
+  Check(mi355gq_moe_scatter_output_dt(Ptr(x), Ptr(indices), x.shape()[0], x.shape()[1], Ptr(out),
+                                      static_cast<int>(model_dtype), StreamOf(x)),
+        "mlc.gq.moe_scatter_output_dt");
+}
+
+void SiluMulDt(TensorView x, int64_t model_dtype, TensorView out) {
+  Check(mi355gq_silu_mul_dt(Ptr(x), x.shape()[0], x.shape()[1] / 2, Ptr(out), static_cast<int>(model_dtype),
+                            StreamOf(x)),
+        "mlc.gq.silu_mul_dt");
+}
+
+void MoeCombineDt(TensorView y, Optional<TensorView> slot_positions, TensorView weights, int64_t model_dtype,
+                  TensorView out) {
+  Check(mi355gq_moe_combine_dt(Ptr(y), slot_positions.has_value() ? Ptr(slot_positions.value()) : nullptr,
+                               Ptr(weights), weights.shape()[0], weights.shape()[1], out.shape()[1], Ptr(out),
+                               static_cast<int>(model_dtype), StreamOf(y)),
+        "mlc.gq.moe_combine_dt");
+}
+
 TVM_FFI_STATIC_INIT_BLOCK() {
   namespace refl = tvm::ffi::reflection;
   refl::GlobalDef()
@@ -321,6 +354,11 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.linear_dt", LinearDt)
       .def("mlc.gq.linear_dt_workspace_bytes", LinearDtWorkspaceBytes)
       .def("mlc.gq.linear_residual_dt", LinearResidualDt)
+      .def("mlc.gq.gating_softmax_topk_dt", GatingSoftmaxTopkDt)
+      .def("mlc.gq.take_rows_dt", TakeRowsDt)
+      .def("mlc.gq.moe_scatter_output_dt", ScatterOutputDt)
+      .def("mlc.gq.silu_mul_dt", SiluMulDt)
+      .def("mlc.gq.moe_combine_dt", MoeCombineDt)
       .def("mlc.gq.moe_gemv_dt", MoeGemvDt)
       .def("mlc.gq.moe_group_gemm_dt", MoeGroupGemmDt);
 }

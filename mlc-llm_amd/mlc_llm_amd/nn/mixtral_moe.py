@@ -34,13 +34,13 @@ class MixtralMoE(nn.Module):
         return self.e2(self.e1_e3(x, indptr, silu_mul_halves=True), indptr)
 
     def forward(self, x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
-        """x fp16 [batch, seq, hidden]; gate fp16 [batch * seq, num_local_experts] router logits."""
+        """x [batch, seq, hidden]; gate [batch * seq, num_local_experts] router logits, both in the model dtype."""
         experts_per_tok = self.num_experts_per_tok
         local_experts = self.num_local_experts
         batch_size, seq_len, hidden_size = x.shape
         num_tokens = batch_size * seq_len
         x = x.reshape(num_tokens, hidden_size).contiguous()
-        if num_tokens > 1:
+        if num_tokens > 1 and x.dtype == torch.float16:  # (the gather inside the expert matmul is a float16 form)
             try:
                 # routing in one launch; the gather rides in e1_e3's row addressing, the scatter in the
                 # combine's: four launches where the op-by-op sequence below takes nine

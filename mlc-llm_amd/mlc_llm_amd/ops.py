@@ -342,41 +342,41 @@ def moe_route(logits: torch.Tensor, top_k: int, indptr_dtype=torch.int32):
     """The routing of a MoE layer in one launch.  Returns (weights [T, k] fp16, ids [T, k] int32,
     token_indices [T * k], reverse_indices [T * k], slot_positions [T * k], indptr [experts + 1]).
     Raises Mi355gqError with code ERR_UNSUPPORTED for batches past the single-workgroup form."""
-    _chk(logits, torch.float16, "logits")
+    _chk(logits, _FLOATS, "logits")
     t, ne = logits.shape
     dev = logits.device
-    w = torch.empty((t, top_k), dtype=torch.float16, device=dev)
+    w = torch.empty((t, top_k), dtype=logits.dtype, device=dev)
     ids = torch.empty((t, top_k), dtype=torch.int32, device=dev)
     tok, rev, pos = (torch.empty((t * top_k,), dtype=torch.int32, device=dev) for _ in range(3))
     indptr = torch.empty((ne + 1,), dtype=indptr_dtype, device=dev)
-    _lib.call("mi355gq_moe_route", logits.data_ptr(), t, ne, top_k, w.data_ptr(), ids.data_ptr(), tok.data_ptr(),
+    _lib.call("mi355gq_moe_route_dt", logits.data_ptr(), t, ne, top_k, w.data_ptr(), ids.data_ptr(), tok.data_ptr(),
               rev.data_ptr(), pos.data_ptr(), indptr.data_ptr(),
-              _lib.I64 if indptr_dtype == torch.int64 else _lib.I32, _stream())
+              _lib.I64 if indptr_dtype == torch.int64 else _lib.I32, _MODEL_DTYPES[logits.dtype], _stream())
     return w, ids, tok, rev, pos, indptr
 
 
 def moe_combine_sorted(y: torch.Tensor, slot_positions: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
     """y fp16 [T * k, H] in expert-sorted order, slot_positions int32 [T * k], weights fp16 [T, k] -> [T, H]."""
-    _chk(y, torch.float16, "y")
+    _chk(y, _FLOATS, "y")
     _chk(slot_positions, torch.int32, "slot_positions")
-    _chk(weights, torch.float16, "weights")
+    _chk(weights, y.dtype, "weights")
     t, k = weights.shape
     if y.shape[0] != t * k or slot_positions.numel() != t * k:
         raise ValueError("moe_combine_sorted: y and slot_positions must have T * k rows")
     h = y.shape[1]
-    out = torch.empty((t, h), dtype=torch.float16, device=y.device)
-    _lib.call("mi355gq_moe_combine_sorted", y.data_ptr(), slot_positions.data_ptr(), weights.data_ptr(), t, k, h,
-              out.data_ptr(), _stream())
+    out = torch.empty((t, h), dtype=y.dtype, device=y.device)
+    _lib.call("mi355gq_moe_combine_dt", y.data_ptr(), slot_positions.data_ptr(), weights.data_ptr(), t, k, h,
+              out.data_ptr(), _MODEL_DTYPES[y.dtype], _stream())
     return out
 
 
 def gating_softmax_topk(logits: torch.Tensor, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
-    _chk(logits, torch.float16, "logits")
+    _chk(logits, _FLOATS, "logits")
     t, ne = logits.shape
-    w = torch.empty((t, top_k), dtype=torch.float16, device=logits.device)
+    w = torch.empty((t, top_k), dtype=logits.dtype, device=logits.device)
     ids = torch.empty((t, top_k), dtype=torch.int32, device=logits.device)
-    _lib.call("mi355gq_gating_softmax_topk", logits.data_ptr(), t, ne, top_k, w.data_ptr(),
-              ids.data_ptr(), _stream())
+    _lib.call("mi355gq_gating_softmax_topk_dt", logits.data_ptr(), t, ne, top_k, w.data_ptr(),
+              ids.data_ptr(), _MODEL_DTYPES[logits.dtype], _stream())
     return w, ids
 
 
@@ -414,39 +414,39 @@ def get_indptr(cumsum: torch.Tensor, num_local_experts: int, batch_size: int, in
 
 
 def take_rows(x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
-    _chk(x, torch.float16, "x")
+    _chk(x, _FLOATS, "x")
     _chk(indices, torch.int32, "indices")
     r, h = indices.numel(), x.shape[1]
-    out = torch.zeros((r, h), dtype=torch.float16, device=x.device)
-    _lib.call("mi355gq_take_rows", x.data_ptr(), indices.data_ptr(), r, h, x.shape[0],
-              out.data_ptr(), _stream())
+    out = torch.zeros((r, h), dtype=x.dtype, device=x.device)
+    _lib.call("mi355gq_take_rows_dt", x.data_ptr(), indices.data_ptr(), r, h, x.shape[0],
+              out.data_ptr(), _MODEL_DTYPES[x.dtype], _stream())
     return out
 
 
 def scatter_output(x: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
-    _chk(x, torch.float16, "x")
+    _chk(x, _FLOATS, "x")
     _chk(indices, torch.int32, "indices")
     r, h = x.shape
     out = torch.zeros_like(x)
-    _lib.call("mi355gq_moe_scatter_output", x.data_ptr(), indices.data_ptr(), r, h,
-              out.data_ptr(), _stream())
+    _lib.call("mi355gq_moe_scatter_output_dt", x.data_ptr(), indices.data_ptr(), r, h,
+              out.data_ptr(), _MODEL_DTYPES[x.dtype], _stream())
     return out
 
 
 def silu_mul(x: torch.Tensor) -> torch.Tensor:
-    _chk(x, torch.float16, "x")
+    _chk(x, _FLOATS, "x")
     r, two_i = x.shape
-    out = torch.empty((r, two_i // 2), dtype=torch.float16, device=x.device)
-    _lib.call("mi355gq_silu_mul", x.data_ptr(), r, two_i // 2, out.data_ptr(), _stream())
+    out = torch.empty((r, two_i // 2), dtype=x.dtype, device=x.device)
+    _lib.call("mi355gq_silu_mul_dt", x.data_ptr(), r, two_i // 2, out.data_ptr(), _MODEL_DTYPES[x.dtype], _stream())
     return out
 
 
 def moe_combine(y: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
-    """y fp16 [T, k, H], weights fp16 [T, k] -> fp16 [T, H]."""
-    _chk(y, torch.float16, "y")
-    _chk(weights, torch.float16, "weights")
+    """y [T, k, H], weights [T, k] -> [T, H], all in the model dtype."""
+    _chk(y, _FLOATS, "y")
+    _chk(weights, y.dtype, "weights")
     t, k, h = y.shape
-    out = torch.empty((t, h), dtype=torch.float16, device=y.device)
-    _lib.call("mi355gq_moe_combine", y.data_ptr(), weights.data_ptr(), t, k, h, out.data_ptr(),
-              _stream())
+    out = torch.empty((t, h), dtype=y.dtype, device=y.device)
+    _lib.call("mi355gq_moe_combine_dt", y.data_ptr(), None, weights.data_ptr(), t, k, h, out.data_ptr(),
+              _MODEL_DTYPES[y.dtype], _stream())
     return out

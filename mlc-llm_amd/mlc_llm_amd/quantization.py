@@ -355,6 +355,9 @@ class GroupQuantizeMixtralExperts(nn.Module):
         assert x.dim() == 2
         if self.config.model_dtype not in MOE_MODEL_DTYPES:
             raise NotImplementedError(f"{self.config.name}: the expert matmuls are built for {MOE_MODEL_DTYPES} models")
+        if silu_mul_halves and x.dtype != torch.float16:
+            # the folded activation exists for float16 models; the others run the two steps
+            return ops.silu_mul(self.forward(x, indptr))
         if indptr.dim() == 2:
             assert indptr.shape[0] == 1
             return ops.moe_gemv(x, self.q_weight, self.q_scale, indptr, self.config.bits,

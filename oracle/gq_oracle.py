@@ -415,6 +415,64 @@ def silu_mul_f16(x1_x3: np.ndarray) -> np.ndarray:
     return (silu * x3).astype(F16)
 
 
+def gating_softmax_topk_dt(x32: np.ndarray, k: int, model_dtype: str):
+    """gating_softmax_topk for logits of any model dtype (float32 carriers): the same top-k and fp32 softmax,
+    weights rounded to the model dtype."""
+    t, ne = x32.shape
+    vals = np.full((t, k), -np.inf, np.float64)
+    idx = np.zeros((t, k), np.int32)
+    for row in range(t):
+        for e in range(ne):
+            v = float(x32[row, e])
+            for i in range(k):
+                if v > vals[row, i]:
+                    vals[row, i + 1 :] = vals[row, i:-1].copy()
+                    idx[row, i + 1 :] = idx[row, i:-1].copy()
+                    vals[row, i] = v
+                    idx[row, i] = e
+                    break
+    v32 = vals.astype(F32)
+    ex = np.exp(v32 - v32.max(axis=1, keepdims=True), dtype=F32)
+    den = ex[:, 0].copy()
+    for i in range(1, k):
+        den = den + ex[:, i]
+    return round_to(ex / den[:, None], model_dtype), idx
+
+
+def silu_mul_dt(x1_x3: np.ndarray, model_dtype: str) -> np.ndarray:
+    """silu_mul_f16 with the model dtype's roundings (float32 carriers): silu in fp32, rounded, product rounded.
+    PARITY UNPINNED like silu_mul_f16."""
+    h = x1_x3.shape[-1] // 2
+    x1, x3 = x1_x3[..., :h].astype(F32), x1_x3[..., h:].astype(F32)
+    silu = round_to(x1 / (F32(1) + np.exp(-x1)), model_dtype)
+    return round_to(silu * x3, model_dtype)
+
+
+def mixtral_moe_dt(x, gate_logits, w13, s13, w2, s2, scheme: Scheme, model_dtype: str, top_k: int = 2):
+    """mixtral_moe for a float32 / bfloat16 model: float32 carriers, every stored tensor rounded to the model
+    dtype, expert matmuls exact in float64 over the dtype-dequantised weights."""
+    t, hdim = x.shape
+    ne = w13.shape[0]
+    weights, ids = gating_softmax_topk_dt(gate_logits, top_k, model_dtype)
+    if t == 1:
+        y = round_to(moe_dequantize_gemv_dt_fp64(x, w13, s13, ids, scheme, model_dtype).astype(F32), model_dtype)
+        y = silu_mul_dt(y, model_dtype)
+        y = round_to(moe_dequantize_gemv_dt_fp64(y, w2, s2, ids, scheme, model_dtype).astype(F32), model_dtype)
+    else:
+        cs = moe_cumsum(ids, ne)
+        rev, tok = get_indices(cs, ids)
+        indptr = get_indptr(cs, ne, t, inclusive=False)
+        y = round_to(dequantize_group_gemm_dt_fp64(x[tok], w13, s13, indptr, scheme, model_dtype).astype(F32), model_dtype)
+        y = silu_mul_dt(y, model_dtype)
+        y = round_to(dequantize_group_gemm_dt_fp64(y, w2, s2, indptr, scheme, model_dtype).astype(F32), model_dtype)
+        y = scatter_output(y, rev)
+    y = round_to(y.reshape(t, top_k, hdim) * weights.reshape(t, top_k, 1), model_dtype)
+    out = y[:, 0]
+    for j in range(1, top_k):
+        out = round_to(out + y[:, j], model_dtype)
+    return out
+
+
 def mixtral_moe(x, gate_logits, w13, s13, w2, s2, scheme: Scheme, top_k: int = 2):
     """MixtralMoE.forward (mixtral_model.py:64-117) given the router logits.
 

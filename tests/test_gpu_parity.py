@@ -1083,6 +1083,76 @@ def test_linear_residual_other_model_dtypes(model_dtype, m, n, k):
     assert torch.equal(acc, y)
 
 
+@pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
+def test_routing_glue_other_model_dtypes(model_dtype):
+    """gating_softmax_topk, moe_route, take_rows / scatter_output, silu_mul and the combine with logits,
+    weights and activations in the model dtype."""
+    dt = _TORCH_OF[model_dtype]
+    rng = np.random.default_rng(5)
+    for t, ne, k in ((1, 8, 2), (7, 8, 2), (33, 6, 3), (300, 8, 2)):
+        lg32 = o.round_to((rng.standard_normal((t, ne)) * 2).astype(np.float32), model_dtype)
+        lg = torch.from_numpy(lg32).to(dt).to(DEV)
+        w, ids = ops.gating_softmax_topk(lg, k)
+        w_ref, ids_ref = o.gating_softmax_topk_dt(lg32, k, model_dtype)
+        assert w.dtype == dt and np.array_equal(ids.cpu().numpy(), ids_ref)
+        # the softmax runs in fp32 on both sides with different exp implementations: one ulp of the dtype
+        assert np.abs(_carrier(w) - w_ref).max() <= (2.0 ** -8 if model_dtype == "bfloat16" else 1e-6)
+        w2, ids2, tok, rev, pos, indptr = ops.moe_route(lg, k)
+        assert torch.equal(w2, w) and torch.equal(ids2, ids)
+        cs = o.moe_cumsum(ids_ref, ne)
+        rev_ref, tok_ref = o.get_indices(cs, ids_ref)
+        assert np.array_equal(tok.cpu().numpy(), tok_ref) and np.array_equal(rev.cpu().numpy(), rev_ref)
+        assert np.array_equal(indptr.cpu().numpy(), o.get_indptr(cs, ne, t, inclusive=False))
+        x32 = o.round_to(rng.standard_normal((t, 40)).astype(np.float32), model_dtype)
+        x = torch.from_numpy(x32).to(dt).to(DEV)
+        g = ops.take_rows(x, tok)
+        assert g.dtype == dt and np.array_equal(_carrier(g), x32[tok_ref])
+        sc = ops.scatter_output(g, rev)
+        assert np.array_equal(_carrier(sc), o.scatter_output(x32[tok_ref], rev_ref))
+        # combine: slot order and expert-sorted order
+        y32 = o.round_to(rng.standard_normal((t * k, 24)).astype(np.float32), model_dtype)
+        y = torch.from_numpy(y32).to(dt).to(DEV)
+        prod = o.round_to(y32.reshape(t, k, 24) * _carrier(w).reshape(t, k, 1), model_dtype)
+        want = prod[:, 0]
+        for j in range(1, k):
+            want = o.round_to(want + prod[:, j], model_dtype)
+        assert np.array_equal(_carrier(ops.moe_combine(y.reshape(t, k, 24), w)), want)
+        y_sorted = torch.from_numpy(y32[rev_ref]).to(dt).to(DEV)  # row p of the sorted order is slot rev[p]
+        assert np.array_equal(_carrier(ops.moe_combine_sorted(y_sorted, pos, w)), want)
+    a32 = o.round_to((rng.standard_normal((5, 192)) * 3).astype(np.float32), model_dtype)
+    got = _carrier(ops.silu_mul(torch.from_numpy(a32).to(dt).to(DEV)))
+    ref = o.silu_mul_dt(a32, model_dtype)
+    assert np.abs(got - ref).max() <= np.abs(ref).max() * (2.0 ** -7 if model_dtype == "bfloat16" else 1e-6)
+
+
+@pytest.mark.parametrize("model_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("t", [1, 9, 70])
+def test_mixtral_moe_layer_other_model_dtypes(model_dtype, t):
+    from mlc_llm_amd.nn import MixtralMoE
+
+    cfg = gq.QUANTIZATION["q4f32_1" if model_dtype == "float32" else "q4bf16_1"]
+    dt = _TORCH_OF[model_dtype]
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(60 + t)
+    h, inter, ne = 128, 192, 4
+    w13 = o.round_to((rng.standard_normal((ne, 2 * inter, h)) * 0.08).astype(np.float32), model_dtype)
+    w2 = o.round_to((rng.standard_normal((ne, h, inter)) * 0.08).astype(np.float32), model_dtype)
+    q13, s13 = o.quantize_dt(w13, s, model_dtype)
+    q2, s2 = o.quantize_dt(w2, s, model_dtype)
+    x32 = o.round_to(rng.standard_normal((t, h)).astype(np.float32), model_dtype)
+    lg32 = o.round_to(rng.standard_normal((t, ne)).astype(np.float32), model_dtype)
+    moe = MixtralMoE(h, inter, ne, 2, cfg, device=DEV)
+    moe.e1_e3.q_weight.data, moe.e1_e3.q_scale.data = dev(q13), torch.from_numpy(s13).to(dt).to(DEV)
+    moe.e2.q_weight.data, moe.e2.q_scale.data = dev(q2), torch.from_numpy(s2).to(dt).to(DEV)
+    y = moe(torch.from_numpy(x32).to(dt).to(DEV).reshape(1, t, h), torch.from_numpy(lg32).to(dt).to(DEV))
+    assert y.dtype == dt
+    y = y.reshape(t, h).double().cpu().numpy()
+    ref = o.mixtral_moe_dt(x32, lg32, q13, s13, q2, s2, s, model_dtype).astype(np.float64)
+    rel = np.linalg.norm(y - ref) / np.linalg.norm(ref)
+    # two chained matmuls and the glue's roundings in the model dtype
+    assert rel <= (1.5e-2 if model_dtype == "bfloat16" else 1e-5), rel
+
+
 def test_linear_other_model_dtypes_through_the_modules():
     for name in ("q4f32_1", "q4bf16_1", "q4bf16_0"):
         cfg = gq.QUANTIZATION[name]

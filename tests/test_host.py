@@ -117,6 +117,19 @@ def test_argument_validation_of_the_later_entry_points():
     assert "null" in _err()
     assert lib.mi355gq_moe_group_gemm_dt(None, 0, None, None, None, 0, 8, 16, 32, 4, 32, 2, None, None) == 0
     assert lib.mi355gq_moe_gemv_dt(None, 1, None, None, None, 0, 8, 16, 32, 4, 32, 1, None, None) == 0
+    # routing glue in the other model dtypes
+    assert lib.mi355gq_gating_softmax_topk_dt(P(0x1000), 4, 8, 9, P(0x2000), P(0x3000), 2, None) == -1
+    assert "top_k" in _err()
+    assert lib.mi355gq_gating_softmax_topk_dt(P(0x1000), 4, 8, 2, P(0x2000), P(0x3000), 9, None) == -1
+    assert "model_dtype" in _err()
+    assert lib.mi355gq_silu_mul_dt(None, 4, 8, None, 1, None) == -1
+    assert lib.mi355gq_silu_mul_dt(None, 0, 8, None, 2, None) == 0
+    assert lib.mi355gq_take_rows_dt(P(0x1002), P(0x2000), 4, 8, 4, P(0x3000), 1, None) == -1
+    assert "misaligned" in _err()
+    assert lib.mi355gq_moe_scatter_output_dt(None, None, 0, 8, None, 2, None) == 0
+    assert lib.mi355gq_moe_combine_dt(None, None, None, 4, 0, 8, None, 1, None) == -1
+    assert lib.mi355gq_moe_route_dt(P(0x1000), 9000, 8, 2, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
+                                    P(0x7000), 0, 2, None) == _lib.ERR_UNSUPPORTED
     assert lib.mi355gq_quantize_dt(None, 0, 32, 4, 32, 0, 2, None, None, None) == 0
     assert lib.mi355gq_embedding_take_dt(None, 0, None, None, 10, 32, 4, 32, 1, None, None) == 0
 
