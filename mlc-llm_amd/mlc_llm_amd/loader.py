@@ -1,5 +1,5 @@
-"""HuggingFace checkpoint -> MLC parameters for the Llama and Mixtral families, quantised on the
-GPU while loading, written as an MLC weight directory.
+"""HuggingFace checkpoint -> MLC parameters for the Llama / Mistral, Mixtral, Qwen2 / Qwen3, Gemma / Gemma2 and
+Phi-3 families, quantised on the GPU while loading, written as an MLC weight directory.
 
 Mirrors the reference's conversion path for exactly the parameters this package's kernels
 consume:
@@ -135,10 +135,116 @@ def mixtral_huggingface(config: Dict[str, Any]) -> Tuple[ExternMapping, List[str
     return mapping, quantized
 
 
+def _plus_one(x: np.ndarray) -> np.ndarray:
+    return (x.astype(np.float32) + 1.0).astype(x.dtype)
+
+
+def _standard_decoder(config: Dict[str, Any], *, qkv_target: str = "qkv_proj", qkv_bias: bool = False,
+                      qk_norm: bool = False, norm_plus_one: bool = False, always_tied: bool = False,
+                      layer_norms: Tuple[str, ...] = ("input_layernorm", "post_attention_layernorm"),
+                      ) -> Tuple[ExternMapping, List[str]]:
+    """The reference's standard HF mapping (python/mlc_llm/loader/standard_loader.py:22-167) over a decoder
+    whose layers hold ``self_attn.<qkv_target>`` (+ bias), ``self_attn.o_proj``, optional per-head
+    ``q_norm`` / ``k_norm``, ``mlp.gate_up_proj`` / ``mlp.down_proj`` and the given RMSNorm weights;
+    parameter order follows the module trees (attention, MLP, norms)."""
+    mapping, quantized = ExternMapping(), []
+    norm_func = _plus_one if norm_plus_one else _identity
+    mapping.add_mapping("model.embed_tokens.weight", ["model.embed_tokens.weight"], _identity)
+    quantized.append("model.embed_tokens.weight")
+    for i in range(_cfg(config, "num_hidden_layers")):
+        attn, mlp = f"model.layers.{i}.self_attn", f"model.layers.{i}.mlp"
+        mapping.add_mapping(f"{attn}.{qkv_target}.weight",
+                            [f"{attn}.q_proj.weight", f"{attn}.k_proj.weight", f"{attn}.v_proj.weight"], _concat0)
+        quantized.append(f"{attn}.{qkv_target}.weight")
+        if qkv_bias:
+            mapping.add_mapping(f"{attn}.{qkv_target}.bias",
+                                [f"{attn}.q_proj.bias", f"{attn}.k_proj.bias", f"{attn}.v_proj.bias"], _concat0)
+        mapping.add_mapping(f"{attn}.o_proj.weight", [f"{attn}.o_proj.weight"], _identity)
+        quantized.append(f"{attn}.o_proj.weight")
+        if qk_norm:
+            for name in (f"{attn}.q_norm.weight", f"{attn}.k_norm.weight"):
+                mapping.add_mapping(name, [name], norm_func)
+        mapping.add_unused(f"{attn}.rotary_emb.inv_freq")
+        mapping.add_mapping(f"{mlp}.gate_up_proj.weight", [f"{mlp}.gate_proj.weight", f"{mlp}.up_proj.weight"],
+                            _concat0)
+        mapping.add_mapping(f"{mlp}.down_proj.weight", [f"{mlp}.down_proj.weight"], _identity)
+        quantized += [f"{mlp}.gate_up_proj.weight", f"{mlp}.down_proj.weight"]
+        for norm in layer_norms:
+            name = f"model.layers.{i}.{norm}.weight"
+            mapping.add_mapping(name, [name], norm_func)
+    mapping.add_mapping("model.norm.weight", ["model.norm.weight"], norm_func)
+    if always_tied or config.get("tie_word_embeddings", False):
+        mapping.add_unused("lm_head.weight")
+    else:
+        mapping.add_mapping("lm_head.weight", ["lm_head.weight"], _identity)
+        quantized.append("lm_head.weight")
+    return mapping, quantized
+
+
+def qwen2_huggingface(config: Dict[str, Any]) -> Tuple[ExternMapping, List[str]]:
+    """``Qwen2ForCausalLM`` (python/mlc_llm/model/qwen2/qwen2_loader.py:10-15, qwen2_model.py:96-232): the fused
+    projection is ``c_attn`` and carries a bias, which stays in the model dtype."""
+    return _standard_decoder(config, qkv_target="c_attn", qkv_bias=True)
+
+
+def qwen3_huggingface(config: Dict[str, Any]) -> Tuple[ExternMapping, List[str]]:
+    """``Qwen3ForCausalLM`` (python/mlc_llm/model/qwen3/qwen3_loader.py:94-150, qwen3_model.py:119-130): ``c_attn``
+    (a bias only with ``attention_bias``) and the per-head q / k RMSNorm weights."""
+    return _standard_decoder(config, qkv_target="c_attn", qkv_bias=bool(config.get("attention_bias", False)),
+                             qk_norm=True)
+
+
+def gemma_huggingface(config: Dict[str, Any]) -> Tuple[ExternMapping, List[str]]:
+    """``GemmaForCausalLM`` (python/mlc_llm/model/gemma/gemma_loader.py:15-48): RMSNorm weights are stored minus one
+    in the checkpoint, the output projection is the embedding (gemma_model.py:228-260)."""
+    return _standard_decoder(config, norm_plus_one=True, always_tied=True)
+
+
+def gemma2_huggingface(config: Dict[str, Any]) -> Tuple[ExternMapping, List[str]]:
+    """``Gemma2ForCausalLM`` (python/mlc_llm/model/gemma2/gemma2_loader.py): Gemma plus the two feed-forward norms."""
+    return _standard_decoder(config, norm_plus_one=True, always_tied=True,
+                             layer_norms=("input_layernorm", "post_attention_layernorm",
+                                          "pre_feedforward_layernorm", "post_feedforward_layernorm"))
+
+
+def phi3_huggingface(config: Dict[str, Any]) -> Tuple[ExternMapping, List[str]]:
+    """``Phi3ForCausalLM`` (python/mlc_llm/model/phi3/phi3_loader.py:40-78): the checkpoint already holds fused
+    ``qkv_proj`` / ``gate_up_proj``; only the names differ (``transformer.h.<i>.mixer`` ...)."""
+    mapping, quantized = ExternMapping(), []
+    if not config.get("tie_word_embeddings", False):
+        mapping.add_mapping("lm_head.weight", ["lm_head.weight"], _identity)
+        quantized.append("lm_head.weight")
+    else:
+        mapping.add_unused("lm_head.weight")
+    mapping.add_mapping("transformer.norm.weight", ["model.norm.weight"], _identity)
+    mapping.add_mapping("transformer.embd.weight", ["model.embed_tokens.weight"], _identity)
+    quantized.append("transformer.embd.weight")
+    for i in range(_cfg(config, "num_hidden_layers")):
+        mlc, hf = f"transformer.h.{i}", f"model.layers.{i}"
+        mapping.add_mapping(f"{mlc}.ln.weight", [f"{hf}.input_layernorm.weight"], _identity)
+        for mlc_name, hf_name in ((f"{mlc}.mlp.down_proj.weight", f"{hf}.mlp.down_proj.weight"),
+                                  (f"{mlc}.mlp.gate_up_proj.weight", f"{hf}.mlp.gate_up_proj.weight")):
+            mapping.add_mapping(mlc_name, [hf_name], _identity)
+            quantized.append(mlc_name)
+        mapping.add_mapping(f"{mlc}.post_attention_layernorm.weight", [f"{hf}.post_attention_layernorm.weight"],
+                            _identity)
+        for mlc_name, hf_name in ((f"{mlc}.mixer.out_proj.weight", f"{hf}.self_attn.o_proj.weight"),
+                                  (f"{mlc}.mixer.qkv_proj.weight", f"{hf}.self_attn.qkv_proj.weight")):
+            mapping.add_mapping(mlc_name, [hf_name], _identity)
+            quantized.append(mlc_name)
+        mapping.add_unused(f"{hf}.self_attn.rotary_emb.inv_freq")
+    return mapping, quantized
+
+
 MODEL_MAPPINGS: Dict[str, Callable[[Dict[str, Any]], Tuple[ExternMapping, List[str]]]] = {
     "llama": llama_huggingface,
     "mistral": llama_huggingface,  # same module tree and HF names
     "mixtral": mixtral_huggingface,
+    "qwen2": qwen2_huggingface,
+    "qwen3": qwen3_huggingface,
+    "gemma": gemma_huggingface,
+    "gemma2": gemma2_huggingface,
+    "phi3": phi3_huggingface,
 }
 
 

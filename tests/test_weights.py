@@ -20,6 +20,7 @@ from oracle import gq_oracle as o
 
 LLAMA = {"model_type": "llama", "hidden_size": 64, "intermediate_size": 160, "num_hidden_layers": 2,
          "num_attention_heads": 4, "num_key_value_heads": 2, "vocab_size": 96, "tie_word_embeddings": False}
+QWEN2 = dict(LLAMA, model_type="qwen2", tie_word_embeddings=True)
 MIXTRAL = {"model_type": "mixtral", "hidden_size": 64, "intermediate_size": 96, "num_hidden_layers": 1,
            "num_attention_heads": 4, "num_key_value_heads": 2, "vocab_size": 80, "num_local_experts": 3,
            "num_experts_per_tok": 2}
@@ -43,6 +44,9 @@ def _hf_tensors(cfg, seed=0):
         t[f"{p}.input_layernorm.weight"] = w(h)
         t[f"{p}.post_attention_layernorm.weight"] = w(h)
         t[f"{p}.self_attn.rotary_emb.inv_freq"] = w(8)
+        if cfg["model_type"] == "qwen2":
+            t[f"{p}.self_attn.q_proj.bias"], t[f"{p}.self_attn.k_proj.bias"] = w(h), w(kv)
+            t[f"{p}.self_attn.v_proj.bias"] = w(kv)
         if cfg["model_type"] == "mixtral":
             t[f"{p}.block_sparse_moe.gate.weight"] = w(cfg["num_local_experts"], h)
             for e in range(cfg["num_local_experts"]):
@@ -197,6 +201,73 @@ def test_mixtral_mapping_stacks_experts():
     assert {"model.layers.0.moe.e1_e3.weight", "model.layers.0.moe.e2.weight"} <= set(quantized)
 
 
+def test_other_family_mappings():
+    """Qwen2 / Qwen3 (c_attn, bias, q / k norms), Gemma / Gemma2 (norm + 1, tied output projection) and Phi-3
+    (already fused in the checkpoint, renamed): names, transforms and which parameters are quantised."""
+    base = dict(LLAMA)
+    t = {k: v.numpy() for k, v in _hf_tensors(LLAMA).items()}
+    rng = np.random.default_rng(3)
+    for i in range(LLAMA["num_hidden_layers"]):
+        attn = f"model.layers.{i}.self_attn"
+        for n, rows in (("q_proj", 64), ("k_proj", 32), ("v_proj", 32)):
+            t[f"{attn}.{n}.bias"] = rng.standard_normal(rows).astype(np.float16)
+        t[f"{attn}.q_norm.weight"] = rng.standard_normal(16).astype(np.float16)
+        t[f"{attn}.k_norm.weight"] = rng.standard_normal(16).astype(np.float16)
+        for n in ("pre_feedforward_layernorm", "post_feedforward_layernorm"):
+            t[f"model.layers.{i}.{n}.weight"] = rng.standard_normal(64).astype(np.float16)
+
+    def build(mapping, name):
+        return mapping.map_func[name](*[t[n] for n in mapping.param_map[name]])
+
+    # Qwen2: fused projection named c_attn, with a concatenated bias that is not quantised
+    m, q = loader.MODEL_MAPPINGS["qwen2"](dict(base, model_type="qwen2"))
+    w = build(m, "model.layers.1.self_attn.c_attn.weight")
+    b = build(m, "model.layers.1.self_attn.c_attn.bias")
+    assert w.shape == (128, 64) and b.shape == (128,)
+    assert np.array_equal(b[64:96], t["model.layers.1.self_attn.k_proj.bias"])
+    assert "model.layers.1.self_attn.c_attn.weight" in q and "model.layers.1.self_attn.c_attn.bias" not in q
+    assert "model.layers.0.self_attn.qkv_proj.weight" not in m.param_map
+    unused = loader.check_parameter_usage(m, set(t))
+    assert all("q_norm" in n or "k_norm" in n or "feedforward" in n for n in unused)
+    # Qwen3: the per-head norms pass through unquantised; a bias only when the config says so
+    m, q = loader.MODEL_MAPPINGS["qwen3"](dict(base, model_type="qwen3"))
+    assert np.array_equal(build(m, "model.layers.0.self_attn.q_norm.weight"), t["model.layers.0.self_attn.q_norm.weight"])
+    assert "model.layers.0.self_attn.c_attn.bias" not in m.param_map and not any("norm" in n for n in q)
+    m, _ = loader.MODEL_MAPPINGS["qwen3"](dict(base, model_type="qwen3", attention_bias=True))
+    assert "model.layers.0.self_attn.c_attn.bias" in m.param_map
+    # Gemma: norm weights + 1, no lm_head parameter whatever the config says; Gemma2 adds two norms per layer
+    m, q = loader.MODEL_MAPPINGS["gemma"](dict(base, model_type="gemma"))
+    n0 = "model.layers.0.input_layernorm.weight"
+    want = (t[n0].astype(np.float32) + 1.0).astype(np.float16)
+    assert np.array_equal(build(m, n0), want) and build(m, n0).dtype == np.float16
+    assert np.array_equal(build(m, "model.norm.weight"), (t["model.norm.weight"].astype(np.float32) + 1).astype(np.float16))
+    assert "lm_head.weight" not in m.param_map and "lm_head.weight" not in q
+    assert np.array_equal(build(m, "model.layers.0.self_attn.qkv_proj.weight")[:64], t["model.layers.0.self_attn.q_proj.weight"])
+    m2, _ = loader.MODEL_MAPPINGS["gemma2"](dict(base, model_type="gemma2"))
+    extra = set(m2.param_map) - set(m.param_map)
+    assert extra == {f"model.layers.{i}.{n}.weight" for i in range(2)
+                     for n in ("pre_feedforward_layernorm", "post_feedforward_layernorm")}
+    # Phi-3: fused tensors pass through under the transformer.h.<i>.mixer / mlp names
+    p3 = {"model.embed_tokens.weight": t["model.embed_tokens.weight"], "model.norm.weight": t["model.norm.weight"],
+          "lm_head.weight": t["lm_head.weight"]}
+    for i in range(2):
+        hf = f"model.layers.{i}"
+        p3[f"{hf}.self_attn.qkv_proj.weight"] = rng.standard_normal((128, 64)).astype(np.float16)
+        p3[f"{hf}.self_attn.o_proj.weight"] = t[f"{hf}.self_attn.o_proj.weight"]
+        p3[f"{hf}.mlp.gate_up_proj.weight"] = rng.standard_normal((320, 64)).astype(np.float16)
+        p3[f"{hf}.mlp.down_proj.weight"] = t[f"{hf}.mlp.down_proj.weight"]
+        p3[f"{hf}.input_layernorm.weight"] = t[f"{hf}.input_layernorm.weight"]
+        p3[f"{hf}.post_attention_layernorm.weight"] = t[f"{hf}.post_attention_layernorm.weight"]
+    m, q = loader.MODEL_MAPPINGS["phi3"](dict(base, model_type="phi3"))
+    assert m.param_map["transformer.h.1.mixer.qkv_proj.weight"] == ["model.layers.1.self_attn.qkv_proj.weight"]
+    assert m.param_map["transformer.h.0.ln.weight"] == ["model.layers.0.input_layernorm.weight"]
+    assert m.param_map["transformer.embd.weight"] == ["model.embed_tokens.weight"]
+    assert set(q) == {"lm_head.weight", "transformer.embd.weight"} | {
+        f"transformer.h.{i}.{n}.weight" for i in range(2)
+        for n in ("mixer.qkv_proj", "mixer.out_proj", "mlp.gate_up_proj", "mlp.down_proj")}
+    assert loader.check_parameter_usage(m, set(p3)) == set()
+
+
 def test_convert_weight_unquantised_on_cpu(tmp_path):
     src, dst = str(tmp_path / "hf"), str(tmp_path / "mlc")
     tensors = _hf_tensors(LLAMA, seed=5)
@@ -214,7 +285,7 @@ def test_convert_weight_unquantised_on_cpu(tmp_path):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("scheme", ["q4f16_1", "q3f16_1"])
-@pytest.mark.parametrize("cfg", [LLAMA, MIXTRAL], ids=["llama", "mixtral"])
+@pytest.mark.parametrize("cfg", [LLAMA, MIXTRAL, QWEN2], ids=["llama", "mixtral", "qwen2"])
 def test_convert_weight_quantised_matches_oracle(tmp_path, cfg, scheme):
     import mlc_llm_amd as gq
     from mlc_llm_amd import ops
@@ -239,12 +310,15 @@ def test_convert_weight_quantised_matches_oracle(tmp_path, cfg, scheme):
         else:
             assert np.array_equal(params[name].numpy(), full), name
     # the converted directory feeds the kernels: one projection against the oracle
-    name = "model.layers.0.self_attn.qkv_proj"
+    name = "model.layers.0.self_attn." + ("c_attn" if cfg["model_type"] == "qwen2" else "qkv_proj")
     dev = torch.device("cuda:0")
     x = np.random.default_rng(1).standard_normal((3, cfg["hidden_size"])).astype(np.float16)
+    bias = params.get(f"{name}.bias")  # Qwen2: the concatenated q / k / v bias, kept in float16
+    assert (bias is not None) == (cfg["model_type"] == "qwen2")
     y = ops.linear(torch.from_numpy(x).to(dev), params[f"{name}.q_weight"].to(dev), params[f"{name}.q_scale"].to(dev),
-                   s.bits, s.group_size)
-    ref = o.linear_fp32(x, params[f"{name}.q_weight"].numpy().view(np.uint32), params[f"{name}.q_scale"].numpy(), s)
+                   s.bits, s.group_size, bias.to(dev) if bias is not None else None)
+    ref = o.linear_fp32(x, params[f"{name}.q_weight"].numpy().view(np.uint32), params[f"{name}.q_scale"].numpy(), s,
+                        bias.numpy() if bias is not None else None)
     err, bound, rel = o.check_linear(y.float().cpu().numpy(), ref, x, cfg["hidden_size"])
     assert err <= bound and rel <= 2e-3  # the linear tolerance of the hot path
 
