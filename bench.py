@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the group-quantized linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--skip-extra] [--skip-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-graph] [--skip-extra] [--skip-cpu] [--prefill-only]
 
 A "step" is one decode token's worth of q4f16_1 GEMVs at Llama-3-8B shapes, batch 1:
 32 layers x (fused qkv 6144x4096, o_proj 4096x4096, fused gate_up 28672x4096, down 4096x14336)
@@ -58,6 +58,9 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--skip-extra", action="store_true")
     ap.add_argument("--skip-cpu", action="store_true")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="time only the prefill GEMM (gate_up 28672x4096, M = 2048): the run the MFMA counters "
+                         "under profiles/ are collected on")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device copy (known bytes) so that a rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE run of this command can scale its counters")
@@ -88,6 +91,28 @@ def main() -> int:
         g = torch.Generator(device=dev).manual_seed(seed)
         w = (torch.randn((n, k), generator=g, device=dev, dtype=torch.float32) * 0.02).half()
         return ops.quantize(w, BITS, G)
+
+    if args.prefill_only:
+        n, k, m = *SHAPES["gate_up"], 2048
+        qw, qs = make_weight(n, k, 2)
+        xm = torch.randn((m, k), generator=torch.Generator(device=dev).manual_seed(1), device=dev).half()
+        ym = torch.empty((m, n), dtype=torch.float16, device=dev)
+        for _ in range(args.warmup):
+            ops.linear(xm, qw, qs, BITS, G, None, torch.float16, ym)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            ops.linear(xm, qw, qs, BITS, G, None, torch.float16, ym)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / args.steps
+        tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+        print(json.dumps({"metric": "q4f16_1 prefill GEMM, gate_up 28672x4096, M=2048", "value": round(tf, 1),
+                          "unit": "TFLOP/s", "us_per_call": round(ms * 1e3, 1), "steps": args.steps,
+                          "warmup": args.warmup, "frac_mfma": round(tf / MFMA_F16_PEAK_TFLOPS, 3),
+                          "flop_per_call": 2 * m * n * k}))
+        return 0
 
     layers = []
     for layer in range(LAYERS):
@@ -230,7 +255,7 @@ def main() -> int:
 
             def call(qw=qw, qs=qs, k=k, ym=ym):
                 ops.linear(xm[k], qw, qs, BITS, G, None, torch.float16, ym)
-            ms = timed(call, 5, 2, False)
+            ms = timed(call, 20, 8, False)  # (the first launches of a process run 5-30 % slow while clocks settle)
             tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
             gemm[f"{name}_m{m}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
                                     "frac_mfma": round(tf / MFMA_F16_PEAK_TFLOPS, 3)}
@@ -241,7 +266,7 @@ def main() -> int:
             xm2 = torch.randn((m2, k), generator=gx, device=dev).half()
             ym2 = torch.empty((m2, n), dtype=torch.float16, device=dev)
             qw, qs = layers[0]["gate_up"]
-            ms = timed(lambda: ops.linear(xm2, qw, qs, BITS, G, None, torch.float16, ym2), 5, 2, False)
+            ms = timed(lambda: ops.linear(xm2, qw, qs, BITS, G, None, torch.float16, ym2), 10, 4, False)
             tf = 2.0 * m2 * n * k / (ms * 1e-3) / 1e12
             gemm[f"gate_up_m{m2}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),
                                       "frac_mfma": round(tf / MFMA_F16_PEAK_TFLOPS, 3)}
@@ -252,7 +277,7 @@ def main() -> int:
         for name in ("gate_up", "down"):
             n, k = SHAPES[name]
             wd = (torch.randn((n, k), generator=gx, device=dev) * 0.02).half()
-            ms = timed(lambda: torch.nn.functional.linear(xm[k], wd), 5, 2, False)
+            ms = timed(lambda: torch.nn.functional.linear(xm[k], wd), 20, 8, False)
             lib[f"{name}_m{m}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(2.0 * m * n * k / (ms * 1e-3) / 1e12, 1)}
             del wd
         extra["library_dense_fp16_gemm_reference"] = lib
