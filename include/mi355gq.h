@@ -315,6 +315,26 @@ MI355GQ_API int mi355gq_moe_combine_sorted(const void* y, const void* slot_posit
                                int64_t T, int64_t top_k, int64_t H, void* out, mi355gq_stream_t stream);
 
 /*
+ * The folded gate/up activation (mi355gq_linear_silu_mul, mi355gq_moe_gemv_silu_mul, mi355gq_moe_group_gemm_silu_mul)
+ * for bfloat16 models: y / out in bfloat16 [.., N / 2], equal bit for bit to the plain entry followed by
+ * mi355gq_silu_mul_dt.  MI355GQ_F16 forwards to the float16 entries; MI355GQ_F32 and shapes without a fused kernel
+ * return MI355GQ_ERR_UNSUPPORTED (run the two steps).
+ */
+MI355GQ_API int64_t mi355gq_linear_silu_mul_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits,
+                                                   int group_size, int model_dtype);
+MI355GQ_API int mi355gq_linear_silu_mul_dt(const void* x, const void* q_weight, const void* q_scale, int64_t M,
+                               int64_t N, int64_t K, int bits, int group_size, int model_dtype, void* y,
+                               void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_moe_gemv_silu_mul_dt(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                                 const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N,
+                                 int64_t K, int bits, int group_size, int model_dtype, void* out,
+                                 mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_moe_group_gemm_silu_mul_dt(const void* x, int64_t rows, const void* q_weight,
+                                       const void* q_scale, const void* indptr, int indptr_dtype,
+                                       int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,
+                                       int model_dtype, void* out, mi355gq_stream_t stream);
+
+/*
  * The routing glue for the other model dtypes (logits, weights, activations and results in model_dtype =
  * MI355GQ_F32 or MI355GQ_BF16; MI355GQ_F16 is the entries above): the same operations with every
  * intermediate the reference stores rounded to that dtype (softmax in fp32 as in moe_misc.py:205-219; silu in

@@ -445,14 +445,20 @@ static int moe_gemv_impl(const void* x, int64_t x_rows, const void* q_weight, co
   return hip_result(e, "moe_gemv launch");
 }
 
+// paired: the fused gate/up form (y in the model dtype, [M, N / 2]); float16 and bfloat16 models
 static int linear_dt_impl(const void* x, const void* q_weight, const void* q_scale, const void* bias,
                           const void* residual, int64_t M, int64_t N, int64_t K, int bits, int group_size,
                           int model_dtype, int out_dtype, void* y, void* workspace, int64_t workspace_bytes,
-                          mi355gq_stream_t stream) {
+                          mi355gq_stream_t stream, bool paired = false) {
   GQ_CHECK(check_model_dtype(model_dtype, "linear_dt"));
   if (model_dtype == MI355GQ_F16)
     return linear_impl(x, q_weight, q_scale, bias, residual, M, N, K, bits, group_size, out_dtype, y, workspace,
-                       workspace_bytes, stream);
+                       workspace_bytes, stream, paired);
+  if (paired) {
+    GQ_REQUIRE((N & 1) == 0, "linear_silu_mul_dt: N=%lld must be even", (long long)N);
+    if (model_dtype != MI355GQ_BF16)
+      return fail(MI355GQ_ERR_UNSUPPORTED, "linear_silu_mul_dt: no fused kernel for float32 models");
+  }
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(M >= 0 && N >= 0 && K >= 1 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
              "linear_dt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
@@ -478,9 +484,16 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
     a.M = M; a.N = N; a.K = K; a.slots = 1; a.x_slot_stride = 0; a.num_experts = 1;
     a.bits = bits; a.group_size = group_size; a.out_f32 = out_dtype == MI355GQ_F32;
     a.bf16 = 1;
+    a.paired = paired;
     const hipError_t e = gq::launch_gemv(a, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemv launch");
+    // (one or two rows: the plain linear may still take the GEMV where its fused form does not exist, so the
+    //  caller runs the two steps and the result stays the same bit for bit)
+    if (paired) return fail(MI355GQ_ERR_UNSUPPORTED, "linear_silu_mul_dt: no fused GEMV for M=%lld K=%lld",
+                            (long long)M, (long long)K);
   }
+  if (paired && M <= 2)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "linear_silu_mul_dt: x must be 16-byte aligned");
   if (model_dtype == MI355GQ_BF16 && M > 1 && (K & 7) == 0 && aligned16(x)) {
     gq::GemmArgs g{};
     g.x = static_cast<const uint16_t*>(x);
@@ -494,6 +507,7 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
     g.bits = bits; g.group_size = group_size; g.out_f32 = out_dtype == MI355GQ_F32;
     g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
     g.bf16 = 1;
+    g.paired = paired;
     // up to 8 rows: the float16 path's quad-row kernel on the bf16 4x4x4 matrix instruction
     if (M <= 8) {
       const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
@@ -503,6 +517,9 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemm launch");
   }
+  if (paired)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "linear_silu_mul_dt: no fused kernel for M=%lld N=%lld K=%lld (K %% 8 != 0?)",
+                (long long)M, (long long)N, (long long)K);
   return hip_result(gq::launch_linear_dt(x, static_cast<const uint32_t*>(q_weight), q_scale, bias, residual, M, N, K,
                                          bits, group_size, model_dtype, out_dtype, y, as_stream(stream)),
                     "linear_dt launch");
@@ -513,6 +530,20 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
                       void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
   return linear_dt_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, model_dtype, out_dtype, y,
                         workspace, workspace_bytes, stream);
+}
+
+int64_t mi355gq_linear_silu_mul_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size,
+                                                   int model_dtype) {
+  if (model_dtype == MI355GQ_F16) return mi355gq_linear_silu_mul_workspace_bytes(M, N, K, bits, group_size);
+  if ((N % 64) != 0) return 0;  // the partial sums of the fused form need whole 32 + 32 column blocks
+  return mi355gq_linear_dt_workspace_bytes(M, N, K, bits, group_size, model_dtype);
+}
+
+int mi355gq_linear_silu_mul_dt(const void* x, const void* q_weight, const void* q_scale, int64_t M, int64_t N,
+                               int64_t K, int bits, int group_size, int model_dtype, void* y, void* workspace,
+                               int64_t workspace_bytes, mi355gq_stream_t stream) {
+  return linear_dt_impl(x, q_weight, q_scale, nullptr, nullptr, M, N, K, bits, group_size, model_dtype, model_dtype, y,
+                        workspace, workspace_bytes, stream, true);
 }
 
 int mi355gq_linear_residual_dt(const void* x, const void* q_weight, const void* q_scale, const void* bias,
@@ -622,13 +653,17 @@ int mi355gq_moe_experts(const void* x, int64_t x_rows, const void* x_row_index, 
                              x_rows);
 }
 
-int mi355gq_moe_gemv_dt(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
-                        const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N, int64_t K, int bits,
-                        int group_size, int model_dtype, void* out, mi355gq_stream_t stream) {
+static int moe_gemv_dt_impl(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                            const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N, int64_t K,
+                            int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream,
+                            bool paired) {
   GQ_CHECK(check_model_dtype(model_dtype, "moe_gemv_dt"));
   if (model_dtype == MI355GQ_F16)
     return moe_gemv_impl(x, x_rows, q_weight, q_scale, expert_ids, top_k, num_experts, N, K, bits, group_size, out,
-                         stream, false);
+                         stream, paired);
+  GQ_REQUIRE(!paired || (N & 1) == 0, "moe_gemv_silu_mul_dt: N=%lld must be even", (long long)N);
+  if (paired && model_dtype != MI355GQ_BF16)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_gemv_silu_mul_dt: no fused kernel for float32 models");
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(top_k >= 0 && top_k <= 65535 && N >= 0 && K >= 1 && N < kMaxDim && K < kMaxDim && num_experts > 0 &&
                  num_experts < kMaxDim,
@@ -654,22 +689,44 @@ int mi355gq_moe_gemv_dt(const void* x, int64_t x_rows, const void* q_weight, con
     a.num_experts = num_experts;
     a.bits = bits; a.group_size = group_size; a.out_f32 = 0;
     a.bf16 = 1;
+    a.paired = paired;
     const hipError_t e = gq::launch_gemv(a, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "moe_gemv_dt gemv launch");
   }
+  if (paired)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_gemv_silu_mul_dt: no fused kernel for N=%lld K=%lld", (long long)N,
+                (long long)K);
   return hip_result(gq::launch_moe_gemv_dt(x, x_rows == 1, static_cast<const uint32_t*>(q_weight), q_scale,
                                            static_cast<const int32_t*>(expert_ids), top_k, num_experts, N, K, bits,
                                            group_size, model_dtype, out, as_stream(stream)),
                     "moe_gemv_dt launch");
 }
 
-int mi355gq_moe_group_gemm_dt(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
-                              const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N, int64_t K,
-                              int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream) {
+int mi355gq_moe_gemv_dt(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                        const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N, int64_t K, int bits,
+                        int group_size, int model_dtype, void* out, mi355gq_stream_t stream) {
+  return moe_gemv_dt_impl(x, x_rows, q_weight, q_scale, expert_ids, top_k, num_experts, N, K, bits, group_size,
+                          model_dtype, out, stream, false);
+}
+
+int mi355gq_moe_gemv_silu_mul_dt(const void* x, int64_t x_rows, const void* q_weight, const void* q_scale,
+                                 const void* expert_ids, int64_t top_k, int64_t num_experts, int64_t N, int64_t K,
+                                 int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream) {
+  return moe_gemv_dt_impl(x, x_rows, q_weight, q_scale, expert_ids, top_k, num_experts, N, K, bits, group_size,
+                          model_dtype, out, stream, true);
+}
+
+static int moe_group_gemm_dt_impl(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                                  const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N, int64_t K,
+                                  int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream,
+                                  bool paired) {
   GQ_CHECK(check_model_dtype(model_dtype, "moe_group_gemm_dt"));
   if (model_dtype == MI355GQ_F16)
     return moe_group_gemm_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
-                               group_size, out, stream, false);
+                               group_size, out, stream, paired);
+  GQ_REQUIRE(!paired || (N & 1) == 0, "moe_group_gemm_silu_mul_dt: N=%lld must be even", (long long)N);
+  if (paired && model_dtype != MI355GQ_BF16)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul_dt: no fused kernel for float32 models");
   GQ_CHECK(check_scheme(bits, group_size));
   GQ_REQUIRE(rows >= 0 && N >= 0 && K >= 1 && rows < kMaxDim && N < kMaxDim && K < kMaxDim && num_experts > 0 &&
                  num_experts <= 65536,
@@ -696,6 +753,7 @@ int mi355gq_moe_group_gemm_dt(const void* x, int64_t rows, const void* q_weight,
     g.rows = rows; g.N = N; g.K = K; g.num_experts = num_experts;
     g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
     g.bf16 = 1;
+    g.paired = paired;
     // few rows in total: every expert streams its weights for a handful of rows (as in float16)
     const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;
     if (rows <= quad_rows && rows <= 128) {
@@ -705,10 +763,28 @@ int mi355gq_moe_group_gemm_dt(const void* x, int64_t rows, const void* q_weight,
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "moe_group_gemm_dt gemm launch");
   }
+  if (paired)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul_dt: no fused kernel for N=%lld K=%lld",
+                (long long)N, (long long)K);
   return hip_result(gq::launch_moe_group_gemm_dt(x, static_cast<const uint32_t*>(q_weight), q_scale, indptr,
                                                  indptr_dtype == MI355GQ_I64, rows, num_experts, N, K, bits,
                                                  group_size, model_dtype, out, as_stream(stream)),
                     "moe_group_gemm_dt launch");
+}
+
+int mi355gq_moe_group_gemm_dt(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                              const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N, int64_t K,
+                              int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream) {
+  return moe_group_gemm_dt_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
+                                group_size, model_dtype, out, stream, false);
+}
+
+int mi355gq_moe_group_gemm_silu_mul_dt(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
+                                       const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
+                                       int64_t K, int bits, int group_size, int model_dtype, void* out,
+                                       mi355gq_stream_t stream) {
+  return moe_group_gemm_dt_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
+                                group_size, model_dtype, out, stream, true);
 }
 
 static int gating_impl(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights, void* ids,

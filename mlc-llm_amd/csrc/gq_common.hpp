@@ -87,6 +87,18 @@ __device__ __forceinline__ uint16_t silu_mul_h(float gate, float up) {
   const float silu = h2f(f2h(g * __builtin_amdgcn_rcpf(1.0f + e)));
   return f2h(silu * u);
 }
+// the same for a bfloat16 model: bfloat16 rounding points, hardware exp2 / reciprocal (1 ulp each, far inside
+// the bfloat16 rounding); the element-wise silu_mul kernel of the bfloat16 models calls this very function
+__device__ __forceinline__ uint16_t silu_mul_bf(float gate, float up) {
+  const float g = bf2f(f2bf(gate)), u = bf2f(f2bf(up));
+  const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896341f);
+  const float silu = bf2f(f2bf(g * __builtin_amdgcn_rcpf(1.0f + e)));
+  return f2bf(silu * u);
+}
+template <bool BF>
+__device__ __forceinline__ uint16_t silu_mul_t(float gate, float up) {
+  return BF ? silu_mul_bf(gate, up) : silu_mul_h(gate, up);
+}
 
 // Sum over the 64 lanes of a wave; every lane ends up with the total.
 // quad_perm and row-mirror steps are DPP moves, the two widest steps cross rows via bpermute.

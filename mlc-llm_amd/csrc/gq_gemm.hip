@@ -242,7 +242,7 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
       if (p.paired) {
         hipLaunchKernelGGL(splitk_reduce_silu_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,
                            p.partial, split, a.rows, p.N, gemm_pipe_pair_block(p, a.bits),
-                           static_cast<uint16_t*>(p.y));
+                           static_cast<uint16_t*>(p.y), p.bf16);
         return hipGetLastError();
       }
       hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s,

@@ -59,7 +59,7 @@ __global__ void splitk_reduce_kernel(const float* partial, int split, int64_t co
                                      const uint16_t* bias, const uint16_t* residual, void* y, int out_f32, int bf16);
 // fused gate/up form: partial[split][rows][N] in the block-interleaved column order -> y fp16 [rows, N / 2]
 __global__ void splitk_reduce_silu_kernel(const float* partial, int split, int64_t rows, int N, int pb,
-                                          uint16_t* y);
+                                          uint16_t* y, int bf16);
 // gate rows per column block (32 | 16) of the tile launch_gemm_pipe picks for these parameters
 int gemm_pipe_pair_block(const GemmParams& p, int bits);
 

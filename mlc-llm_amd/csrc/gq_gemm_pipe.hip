@@ -235,7 +235,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
             const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             if (row < seg_hi && col < half)
               static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * half + col] =
-                  silu_mul_h(acc[i][2 * jj][r], acc[i][2 * jj + 1][r]);
+                  silu_mul_t<BF>(acc[i][2 * jj][r], acc[i][2 * jj + 1][r]);
           }
         }
       }
@@ -250,7 +250,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
           const float up = __shfl_xor(acc[i][0][r], 16, 64);  // every lane takes part
           const int row = m0 + wm0 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
           if ((lane & 16) == 0 && row < seg_hi && col < half)
-            static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * half + col] = silu_mul_h(acc[i][0][r], up);
+            static_cast<uint16_t*>(p.y)[static_cast<int64_t>(row) * half + col] = silu_mul_t<BF>(acc[i][0][r], up);
         }
       }
     }
@@ -366,7 +366,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restr
 
 __global__ __launch_bounds__(256) void splitk_reduce_silu_kernel(const float* __restrict__ partial, int split,
                                                                  int64_t rows, int N, int pb,
-                                                                 uint16_t* __restrict__ y) {
+                                                                 uint16_t* __restrict__ y, int bf16) {
   const int half = N >> 1;
   const int64_t count = rows * N, outs = rows * half;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -379,7 +379,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_silu_kernel(const float* __
       g += partial[sidx * count + at];
       u += partial[sidx * count + at + pb];
     }
-    y[i] = silu_mul_h(g, u);
+    y[i] = bf16 ? silu_mul_bf(g, u) : silu_mul_h(g, u);
   }
 }
 
@@ -426,11 +426,13 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   if (p.paired && (p.N & 1)) return hipErrorNotSupported;
   if (p.bf16) {
     // bfloat16 models: plain and grouped matmul (no folded activation)
-    if (p.paired || p.x_rows != nullptr) return hipErrorNotSupported;
+    if (p.x_rows != nullptr) return hipErrorNotSupported;
     if (p.bm_hint > 0 && p.indptr == nullptr) {  // few rows, K possibly split (see plan_split_k)
       if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4, true>(p, s);
       if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4, true>(p, s);
       if (bits == 4) return launch_pipe_cfg<4, 128, 128, 64, 64, 2, true>(p, s);
+      if (p.bm_hint == 32) return launch_pipe_cfg<3, 32, 128, 32, 32, 4, true>(p, s);
+      if (p.bm_hint == 64) return launch_pipe_cfg<3, 64, 128, 32, 64, 4, true>(p, s);
       return launch_pipe_cfg<3, 128, 128, 64, 64, 2, true>(p, s);
     }
     if (p.partial != nullptr) return hipErrorNotSupported;

@@ -26,7 +26,6 @@ template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false>
 __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int nsets) {
   using T = GemvTraits<BITS>;
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;
-  static_assert(!(BF && PAIRED), "the fused gate/up form is float16 only");
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
   static_assert(!PAIRED || R % 2 == 0, "a set holds whole (gate, up) pairs");
   constexpr int G = T::G;
@@ -176,7 +175,7 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
 #pragma unroll
             for (int b = 0; b < NB; ++b)
               static_cast<uint16_t*>(p.y)[static_cast<int64_t>(slot + b) * (p.N >> 1) + col] =
-                  silu_mul_h(acc[r][b], acc[r + 1][b]);
+                  silu_mul_t<BF>(acc[r][b], acc[r + 1][b]);
           }
         }
       }
@@ -223,7 +222,13 @@ static hipError_t launch_k(const GemvParams& p, int slots, int blocks, int nsets
   const size_t lds = static_cast<size_t>(NB) * p.ng * GemvTraits<BITS>::G * 2;
   const dim3 grid(blocks, slots);
   if (p.bf16) {
-    if (p.paired) return hipErrorNotSupported;
+    if (p.paired) {
+      if constexpr (R % 2 == 0)
+        hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 2, true>), grid, dim3(threads), lds, s, p, nsets);
+      else
+        return hipErrorNotSupported;
+      return hipGetLastError();
+    }
     if (p.bias != nullptr || p.residual != nullptr)
       hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 1, true>), grid, dim3(threads), lds, s, p, nsets);
     else

@@ -299,6 +299,8 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const void* __restrict__ 
   const float x3 = Elem<DT>::load(x, r * 2 * I + I + c);
   if constexpr (DT == MODEL_F16) {
     static_cast<uint16_t*>(out)[i] = silu_mul_h(x1, x3);
+  } else if constexpr (DT == MODEL_BF16) {
+    static_cast<uint16_t*>(out)[i] = silu_mul_bf(x1, x3);  // (shared with the matmul kernels' folded form)
   } else {
     const float silu = Elem<DT>::rnd(x1 / (1.0f + expf(-x1)));
     Elem<DT>::store(out, i, silu * x3);

@@ -85,7 +85,6 @@ __device__ __forceinline__ float4_t mfma4_bf16(uint32_t a0, uint32_t a1, uint32_
 template <int BITS, int NBQ, int U, int MODE, bool BF = false>
 __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;  // 2: fused gate/up form, quad = 2 (gate, up) pairs
-  static_assert(!(BF && PAIRED), "the fused gate/up form is float16 only");
   constexpr uint32_t kMagic = BF ? 0x43004300u : 0x64006400u;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
   auto to_out = [](float v) { return BF ? f2bf(v) : f2h(v); };
@@ -371,8 +370,8 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
               const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
               if constexpr (PAIRED) {
                 *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p.y) + (oi >> 1)) =
-                    static_cast<uint32_t>(silu_mul_h(v[0], v[1])) |
-                    (static_cast<uint32_t>(silu_mul_h(v[2], v[3])) << 16);
+                    static_cast<uint32_t>(silu_mul_t<BF>(v[0], v[1])) |
+                    (static_cast<uint32_t>(silu_mul_t<BF>(v[2], v[3])) << 16);
               } else if (p.out_f32) {
                 *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) =
                     make_float4(v[0], v[1], v[2], v[3]);
@@ -419,7 +418,7 @@ template <int BITS, int NBQ, int U>
 static hipError_t launch_quad_cfg(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                   hipStream_t s) {
   if (p.bf16) {
-    if (p.paired) return hipErrorNotSupported;
+    if (p.paired) return launch_quad_extra<BITS, NBQ, U, 2, true>(p, grid, threads, lds, s);
     return (p.bias != nullptr || p.residual != nullptr)
                ? launch_quad_extra<BITS, NBQ, U, 1, true>(p, grid, threads, lds, s)
                : launch_quad_extra<BITS, NBQ, U, 0, true>(p, grid, threads, lds, s);

@@ -297,6 +297,41 @@ void MoeGroupGemmDt(TensorView x, TensorView q_weight, TensorView q_scale, Tenso
         "mlc.gq.moe_group_gemm_dt");
 }
 
+// the folded gate/up activation for bfloat16 models (y / out are [.., N / 2] in the model dtype)
+void LinearSiluMulDt(TensorView x, TensorView q_weight, TensorView q_scale, int64_t bits, int64_t group_size,
+                     int64_t model_dtype, Optional<TensorView> workspace, TensorView y) {
+  const int64_t K = x.shape()[x.ndim() - 1], N = q_weight.shape()[0];
+  void* ws = workspace.has_value() ? Ptr(workspace.value()) : nullptr;
+  int64_t ws_bytes = 0;
+  if (workspace.has_value()) {
+    ws_bytes = (workspace.value().dtype().bits + 7) / 8;
+    for (int i = 0; i < workspace.value().ndim(); ++i) ws_bytes *= workspace.value().shape()[i];
+  }
+  Check(mi355gq_linear_silu_mul_dt(Ptr(x), Ptr(q_weight), Ptr(q_scale), Rows(x), N, K, static_cast<int>(bits),
+                                   static_cast<int>(group_size), static_cast<int>(model_dtype), Ptr(y), ws,
+                                   ws_bytes, StreamOf(x)),
+        "mlc.gq.linear_silu_mul_dt");
+}
+
+void MoeGemvSiluMulDt(TensorView x, TensorView q_weight, TensorView q_scale, TensorView expert_ids, int64_t bits,
+                      int64_t group_size, int64_t model_dtype, TensorView out) {
+  Check(mi355gq_moe_gemv_silu_mul_dt(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(expert_ids),
+                                     expert_ids.shape()[1], q_weight.shape()[0], q_weight.shape()[1], x.shape()[1],
+                                     static_cast<int>(bits), static_cast<int>(group_size),
+                                     static_cast<int>(model_dtype), Ptr(out), StreamOf(x)),
+        "mlc.gq.moe_gemv_silu_mul_dt");
+}
+
+void MoeGroupGemmSiluMulDt(TensorView x, TensorView q_weight, TensorView q_scale, TensorView indptr, int64_t bits,
+                           int64_t group_size, int64_t model_dtype, TensorView out) {
+  Check(mi355gq_moe_group_gemm_silu_mul_dt(Ptr(x), x.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(indptr),
+                                           indptr.dtype().bits == 64 ? MI355GQ_I64 : MI355GQ_I32,
+                                           q_weight.shape()[0], q_weight.shape()[1], x.shape()[1],
+                                           static_cast<int>(bits), static_cast<int>(group_size),
+                                           static_cast<int>(model_dtype), Ptr(out), StreamOf(x)),
+        "mlc.gq.moe_group_gemm_silu_mul_dt");
+}
+
 // routing glue with logits, weights and activations in model_dtype
 void GatingSoftmaxTopkDt(TensorView logits, int64_t top_k, int64_t model_dtype, TensorView weights, TensorView ids) {
   Check(mi355gq_gating_softmax_topk_dt(Ptr(logits), logits.shape()[0], logits.shape()[1], top_k, Ptr(weights),
@@ -354,6 +389,9 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.linear_dt", LinearDt)
       .def("mlc.gq.linear_dt_workspace_bytes", LinearDtWorkspaceBytes)
       .def("mlc.gq.linear_residual_dt", LinearResidualDt)
+      .def("mlc.gq.linear_silu_mul_dt", LinearSiluMulDt)
+      .def("mlc.gq.moe_gemv_silu_mul_dt", MoeGemvSiluMulDt)
+      .def("mlc.gq.moe_group_gemm_silu_mul_dt", MoeGroupGemmSiluMulDt)
       .def("mlc.gq.gating_softmax_topk_dt", GatingSoftmaxTopkDt)
       .def("mlc.gq.take_rows_dt", TakeRowsDt)
       .def("mlc.gq.moe_scatter_output_dt", ScatterOutputDt)

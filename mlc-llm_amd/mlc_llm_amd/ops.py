@@ -204,9 +204,9 @@ def linear_silu_mul(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tens
     """silu(x1) * x2 with x1, x2 = split(linear(x), 2, axis=-1): the gate_up projection of an MLP
     with its activation folded into the matmul kernel.  Bit-identical to linear then silu_mul;
     shapes without a fused kernel run exactly those two calls."""
-    _chk(x, torch.float16, "x")
+    _chk(x, _FLOATS, "x")
     _chk(q_weight, _STORAGE, "q_weight")
-    _chk(q_scale, torch.float16, "q_scale")
+    _chk(q_scale, x.dtype, "q_scale")
     k = x.shape[-1]
     n = q_weight.shape[0]
     _check_qshapes(q_weight, q_scale, (n,), k, bits, group_size)
@@ -215,12 +215,13 @@ def linear_silu_mul(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tens
     m = 1
     for d in x.shape[:-1]:
         m *= d
-    out = torch.empty((*x.shape[:-1], n // 2), dtype=torch.float16, device=x.device)
-    ws_bytes = _lib.lib().mi355gq_linear_silu_mul_workspace_bytes(m, n, k, bits, group_size)
+    out = torch.empty((*x.shape[:-1], n // 2), dtype=x.dtype, device=x.device)
+    dt = _MODEL_DTYPES[x.dtype]
+    ws_bytes = _lib.lib().mi355gq_linear_silu_mul_dt_workspace_bytes(m, n, k, bits, group_size, dt)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
     try:
-        _lib.call("mi355gq_linear_silu_mul", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(), m, n, k,
-                  bits, group_size, out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
+        _lib.call("mi355gq_linear_silu_mul_dt", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(), m, n, k,
+                  bits, group_size, dt, out.data_ptr(), ws.data_ptr() if ws is not None else None, ws_bytes,
                   _stream())
     except _lib.Mi355gqError as err:
         if not _unsupported(err):
@@ -245,12 +246,21 @@ def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
     _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
     top_k = expert_ids.shape[1]
     if x.dtype != torch.float16:
+        dt_args = (x.data_ptr(), x.shape[0], q_weight.data_ptr(), q_scale.data_ptr(), expert_ids.data_ptr(), top_k, ne,
+                   n, k, bits, group_size, _MODEL_DTYPES[x.dtype])
         if silu_mul_halves:
-            raise NotImplementedError("moe_gemv: the SiLU epilogue exists for float16 models only")
+            if n % 2:
+                raise ValueError(f"moe_gemv: {n} rows cannot be split into gate and up halves")
+            out = torch.empty((top_k, n // 2), dtype=x.dtype, device=x.device)
+            try:
+                _lib.call("mi355gq_moe_gemv_silu_mul_dt", *dt_args, out.data_ptr(), _stream())
+                return out
+            except _lib.Mi355gqError as err:
+                if not _unsupported(err):
+                    raise
+                return silu_mul(moe_gemv(x, q_weight, q_scale, expert_ids, bits, group_size))
         out = torch.empty((top_k, n), dtype=x.dtype, device=x.device)
-        _lib.call("mi355gq_moe_gemv_dt", x.data_ptr(), x.shape[0], q_weight.data_ptr(), q_scale.data_ptr(),
-                  expert_ids.data_ptr(), top_k, ne, n, k, bits, group_size, _MODEL_DTYPES[x.dtype], out.data_ptr(),
-                  _stream())
+        _lib.call("mi355gq_moe_gemv_dt", *dt_args, out.data_ptr(), _stream())
         return out
     args = (x.data_ptr(), x.shape[0], q_weight.data_ptr(), q_scale.data_ptr(), expert_ids.data_ptr(), top_k, ne,
             n, k, bits, group_size)
@@ -284,12 +294,22 @@ def moe_group_gemm(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tenso
     if tuple(indptr.shape) != (ne + 1,):
         raise ValueError(f"indptr shape {tuple(indptr.shape)}, expected {(ne + 1,)}")
     if x.dtype != torch.float16:
+        dt_args = (x.data_ptr(), rows, q_weight.data_ptr(), q_scale.data_ptr(), indptr.data_ptr(),
+                   _lib.I64 if indptr.dtype == torch.int64 else _lib.I32, ne, n, k, bits, group_size,
+                   _MODEL_DTYPES[x.dtype])
         if silu_mul_halves:
-            raise NotImplementedError("moe_group_gemm: the SiLU epilogue exists for float16 models only")
+            if n % 2:
+                raise ValueError(f"moe_group_gemm: {n} rows cannot be split into gate and up halves")
+            out = torch.zeros((rows, n // 2), dtype=x.dtype, device=x.device)
+            try:
+                _lib.call("mi355gq_moe_group_gemm_silu_mul_dt", *dt_args, out.data_ptr(), _stream())
+                return out
+            except _lib.Mi355gqError as err:
+                if not _unsupported(err):
+                    raise
+                return silu_mul(moe_group_gemm(x, q_weight, q_scale, indptr, bits, group_size))
         out = torch.zeros((rows, n), dtype=x.dtype, device=x.device)
-        _lib.call("mi355gq_moe_group_gemm_dt", x.data_ptr(), rows, q_weight.data_ptr(), q_scale.data_ptr(),
-                  indptr.data_ptr(), _lib.I64 if indptr.dtype == torch.int64 else _lib.I32, ne, n, k, bits,
-                  group_size, _MODEL_DTYPES[x.dtype], out.data_ptr(), _stream())
+        _lib.call("mi355gq_moe_group_gemm_dt", *dt_args, out.data_ptr(), _stream())
         return out
     args = (x.data_ptr(), rows, q_weight.data_ptr(), q_scale.data_ptr(), indptr.data_ptr(),
             _lib.I64 if indptr.dtype == torch.int64 else _lib.I32, ne, n, k, bits, group_size)

@@ -262,9 +262,7 @@ class GroupQuantizeLinear(nn.Module):
         """For a gate_up projection: `x1, x2 = split(self(x), 2, axis=-1); silu(x1) * x2` of the MLP
         (model/llama/llama_model.py:122-125) in one kernel; same bits as the two steps."""
         self.config._require_built()
-        if self.config.model_dtype != "float16":
-            raise NotImplementedError(f"{self.config.name}: silu * mul (folded or not) is built for float16 models")
-        if self.bias is not None or self.out_dtype not in (None, "float16"):
+        if self.bias is not None or self.out_dtype not in (None, self.config.model_dtype):
             return ops.silu_mul(self.forward(x).reshape(-1, self.out_features)).reshape(*x.shape[:-1], -1)
         q_weight, q_scale = self._nk_tensors()
         return ops.linear_silu_mul(x, q_weight, q_scale, self.config.bits, self.config.group_size)
@@ -355,9 +353,6 @@ class GroupQuantizeMixtralExperts(nn.Module):
         assert x.dim() == 2
         if self.config.model_dtype not in MOE_MODEL_DTYPES:
             raise NotImplementedError(f"{self.config.name}: the expert matmuls are built for {MOE_MODEL_DTYPES} models")
-        if silu_mul_halves and x.dtype != torch.float16:
-            # the folded activation exists for float16 models; the others run the two steps
-            return ops.silu_mul(self.forward(x, indptr))
         if indptr.dim() == 2:
             assert indptr.shape[0] == 1
             return ops.moe_gemv(x, self.q_weight, self.q_scale, indptr, self.config.bits,

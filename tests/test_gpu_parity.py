@@ -1153,6 +1153,61 @@ def test_mixtral_moe_layer_other_model_dtypes(model_dtype, t):
     assert rel <= (1.5e-2 if model_dtype == "bfloat16" else 1e-5), rel
 
 
+@pytest.mark.parametrize("bits_name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("m,n,k", [(1, 256, 4096), (1, 128, 8192), (1, 64, 14336), (2, 256, 4096), (2, 128, 8192),
+                                   (4, 132, 2048), (8, 64, 1000), (3, 64, 13), (16, 128, 8192), (40, 192, 4096),
+                                   (100, 200, 1024), (130, 256, 1024), (600, 384, 512)])
+def test_linear_silu_mul_bfloat16_equals_the_two_steps(bits_name, m, n, k):
+    """The folded gate/up activation of a bfloat16 model in every kernel family; shapes without a fused kernel
+    run the two steps, so the equality holds for all of them."""
+    s = SCHEMES[bits_name]
+    rng = np.random.default_rng(m + n + k)
+    w32 = o.round_to((rng.standard_normal((n, k)) * 0.05).astype(np.float32), "bfloat16")
+    qw_ref, qs_ref = o.quantize_dt(w32, s, "bfloat16")
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).bfloat16().to(DEV)
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).bfloat16().to(DEV)
+    fused = ops.linear_silu_mul(x, qw, qs, s.bits, s.group_size)
+    assert fused.dtype == torch.bfloat16 and tuple(fused.shape) == (m, n // 2)
+    plain = ops.linear(x, qw, qs, s.bits, s.group_size)
+    two = ops.silu_mul(plain)
+    # a fused GEMM whose plain counterpart splits K sums in another order (N % 64 != 0 keeps the fused one unsplit)
+    split_differs = m > 8 and n % 64 != 0 and gq._lib.lib().mi355gq_linear_dt_workspace_bytes(m, n, k, s.bits, s.group_size, 2) > 0
+    if split_differs:
+        assert (fused.float() - two.float()).abs().max() <= 2.0 ** -6 * two.float().abs().max()
+    else:
+        assert torch.equal(fused, two), f"{(fused != two).sum().item()} of {fused.numel()} differ"
+    # and the value: silu(g) * u of the oracle's product, at the matmul tolerance carried through the two factors
+    ref = o.linear_dt_fp64(_carrier(x), qw_ref, qs_ref, s, "bfloat16")
+    g, u = ref[:, : n // 2], ref[:, n // 2:]
+    want = g / (1.0 + np.exp(-g)) * u
+    err = np.abs(fused.double().cpu().numpy() - want)
+    tol = 1e-2 * float(x.float().abs().max()) * np.sqrt(k) / 64
+    bound = tol * (1.1 * np.abs(u) + np.abs(g / (1.0 + np.exp(-g)))) + 3 * 2.0 ** -8 * np.abs(want) + 2.0 ** -14
+    assert (err <= bound).all(), (err - bound).max()
+
+
+def test_moe_silu_mul_bfloat16_equals_the_two_steps():
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(92)
+    ne, n, k = 4, 512, 1280
+    w32 = o.round_to((rng.standard_normal((ne, n, k)) * 0.05).astype(np.float32), "bfloat16")
+    qw_ref, qs_ref = o.quantize_dt(w32, s, "bfloat16")
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).bfloat16().to(DEV)
+    x1 = torch.from_numpy(rng.standard_normal((1, k)).astype(np.float32)).bfloat16().to(DEV)
+    ids = torch.tensor([[3, 1]], dtype=torch.int32, device=DEV)
+    y = ops.moe_gemv(x1, qw, qs, ids, 4, 32, silu_mul_halves=True)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (2, n // 2)
+    assert torch.equal(y, ops.silu_mul(ops.moe_gemv(x1, qw, qs, ids, 4, 32)))
+    for rows, indptr in ((20, [0, 7, 7, 15, 20]), (50, [0, 20, 21, 21, 50]), (100, [0, 40, 41, 41, 100]),
+                         (700, [0, 300, 380, 700, 700])):
+        x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).bfloat16().to(DEV)
+        ip = torch.tensor(indptr, dtype=torch.int32, device=DEV)
+        y = ops.moe_group_gemm(x, qw, qs, ip, 4, 32, silu_mul_halves=True)
+        assert tuple(y.shape) == (rows, n // 2)
+        two = ops.silu_mul(ops.moe_group_gemm(x, qw, qs, ip, 4, 32))
+        assert torch.equal(y, two), f"rows={rows}: {(y != two).sum().item()} differ"
+
+
 def test_linear_other_model_dtypes_through_the_modules():
     for name in ("q4f32_1", "q4bf16_1", "q4bf16_0"):
         cfg = gq.QUANTIZATION[name]

@@ -117,6 +117,15 @@ def test_argument_validation_of_the_later_entry_points():
     assert "null" in _err()
     assert lib.mi355gq_moe_group_gemm_dt(None, 0, None, None, None, 0, 8, 16, 32, 4, 32, 2, None, None) == 0
     assert lib.mi355gq_moe_gemv_dt(None, 1, None, None, None, 0, 8, 16, 32, 4, 32, 1, None, None) == 0
+    # folded activation in the other model dtypes: float32 has no fused kernel, odd N is an error
+    assert lib.mi355gq_linear_silu_mul_dt(P(0x1000), P(0x2000), P(0x3000), 2, 8, 64, 4, 32, 1, P(0x4000), None, 0,
+                                          None) == _lib.ERR_UNSUPPORTED
+    assert lib.mi355gq_linear_silu_mul_dt(P(0x1000), P(0x2000), P(0x3000), 2, 7, 64, 4, 32, 2, P(0x4000), None, 0,
+                                          None) == -1
+    assert lib.mi355gq_moe_gemv_silu_mul_dt(P(0x1000), 1, P(0x2000), P(0x3000), P(0x4000), 2, 8, 16, 32, 4, 32, 1,
+                                            P(0x5000), None) == _lib.ERR_UNSUPPORTED
+    assert lib.mi355gq_linear_silu_mul_dt_workspace_bytes(40, 100, 4096, 4, 32, 2) == 0  # N % 64 != 0
+    assert lib.mi355gq_linear_silu_mul_dt_workspace_bytes(40, 128, 4096, 4, 32, 2) > 0
     # routing glue in the other model dtypes
     assert lib.mi355gq_gating_softmax_topk_dt(P(0x1000), 4, 8, 9, P(0x2000), P(0x3000), 2, None) == -1
     assert "top_k" in _err()
