@@ -334,6 +334,12 @@ MI355GQ_API int mi355gq_moe_group_gemm_silu_mul_dt(const void* x, int64_t rows, 
                                        int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,
                                        int model_dtype, void* out, mi355gq_stream_t stream);
 
+/* mi355gq_moe_experts for bfloat16 models (float32: MI355GQ_ERR_UNSUPPORTED when x_row_index is given). */
+MI355GQ_API int mi355gq_moe_experts_dt(const void* x, int64_t x_rows, const void* x_row_index, int64_t rows,
+                           const void* q_weight, const void* q_scale, const void* indptr, int indptr_dtype,
+                           int64_t num_experts, int64_t N, int64_t K, int bits, int group_size, int epilogue,
+                           int model_dtype, void* out, mi355gq_stream_t stream);
+
 /*
  * The routing glue for the other model dtypes (logits, weights, activations and results in model_dtype =
  * MI355GQ_F32 or MI355GQ_BF16; MI355GQ_F16 is the entries above): the same operations with every

@@ -719,11 +719,15 @@ int mi355gq_moe_gemv_silu_mul_dt(const void* x, int64_t x_rows, const void* q_we
 static int moe_group_gemm_dt_impl(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
                                   const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N, int64_t K,
                                   int bits, int group_size, int model_dtype, void* out, mi355gq_stream_t stream,
-                                  bool paired) {
+                                  bool paired, const void* x_row_index = nullptr, int64_t x_rows = 0) {
   GQ_CHECK(check_model_dtype(model_dtype, "moe_group_gemm_dt"));
   if (model_dtype == MI355GQ_F16)
     return moe_group_gemm_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits,
-                               group_size, out, stream, paired);
+                               group_size, out, stream, paired, x_row_index, x_rows);
+  if (x_row_index != nullptr && model_dtype != MI355GQ_BF16)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_experts_dt: the gather is folded in for float16 and bfloat16 models");
+  GQ_REQUIRE(x_row_index == nullptr || (x_rows >= 1 && x_rows < kMaxDim && aligned4(x_row_index)),
+             "moe_experts_dt: x has %lld rows", (long long)x_rows);
   GQ_REQUIRE(!paired || (N & 1) == 0, "moe_group_gemm_silu_mul_dt: N=%lld must be even", (long long)N);
   if (paired && model_dtype != MI355GQ_BF16)
     return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul_dt: no fused kernel for float32 models");
@@ -754,6 +758,10 @@ static int moe_group_gemm_dt_impl(const void* x, int64_t rows, const void* q_wei
     g.bits = bits; g.group_size = group_size; g.out_f32 = 0;
     g.bf16 = 1;
     g.paired = paired;
+    if (x_row_index != nullptr) {
+      g.x_rows = static_cast<const int32_t*>(x_row_index);
+      g.x_src_rows = x_rows;
+    }
     // few rows in total: every expert streams its weights for a handful of rows (as in float16)
     const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;
     if (rows <= quad_rows && rows <= 128) {
@@ -763,8 +771,8 @@ static int moe_group_gemm_dt_impl(const void* x, int64_t rows, const void* q_wei
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "moe_group_gemm_dt gemm launch");
   }
-  if (paired)
-    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul_dt: no fused kernel for N=%lld K=%lld",
+  if (paired || x_row_index != nullptr)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_dt: no fused kernel for N=%lld K=%lld (K %% 8 != 0?)",
                 (long long)N, (long long)K);
   return hip_result(gq::launch_moe_group_gemm_dt(x, static_cast<const uint32_t*>(q_weight), q_scale, indptr,
                                                  indptr_dtype == MI355GQ_I64, rows, num_experts, N, K, bits,
@@ -800,6 +808,18 @@ static int gating_impl(const void* logits, int64_t T, int64_t num_experts, int64
   return hip_result(gq::launch_topk_softmax(logits, T, static_cast<int>(num_experts), static_cast<int>(top_k), weights,
                                             static_cast<int32_t*>(ids), model_dtype, as_stream(stream)),
                     "gating_softmax_topk launch");
+}
+
+int mi355gq_moe_experts_dt(const void* x, int64_t x_rows, const void* x_row_index, int64_t rows, const void* q_weight,
+                           const void* q_scale, const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
+                           int64_t K, int bits, int group_size, int epilogue, int model_dtype, void* out,
+                           mi355gq_stream_t stream) {
+  GQ_REQUIRE(epilogue == MI355GQ_EPILOGUE_NONE || epilogue == MI355GQ_EPILOGUE_SILU_MUL, "moe_experts_dt: epilogue=%d",
+             epilogue);
+  GQ_REQUIRE(x_row_index != nullptr || x_rows == rows, "moe_experts_dt: x has %lld rows, expected %lld",
+             (long long)x_rows, (long long)rows);
+  return moe_group_gemm_dt_impl(x, rows, q_weight, q_scale, indptr, indptr_dtype, num_experts, N, K, bits, group_size,
+                                model_dtype, out, stream, epilogue == MI355GQ_EPILOGUE_SILU_MUL, x_row_index, x_rows);
 }
 
 int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,

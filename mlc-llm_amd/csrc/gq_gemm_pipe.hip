@@ -426,7 +426,6 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   if (p.paired && (p.N & 1)) return hipErrorNotSupported;
   if (p.bf16) {
     // bfloat16 models: plain and grouped matmul (no folded activation)
-    if (p.x_rows != nullptr) return hipErrorNotSupported;
     if (p.bm_hint > 0 && p.indptr == nullptr) {  // few rows, K possibly split (see plan_split_k)
       if (bits == 4 && p.bm_hint == 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4, true>(p, s);
       if (bits == 4 && p.bm_hint == 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4, true>(p, s);

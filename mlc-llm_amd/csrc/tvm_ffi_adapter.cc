@@ -332,6 +332,18 @@ void MoeGroupGemmSiluMulDt(TensorView x, TensorView q_weight, TensorView q_scale
         "mlc.gq.moe_group_gemm_silu_mul_dt");
 }
 
+void MoeExpertsDt(TensorView x, Optional<TensorView> x_row_index, TensorView q_weight, TensorView q_scale,
+                  TensorView indptr, int64_t bits, int64_t group_size, int64_t epilogue, int64_t model_dtype,
+                  TensorView out) {
+  Check(mi355gq_moe_experts_dt(Ptr(x), x.shape()[0], x_row_index.has_value() ? Ptr(x_row_index.value()) : nullptr,
+                               out.shape()[0], Ptr(q_weight), Ptr(q_scale), Ptr(indptr),
+                               indptr.dtype().bits == 64 ? MI355GQ_I64 : MI355GQ_I32, q_weight.shape()[0],
+                               q_weight.shape()[1], x.shape()[1], static_cast<int>(bits),
+                               static_cast<int>(group_size), static_cast<int>(epilogue),
+                               static_cast<int>(model_dtype), Ptr(out), StreamOf(x)),
+        "mlc.gq.moe_experts_dt");
+}
+
 // routing glue with logits, weights and activations in model_dtype
 void GatingSoftmaxTopkDt(TensorView logits, int64_t top_k, int64_t model_dtype, TensorView weights, TensorView ids) {
   Check(mi355gq_gating_softmax_topk_dt(Ptr(logits), logits.shape()[0], logits.shape()[1], top_k, Ptr(weights),
@@ -392,6 +404,7 @@ TVM_FFI_STATIC_INIT_BLOCK() {
       .def("mlc.gq.linear_silu_mul_dt", LinearSiluMulDt)
       .def("mlc.gq.moe_gemv_silu_mul_dt", MoeGemvSiluMulDt)
       .def("mlc.gq.moe_group_gemm_silu_mul_dt", MoeGroupGemmSiluMulDt)
+      .def("mlc.gq.moe_experts_dt", MoeExpertsDt)
       .def("mlc.gq.gating_softmax_topk_dt", GatingSoftmaxTopkDt)
       .def("mlc.gq.take_rows_dt", TakeRowsDt)
       .def("mlc.gq.moe_scatter_output_dt", ScatterOutputDt)

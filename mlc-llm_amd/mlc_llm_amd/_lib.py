@@ -52,6 +52,7 @@ SIGNATURES = {
     "mi355gq_linear_silu_mul_dt": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_moe_gemv_silu_mul_dt": (_I, [_P, _L, _P, _P, _P, _L, _L, _L, _L, _I, _I, _I, _P, _P]),
     "mi355gq_moe_group_gemm_silu_mul_dt": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _I, _P, _P]),
+    "mi355gq_moe_experts_dt": (_I, [_P, _L, _P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _I, _I, _P, _P]),
     "mi355gq_gating_softmax_topk_dt": (_I, [_P, _L, _L, _L, _P, _P, _I, _P]),
     "mi355gq_moe_route_dt": (_I, [_P, _L, _L, _L, _P, _P, _P, _P, _P, _P, _I, _I, _P]),
     "mi355gq_take_rows_dt": (_I, [_P, _P, _L, _L, _L, _P, _I, _P]),

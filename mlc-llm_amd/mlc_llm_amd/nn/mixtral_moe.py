@@ -40,7 +40,7 @@ class MixtralMoE(nn.Module):
         batch_size, seq_len, hidden_size = x.shape
         num_tokens = batch_size * seq_len
         x = x.reshape(num_tokens, hidden_size).contiguous()
-        if num_tokens > 1 and x.dtype == torch.float16:  # (the gather inside the expert matmul is a float16 form)
+        if num_tokens > 1:
             try:
                 # routing in one launch; the gather rides in e1_e3's row addressing, the scatter in the
                 # combine's: four launches where the op-by-op sequence below takes nine

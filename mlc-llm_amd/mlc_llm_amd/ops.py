@@ -333,10 +333,11 @@ def moe_experts(x: torch.Tensor, x_row_index: Optional[torch.Tensor], q_weight: 
                 q_scale: torch.Tensor, indptr: torch.Tensor, bits: int, group_size: int,
                 silu_mul_halves: bool = False) -> torch.Tensor:
     """moe_group_gemm on x[x_row_index] (the layer's gather folded into the matmul's row addressing);
-    x_row_index None: x is already in expert order."""
-    _chk(x, torch.float16, "x")
+    x_row_index None: x is already in expert order.  Float16 and bfloat16 models; anything without such a
+    kernel (float32 models, odd shapes) runs take_rows and moe_group_gemm."""
+    _chk(x, _FLOATS, "x")
     _chk(q_weight, _STORAGE, "q_weight")
-    _chk(q_scale, torch.float16, "q_scale")
+    _chk(q_scale, x.dtype, "q_scale")
     _chk(indptr, (torch.int32, torch.int64), "indptr")
     ne, n, _ = q_weight.shape
     x_rows, k = x.shape
@@ -349,12 +350,18 @@ def moe_experts(x: torch.Tensor, x_row_index: Optional[torch.Tensor], q_weight: 
         rows = x_row_index.numel()
     if silu_mul_halves and n % 2:
         raise ValueError(f"moe_experts: {n} rows cannot be split into gate and up halves")
-    out = torch.zeros((rows, n // 2 if silu_mul_halves else n), dtype=torch.float16, device=x.device)
-    _lib.call("mi355gq_moe_experts", x.data_ptr(), x_rows,
-              x_row_index.data_ptr() if x_row_index is not None else None, rows, q_weight.data_ptr(),
-              q_scale.data_ptr(), indptr.data_ptr(), _lib.I64 if indptr.dtype == torch.int64 else _lib.I32,
-              ne, n, k, bits, group_size, _lib.EPILOGUE_SILU_MUL if silu_mul_halves else _lib.EPILOGUE_NONE,
-              out.data_ptr(), _stream())
+    out = torch.zeros((rows, n // 2 if silu_mul_halves else n), dtype=x.dtype, device=x.device)
+    try:
+        _lib.call("mi355gq_moe_experts_dt", x.data_ptr(), x_rows,
+                  x_row_index.data_ptr() if x_row_index is not None else None, rows, q_weight.data_ptr(),
+                  q_scale.data_ptr(), indptr.data_ptr(), _lib.I64 if indptr.dtype == torch.int64 else _lib.I32,
+                  ne, n, k, bits, group_size, _lib.EPILOGUE_SILU_MUL if silu_mul_halves else _lib.EPILOGUE_NONE,
+                  _MODEL_DTYPES[x.dtype], out.data_ptr(), _stream())
+    except _lib.Mi355gqError as err:
+        if not _unsupported(err):
+            raise
+        gathered = take_rows(x, x_row_index) if x_row_index is not None else x
+        return moe_group_gemm(gathered, q_weight, q_scale, indptr, bits, group_size, silu_mul_halves)
     return out
 
 

@@ -1208,6 +1208,32 @@ def test_moe_silu_mul_bfloat16_equals_the_two_steps():
         assert torch.equal(y, two), f"rows={rows}: {(y != two).sum().item()} differ"
 
 
+def test_moe_experts_gather_bfloat16():
+    """The gather folded into the expert matmul for a bfloat16 model equals take_rows + moe_group_gemm bit for
+    bit (quad-row kernel and GEMM tiles; with and without the folded activation)."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(93)
+    ne, n, k, t = 4, 256, 1024, 90
+    w32 = o.round_to((rng.standard_normal((ne, n, k)) * 0.05).astype(np.float32), "bfloat16")
+    qw_ref, qs_ref = o.quantize_dt(w32, s, "bfloat16")
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).bfloat16().to(DEV)
+    x = torch.from_numpy(rng.standard_normal((t, k)).astype(np.float32)).bfloat16().to(DEV)
+    for rows, indptr in ((12, [0, 3, 3, 8, 12]), (60, [0, 20, 21, 21, 60]), (180, [0, 40, 90, 91, 180])):
+        idx = torch.from_numpy(rng.integers(0, t, rows).astype(np.int32)).to(DEV)
+        ip = torch.tensor(indptr, dtype=torch.int32, device=DEV)
+        for fold in (False, True):
+            got = ops.moe_experts(x, idx, qw, qs, ip, 4, 32, silu_mul_halves=fold)
+            want = ops.moe_group_gemm(ops.take_rows(x, idx), qw, qs, ip, 4, 32, silu_mul_halves=fold)
+            assert got.dtype == torch.bfloat16 and torch.equal(got, want), (rows, fold)
+    # float32 models have no such kernel: the call still answers, through the two steps
+    x32 = x.float()
+    qs32 = qs.float()
+    idx = torch.arange(12, dtype=torch.int32, device=DEV)
+    ip = torch.tensor([0, 3, 3, 8, 12], dtype=torch.int32, device=DEV)
+    got = ops.moe_experts(x32, idx, qw, qs32, ip, 4, 32)
+    assert got.dtype == torch.float32 and torch.equal(got, ops.moe_group_gemm(x32[:12].contiguous(), qw, qs32, ip, 4, 32))
+
+
 def test_linear_other_model_dtypes_through_the_modules():
     for name in ("q4f32_1", "q4bf16_1", "q4bf16_0"):
         cfg = gq.QUANTIZATION[name]
