@@ -639,7 +639,7 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
   const int mr = rows_max <= 4 ? 4 : (rows_max <= 8 ? 8 : 16);
   // row tiles per workgroup: enough workgroups for 256 CUs first, then fewer re-reads of x
   const int64_t tiles = (a.N + 15) / 16 * experts * mtiles;
-  // Measured: below ~1000 row tiles the chunk-pipelined kernel (one tile per workgroup) wins, above
+  // Measured: below ~800 row tiles the chunk-pipelined kernel (one tile per workgroup) wins, above
   // it the unpipelined one with 2-4 tiles per workgroup (occupancy hides the latency instead).
   const int mode = options().gemv_variant;  // tuning override: 2 simple, 3 pipelined, 4 persistent, 5 never persistent
   // persistent kernel whenever the activations fit LDS whole (k padded to 1024)
@@ -671,9 +671,12 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
       return launch(skinny_q4_persist_kernel<16>);
     }
   }
-  const bool pipelined = mode == 3 ? true : (mode == 2 ? false : tiles < 1024);
+  // (a sweep over 7B..70B projection shapes put the hand-over between 640 and 960 tiles: 70B qkv, 640 tiles,
+  //  27.5 us pipelined against 30-36 unpipelined; 13B qkv, 960 tiles, 29.4 against 24.1-24.9; and four row tiles
+  //  per workgroup from about 3000 tiles on: 70B gate_up 98-106 us against 107-113 with two)
+  const bool pipelined = mode == 3 ? true : (mode == 2 ? false : tiles < 800);
   int rt = options().gemv_rows_per_wave;  // tuning override
-  if (rt != 1 && rt != 2 && rt != 4) rt = pipelined ? 1 : (tiles >= 4096 ? 4 : 2);
+  if (rt != 1 && rt != 2 && rt != 4) rt = pipelined ? 1 : (tiles >= 3072 ? 4 : 2);
   if (mr == 4) {
     if (rt == 4) return launch_skinny_cfg<4, 4>(p, experts, mtiles, pipelined, s);
     if (rt == 2) return launch_skinny_cfg<4, 2>(p, experts, mtiles, pipelined, s);
