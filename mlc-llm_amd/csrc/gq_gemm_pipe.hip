@@ -420,6 +420,33 @@ int gemm_pipe_pair_block(const GemmParams& p, int bits) {
   return (p.bm_hint == 32 && options().gemm_variant < 0) ? 16 : 32;  // the 32 x 128 tile below
 }
 
+// Which of the three regular tiles a plain matmul of this shape should run: 2 = 256 x 256, 1 = 128 x 256,
+// 0 = 128 x 128.  A launch costs rounds x (time of one tile), rounds = ceil(tiles / resident workgroups) (256 for
+// the two large tiles, 512 for 128 x 128), tile times from the per-tile rates measured with balanced rounds (q4:
+// 1035 / 870 / 806 TFLOP/s; q3, whose K tile does not fit the largest one: 739 / 566).  What the model is for is the
+// last, partly filled round: 300 tiles of 256 x 256 take two rounds where 540 of 128 x 256 take three half-sized
+// ones (13B qkv at 1025 rows: 584 -> 621 TFLOP/s; gate_up at 1025 rows: 699 -> 785; qkv 6144 x 4096 at 1536 rows, the
+// other way round: 568 -> 706).
+int pick_regular_tile(int64_t rows, int64_t N, int bits) {
+  const int64_t ntw = (N + 255) / 256, ntn = (N + 127) / 128;
+  const int64_t big = ((rows + 255) / 256) * ntw, mid = ((rows + 127) / 128) * ntw, small = ((rows + 127) / 128) * ntn;
+  const double t_big = 65536.0 / (1035.0 / 256), t_mid = 32768.0 / ((bits == 4 ? 870.0 : 739.0) / 256),
+               t_small = 16384.0 / ((bits == 4 ? 806.0 : 566.0) / 512);
+  const double c_big = bits == 4 ? static_cast<double>((big + 255) / 256) * t_big : 1e30;
+  const double c_mid = static_cast<double>((mid + 255) / 256) * t_mid;
+  // 128 x 128: two workgroups share a CU; one on its own runs faster than its half of a pair (0.72 of the
+  // pair's time fits 13B o_proj at 640 rows, 200 such tiles: 539 TFLOP/s against 420 on 100 tiles of 128 x 256)
+  const int64_t per_cu = (small + 255) / 256;
+  const double c_small = static_cast<double>(per_cu / 2) * t_small + static_cast<double>(per_cu % 2) * 0.72 * t_small;
+  // a partly filled last round runs faster than a full one (the part is power-limited), which favours the larger
+  // tile: a smaller tile has to win by 8 % on paper
+  int pick = 2;
+  double best = c_big;
+  if (c_mid < 0.92 * best) { pick = 1; best = c_mid; }
+  if (c_small < 0.92 * best) pick = 0;
+  return pick;
+}
+
 hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
   if ((p.K & 7) != 0 || p.ng == 0) return hipErrorNotSupported;
   const int variant = options().gemm_variant;
@@ -448,17 +475,16 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
       return wide ? launch_pipe_cfg<3, 128, 256, 64, 64, 2, true>(p, s)
                   : launch_pipe_cfg<3, 128, 128, 64, 64, 2, true>(p, s);
     }
-    const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
-    const int64_t mid_tiles = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
     if (bits == 4) {
       // few rows: tile height follows the rows (the float16 path's few-row tiles, unsplit)
       if (p.rows <= 32) return launch_pipe_cfg<4, 32, 128, 32, 32, 4, true>(p, s);
       if (p.rows <= 64) return launch_pipe_cfg<4, 64, 128, 32, 64, 4, true>(p, s);
-      if (big_tiles >= 160) return launch_pipe_cfg<4, 256, 256, 128, 64, 2, true>(p, s);
-      if (mid_tiles >= 160) return launch_pipe_cfg<4, 128, 256, 64, 64, 2, true>(p, s);
+      const int tile = pick_regular_tile(p.rows, p.N, 4);
+      if (tile == 2) return launch_pipe_cfg<4, 256, 256, 128, 64, 2, true>(p, s);
+      if (tile == 1) return launch_pipe_cfg<4, 128, 256, 64, 64, 2, true>(p, s);
       return launch_pipe_cfg<4, 128, 128, 64, 64, 2, true>(p, s);
     }
-    if (mid_tiles >= 160) return launch_pipe_cfg<3, 128, 256, 64, 64, 2, true>(p, s);
+    if (pick_regular_tile(p.rows, p.N, 3) == 1) return launch_pipe_cfg<3, 128, 256, 64, 64, 2, true>(p, s);
     return launch_pipe_cfg<3, 128, 128, 64, 64, 2, true>(p, s);
   }
   if (p.bm_hint > 0 && variant < 0) {
@@ -476,16 +502,12 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
       if (p.rows <= 16 * p.num_experts) return launch_pipe_cfg<4, 32, 128, 32, 32, 4>(p, s);
       if (p.rows <= 48 * p.num_experts) return launch_pipe_cfg<4, 64, 128, 32, 64, 4>(p, s);
     }
-    const int64_t big_tiles = ((static_cast<int64_t>(p.rows) + 255) / 256) * ((p.N + 255) / 256);
-    const bool big = variant == 7 ? true : (variant == 6 ? false : (p.indptr == nullptr && big_tiles >= 160));
+    // plain matmul: the tile whose rounds of workgroups cost least (variants 6 / 7 / 9 force one)
+    const int tile = p.indptr != nullptr ? 0 : pick_regular_tile(p.rows, p.N, 4);
+    const bool big = variant == 7 ? true : (variant == 6 ? false : tile == 2);
     if (variant == 9) return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     if (big) return launch_pipe_cfg<4, 256, 256, 128, 64>(p, s);
-    // too few 256x256 tiles for 256 CUs (o_proj, down at M = 2048): halve the tile along M
-    // (from 160 such tiles on: 5120-wide 13B projections at 1024 rows ran 589-659 TFLOP/s on them against
-    //  517-572 on twice as many 128x128 tiles)
-    const int64_t mid_tiles = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
-    if (variant != 6 && p.indptr == nullptr && mid_tiles >= 160)
-      return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
+    if (variant != 6 && tile == 1) return launch_pipe_cfg<4, 128, 256, 64, 64>(p, s);
     // grouped: the wider tile once the experts' row tiles alone make several rounds of workgroups
     if (variant != 6 && p.indptr != nullptr && p.rows >= 96 * p.num_experts &&
         (static_cast<int64_t>(p.rows) / 128 + p.num_experts) * ((p.N + 255) / 256) >= 768)
@@ -497,10 +519,10 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     if (p.rows <= 48 * p.num_experts) return launch_pipe_cfg<3, 64, 128, 32, 64, 4>(p, s);
   }
   // q3: a K tile is 80 wide, so the 256 x 256 tile does not fit LDS; 128 x 256 does
-  const int64_t mid_tiles3 = ((static_cast<int64_t>(p.rows) + 127) / 128) * ((p.N + 255) / 256);
+  const bool plain_wide = p.indptr == nullptr && pick_regular_tile(p.rows, p.N, 3) == 1;
   const bool grouped_wide = p.indptr != nullptr && p.rows >= 96 * p.num_experts &&
                             (static_cast<int64_t>(p.rows) / 128 + p.num_experts) * ((p.N + 255) / 256) >= 768;
-  if (variant == 9 || (variant != 6 && ((p.indptr == nullptr && mid_tiles3 >= 160) || grouped_wide)))
+  if (variant == 9 || (variant != 6 && (plain_wide || grouped_wide)))
     return launch_pipe_cfg<3, 128, 256, 64, 64>(p, s);
   return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
 }
