@@ -319,7 +319,7 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     // the regimes of the plain linear: register GEMV up to 2 rows, quad-row kernel up to 8 (q3: 16),
     // skinny kernel up to 16 (q4), else the pipelined GEMM
     hipError_t e = hipErrorNotSupported;
-    if ((M == 2 && (K > 8192 || N * K >= (1ll << 28))) || (M <= 2 && K > 16384))  // as the plain linear
+    if ((M == 2 && (K > 8192 || N * K >= (1ll << 28))) || (M <= 2 && K > 24576))  // as the plain linear
       e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     if (e != hipErrorNotSupported) {
       // served above
@@ -355,8 +355,8 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   }
   // two rows of a long K (down_proj): the register GEMV holds 6-7 groups per lane there and measured 19.0 us (q4)
   // / 17.9 us (q3) on 4096 x 14336 against 14.3-16.4 us for the quad-row kernel at 3-4 rows
-  // (beyond K = 16 Ki the register GEMV does not apply at all and the quad-row kernel also takes single rows)
-  const bool long_k = (M == 2 && K > 8192) || K > 16384;
+  // (beyond K = 24 Ki the register GEMV does not apply at all and the quad-row kernel also takes single rows)
+  const bool long_k = (M == 2 && K > 8192) || K > 24576;
   // ... and two rows of a very large matrix (lm_head 128256 x 4096: 56 us against 70; 70B gate_up 58 against 66)
   const bool huge2 = M == 2 && N * K >= (1ll << 28);
   if (M <= 2 && gm < 0 && ((gv < 0 && (long_k || huge2)) || (gv >= 6 && gv <= 8))) {

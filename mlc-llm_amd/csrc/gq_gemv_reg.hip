@@ -260,6 +260,9 @@ static hipError_t launch_iters(const GemvParams& p, int slots, int iters, int bl
     case 6: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 6>(p, slots, blocks, nsets, s); break;
     case 7: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 7>(p, slots, blocks, nsets, s); break;
     case 8: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 8>(p, slots, blocks, nsets, s); break;
+    // K up to 24 Ki (q3: 30 Ki): Qwen2-7B's down_proj, 3584 x 18944, runs 10 groups per lane
+    case 9: case 10: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 10>(p, slots, blocks, nsets, s); break;
+    case 11: case 12: if constexpr (R * NB == 1) return launch_k<BITS, NB, R, 12>(p, slots, blocks, nsets, s); break;
     default: break;
   }
   return hipErrorNotSupported;
@@ -268,7 +271,7 @@ static hipError_t launch_iters(const GemvParams& p, int slots, int iters, int bl
 template <int BITS>
 static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_t s) {
   const int iters = (p.ng + 63) / 64;
-  if (iters < 1 || iters > 8) return hipErrorNotSupported;
+  if (iters < 1 || iters > 12) return hipErrorNotSupported;
   // register budget: R * ITERS loads in flight, NB * ITERS x slices resident
   int rmax = iters <= 2 ? 4 : (iters <= 4 ? 2 : 1);
   if (nb == 2) rmax = iters <= 2 ? 2 : (iters <= 4 ? 1 : 0);

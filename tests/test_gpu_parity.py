@@ -216,10 +216,11 @@ def _linear_case(s, m, n, k, seed, bias=False, scale=0.02):
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("m,n,k", [(1, 64, 20480), (2, 64, 20480), (1, 36, 28672), (2, 128, 9000), (1, 62, 20481),
-                                   (2, 62, 20004)])
+                                   (2, 62, 20004), (1, 130, 18944), (1, 64, 24576), (1, 64, 24584)])
 def test_one_and_two_rows_of_a_long_k(name, m, n, k):
-    # K past what the register GEMV holds per lane: the quad-row kernel takes over (two rows: from K > 8192;
-    # one row: from K > 16384), the LDS GEMV where that one declines the shape (N % 4, K % 8)
+    # K past what the register GEMV holds per lane (12 groups for one row, 4 for two): the quad-row kernel takes
+    # over (two rows: from K > 8192; one row: from K > 24576), the LDS GEMV where that one declines the shape
+    # (N % 4, K % 8)
     s = SCHEMES[name]
     x, qw, qs, b = _linear_case(s, m, n, k, 7 * m + n + k, bias=True)
     y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
