@@ -41,6 +41,32 @@ struct Elem<MODEL_BF16> {
   static constexpr float kLowest = -3.3895313892515355e38f;  // min_value(bfloat16)
 };
 
+// softmax over the k selected logits in fp32, in slot order, and the stores of one token's results
+template <int KMAX, int DT>
+__device__ __forceinline__ void softmax_store(const float (&val)[KMAX], const int (&idx)[KMAX], int k,
+                                              void* __restrict__ w, int64_t w0, int32_t* __restrict__ ids) {
+  float mx = val[0];
+#pragma unroll
+  for (int i = 1; i < KMAX; ++i)
+    if (i < k) mx = fmaxf(mx, val[i]);
+  float ex[KMAX];
+  float den = 0.f;
+#pragma unroll
+  for (int i = 0; i < KMAX; ++i) {
+    if (i < k) {
+      ex[i] = expf(val[i] - mx);
+      den = (i == 0) ? ex[0] : den + ex[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < KMAX; ++i) {
+    if (i < k) {
+      Elem<DT>::store(w, w0 + i, ex[i] / den);
+      ids[i] = idx[i];
+    }
+  }
+}
+
 // One thread per token: insertion top-k with strict '>' (ties keep the lower expert index),
 // then softmax over the k selected logits in fp32.
 // KMAX: slots kept (k <= KMAX); the insertion is a chain of KMAX * KMAX predicated moves per expert,
@@ -75,26 +101,7 @@ __device__ __forceinline__ void topk_softmax_slots(const void* __restrict__ logi
       }
     }
   }
-  float mx = val[0];
-#pragma unroll
-  for (int i = 1; i < kMaxTopK; ++i)
-    if (i < k) mx = fmaxf(mx, val[i]);
-  float ex[kMaxTopK];
-  float den = 0.f;
-#pragma unroll
-  for (int i = 0; i < kMaxTopK; ++i) {
-    if (i < k) {
-      ex[i] = expf(val[i] - mx);
-      den = (i == 0) ? ex[0] : den + ex[i];
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < kMaxTopK; ++i) {
-    if (i < k) {
-      Elem<DT>::store(w, w0 + i, ex[i] / den);
-      ids[i] = idx[i];
-    }
-  }
+  softmax_store<KMAX, DT>(val, idx, k, w, w0, ids);
 }
 
 // token t: logits[t, :] -> w[t, :k], ids[t, :k]
@@ -112,6 +119,98 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const void* __restric
   const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (t >= T) return;
   topk_softmax_token<DT>(logits, t, ne, k, w, ids);
+}
+
+// One wave per token, for many experts or many slots (the thread-per-token insertion above costs
+// ne * k * k predicated moves on one lane): lane l holds the logits of experts l, l + 64, ...; k rounds
+// of a wave-wide arg-max (larger value first, equal values by lower expert index: the order the
+// insertion produces) pick the slots, and lane 0 finishes with the same softmax.  Logits that are not
+// above min_value(dtype), NaN included, are never picked; slots left empty keep (min_value, expert 0).
+constexpr int kWaveTopkChunks = 8;  // experts per lane: ne <= 512
+template <int DT>
+__device__ __forceinline__ void topk_softmax_wave(const void* __restrict__ logits, int64_t t, int ne, int k,
+                                                  void* __restrict__ w, int32_t* __restrict__ ids) {
+  const int lane = threadIdx.x & 63;
+  const int nch = (ne + 63) >> 6;
+  float v[kWaveTopkChunks];
+  unsigned out_of_running = 0;  // bit c: expert lane + 64 * c is absent, not placeable or already picked
+#pragma unroll
+  for (int c = 0; c < kWaveTopkChunks; ++c) {
+    const int e = lane + 64 * c;
+    v[c] = Elem<DT>::kLowest;
+    if (c < nch && e < ne) v[c] = Elem<DT>::load(logits, t * ne + e);
+    if (!(v[c] > Elem<DT>::kLowest)) out_of_running |= 1u << c;
+  }
+  constexpr int kNone = 0x7fffffff;
+  float val[kMaxTopK];
+  int idx[kMaxTopK];
+  if (nch == 1) {
+    // up to 64 experts: every lane counts the experts that come before its own in that order (its rank)
+    // from lane broadcasts, with no trip through the LDS crossbar; slot i is the lane of rank i
+    const bool placeable = !(out_of_running & 1u);
+    int rank = 0;
+#pragma unroll
+    for (int l = 0; l < 64; ++l) {
+      const float ov = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[0]), l));
+      rank += (ov > v[0] || (ov == v[0] && l < lane)) ? 1 : 0;  // a logit that cannot be placed never wins here
+    }
+#pragma unroll
+    for (int i = 0; i < kMaxTopK; ++i) {
+      val[i] = Elem<DT>::kLowest;
+      idx[i] = 0;
+      if (i < k) {
+        const unsigned long long m = __ballot(placeable && rank == i);
+        if (m != 0ull) {
+          const int src = __builtin_ctzll(m);
+          val[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[0]), src));
+          idx[i] = src;
+        }
+      }
+    }
+    if (lane == 0) softmax_store<kMaxTopK, DT>(val, idx, k, w, t * k, ids + t * k);
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < kMaxTopK; ++i) {
+    val[i] = Elem<DT>::kLowest;
+    idx[i] = 0;
+    if (i < k) {  // uniform
+      float bv = Elem<DT>::kLowest;
+      int be = kNone;
+#pragma unroll
+      for (int c = 0; c < kWaveTopkChunks; ++c)
+        if (c < nch && !((out_of_running >> c) & 1u) && (be == kNone || v[c] > bv)) {
+          bv = v[c];
+          be = lane + 64 * c;
+        }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off);
+        const int oe = __shfl_xor(be, off);
+        if (oe != kNone && (be == kNone || ov > bv || (ov == bv && oe < be))) {
+          bv = ov;
+          be = oe;
+        }
+      }
+      if (be != kNone) {  // uniform: every lane ends with the same winner
+        val[i] = bv;
+        idx[i] = be;
+        if ((be & 63) == lane) out_of_running |= 1u << (be >> 6);
+      }
+    }
+  }
+  if (lane == 0) softmax_store<kMaxTopK, DT>(val, idx, k, w, t * k, ids + t * k);
+}
+
+static inline bool use_wave_topk(int ne, int k) { return ne * k > 64 && ne <= 64 * kWaveTopkChunks; }
+
+template <int DT>
+__global__ __launch_bounds__(256) void topk_softmax_wave_kernel(const void* __restrict__ logits, int64_t T, int ne,
+                                                                int k, void* __restrict__ w,
+                                                                int32_t* __restrict__ ids) {
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+  if (t >= T) return;  // whole waves
+  topk_softmax_wave<DT>(logits, t, ne, k, w, ids);
 }
 
 // The whole routing step of a MoE layer in one workgroup, for batches a single workgroup can scan:
@@ -177,6 +276,100 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict_
     if (tid == 0) {
       if (out_i64) static_cast<int64_t*>(indptr)[e + 1] = base;
       else static_cast<int32_t*>(indptr)[e + 1] = base;
+    }
+  }
+}
+
+// The same routing step organised by slot, for up to 8 slots per thread and up to 64 experts: thread
+// tid owns slots tid, tid + nthreads, ...; one pass of wave ballots per expert gives every slot its rank
+// among its wave's slots of the same expert and every (expert, 64-slot chunk) its count; a scan of that
+// table in (expert, chunk) order turns the counts into offsets.  Three barriers in all, where the
+// kernel above takes one per expert and round and re-reads k ids per token and expert.
+// do_topk 0: ids (and w) were produced by an earlier launch.  wave_topk: one wave per token.
+template <int DT>
+__global__ __launch_bounds__(1024) void moe_route_slots_kernel(const void* __restrict__ logits, int T, int ne, int k,
+                                                               void* __restrict__ w, int32_t* __restrict__ ids,
+                                                               int32_t* __restrict__ tok, int32_t* __restrict__ rev,
+                                                               int32_t* __restrict__ pos_of_slot, int out_i64,
+                                                               void* indptr, int do_topk, int wave_topk) {
+  constexpr int kSlotsPerThread = 8;
+  __shared__ int wave_tot[16];
+  extern __shared__ int32_t cnt[];  // [ne, nchunks]: counts, then exclusive offsets
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
+  const int S = T * k, nchunks = (S + 63) >> 6, N = ne * nchunks;
+  if (do_topk) {
+    if (wave_topk)
+      for (int t = wave; t < T; t += nwaves) topk_softmax_wave<DT>(logits, t, ne, k, w, ids);
+    else
+      for (int t = tid; t < T; t += nthreads) topk_softmax_token<DT>(logits, t, ne, k, w, ids);
+    __syncthreads();  // ids written above are read back by other threads below
+  }
+  const unsigned long long lower = (1ull << lane) - 1ull;
+  int myid[kSlotsPerThread], before[kSlotsPerThread];
+#pragma unroll
+  for (int r = 0; r < kSlotsPerThread; ++r) {
+    const int s = r * nthreads + tid;
+    myid[r] = -1;  // no slot, or a repeated id of its token (the mask is boolean: it counts once)
+    before[r] = 0;
+    if (r * nthreads + wave * 64 < S) {  // per wave: its 64-slot chunk exists
+      if (s < S) {
+        const int id = ids[s], j = s % k;
+        bool repeated = false;
+#pragma unroll
+        for (int jj = 0; jj < kMaxTopK - 1; ++jj)  // unconditional loads (its own id past j), all in flight together
+          repeated |= (ids[s - j + (jj < j ? jj : j)] == id) & (jj < j);
+        if (!repeated) myid[r] = id;
+      }
+      int mine = 0;  // lane e: slots of expert e in this wave's chunk
+      for (int e = 0; e < ne; ++e) {
+        const unsigned long long m = __ballot(myid[r] == e);
+        if (myid[r] == e) before[r] = __popcll(m & lower);
+        if (lane == e) mine = __popcll(m);
+      }
+      if (lane < ne) cnt[lane * nchunks + r * nwaves + wave] = mine;
+    }
+  }
+  __syncthreads();
+  // exclusive scan of cnt[0, N): consecutive runs per thread, a wave scan of the run sums, wave totals
+  const int per = (N + nthreads - 1) / nthreads;
+  const int i0 = tid * per, i1 = (i0 + per < N) ? i0 + per : N;
+  int sum = 0;
+  for (int i = i0; i < i1; ++i) sum += cnt[i];
+  int inc = sum;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(inc, off);
+    if (lane >= off) inc += o;
+  }
+  if (lane == 63) wave_tot[wave] = inc;
+  __syncthreads();
+  int pre = 0, total = 0;
+  for (int wv = 0; wv < nwaves; ++wv) {
+    const int c = wave_tot[wv];
+    if (wv < wave) pre += c;
+    total += c;
+  }
+  int run = pre + inc - sum;
+  for (int i = i0; i < i1; ++i) {
+    const int c = cnt[i];
+    cnt[i] = run;
+    run += c;
+  }
+  __syncthreads();
+  for (int e = tid; e <= ne; e += nthreads) {
+    const int v = e == 0 ? 0 : (e < ne ? cnt[e * nchunks] : total);
+    if (out_i64) static_cast<int64_t*>(indptr)[e] = v;
+    else static_cast<int32_t*>(indptr)[e] = v;
+  }
+#pragma unroll
+  for (int r = 0; r < kSlotsPerThread; ++r) {
+    if (myid[r] >= 0) {
+      const int s = r * nthreads + tid;
+      const int pos = cnt[myid[r] * nchunks + r * nwaves + wave] + before[r];  // < S: distinct (t, j) pairs
+      tok[pos] = s / k;
+      rev[pos] = s;
+      pos_of_slot[s] = pos;
     }
   }
 }
@@ -344,9 +537,14 @@ static hipError_t by_dtype(int model_dtype, Fn fn) {
 hipError_t launch_topk_softmax(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int model_dtype,
                                hipStream_t s) {
   if (T == 0) return hipSuccess;
+  const bool by_wave = use_wave_topk(ne, k);
   return by_dtype(model_dtype, [&](auto dt) {
-    hipLaunchKernelGGL(topk_softmax_kernel<decltype(dt)::value>, dim3(blocks_for(T, 256)), dim3(256), 0, s, logits, T,
-                       ne, k, w, ids);
+    if (by_wave)
+      hipLaunchKernelGGL(topk_softmax_wave_kernel<decltype(dt)::value>, dim3(blocks_for(T, 4)), dim3(256), 0, s,
+                         logits, T, ne, k, w, ids);
+    else
+      hipLaunchKernelGGL(topk_softmax_kernel<decltype(dt)::value>, dim3(blocks_for(T, 256)), dim3(256), 0, s, logits,
+                         T, ne, k, w, ids);
   });
 }
 
@@ -408,6 +606,26 @@ hipError_t launch_moe_combine(const void* y, const void* w, const int32_t* pos, 
 hipError_t launch_moe_route(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int32_t* tok,
                             int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr, int model_dtype,
                             hipStream_t s) {
+  const int64_t slots = T * k;
+  if (slots > 0 && slots <= 8 * 1024 && ne <= 64) {
+    // by slot; with many experts the top-k runs one wave per token, inside the kernel while one
+    // workgroup has a wave for every token, as a launch of its own across the chip beyond that
+    const bool by_wave = use_wave_topk(ne, k);
+    const bool topk_first = by_wave && T > 16;
+    if (topk_first) {
+      const hipError_t err = launch_topk_softmax(logits, T, ne, k, w, ids, model_dtype, s);
+      if (err != hipSuccess) return err;
+    }
+    int threads = static_cast<int>((slots + 63) / 64) * 64;
+    if (by_wave && !topk_first && threads < 64 * T) threads = static_cast<int>(64 * T);
+    threads = threads > 1024 ? 1024 : threads;
+    const size_t lds = static_cast<size_t>(ne) * ((slots + 63) / 64) * sizeof(int32_t);
+    return by_dtype(model_dtype, [&](auto dt) {
+      hipLaunchKernelGGL(moe_route_slots_kernel<decltype(dt)::value>, dim3(1), dim3(threads), lds, s, logits,
+                         static_cast<int>(T), ne, k, w, ids, tok, rev, pos_of_slot, out_i64, indptr,
+                         topk_first ? 0 : 1, by_wave ? 1 : 0);
+    });
+  }
   int threads = static_cast<int>((T + 63) / 64) * 64;
   threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
   const size_t lds = static_cast<size_t>(T) * k * sizeof(int32_t);

@@ -1429,8 +1429,41 @@ def test_moe_route_equals_the_four_calls(t, ne, k):
     assert torch.equal(ops.moe_route(logits, k, torch.int64)[5], indptr0.long())
 
 
+@pytest.mark.parametrize("t,ne,k", [(1, 64, 8), (2, 64, 8), (16, 64, 8), (17, 60, 4), (200, 64, 6), (1024, 64, 8),
+                                    (40, 160, 6), (3, 256, 8), (5, 200, 8), (1100, 33, 7), (7, 65, 1)])
+def test_many_expert_routing_against_oracle(t, ne, k):
+    """Many experts or many slots: the top-k runs one wave per token and the route step by slot.  Logits
+    drawn from a few values so that ties abound, plus rows that cannot fill their k slots."""
+    rng = np.random.default_rng(t * 1000 + ne + k)
+    logits = rng.standard_normal((t, ne)).astype(np.float16)
+    logits[::3] = rng.integers(-3, 4, logits[::3].shape).astype(np.float16)  # ties: the lower index first
+    logits[-1, :] = np.float16(-65504.0)  # nothing exceeds min_value: every slot stays (min_value, expert 0)
+    if t > 2:
+        logits[1, :] = -np.inf
+        logits[1, ne // 2] = 1.0  # one placeable logit
+    w_ref, ids_ref = o.gating_softmax_topk(logits, k)
+    w, ids = ops.gating_softmax_topk(dev(logits), k)
+    assert (ids.cpu().numpy() == ids_ref).all()
+    dw = np.abs(w.cpu().numpy().astype(np.float32) - w_ref.astype(np.float32))
+    assert (dw <= 2.0**-11).all(), dw.max()  # one fp16 ulp between libms, as for the golden vectors
+    if ne <= 64:
+        w2, ids2, tok, rev, pos, indptr = ops.moe_route(dev(logits), k)
+        assert torch.equal(w2, w) and torch.equal(ids2, ids)
+        cs_ref = o.moe_cumsum(ids_ref, ne)
+        rev_ref, tok_ref = o.get_indices(cs_ref, ids_ref)
+        n_pairs = int(cs_ref.reshape(-1)[-1])  # rows with repeated ids leave the tail of the order unwritten
+        indptr_ref = o.get_indptr(cs_ref, ne, t, inclusive=False)
+        assert (indptr.cpu().numpy() == indptr_ref).all()
+        tok_h, rev_h = tok.cpu().numpy()[:n_pairs], rev.cpu().numpy()[:n_pairs]
+        assert (tok_h == tok_ref[:n_pairs]).all() and (rev_h // k == tok_h).all()
+        distinct = np.array([len(set(row)) == k for row in ids_ref.tolist()])[tok_h]  # a repeated id counts once,
+        assert (rev_h[distinct] == rev_ref[:n_pairs][distinct]).all()  # under its first slot here
+        assert (ids_ref.reshape(-1)[rev_h] == np.repeat(np.arange(ne), np.diff(indptr_ref))).all()
+        assert torch.equal(pos[rev[:n_pairs].long()], torch.arange(n_pairs, dtype=torch.int32, device=DEV))
+
+
 def test_moe_route_past_one_workgroup_is_unsupported():
-    for t, ne in ((9000, 8), (16, 100), (4096, 32)):
+    for t, ne in ((9000, 8), (16, 100), (4097, 32)):
         with pytest.raises(gq._lib.Mi355gqError) as e:
             ops.moe_route(torch.zeros(t, ne, device=DEV).half(), 2)
         assert e.value.code == gq._lib.ERR_UNSUPPORTED
