@@ -569,6 +569,27 @@ int mi355gq_moe_gemv_silu_mul(const void* x, int64_t x_rows, const void* q_weigh
                        out, stream, true);
 }
 
+// Expert-sorted rows, about one per expert: the register GEMV with one grid row per activation row streams an
+// expert's weights once per row, the quad-row kernel once per expert but at well under half the GEMV's rate, so up
+// to num_experts rows (about 1.5 rows per distinct expert under uniform routing) the GEMV is ahead or level.
+// Measured on expert matmuls, quad-row -> GEMV: Mixtral-8x7B e1_e3 T=2 62 -> 38 us, T=4 116 -> 80, e2 35 -> 24 and
+// 72 -> 40; Qwen2-MoE-57B shapes (64 experts, top-8) T=2 58 -> 33, T=4 83 -> 51; past num_experts rows the order flips
+// (Mixtral T=6 132 -> 152).
+static bool moe_rows_by_gemv(const gq::GemmArgs& g) {
+  return g.rows <= (g.num_experts > 4 ? g.num_experts : 4) && g.rows <= 256 && g.num_experts <= 256 && (g.K & 7) == 0;
+}
+
+static hipError_t moe_row_gemv(const gq::GemmArgs& g, hipStream_t s) {
+  gq::GemvArgs a{};
+  a.x = g.x; a.q_weight = g.q_weight; a.q_scale = g.q_scale; a.bias = nullptr; a.y = g.y;
+  a.expert_ids = nullptr;
+  a.M = 1; a.N = g.N; a.K = g.K; a.slots = g.rows; a.x_slot_stride = 0; a.num_experts = g.num_experts;
+  a.bits = g.bits; a.group_size = g.group_size; a.out_f32 = 0; a.paired = g.paired; a.bf16 = g.bf16;
+  a.indptr = g.indptr; a.indptr_i64 = g.indptr_i64;
+  a.x_row_index = g.x_rows; a.x_src_rows = g.x_rows ? g.x_src_rows : g.rows;
+  return gq::launch_gemv(a, s);
+}
+
 static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
                                const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
                                int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream,
@@ -604,6 +625,13 @@ static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight
   }
   // few rows in total: every expert is a skinny problem bound by streaming its weights
   const int gv = gq::options().gemv_variant;
+  if (gv < 0 && moe_rows_by_gemv(g)) {
+    const hipError_t e = moe_row_gemv(g, as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "moe row GEMV launch");
+    // (the unfused form may still take that kernel: the caller runs the two steps and the bits stay the same)
+    if (paired) return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul: no fused GEMV for N=%lld K=%lld",
+                            (long long)N, (long long)K);
+  }
   // (up to about six rows per expert: 8 experts, 40-48 rows 255-263 us for the whole layer against 285 with the
   //  skinny kernel; from 64 rows on the order flips)
   const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;
@@ -761,6 +789,12 @@ static int moe_group_gemm_dt_impl(const void* x, int64_t rows, const void* q_wei
     if (x_row_index != nullptr) {
       g.x_rows = static_cast<const int32_t*>(x_row_index);
       g.x_src_rows = x_rows;
+    }
+    if (gq::options().gemv_variant < 0 && moe_rows_by_gemv(g)) {  // about one row per expert (as in float16)
+      const hipError_t e = moe_row_gemv(g, as_stream(stream));
+      if (e != hipErrorNotSupported) return hip_result(e, "moe_group_gemm_dt row GEMV launch");
+      if (paired) return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul_dt: no fused GEMV for N=%lld K=%lld",
+                              (long long)N, (long long)K);
     }
     // few rows in total: every expert streams its weights for a handful of rows (as in float16)
     const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;

@@ -37,6 +37,13 @@ struct GemvParams {
   int out_f32;
   int paired;  // fused gate/up form: y[.., N / 2] = silu(x . W[j]) * (x . W[N / 2 + j]), fp16
   int bf16;    // x, q_scale, bias, residual and a 16-bit y are bfloat16 (register kernel only)
+  // rows sorted by expert instead of expert_ids (register kernel only): slot s belongs to the expert e with
+  // indptr[e] <= s < indptr[e + 1] (slots outside every segment are left alone) and reads x row
+  // x_row_index[s] (null: row s)
+  const void* indptr;
+  int indptr_i64;
+  const int32_t* x_row_index;
+  int x_src_rows;
 };
 
 // sum_k x_k * (field_k - m) for one group, given the 4 storage words and the staged x pairs

@@ -44,7 +44,28 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
   const uint16_t* x = p.x + slot * p.x_slot_stride;
   const uint32_t* qw = p.qw;
   const uint16_t* qs = p.qs;
-  if (p.expert_ids != nullptr) {
+  if (p.indptr != nullptr) {
+    // expert-sorted rows: the segment ends at or before this row number its expert (each wave counts for itself)
+    int e = 0;
+    for (int e0 = 0; e0 < p.num_experts; e0 += 64) {
+      const int i = e0 + lane;
+      int64_t end = 0x7fffffffffffffffll;
+      if (i < p.num_experts)
+        end = p.indptr_i64 ? static_cast<const int64_t*>(p.indptr)[i + 1] : static_cast<const int32_t*>(p.indptr)[i + 1];
+      e += __popcll(__ballot(end <= slot));
+    }
+    if (e >= p.num_experts) return;  // past the last segment (uniform over the workgroup)
+    const int64_t begin = p.indptr_i64 ? static_cast<const int64_t*>(p.indptr)[e] : static_cast<const int32_t*>(p.indptr)[e];
+    if (begin > slot) return;  // before the first segment
+    qw += e * p.expert_w_stride;
+    qs += e * p.expert_s_stride;
+    int row = slot;
+    if (p.x_row_index != nullptr) {
+      row = p.x_row_index[slot];
+      row = row < 0 ? 0 : (row >= p.x_src_rows ? p.x_src_rows - 1 : row);
+    }
+    x = p.x + static_cast<int64_t>(row) * p.K;
+  } else if (p.expert_ids != nullptr) {
     int e = p.expert_ids[slot];
     e = e < 0 ? 0 : (e >= p.num_experts ? p.num_experts - 1 : e);
     qw += e * p.expert_w_stride;
@@ -302,7 +323,10 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
     waves = half <= 3072 ? static_cast<int>(half) : 2048;
     if (waves < 1024) waves = 1024;
   }
-  waves = (waves + slots - 1) / slots;  // grid.y = slots
+  // grid.y = slots: whole workgroups per slot, rounded down, so that the grid stays within the one or two
+  // workgroups per CU the totals above stand for (6 slots rounded up are 516 workgroups: four of them run alone
+  // after the other 512, and 6 rows cost what 8 do)
+  if (slots > 1) waves = waves / (4 * slots) * 4;
   if (waves < 4) waves = 4;
   const int rounds = (nsets + waves - 1) / waves;
   const int blocks = ((nsets + rounds - 1) / rounds + 3) / 4;  // even share of sets per wave

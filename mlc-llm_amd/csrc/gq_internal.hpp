@@ -32,6 +32,12 @@ struct GemvArgs {
   int out_f32;
   int paired = 0;           // fused gate/up form (see gate_up_row): y is [M or slots, N / 2] fp16; N even, no bias / residual
   int bf16 = 0;             // bfloat16 model: x, q_scale, bias, residual and a 16-bit y are bf16 (M <= 2, no fused form)
+  // expert-sorted rows (slots = rows, M = 1, expert_ids null): the expert of a row comes from indptr
+  // [num_experts + 1], its x row from x_row_index (null: the row itself)
+  const void* indptr = nullptr;
+  int indptr_i64 = 0;
+  const int32_t* x_row_index = nullptr;
+  int64_t x_src_rows = 0;
 };
 hipError_t launch_gemv(const GemvArgs& a, hipStream_t s);
 

@@ -749,6 +749,57 @@ def test_moe_group_gemm(name, indptr):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("model_dtype", ["float16", "bfloat16"])
+def test_moe_group_gemm_about_one_row_per_expert(name, model_dtype):
+    """Up to num_experts rows: one grid row of the GEMV per activation row, its expert found from indptr.
+    Empty experts, experts with several rows, rows outside every segment, int64 indptr, the gather index
+    and the fused SiLU form."""
+    s = SCHEMES[name]
+    rng = np.random.default_rng(53)
+    ne, n = 70, 264  # more experts than one wave's lanes
+    k = 1024 if s.bits == 4 else 1000
+    tdt = torch.float16 if model_dtype == "float16" else torch.bfloat16
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs16 = o.quantize(w, s)
+    qs = torch.from_numpy(qs16.astype(np.float32)).to(DEV).to(tdt)
+    qs_ref = qs.float().cpu().numpy()
+    qwd = dev(qw)
+    for rows, cuts in ((1, {69: 1}), (9, {0: 2, 3: 1, 64: 3, 69: 3}), (70, {5: 30, 6: 1, 68: 39}), (33, {1: 7, 40: 20})):
+        counts = np.zeros(ne, np.int64)
+        for e, c in cuts.items():
+            counts[e] = c
+        ip = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)  # the last case covers 27 of 33 rows
+        x = torch.from_numpy(rng.standard_normal((rows, k)).astype(np.float32)).to(DEV).to(tdt)
+        x_ref = x.float().cpu().numpy()
+        out = torch.full((rows, n), 7.0, dtype=tdt, device=DEV)
+        if model_dtype == "float16":
+            gq._lib.call("mi355gq_moe_group_gemm", x.data_ptr(), rows, qwd.data_ptr(), qs.data_ptr(), dev(ip).data_ptr(),
+                         gq._lib.I32, ne, n, k, s.bits, s.group_size, out.data_ptr(), 0)
+        else:
+            gq._lib.call("mi355gq_moe_group_gemm_dt", x.data_ptr(), rows, qwd.data_ptr(), qs.data_ptr(),
+                         dev(ip).data_ptr(), gq._lib.I32, ne, n, k, s.bits, s.group_size, gq._lib.BF16, out.data_ptr(), 0)
+        torch.cuda.synchronize()
+        covered = int(ip[-1])
+        ref = o.dequantize_group_gemm_dt_fp64(x_ref, qw, qs_ref, ip, s, model_dtype)[:covered]
+        got = out.float().cpu().numpy()
+        assert (got[covered:] == 7.0).all()  # rows that no segment covers are left alone
+        err = np.abs(got[:covered] - ref)
+        scale = np.abs(ref).max() + 1e-6
+        assert err.max() <= (2e-3 if model_dtype == "float16" else 1.2e-2) * scale, (rows, err.max(), scale)
+        if covered == rows:
+            out2 = ops.moe_group_gemm(x, qwd, qs, dev(ip.astype(np.int64)), s.bits, s.group_size)
+            assert torch.equal(out2, out)
+            src = torch.from_numpy(rng.standard_normal((rows + 5, k)).astype(np.float32)).to(DEV).to(tdt)
+            idx = torch.from_numpy(rng.integers(0, rows + 5, rows).astype(np.int32)).to(DEV)
+            for silu in (False, True):
+                want = ops.moe_group_gemm(ops.take_rows(src, idx), qwd, qs, dev(ip), s.bits, s.group_size, silu)
+                assert torch.equal(ops.moe_experts(src, idx, qwd, qs, dev(ip), s.bits, s.group_size, silu), want)
+                if silu:
+                    plain = ops.moe_group_gemm(ops.take_rows(src, idx), qwd, qs, dev(ip), s.bits, s.group_size)
+                    assert torch.equal(want, ops.silu_mul(plain))
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 def test_moe_group_gemm_wide_tile(name):
     """Enough rows per expert and enough column tiles for the 128 x 256 grouped tile; ragged segments."""
     s = SCHEMES[name]
