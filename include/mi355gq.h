@@ -258,9 +258,9 @@ MI355GQ_API int mi355gq_moe_experts(const void* x, int64_t x_rows, const void* x
 /*
  * The routing of one MoE layer in one launch: gating_softmax_topk, moe_cumsum, get_indices and
  * get_indptr (moe_misc.py:135-235, 371-605; the sequence of mixtral_model.py:77-106) for batches one
- * workgroup can scan (num_experts <= 64, and T * top_k <= 8192 or else T <= 8192 with
- * num_experts * ceil(T / 1024) <= 64; otherwise MI355GQ_ERR_UNSUPPORTED and the four calls below do
- * the same work).  Outputs as those calls give
+ * workgroup can scan (T * top_k <= 8192 with num_experts * ceil(T * top_k / 64) <= 8192, or else
+ * num_experts <= 64 and T <= 8192 with num_experts * ceil(T / 1024) <= 64; otherwise
+ * MI355GQ_ERR_UNSUPPORTED and the four calls below do the same work).  Outputs as those calls give
  * them: weights fp16 [T, top_k], ids int32 [T, top_k], token_indices / reverse_indices int32
  * [T * top_k], indptr [num_experts + 1] (exclusive form, indptr[0] = 0); plus slot_positions int32
  * [T * top_k], the inverse of reverse_indices (slot t * top_k + j is row slot_positions[...] of the

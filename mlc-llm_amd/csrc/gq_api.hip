@@ -1000,9 +1000,9 @@ static int moe_route_impl(const void* logits, int64_t T, int64_t num_experts, in
   GQ_REQUIRE(indptr_dtype == MI355GQ_I32 || indptr_dtype == MI355GQ_I64, "moe_route: indptr_dtype=%d",
              indptr_dtype);
   GQ_REQUIRE(indptr != nullptr, "moe_route: indptr is null");
-  // one workgroup: by slot up to 8192 (token, slot) pairs, else expert by expert while that is a handful of rounds
-  const bool by_slot = T * top_k <= 8192;
-  if (num_experts > 64 || (!by_slot && (T > 8192 || num_experts * ((T + 1023) / 1024) > 64)))
+  // one workgroup: by slot while the count table fits, else expert by expert while that is a handful of rounds
+  const bool by_slot = gq::moe_route_by_slot(T, static_cast<int>(num_experts), static_cast<int>(top_k));
+  if (!by_slot && (num_experts > 64 || T > 8192 || num_experts * ((T + 1023) / 1024) > 64))
     return fail(MI355GQ_ERR_UNSUPPORTED,
                 "moe_route: T=%lld with %lld experts is past the single-workgroup form; run "
                 "gating_softmax_topk, moe_cumsum, moe_get_indices and moe_get_indptr",

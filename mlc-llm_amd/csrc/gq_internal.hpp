@@ -112,6 +112,7 @@ hipError_t launch_silu_mul(const void* x, int64_t R, int64_t I, void* out, int m
 hipError_t launch_moe_combine(const void* y, const void* w, const int32_t* pos, int64_t T, int k, int64_t H,
                               void* out, int model_dtype, hipStream_t s);
 // fused routing for batches one workgroup can scan (the caller checks T and the expert count)
+bool moe_route_by_slot(int64_t T, int ne, int k);  // the single-workgroup route step has its slot-organised form
 hipError_t launch_moe_route(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int32_t* tok,
                             int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr, int model_dtype,
                             hipStream_t s);

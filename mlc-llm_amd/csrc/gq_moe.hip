@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const void* __restric
 // One wave per token, for many experts or many slots (the thread-per-token insertion above costs
 // ne * k * k predicated moves on one lane): lane l holds the logits of experts l, l + 64, ...; k rounds
 // of a wave-wide arg-max (larger value first, equal values by lower expert index: the order the
-// insertion produces) pick the slots, and lane 0 finishes with the same softmax.  Logits that are not
+// insertion produces) pick the slots (by rank counting up to 128 experts), and lane 0 finishes with the same softmax.  Logits that are not
 // above min_value(dtype), NaN included, are never picked; slots left empty keep (min_value, expert 0).
 constexpr int kWaveTopkChunks = 8;  // experts per lane: ne <= 512
 template <int DT>
@@ -144,26 +144,37 @@ __device__ __forceinline__ void topk_softmax_wave(const void* __restrict__ logit
   constexpr int kNone = 0x7fffffff;
   float val[kMaxTopK];
   int idx[kMaxTopK];
-  if (nch == 1) {
-    // up to 64 experts: every lane counts the experts that come before its own in that order (its rank)
-    // from lane broadcasts, with no trip through the LDS crossbar; slot i is the lane of rank i
-    const bool placeable = !(out_of_running & 1u);
-    int rank = 0;
+  if (nch <= 2) {
+    // up to 128 experts: every lane counts the experts that come before its own in that order (their rank)
+    // from lane broadcasts, with no trip through the LDS crossbar; slot i is the expert of rank i
+    int rank[2] = {0, 0};
 #pragma unroll
-    for (int l = 0; l < 64; ++l) {
-      const float ov = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[0]), l));
-      rank += (ov > v[0] || (ov == v[0] && l < lane)) ? 1 : 0;  // a logit that cannot be placed never wins here
+    for (int c2 = 0; c2 < 2; ++c2) {
+      if (c2 < nch) {  // uniform
+#pragma unroll
+        for (int l = 0; l < 64; ++l) {
+          const float ov = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[c2]), l));
+          const int oe = l + 64 * c2;  // (a logit that cannot be placed never wins the comparisons below)
+          rank[0] += (ov > v[0] || (ov == v[0] && oe < lane)) ? 1 : 0;
+          if (nch == 2) rank[1] += (ov > v[1] || (ov == v[1] && oe < lane + 64)) ? 1 : 0;
+        }
+      }
     }
 #pragma unroll
     for (int i = 0; i < kMaxTopK; ++i) {
       val[i] = Elem<DT>::kLowest;
       idx[i] = 0;
       if (i < k) {
-        const unsigned long long m = __ballot(placeable && rank == i);
-        if (m != 0ull) {
-          const int src = __builtin_ctzll(m);
+        const unsigned long long m0 = __ballot(!(out_of_running & 1u) && rank[0] == i);
+        const unsigned long long m1 = __ballot(nch == 2 && !(out_of_running & 2u) && rank[1] == i);
+        if (m0 != 0ull) {
+          const int src = __builtin_ctzll(m0);
           val[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[0]), src));
           idx[i] = src;
+        } else if (m1 != 0ull) {
+          const int src = __builtin_ctzll(m1);
+          val[i] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v[1]), src));
+          idx[i] = src + 64;
         }
       }
     }
@@ -280,7 +291,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict_
   }
 }
 
-// The same routing step organised by slot, for up to 8 slots per thread and up to 64 experts: thread
+// The same routing step organised by slot, for up to 8 slots per thread and a count table that fits LDS: thread
 // tid owns slots tid, tid + nthreads, ...; one pass of wave ballots per expert gives every slot its rank
 // among its wave's slots of the same expert and every (expert, 64-slot chunk) its count; a scan of that
 // table in (expert, chunk) order turns the counts into offsets.  Three barriers in all, where the
@@ -321,13 +332,16 @@ __global__ __launch_bounds__(1024) void moe_route_slots_kernel(const void* __res
           repeated |= (ids[s - j + (jj < j ? jj : j)] == id) & (jj < j);
         if (!repeated) myid[r] = id;
       }
-      int mine = 0;  // lane e: slots of expert e in this wave's chunk
-      for (int e = 0; e < ne; ++e) {
-        const unsigned long long m = __ballot(myid[r] == e);
-        if (myid[r] == e) before[r] = __popcll(m & lower);
-        if (lane == e) mine = __popcll(m);
+      for (int e0 = 0; e0 < ne; e0 += 64) {
+        int mine = 0;  // lane l: slots of expert e0 + l in this wave's chunk
+        const int e1 = e0 + 64 < ne ? e0 + 64 : ne;
+        for (int e = e0; e < e1; ++e) {
+          const unsigned long long m = __ballot(myid[r] == e);
+          if (myid[r] == e) before[r] = __popcll(m & lower);
+          if (lane == e - e0) mine = __popcll(m);
+        }
+        if (e0 + lane < ne) cnt[(e0 + lane) * nchunks + r * nwaves + wave] = mine;
       }
-      if (lane < ne) cnt[lane * nchunks + r * nwaves + wave] = mine;
     }
   }
   __syncthreads();
@@ -603,11 +617,17 @@ hipError_t launch_moe_combine(const void* y, const void* w, const int32_t* pos, 
   });
 }
 
+// the slot-organised route kernel: 8 slots per thread, [experts, 64-slot chunks] counts in 32 KiB of LDS
+bool moe_route_by_slot(int64_t T, int ne, int k) {
+  const int64_t slots = T * k;
+  return slots <= 8 * 1024 && ne <= 256 && static_cast<int64_t>(ne) * ((slots + 63) / 64) <= 8 * 1024;
+}
+
 hipError_t launch_moe_route(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int32_t* tok,
                             int32_t* rev, int32_t* pos_of_slot, int out_i64, void* indptr, int model_dtype,
                             hipStream_t s) {
   const int64_t slots = T * k;
-  if (slots > 0 && slots <= 8 * 1024 && ne <= 64) {
+  if (moe_route_by_slot(T, ne, k) && slots > 0) {
     // by slot; with many experts the top-k runs one wave per token, inside the kernel while one
     // workgroup has a wave for every token, as a launch of its own across the chip beyond that
     const bool by_wave = use_wave_topk(ne, k);
