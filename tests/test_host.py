@@ -84,7 +84,7 @@ def test_argument_validation_of_the_later_entry_points():
     assert lib.mi355gq_moe_route(P(0x1000), 9000, 8, 2, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
                                  P(0x7000), 0, None) == -3
     assert "four" in _err() or "gating_softmax_topk" in _err()
-    assert lib.mi355gq_moe_route(P(0x1000), 16, 100, 2, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
+    assert lib.mi355gq_moe_route(P(0x1000), 5000, 128, 2, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
                                  P(0x7000), 0, None) == -3
     assert lib.mi355gq_moe_route(P(0x1000), 16, 8, 9, P(0x2000), P(0x3000), P(0x4000), P(0x5000), P(0x6000),
                                  P(0x7000), 0, None) == -1
