@@ -292,8 +292,9 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict_
 }
 
 // The same routing step organised by slot, for up to 8 slots per thread and a count table that fits LDS: thread
-// tid owns slots tid, tid + nthreads, ...; one pass of wave ballots per expert gives every slot its rank
-// among its wave's slots of the same expert and every (expert, 64-slot chunk) its count; a scan of that
+// tid owns slots tid, tid + nthreads, ...; one pass of wave ballots per expert (or, past 16 experts, of
+// pairwise id comparisons among the wave's lanes) gives every slot its rank among its wave's slots of the
+// same expert and every (expert, 64-slot chunk) its count; a scan of that
 // table in (expert, chunk) order turns the counts into offsets.  Three barriers in all, where the
 // kernel above takes one per expert and round and re-reads k ids per token and expert.
 // do_topk 0: ids (and w) were produced by an earlier launch.  wave_topk: one wave per token.
@@ -316,6 +317,10 @@ __global__ __launch_bounds__(1024) void moe_route_slots_kernel(const void* __res
       for (int t = tid; t < T; t += nthreads) topk_softmax_token<DT>(logits, t, ne, k, w, ids);
     __syncthreads();  // ids written above are read back by other threads below
   }
+  if (ne > 16) {  // uniform
+    for (int i = tid; i < N; i += nthreads) cnt[i] = 0;
+    __syncthreads();
+  }
   const unsigned long long lower = (1ull << lane) - 1ull;
   int myid[kSlotsPerThread], before[kSlotsPerThread];
 #pragma unroll
@@ -332,6 +337,18 @@ __global__ __launch_bounds__(1024) void moe_route_slots_kernel(const void* __res
           repeated |= (ids[s - j + (jj < j ? jj : j)] == id) & (jj < j);
         if (!repeated) myid[r] = id;
       }
+      if (ne > 16) {
+        // many experts: the lanes compare ids pairwise instead (64 lane broadcasts whatever the expert count);
+        // the last slot of an expert in the chunk records the expert's count in the zeroed table
+        int after = 0;
+#pragma unroll
+        for (int l = 0; l < 64; ++l) {
+          const int same = __builtin_amdgcn_readlane(myid[r], l) == myid[r] ? 1 : 0;
+          before[r] += l < lane ? same : 0;
+          after += l > lane ? same : 0;
+        }
+        if (myid[r] >= 0 && after == 0) cnt[myid[r] * nchunks + r * nwaves + wave] = before[r] + 1;
+      } else
       for (int e0 = 0; e0 < ne; e0 += 64) {
         int mine = 0;  // lane l: slots of expert e0 + l in this wave's chunk
         const int e1 = e0 + 64 < ne ? e0 + 64 : ne;
@@ -629,9 +646,10 @@ hipError_t launch_moe_route(const void* logits, int64_t T, int ne, int k, void* 
   const int64_t slots = T * k;
   if (moe_route_by_slot(T, ne, k) && slots > 0) {
     // by slot; with many experts the top-k runs one wave per token, inside the kernel while one
-    // workgroup has a wave for every token, as a launch of its own across the chip beyond that
+    // workgroup is a single token's wave, as a launch of its own across the chip beyond that (never slower: T=16
+    // 25.5 -> 18.0 us with 128 experts, and a route step of one or two waves instead of one per token)
     const bool by_wave = use_wave_topk(ne, k);
-    const bool topk_first = by_wave && T > 16;
+    const bool topk_first = by_wave && T > 1;
     if (topk_first) {
       const hipError_t err = launch_topk_softmax(logits, T, ne, k, w, ids, model_dtype, s);
       if (err != hipSuccess) return err;
