@@ -4,6 +4,8 @@
  * Every entry point takes raw device pointers, sizes and a hipStream_t (passed
  * as void*), launches asynchronously on that stream and returns MI355GQ_OK or a
  * negative code; mi355gq_last_error() then holds a thread-local message.
+ * The library holds no process-wide mutable state (a per-device record of kernel attributes already set aside):
+ * entry points may be called from any thread.
  * Nothing allocates, nothing retains pointers, nothing synchronises: outputs
  * (and workspaces, where named) are owned by the caller, exactly as Relax
  * `call_dps_packed` hands them over (destination-passing style, see the
@@ -60,10 +62,6 @@ MI355GQ_API int mi355gq_check_device(void);
  * scale tensors to quote what the device delivers for those bytes without any arithmetic. */
 MI355GQ_API int mi355gq_probe_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,
                               void* sink, mi355gq_stream_t stream);
-
-/* Tuning/diagnostic knob (process-global, not thread-safe against running calls):
- * "gemv_rows_per_wave", "gemv_variant", "gemm_variant" ... ; value < 0 restores the default. */
-MI355GQ_API int mi355gq_set_option(const char* name, int value);
 
 /*
  * GroupQuantize.quantize_weight, NK layout (replaces the Relax function built at
@@ -276,6 +274,19 @@ MI355GQ_API int mi355gq_moe_route(const void* logits, int64_t T, int64_t num_exp
  * Ties keep the lower expert index. top_k <= 8, num_experts <= 256. */
 MI355GQ_API int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
                                 void* weights, void* ids, mi355gq_stream_t stream);
+
+/* gating_topk (moe_misc.py:63-132): scores [T, num_experts] in model_dtype -> the top_k scores as they are
+ * [T, top_k] and their expert ids int32 [T, top_k], by the same insertion (ties keep the lower index). top_k <= 8. */
+MI355GQ_API int mi355gq_gating_topk(const void* scores, int64_t T, int64_t num_experts, int64_t top_k,
+                        void* out_scores, void* ids, int model_dtype, mi355gq_stream_t stream);
+
+/* gating_softmax_topk with its norm_topk_prob argument (moe_misc.py:135-235).  norm_topk_prob != 0 is
+ * mi355gq_gating_softmax_topk(_dt).  norm_topk_prob == 0 is the branch of :234-235: softmax over ALL experts in
+ * fp32, cast to the model dtype, then gating_topk of those rounded scores; the weights are the selected scores,
+ * not renormalised. */
+MI355GQ_API int mi355gq_gating_softmax_topk_ex(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
+                                   int norm_topk_prob, int model_dtype, void* weights, void* ids,
+                                   mi355gq_stream_t stream);
 
 /* moe_cumsum (moe_misc.py:371-450): ids int32 [T, top_k] -> cumsum int32 [num_experts * T],
  * inclusive prefix sum of the expert-major token mask. */

@@ -6,14 +6,35 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/mi355gq.h"
 #include "gq_internal.hpp"
+#include "gq_testing.h"
 
 namespace gq {
 Options& options() {
-  static Options o;
+  thread_local Options o;
   return o;
+}
+
+hipError_t allow_large_lds(const void* kernel) {
+  constexpr int kMaxDevices = 64, kSlots = 512;
+  static std::mutex mu;
+  static const void* seen[kMaxDevices][kSlots];  // kernels already set, per device (a few dozen instantiations exist)
+  static int count[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev >= 0 && dev < kMaxDevices) {
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < count[dev]; ++i)
+      if (seen[dev][i] == kernel) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess && count[dev] < kSlots) seen[dev][count[dev]++] = kernel;
+    return e;
+  }
+  return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
 }
 }  // namespace gq
 
@@ -111,14 +132,28 @@ int mi355gq_check_device(void) {
   return MI355GQ_OK;
 }
 
-int mi355gq_set_option(const char* name, int value) {
+int mi355gq_testing_set_option(const char* name, int value) {
   GQ_REQUIRE(name != nullptr, "option name is null");
   gq::Options& o = gq::options();
-  if (!strcmp(name, "gemv_rows_per_wave")) o.gemv_rows_per_wave = value;
-  else if (!strcmp(name, "gemv_variant")) o.gemv_variant = value;
-  else if (!strcmp(name, "gemm_variant")) o.gemm_variant = value;
-  else if (!strcmp(name, "gemv_split")) o.gemv_split = value;
-  else return fail(MI355GQ_ERR_ARG, "unknown option '%s'", name);
+  if (value < 0) value = -1;  // any negative value restores the heuristic
+  if (!strcmp(name, "gemv_rows_per_wave")) {
+    GQ_REQUIRE(value == -1 || value == 1 || value == 2 || value == 4 || value == 8, "gemv_rows_per_wave=%d (1, 2, 4, 8)", value);
+    o.gemv_rows_per_wave = value;
+  } else if (!strcmp(name, "gemv_variant")) {
+    GQ_REQUIRE(value <= 15, "gemv_variant=%d (-1..15)", value);
+    o.gemv_variant = value;
+  } else if (!strcmp(name, "gemm_variant")) {
+    GQ_REQUIRE(value <= 15, "gemm_variant=%d (-1..15)", value);
+    o.gemm_variant = value;
+  } else if (!strcmp(name, "gemv_waves")) {
+    GQ_REQUIRE(value == -1 || (value >= 4 && value <= 16384), "gemv_waves=%d (4..16384)", value);
+    o.gemv_waves = value;
+  } else if (!strcmp(name, "gemm_split_k")) {
+    GQ_REQUIRE(value == -1 || (value >= 1 && value <= 4096), "gemm_split_k=%d (1..4096)", value);
+    o.gemm_split_k = value;
+  } else {
+    return fail(MI355GQ_ERR_ARG, "unknown option '%s'", name);
+  }
   return MI355GQ_OK;
 }
 
@@ -864,6 +899,37 @@ int mi355gq_gating_softmax_topk(const void* logits, int64_t T, int64_t num_exper
 int mi355gq_gating_softmax_topk_dt(const void* logits, int64_t T, int64_t num_experts, int64_t top_k, void* weights,
                                    void* ids, int model_dtype, mi355gq_stream_t stream) {
   return gating_impl(logits, T, num_experts, top_k, weights, ids, model_dtype, stream);
+}
+
+static int topk_scores_impl(const char* what, const void* x, int64_t T, int64_t num_experts, int64_t top_k,
+                            void* out_scores, void* ids, int model_dtype, bool softmax_first,
+                            mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, what));
+  GQ_REQUIRE(T >= 0 && T < kMaxDim, "%s: bad T", what);
+  GQ_REQUIRE(num_experts >= 1 && num_experts <= 65536, "%s: num_experts=%lld (1..65536)", what, (long long)num_experts);
+  GQ_REQUIRE(top_k >= 1 && top_k <= 8 && top_k <= num_experts, "%s: top_k=%lld (1..min(8, num_experts))", what,
+             (long long)top_k);
+  if (T == 0) return MI355GQ_OK;
+  GQ_REQUIRE(x && out_scores && ids, "%s: null pointer", what);
+  GQ_REQUIRE(aligned4(ids) && (model_dtype == MI355GQ_F32 ? aligned4(x) && aligned4(out_scores)
+                                                          : aligned2(x) && aligned2(out_scores)),
+             "%s: misaligned tensor", what);
+  return hip_result(gq::launch_topk_scores(x, T, static_cast<int>(num_experts), static_cast<int>(top_k), out_scores,
+                                           static_cast<int32_t*>(ids), model_dtype, softmax_first, as_stream(stream)),
+                    what);
+}
+
+int mi355gq_gating_topk(const void* scores, int64_t T, int64_t num_experts, int64_t top_k, void* out_scores,
+                        void* ids, int model_dtype, mi355gq_stream_t stream) {
+  return topk_scores_impl("gating_topk", scores, T, num_experts, top_k, out_scores, ids, model_dtype, false, stream);
+}
+
+int mi355gq_gating_softmax_topk_ex(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
+                                   int norm_topk_prob, int model_dtype, void* weights, void* ids,
+                                   mi355gq_stream_t stream) {
+  if (norm_topk_prob) return gating_impl(logits, T, num_experts, top_k, weights, ids, model_dtype, stream);
+  return topk_scores_impl("gating_softmax_topk_ex", logits, T, num_experts, top_k, weights, ids, model_dtype, true,
+                          stream);
 }
 
 int mi355gq_moe_cumsum(const void* ids, int64_t T, int64_t top_k, int64_t num_experts,

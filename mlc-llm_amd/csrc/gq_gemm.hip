@@ -188,9 +188,7 @@ static hipError_t launch_cfg(const GemmParams& p, hipStream_t s) {
   constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
   auto kern = gemm_kernel<BITS, BM, BN, WM, WN>;
   if (lds > 65536) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             static_cast<int>(lds));
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
     if (e != hipSuccess) return e;
   }
   const int m_tiles = p.indptr ? (p.rows + BM - 1) / BM + p.num_experts : (p.rows + BM - 1) / BM;

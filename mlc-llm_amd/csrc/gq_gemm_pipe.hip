@@ -299,9 +299,7 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
   auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH, BF>;
   if (lds > 65536) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             static_cast<int>(lds));
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
     if (e != hipSuccess) return e;
   }
   const int m_tiles = p.indptr ? (p.rows + BM - 1) / BM + p.num_experts : (p.rows + BM - 1) / BM;
@@ -400,13 +398,13 @@ SplitPlan plan_split_k(int64_t rows, int64_t N, int64_t K, int bits, int group_s
   // Splitting K pays with partial sums (split * rows * N * 8 bytes written and read back): only
   // when the tiles alone leave CUs idle, and never beyond about twice the weight bytes.
   int split = 1;
-  if (tiles < 200 || options().gemv_split > 0) {
+  if (tiles < 200 || options().gemm_split_k > 0) {
     // one workgroup per CU: measured 8-20 % faster than two (o_proj, qkv, down at 17..128 rows), whose
     // partial sums cost more than the second workgroup hides
-    const int64_t want = options().gemv_split > 0 ? options().gemv_split : 256;  // (tuning override)
+    const int64_t want = options().gemm_split_k > 0 ? options().gemm_split_k : 256;  // (tuning override)
     split = static_cast<int>((want + tiles - 1) / tiles);
     const int64_t cap = K / (7 * rows);
-    if (options().gemv_split <= 0 && split > cap) split = static_cast<int>(cap);
+    if (options().gemm_split_k <= 0 && split > cap) split = static_cast<int>(cap);
     if (split > nk / 4) split = nk / 4;  // at least four K tiles per workgroup
     if (split < 1) split = 1;
   }

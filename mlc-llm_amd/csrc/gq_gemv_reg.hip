@@ -313,8 +313,8 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
   }
   const int nsets = (p.N + R - 1) / R;
   int waves;
-  if (options().gemv_split > 0) {
-    waves = options().gemv_split;
+  if (options().gemv_waves > 0) {
+    waves = options().gemv_waves;
   } else if (iters > 2) {
     // one wave per SIMD; two once the registers allow it (up to 4 groups per lane) and the rows keep them busy
     waves = (iters <= 4 && rows_total >= 12288) ? 2048 : 1024;
@@ -341,6 +341,9 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
 
 hipError_t launch_gemv_reg(const GemvParams& p, int bits, int nb, int slots, hipStream_t s) {
   if (p.ng == 0) return hipErrorNotSupported;
+  // the x staging always issues whole 16-byte loads (from the base of x where a chunk is unusable): x must hold
+  // at least 8 halves per row for that address to be readable
+  if (p.K < 8) return hipErrorNotSupported;
   if (static_cast<int64_t>(nb) * p.ng * (bits == 4 ? 32 : 40) * 2 > 65536) return hipErrorNotSupported;
   return bits == 4 ? launch_bits<4>(p, nb, slots, s) : launch_bits<3>(p, nb, slots, s);
 }

@@ -7,13 +7,21 @@
 
 namespace gq {
 
+// Kernel forcing for tests and tuning sweeps.  The state is thread-local and defaults to "heuristics": only the
+// thread that called the test hook (mi355gq_testing_set_option, declared in gq_testing.h and absent from the
+// public header) ever sees anything else, so calls arriving on other threads cannot be steered by it.
 struct Options {
   int gemv_rows_per_wave = -1;  // -1: heuristic
-  int gemv_variant = -1;        // -1: heuristic, 0: dot2 kernel, 1: mfma kernel
+  int gemv_variant = -1;        // -1: heuristic, 0: LDS GEMV, 1: register GEMV, 2..5 skinny forms, 6..8 quad-row forms
   int gemm_variant = -1;
-  int gemv_split = -1;        // total waves of the persistent GEMV grid
+  int gemv_waves = -1;          // total waves of a persistent GEMV / quad-row / skinny grid
+  int gemm_split_k = -1;        // wanted workgroups of the few-row GEMM's split along K
 };
 Options& options();
+
+// hipFuncAttributeMaxDynamicSharedMemorySize = the CU's whole LDS, set once per (kernel, device) and remembered;
+// kernels whose dynamic LDS may exceed 64 KiB call it before launching.
+hipError_t allow_large_lds(const void* kernel);
 
 struct GemvArgs {
   const uint16_t* x;        // [x_rows, K] fp16
@@ -100,6 +108,9 @@ hipError_t launch_dequantize(const int32_t* ids, int64_t out_rows, const uint32_
 // (logits, weights, activations of the routing glue carry model_dtype: MODEL_F16 | MODEL_F32 | MODEL_BF16)
 hipError_t launch_topk_softmax(const void* logits, int64_t T, int ne, int k, void* w, int32_t* ids, int model_dtype,
                                hipStream_t s);
+// gating_topk on given scores, or (softmax_first) fp32 softmax over all experts rounded to the dtype, then that top-k
+hipError_t launch_topk_scores(const void* x, int64_t T, int ne, int k, void* w, int32_t* ids, int model_dtype,
+                              bool softmax_first, hipStream_t s);
 hipError_t launch_moe_cumsum(const int32_t* ids, int64_t T, int k, int ne, int32_t* cumsum,
                              hipStream_t s);
 hipError_t launch_get_indices(const int32_t* cumsum, const int32_t* ids, int64_t T, int k, int ne,

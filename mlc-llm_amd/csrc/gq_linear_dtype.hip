@@ -491,8 +491,7 @@ hipError_t launch_dt(const LinParams& p, hipStream_t s) {
         }
         auto go = [&](auto kern) -> hipError_t {
           if (lds > 65536) {
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
             if (e != hipSuccess) return e;
           }
           hipLaunchKernelGGL(kern, dim3(blocks, segments), dim3(256), lds, s, q, nsets);
@@ -519,8 +518,7 @@ hipError_t launch_dt(const LinParams& p, hipStream_t s) {
   }
   constexpr size_t lds = size_t(2) * 256 * (G + 1) * sizeof(float);
   auto kern = gemm_dt_kernel<BITS, DT>;
-  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+  const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
   if (e != hipSuccess) return e;
   // row tiles: one per one-row segment; grouped, every expert may add a partly filled one
   const int m_tiles = p.ids != nullptr ? p.M : (p.M + 127) / 128 + (p.indptr != nullptr ? p.num_experts : 0);

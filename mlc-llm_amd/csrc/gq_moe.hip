@@ -121,6 +121,67 @@ __global__ __launch_bounds__(256) void topk_softmax_kernel(const void* __restric
   topk_softmax_token<DT>(logits, t, ne, k, w, ids);
 }
 
+// gating_topk (moe_misc.py:63-132) and the norm_topk_prob = False branch of gating_softmax_topk (:234-235), one
+// thread per token: SOFTMAX computes softmax over ALL experts in fp32 (exp(x - max) / sum, summed left to right),
+// rounds each score to the model dtype, and then, in both forms, the same insertion top-k runs on the scores and
+// returns them as they are (no renormalisation).  Scores that round to the same value tie: lower index first.
+template <int KMAX, int DT, bool SOFTMAX>
+__device__ __forceinline__ void topk_scores_slots(const void* __restrict__ x, int64_t row0, int ne, int k,
+                                                  void* __restrict__ w, int64_t w0, int32_t* __restrict__ ids) {
+  float mx = 0.f, den = 0.f;
+  if (SOFTMAX) {
+    mx = Elem<DT>::load(x, row0);
+    for (int e = 1; e < ne; ++e) mx = fmaxf(mx, Elem<DT>::load(x, row0 + e));
+    for (int e = 0; e < ne; ++e) {
+      const float ex = expf(Elem<DT>::load(x, row0 + e) - mx);
+      den = e == 0 ? ex : den + ex;
+    }
+  }
+  float val[KMAX];
+  int idx[KMAX];
+#pragma unroll
+  for (int i = 0; i < KMAX; ++i) {
+    val[i] = Elem<DT>::kLowest;
+    idx[i] = 0;
+  }
+  for (int e = 0; e < ne; ++e) {
+    float v = Elem<DT>::load(x, row0 + e);
+    if (SOFTMAX) v = Elem<DT>::rnd(expf(v - mx) / den);
+    bool placed = false;
+#pragma unroll
+    for (int i = 0; i < KMAX; ++i) {
+      if (i < k && !placed && v > val[i]) {
+#pragma unroll
+        for (int j = KMAX - 1; j > 0; --j) {
+          if (j > i && j < k) {
+            val[j] = val[j - 1];
+            idx[j] = idx[j - 1];
+          }
+        }
+        val[i] = v;
+        idx[i] = e;
+        placed = true;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < KMAX; ++i) {
+    if (i < k) {
+      Elem<DT>::store(w, w0 + i, val[i]);
+      ids[i] = idx[i];
+    }
+  }
+}
+
+template <int DT, bool SOFTMAX>
+__global__ __launch_bounds__(256) void topk_scores_kernel(const void* __restrict__ x, int64_t T, int ne, int k,
+                                                          void* __restrict__ w, int32_t* __restrict__ ids) {
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (t >= T) return;
+  if (k <= 2) topk_scores_slots<2, DT, SOFTMAX>(x, t * ne, ne, k, w, t * k, ids + t * k);
+  else topk_scores_slots<kMaxTopK, DT, SOFTMAX>(x, t * ne, ne, k, w, t * k, ids + t * k);
+}
+
 // One wave per token, for many experts or many slots (the thread-per-token insertion above costs
 // ne * k * k predicated moves on one lane): lane l holds the logits of experts l, l + 64, ...; k rounds
 // of a wave-wide arg-max (larger value first, equal values by lower expert index: the order the
@@ -576,6 +637,19 @@ hipError_t launch_topk_softmax(const void* logits, int64_t T, int ne, int k, voi
     else
       hipLaunchKernelGGL(topk_softmax_kernel<decltype(dt)::value>, dim3(blocks_for(T, 256)), dim3(256), 0, s, logits,
                          T, ne, k, w, ids);
+  });
+}
+
+hipError_t launch_topk_scores(const void* x, int64_t T, int ne, int k, void* w, int32_t* ids, int model_dtype,
+                              bool softmax_first, hipStream_t s) {
+  if (T == 0) return hipSuccess;
+  return by_dtype(model_dtype, [&](auto dt) {
+    if (softmax_first)
+      hipLaunchKernelGGL((topk_scores_kernel<decltype(dt)::value, true>), dim3(blocks_for(T, 256)), dim3(256), 0, s, x,
+                         T, ne, k, w, ids);
+    else
+      hipLaunchKernelGGL((topk_scores_kernel<decltype(dt)::value, false>), dim3(blocks_for(T, 256)), dim3(256), 0, s,
+                         x, T, ne, k, w, ids);
   });
 }
 

@@ -405,9 +405,7 @@ template <int BITS, int NBQ, int U, int MODE, bool BF = false>
 static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                     hipStream_t s) {
   if (lds > 65536) {
-    const hipError_t e =
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF>));
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF>), grid, dim3(threads), lds, s, p);
@@ -480,7 +478,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   // About one quad per wave up to 2048 waves (measured over the projection shapes of 7B..70B models: 13 to 30 %
   // faster than 1024 waves of two to four quads each at 2..8 rows); concurrent passes over the same weights
   // already multiply the grid, and there 1024 measured better (down_proj 8192 x 28672 at 8 rows: 48 vs 66 us).
-  int waves = options().gemv_split > 0 ? options().gemv_split
+  int waves = options().gemv_waves > 0 ? options().gemv_waves
                                        : (a.indptr != nullptr || mtiles == 1 ? 2048 : 1024);
   // workgroups of experts without rows leave at once: share the waves among those that can have rows
   const int busy = p.rows < experts ? p.rows : experts;

@@ -650,7 +650,7 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
     const int64_t tiles_all = (static_cast<int64_t>(p.N) + 15) / 16;
     if (mode != 2 && mode != 3 && mode != 5 && lds_p <= lds_cap && (mode == 4 || tiles_all >= 4096)) {
       const int ntiles = (p.N + 15) / 16;
-      int waves = options().gemv_split > 0 ? options().gemv_split : 2048;
+      int waves = options().gemv_waves > 0 ? options().gemv_waves : 2048;
       waves = (waves + experts * mtiles - 1) / (experts * mtiles);
       const int rounds = (ntiles + waves - 1) / waves;
       const int wpb = options().gemv_rows_per_wave == 4 ? 4 : 8;  // waves per workgroup (8 unless tuning says 4)
@@ -658,9 +658,7 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
       const dim3 grid(blocks, experts, mtiles);
       auto launch = [&](auto kern) -> hipError_t {
         if (lds_p > 65536) {
-          const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   static_cast<int>(lds_p));
+          const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
           if (e != hipSuccess) return e;
         }
         hipLaunchKernelGGL(kern, grid, dim3(64 * wpb), lds_p, s, p, ntiles, nblk);

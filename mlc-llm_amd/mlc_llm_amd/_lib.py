@@ -30,7 +30,6 @@ SIGNATURES = {
     "mi355gq_version": (_I, []),
     "mi355gq_last_error": (c_char_p, []),
     "mi355gq_check_device": (_I, []),
-    "mi355gq_set_option": (_I, [c_char_p, _I]),
     "mi355gq_quantize": (_I, [_P, _L, _L, _I, _I, _I, _P, _P, _P]),
     "mi355gq_dequantize": (_I, [_P, _P, _L, _L, _I, _I, _P, _P]),
     "mi355gq_quantize_dt": (_I, [_P, _L, _L, _I, _I, _I, _I, _P, _P, _P]),
@@ -67,6 +66,8 @@ SIGNATURES = {
     "mi355gq_moe_route": (_I, [_P, _L, _L, _L, _P, _P, _P, _P, _P, _P, _I, _P]),
     "mi355gq_moe_combine_sorted": (_I, [_P, _P, _P, _L, _L, _L, _P, _P]),
     "mi355gq_gating_softmax_topk": (_I, [_P, _L, _L, _L, _P, _P, _P]),
+    "mi355gq_gating_topk": (_I, [_P, _L, _L, _L, _P, _P, _I, _P]),
+    "mi355gq_gating_softmax_topk_ex": (_I, [_P, _L, _L, _L, _I, _I, _P, _P, _P]),
     "mi355gq_moe_cumsum": (_I, [_P, _L, _L, _L, _P, _P]),
     "mi355gq_moe_get_indices": (_I, [_P, _P, _L, _L, _L, _P, _P, _P]),
     "mi355gq_moe_get_indptr": (_I, [_P, _L, _L, _I, _I, _P, _P]),
@@ -74,6 +75,12 @@ SIGNATURES = {
     "mi355gq_moe_scatter_output": (_I, [_P, _P, _L, _L, _P, _P]),
     "mi355gq_silu_mul": (_I, [_P, _L, _L, _P, _P]),
     "mi355gq_moe_combine": (_I, [_P, _P, _L, _L, _L, _P, _P]),
+}
+
+
+# exported for tests and tuning sweeps only (csrc/gq_testing.h); not declared in the public header
+TEST_HOOKS = {
+    "mi355gq_testing_set_option": (_I, [c_char_p, _I]),
 }
 
 
@@ -106,7 +113,7 @@ def lib() -> ctypes.CDLL:
                 "(there is no non-HIP fallback)"
             )
         handle = ctypes.CDLL(LIB_PATH)
-        for name, (res, args) in SIGNATURES.items():
+        for name, (res, args) in {**SIGNATURES, **TEST_HOOKS}.items():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
@@ -123,4 +130,6 @@ def call(name: str, *args) -> None:
 
 
 def set_option(name: str, value: int) -> None:
-    call("mi355gq_set_option", name.encode(), int(value))
+    """Test / tuning hook (csrc/gq_testing.h): force a kernel family or launch shape for later calls of THIS
+    thread; a negative value restores the heuristic."""
+    call("mi355gq_testing_set_option", name.encode(), int(value))

@@ -267,6 +267,21 @@ def check_parameter_usage(mapping: ExternMapping, extern_names: Set[str]) -> Set
     return leftover
 
 
+def param_kind(mlc_name: str) -> str:
+    """Which module of GroupQuantize.quantize_model a quantised parameter belongs to, from its MLC name
+    (python/mlc_llm/quantization/group_quantization.py:105-147): "embedding" (nn.Embedding), "final_fc" (a Linear
+    that is_final_fc names: quantization/utils.py:51-54), "experts" (MixtralExperts) or "linear"."""
+    base = mlc_name[: -len(".weight")] if mlc_name.endswith(".weight") else mlc_name
+    leaf = base.rsplit(".", 1)[-1]
+    if leaf in ("embed_tokens", "embd", "wte"):
+        return "embedding"
+    if base in ("head", "lm_head", "lm_head.linear", "embed_out"):
+        return "final_fc"
+    if leaf in ("e1_e3", "e2"):
+        return "experts"
+    return "linear"
+
+
 class HuggingFaceLoader:
     """Yields (MLC name, tensor) for a safetensors checkpoint directory (or single file),
     quantising on ``device`` the parameters group quantisation replaces."""
@@ -333,14 +348,25 @@ class HuggingFaceLoader:
                 value = torch.from_numpy(np.ascontiguousarray(self.mapping.map_func[mlc_name](*np_parts)))
                 value = value.to(self.model_dtype)
                 self.total_param_num += value.numel()
-                if mlc_name in self.quantized:
-                    q = self.quantization
-                    base = mlc_name[: -len(".weight")]
-                    qw, qs = q.quantize_weight(value.to(device))
-                    yield f"{base}.q_weight", qw
-                    yield f"{base}.q_scale", qs
-                else:
+                q = self.quantization
+                kind = param_kind(mlc_name)
+                # what quantize_model leaves alone (group_quantization.py:117-139): the embedding under
+                # quantize_embedding=False, the final fc under quantize_final_fc=False (q4f16_2)
+                skip = mlc_name not in self.quantized or (kind == "embedding" and not q.quantize_embedding) or \
+                    (kind == "final_fc" and not q.quantize_final_fc)
+                if skip:
                     yield mlc_name, value.to(device)
+                    continue
+                if kind == "experts" and q.linear_weight_layout == "KN":
+                    raise NotImplementedError("GroupQuantizeMixtralExperts does not support the KN layout "
+                                              "(group_quantization.py:584-585)")
+                base = mlc_name[: -len(".weight")]
+                # KN schemes store a Linear's words and scales transposed (:125-130, 299-305); embeddings and
+                # experts always quantise along their last axis and keep that layout
+                transpose = q.linear_weight_layout == "KN" and kind in ("linear", "final_fc")
+                qw, qs = q.quantize_weight(value.to(device), output_transpose=transpose)
+                yield f"{base}.q_weight", qw
+                yield f"{base}.q_scale", qs
         finally:
             self.close()
 
@@ -363,7 +389,11 @@ def convert_weight(source: str, output: str, quantization: str = "q4f16_1",
     elif quantization != "q0f16":
         raise ValueError("unquantised conversion is float16 only")
     mapping, quantized = MODEL_MAPPINGS[model_type](config)
-    loader = HuggingFaceLoader(source, mapping, quantized, quant)
+    from .quantization import _TORCH_DTYPE
+
+    # every tensor is cast to the scheme's model dtype, not to float16 (q4bf16_*, q4f32_1)
+    loader = HuggingFaceLoader(source, mapping, quantized, quant,
+                               _TORCH_DTYPE[quant.model_dtype] if quant is not None else torch.float16)
     total_bytes = 0
     count = 0
 

@@ -20,10 +20,14 @@ def moe_sum(x: torch.Tensor, dim: int) -> torch.Tensor:
 
 def gating_softmax_topk(x: torch.Tensor, k: int, norm_topk_prob: bool = True
                         ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """:135-235.  Returns (expert_weights fp16 [T, k], expert_indices int32 [T, k])."""
-    if not norm_topk_prob:
-        raise NotImplementedError("norm_topk_prob=False (full softmax, then top-k) is not built")
-    return ops.gating_softmax_topk(x, k)
+    """:135-235.  Returns (expert_weights [T, k] in x's dtype, expert_indices int32 [T, k]).
+    norm_topk_prob=False is the branch of :234-235 (softmax over all experts, cast, then gating_topk)."""
+    return ops.gating_softmax_topk(x, k, norm_topk_prob)
+
+
+def gating_topk(scores: torch.Tensor, k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """:63-132.  Returns (the k largest scores as they are [T, k], their expert indices int32 [T, k])."""
+    return ops.gating_topk(scores, k)
 
 
 def moe_cumsum(expert_indices: torch.Tensor, num_local_experts: int) -> torch.Tensor:

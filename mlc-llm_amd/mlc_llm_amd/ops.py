@@ -397,13 +397,24 @@ def moe_combine_sorted(y: torch.Tensor, slot_positions: torch.Tensor, weights: t
     return out
 
 
-def gating_softmax_topk(logits: torch.Tensor, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+def gating_softmax_topk(logits: torch.Tensor, top_k: int, norm_topk_prob: bool = True
+                        ) -> Tuple[torch.Tensor, torch.Tensor]:
     _chk(logits, _FLOATS, "logits")
     t, ne = logits.shape
     w = torch.empty((t, top_k), dtype=logits.dtype, device=logits.device)
     ids = torch.empty((t, top_k), dtype=torch.int32, device=logits.device)
-    _lib.call("mi355gq_gating_softmax_topk_dt", logits.data_ptr(), t, ne, top_k, w.data_ptr(),
-              ids.data_ptr(), _MODEL_DTYPES[logits.dtype], _stream())
+    _lib.call("mi355gq_gating_softmax_topk_ex", logits.data_ptr(), t, ne, top_k, 1 if norm_topk_prob else 0,
+              _MODEL_DTYPES[logits.dtype], w.data_ptr(), ids.data_ptr(), _stream())
+    return w, ids
+
+
+def gating_topk(scores: torch.Tensor, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    _chk(scores, _FLOATS, "scores")
+    t, ne = scores.shape
+    w = torch.empty((t, top_k), dtype=scores.dtype, device=scores.device)
+    ids = torch.empty((t, top_k), dtype=torch.int32, device=scores.device)
+    _lib.call("mi355gq_gating_topk", scores.data_ptr(), t, ne, top_k, w.data_ptr(), ids.data_ptr(),
+              _MODEL_DTYPES[scores.dtype], _stream())
     return w, ids
 
 

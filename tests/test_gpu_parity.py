@@ -357,12 +357,12 @@ def test_quadrow_kernel_k_phases(name, waves, m, n, k):
     s = SCHEMES[name]
     x, qw, qs, b = _linear_case(s, m, n, k, 5 * m + n + k, bias=True)
     gq._lib.set_option("gemv_variant", 7)
-    gq._lib.set_option("gemv_split", waves)
+    gq._lib.set_option("gemv_waves", waves)
     try:
         y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
     finally:
         gq._lib.set_option("gemv_variant", -1)
-        gq._lib.set_option("gemv_split", -1)
+        gq._lib.set_option("gemv_waves", -1)
     assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"quad-row phases {name} {m}x{n}x{k} waves={waves}")
 
 
@@ -477,12 +477,12 @@ def test_few_row_gemm_split_counts_and_missing_workspace(want):
     m, n, k = 40, 260, 8192
     x, qw, qs, b = _linear_case(s, m, n, k, 99, bias=True)
     ref = o.linear_fp32(x, qw, qs, s, b)
-    gq._lib.set_option("gemv_split", want)
+    gq._lib.set_option("gemm_split_k", want)
     try:
         y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b))
         ws = gq._lib.lib().mi355gq_linear_workspace_bytes(m, n, k, 4, 32)
     finally:
-        gq._lib.set_option("gemv_split", -1)
+        gq._lib.set_option("gemm_split_k", -1)
     assert ws > 0
     assert_linear_ok(y, ref, x, k, f"few-row gemm, {want} workgroups wanted")
     # no workspace handed over: same tiles, no split, same answer

@@ -57,7 +57,7 @@ def test_argument_validation_never_launches():
     assert "expected 1 or top_k" in _err()
     assert lib.mi355gq_gating_softmax_topk(None, 4, 8, 9, None, None, None) == -1
     assert lib.mi355gq_moe_cumsum(None, 4, 2, 300, None, None) == -1
-    assert lib.mi355gq_set_option(b"no_such_option", 1) == -1
+    assert lib.mi355gq_testing_set_option(b"no_such_option", 1) == -1
     # misaligned pointers are rejected, not dereferenced
     assert lib.mi355gq_dequantize(ctypes.c_void_p(0x1004), ctypes.c_void_p(0x2000), 1, 32, 4, 32,
                                   ctypes.c_void_p(0x3000), None) == -1
@@ -67,7 +67,7 @@ def test_argument_validation_never_launches():
     assert lib.mi355gq_quantize(None, 0, 32, 4, 32, 0, None, None, None) == 0
     assert lib.mi355gq_embedding_take(None, 0, None, None, 10, 32, 4, 32, None, None) == 0
     with pytest.raises(_lib.Mi355gqError) as ei:
-        _lib.call("mi355gq_set_option", b"bogus", 0)
+        _lib.call("mi355gq_testing_set_option", b"bogus", 0)
     assert ei.value.code == -1 and "bogus" in str(ei.value)
 
 

@@ -420,3 +420,199 @@ def test_float32_scheme_closed_forms():
     d = o.dequantize_dt(qw, qs, s, 96, "float32")
     assert np.array_equal(d, (q.astype(np.float32) - 7) * np.repeat(qs, 32, -1))
     assert np.abs(d - w).max() <= np.abs(qs).max() * 0.5000001
+
+
+# --------------------------------------------------------------------------- silu * mul and the composed layer
+#
+# What fixes these without a run of the reference: silu(x) = x * sigmoid(x) is a closed form, so the fp32
+# evaluation rounded once to the dtype is compared with torch's own silu (an independent implementation)
+# and with float64 mathematics; the product of two halves is a single correctly rounded operation.  The
+# composed layer is compared with a dense per-token form that has no gather, scatter, cumsum or indptr
+# in it, over weights dequantised by the repeat-and-index formulation of the reference's own test.
+
+def _ulp16_diff(a, b):
+    """distance in fp16 representation steps (sign-magnitude to a monotone integer line)"""
+    def line(v):
+        u = np.asarray(v, np.float16).view(np.uint16).astype(np.int64)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(line(a) - line(b))
+
+
+def test_silu_mul_f16_against_closed_form_and_torch():
+    import torch
+
+    rng = np.random.default_rng(31)
+    x1 = np.concatenate([rng.standard_normal(4000) * 3, np.linspace(-20, 20, 801),
+                         np.array([0.0, -0.0, 1e-4, -1e-4, 30.0, -30.0, 65504.0, -65504.0, 6e-8])]).astype(np.float16)
+    x3 = np.concatenate([rng.standard_normal(4000) * 2, rng.standard_normal(801),
+                         np.array([5.0, 5.0, -3.0, 7.0, 2.0, 2.0, 1.0, 1.0, 1.0])]).astype(np.float16)
+    got = o.silu_mul_f16(np.concatenate([x1, x3])[None, :])[0]
+    # silu in float64 mathematics, rounded once to half, then the exact product rounded once to half
+    x64 = x1.astype(np.float64)
+    with np.errstate(over="ignore"):
+        silu64 = x64 / (1.0 + np.exp(-x64))
+    silu16 = silu64.astype(np.float16)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = (silu16.astype(np.float64) * x3.astype(np.float64)).astype(np.float16)
+    # the oracle evaluates silu in fp32 before the rounding to half: it may land on the other side of a rounding
+    # boundary of the float64 value in rare cases, never further
+    ok = ~(np.isnan(want.astype(np.float32)) | np.isinf(want.astype(np.float32)))
+    assert _ulp16_diff(got[ok], want[ok]).max() <= 1
+    assert (got[ok].view(np.uint16) == want[ok].view(np.uint16)).mean() > 0.995
+    # torch's silu on float32 (an independent implementation), rounded once, times x3 in half
+    t_silu = torch.nn.functional.silu(torch.from_numpy(x1.astype(np.float32))).half()
+    t_out = (t_silu * torch.from_numpy(x3)).numpy()
+    assert _ulp16_diff(got[ok], t_out[ok]).max() <= 1
+    # fixed points: silu(0) = 0 (either sign of zero gives a zero), silu(x) -> x for large x, -> -0 for large -x
+    z = o.silu_mul_f16(np.array([[0.0, -0.0, 30.0, -30.0, 5.0, 5.0, 2.0, 2.0]], np.float16))[0]
+    assert z[0] == 0 and z[1] == 0 and float(z[2]) == 60.0 and abs(float(z[3])) < 1e-6
+    # the halves are not interchangeable: silu applies to the FIRST half (mixtral_model.py:66-68)
+    a = o.silu_mul_f16(np.array([[4.0, 0.5]], np.float16))[0, 0]
+    b = o.silu_mul_f16(np.array([[0.5, 4.0]], np.float16))[0, 0]
+    assert float(a) == float(np.float16(np.float16(4.0 / (1 + np.exp(-4.0))) * np.float16(0.5)))
+    assert float(a) != float(b)
+
+
+@pytest.mark.parametrize("md", ["float32", "bfloat16", "float16"])
+def test_silu_mul_dt_against_closed_form(md):
+    rng = np.random.default_rng(37)
+    x1 = o.round_to(np.concatenate([rng.standard_normal(3000) * 3, np.linspace(-15, 15, 301)]).astype(np.float32), md)
+    x3 = o.round_to((rng.standard_normal(3301) * 2).astype(np.float32), md)
+    got = o.silu_mul_dt(np.concatenate([x1, x3])[None, :], md)[0]
+    x64 = x1.astype(np.float64)
+    silu = o.round_to((x64 / (1.0 + np.exp(-x64))).astype(np.float32), md)
+    want = o.round_to((silu.astype(np.float64) * x3.astype(np.float64)).astype(np.float32), md)
+    # one unit of the dtype at most (fp32 evaluation against float64 before the rounding)
+    # (float32: the fp32 exp, add and divide each round, a few units of the last place in all)
+    eps = {"float32": 2.0 ** -20, "bfloat16": 2.0 ** -7, "float16": 2.0 ** -10}[md]
+    assert (np.abs(got - want) <= eps * np.abs(want) + 1e-30).all()
+    if md != "float32":
+        assert (got == want).mean() > 0.99
+    if md == "float16":  # the generic form is the float16 form
+        h = o.silu_mul_f16(np.concatenate([x1, x3]).astype(np.float16)[None, :])[0]
+        assert np.array_equal(h.astype(np.float32), got)
+
+
+def _dense_moe_bruteforce(x, logits, q13, s13, q2, s2, s, top_k):
+    """MixtralMoE.forward (mixtral_model.py:64-117) token by token, with no gather / scatter / cumsum / indptr:
+    out[t] = sum_j w[t, j] * e2_id(silu(e1_id x) * e3_id x), fp16 wherever the reference stores fp16."""
+    t, h = x.shape
+    ne, n13, _ = q13.shape
+    inter = n13 // 2
+    w13 = np.stack([_dequant_by_repeat(s, q13[e], s13[e], (n13, h)) for e in range(ne)]).astype(np.float16)
+    w2 = np.stack([_dequant_by_repeat(s, q2[e], s2[e], (h, inter)) for e in range(ne)]).astype(np.float16)
+    out = np.zeros((t, h), np.float16)
+    for ti in range(t):
+        lg = logits[ti].astype(np.float64)
+        order = sorted(range(ne), key=lambda e: (-lg[e], e))[:top_k]
+        p = np.exp(lg[order] - lg[order].max())
+        wts = (p / p.sum()).astype(np.float16)
+        acc = None
+        for j, e in enumerate(order):
+            y13 = (w13[e].astype(np.float64) @ x[ti].astype(np.float64)).astype(np.float16)
+            g64 = y13[:inter].astype(np.float64)
+            act = (g64 / (1.0 + np.exp(-g64))).astype(np.float16)
+            a = (act.astype(np.float64) * y13[inter:].astype(np.float64)).astype(np.float16)
+            y2 = (w2[e].astype(np.float64) @ a.astype(np.float64)).astype(np.float16)
+            term = (wts[j].astype(np.float64) * y2.astype(np.float64)).astype(np.float16)
+            acc = term if acc is None else (acc.astype(np.float64) + term.astype(np.float64)).astype(np.float16)
+        out[ti] = acc
+    return out
+
+
+@pytest.mark.parametrize("t", [1, 2, 3, 9, 40])
+def test_mixtral_moe_against_dense_bruteforce(t):
+    rng = np.random.default_rng(41 + t)
+    ne, h, inter, top_k = 8, 64, 96, 2
+    w13 = (rng.standard_normal((ne, 2 * inter, h)) * 0.2).astype(np.float16)
+    w2 = (rng.standard_normal((ne, h, inter)) * 0.2).astype(np.float16)
+    q13, s13 = o.quantize(w13, Q4)
+    q2, s2 = o.quantize(w2, Q4)
+    x = rng.standard_normal((t, h)).astype(np.float16)
+    logits = rng.standard_normal((t, ne)).astype(np.float16)
+    if t >= 3:
+        logits[1] = logits[0]  # two tokens with the same experts, in order
+        logits[2, :] = 0.5     # a full tie: experts 0 and 1
+    got = o.mixtral_moe(x, logits, q13, s13, q2, s2, Q4, top_k)
+    want = _dense_moe_bruteforce(x, logits, q13, s13, q2, s2, Q4, top_k)
+    # rounding points are the same; the fp32 softmax / silu of the oracle may differ from float64 by a unit in
+    # rare places, which the second matmul spreads: a few units at most, nothing like a wrong index or order
+    d = _ulp16_diff(got, want)
+    scale = np.abs(want.astype(np.float64)).max()
+    assert np.abs(got.astype(np.float64) - want.astype(np.float64)).max() <= 4e-3 * scale
+    assert (d <= 1).mean() > 0.98
+    # the same check must reject a swapped weight order and a shifted scatter
+    ids = o.gating_softmax_topk(logits, top_k)[1]
+    if t > 1 and len(np.unique(ids)) > 2:
+        wrong = o.mixtral_moe(x[::-1].copy(), logits, q13, s13, q2, s2, Q4, top_k)
+        assert np.abs(wrong.astype(np.float64) - want.astype(np.float64)).max() > 0.05 * scale
+
+
+@pytest.mark.parametrize("md", ["float32", "bfloat16"])
+def test_mixtral_moe_dt_against_dense_bruteforce(md):
+    rng = np.random.default_rng(43)
+    ne, h, inter, top_k = 4, 64, 64, 2
+    for t in (1, 7):
+        w13 = o.round_to((rng.standard_normal((ne, 2 * inter, h)) * 0.2).astype(np.float32), md)
+        w2 = o.round_to((rng.standard_normal((ne, h, inter)) * 0.2).astype(np.float32), md)
+        q13, s13 = o.quantize_dt(w13, Q4, md)
+        q2, s2 = o.quantize_dt(w2, Q4, md)
+        x = o.round_to(rng.standard_normal((t, h)).astype(np.float32), md)
+        logits = o.round_to(rng.standard_normal((t, ne)).astype(np.float32), md)
+        got = o.mixtral_moe_dt(x, logits, q13, s13, q2, s2, Q4, md, top_k)
+        r = lambda a: o.round_to(np.asarray(a, np.float64).astype(np.float32), md).astype(np.float64)
+        d13 = np.stack([r((o.unpack(q13[e], Q4, h).astype(np.float64) - 7) * np.repeat(s13[e].astype(np.float64), 32, -1))
+                        for e in range(ne)])
+        d2 = np.stack([r((o.unpack(q2[e], Q4, inter).astype(np.float64) - 7) * np.repeat(s2[e].astype(np.float64), 32, -1))
+                       for e in range(ne)])
+        want = np.zeros((t, h))
+        for ti in range(t):
+            lg = logits[ti].astype(np.float64)
+            order = sorted(range(ne), key=lambda e: (-lg[e], e))[:top_k]
+            p = np.exp(lg[order] - lg[order].max())
+            wts = r(p / p.sum())
+            acc = None
+            for j, e in enumerate(order):
+                y13 = r(d13[e] @ x[ti].astype(np.float64))
+                a = r(r(y13[:inter] / (1.0 + np.exp(-y13[:inter]))) * y13[inter:])
+                term = r(wts[j] * r(d2[e] @ a))
+                acc = term if acc is None else r(acc + term)
+            want[ti] = acc
+        scale = np.abs(want).max()
+        tol = {"float32": 2e-5, "bfloat16": 3e-2}[md]
+        assert np.abs(got.astype(np.float64) - want).max() <= tol * scale
+
+
+def test_gating_topk_and_full_softmax_branch_brute_force():
+    # moe_misc.py:63-132 and :234-235 (norm_topk_prob=False): softmax over all experts in fp32, cast to the
+    # model dtype, then top-k of the ROUNDED scores with ties to the lower index
+    rng = np.random.default_rng(47)
+    t, ne, k = 64, 8, 2
+    logits = rng.standard_normal((t, ne)).astype(np.float16)
+    logits[5, :] = 1.0                      # all equal: scores all 1/8, experts 0, 1
+    logits[6, [2, 6]] = 3.0                 # an exact tie at the top: 2 before 6
+    logits[7] = np.array([0, 0, 0, 0, 0, 0, 0, 9], np.float16)
+    w, ids = o.gating_softmax_topk_full(logits, k)
+    assert ids[5].tolist() == [0, 1] and float(w[5, 0]) == 0.125 and float(w[5, 1]) == 0.125
+    assert ids[6].tolist() == [2, 6] and w[6, 0] == w[6, 1]
+    assert ids[7, 0] == 7
+    p = np.exp(logits.astype(np.float64) - logits.astype(np.float64).max(-1, keepdims=True))
+    p = p / p.sum(-1, keepdims=True)
+    p16 = p.astype(np.float16)
+    assert _ulp16_diff(o.softmax_fp32(logits.astype(np.float32)).astype(np.float16), p16).max() <= 1
+    for r in range(t):
+        s16 = o.softmax_fp32(logits[r: r + 1].astype(np.float32)).astype(np.float16)[0]
+        order = sorted(range(ne), key=lambda e: (-float(s16[e]), e))[:k]
+        assert ids[r].tolist() == order            # top-k of the rounded scores, ties to the lower index
+        assert (w[r] == s16[order]).all()          # and the scores are returned as they are (no renormalisation)
+        assert abs(float(w[r].astype(np.float64).sum())) <= 1.0 + 1e-3
+    # unlike the norm_topk_prob=True branch the weights do not sum to one
+    w_norm, ids_norm = o.gating_softmax_topk(logits, k)
+    assert (ids_norm[8:] == ids[8:]).mean() > 0.95  # same experts away from rounding ties
+    assert (w.astype(np.float32).sum(-1)[8:] < w_norm.astype(np.float32).sum(-1)[8:] - 0.05).all()
+    # gating_topk alone: scores pass through unchanged
+    sc = rng.random((5, 6)).astype(np.float16)
+    v, i = o.gating_topk(sc, 3)
+    for r in range(5):
+        order = sorted(range(6), key=lambda e: (-float(sc[r, e]), e))[:3]
+        assert i[r].tolist() == order and (v[r] == sc[r, order]).all()

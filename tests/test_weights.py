@@ -281,7 +281,113 @@ def test_convert_weight_unquantised_on_cpu(tmp_path):
     assert json.load(open(os.path.join(dst, "mlc-chat-config.json")))["quantization"] == "q0f16"
 
 
+def test_param_kind_and_scheme_flags_on_cpu(tmp_path, monkeypatch):
+    """Names, shapes and dtypes of a converted directory for the schemes that differ from q4f16_1 in layout or in
+    what they leave alone: q4f16_0 (KN: a Linear's words and scales transposed), q4f16_2 (embedding and final fc
+    stay in floating point), q4bf16_1 (everything in bfloat16).  The packing itself is the GPU kernel's job (checked
+    bit for bit in the gpu tests below); here the oracle stands in for it so that the host logic runs without one."""
+    from mlc_llm_amd import ops
+
+    assert loader.param_kind("model.embed_tokens.weight") == "embedding"
+    assert loader.param_kind("transformer.embd.weight") == "embedding"
+    assert loader.param_kind("lm_head.weight") == "final_fc"
+    assert loader.param_kind("model.layers.3.moe.e1_e3.weight") == "experts"
+    assert loader.param_kind("model.layers.3.moe.e2.weight") == "experts"
+    assert loader.param_kind("model.layers.3.mlp.down_proj.weight") == "linear"
+    assert loader.param_kind("model.layers.0.self_attn.c_attn.weight") == "linear"
+
+    def fake_quantize(w, bits, group_size, round_mode=0):
+        md = {torch.float16: "float16", torch.float32: "float32", torch.bfloat16: "bfloat16"}[w.dtype]
+        qw, qs = o.quantize_dt(w.float().numpy(), o.SCHEMES["q4f16_1" if bits == 4 else "q3f16_1"], md)
+        return torch.from_numpy(qw.view(np.int32)), torch.from_numpy(qs).to(w.dtype)
+
+    monkeypatch.setattr(ops, "quantize", fake_quantize)
+    src = str(tmp_path / "hf")
+    tensors = _hf_tensors(LLAMA, seed=9)
+    _write_checkpoint(src, LLAMA, tensors)
+    h, inter, v = LLAMA["hidden_size"], LLAMA["intermediate_size"], LLAMA["vocab_size"]
+
+    # q4f16_0: KN layout for every Linear (final fc included), embedding stays [vocab, words]
+    dst = str(tmp_path / "kn")
+    loader.convert_weight(src, dst, quantization="q4f16_0", device="cpu")
+    p, _ = tensor_cache.load_tensor_cache(dst)
+    assert tuple(p["model.layers.0.mlp.down_proj.q_weight"].shape) == (inter // 8, h)
+    assert tuple(p["model.layers.0.mlp.down_proj.q_scale"].shape) == (inter // 32, h)
+    assert tuple(p["model.layers.0.self_attn.qkv_proj.q_weight"].shape) == (h // 8, 2 * h)
+    assert tuple(p["lm_head.q_weight"].shape) == (h // 8, v) and tuple(p["lm_head.q_scale"].shape) == (h // 32, v)
+    assert tuple(p["model.embed_tokens.q_weight"].shape) == (v, h // 8)
+    nk, _ = o.quantize(tensors["model.layers.0.mlp.down_proj.weight"].numpy(), o.SCHEMES["q4f16_1"])
+    assert np.array_equal(p["model.layers.0.mlp.down_proj.q_weight"].numpy().view(np.uint32), nk.T)
+
+    # q4f16_2: embedding and final fc are left in float16 under their .weight names
+    dst = str(tmp_path / "f2")
+    loader.convert_weight(src, dst, quantization="q4f16_2", device="cpu")
+    p, _ = tensor_cache.load_tensor_cache(dst)
+    assert "model.embed_tokens.q_weight" not in p and "lm_head.q_weight" not in p
+    assert p["model.embed_tokens.weight"].dtype == torch.float16 and tuple(p["lm_head.weight"].shape) == (v, h)
+    assert torch.equal(p["lm_head.weight"], tensors["lm_head.weight"])
+    assert tuple(p["model.layers.1.mlp.gate_up_proj.q_weight"].shape) == (2 * inter, h // 8)
+
+    # q4bf16_1: norms and scales in bfloat16; values come straight from the checkpoint, not through float16
+    big = dict(tensors)
+    big["model.norm.weight"] = torch.full((h,), 1.0e5, dtype=torch.float32).bfloat16()  # overflows float16
+    src2 = str(tmp_path / "hf_bf16")
+    _write_checkpoint(src2, LLAMA, {k: (t if k == "model.norm.weight" else t.bfloat16()) for k, t in big.items()})
+    dst = str(tmp_path / "bf")
+    loader.convert_weight(src2, dst, quantization="q4bf16_1", device="cpu")
+    p, _ = tensor_cache.load_tensor_cache(dst)
+    assert p["model.norm.weight"].dtype == torch.bfloat16 and torch.isfinite(p["model.norm.weight"].float()).all()
+    assert float(p["model.norm.weight"][0]) == float(torch.tensor(1.0e5).bfloat16())
+    assert p["model.layers.0.mlp.down_proj.q_scale"].dtype == torch.bfloat16
+    qw, qs = o.quantize_dt(tensors["model.layers.0.mlp.down_proj.weight"].bfloat16().float().numpy(),
+                           o.SCHEMES["q4f16_1"], "bfloat16")
+    assert np.array_equal(p["model.layers.0.mlp.down_proj.q_weight"].numpy().view(np.uint32), qw)
+    assert np.array_equal(p["model.layers.0.mlp.down_proj.q_scale"].float().numpy(), qs)
+
+    # experts have no KN form (group_quantization.py:584-585)
+    srcm = str(tmp_path / "hf_mixtral")
+    _write_checkpoint(srcm, MIXTRAL, _hf_tensors(MIXTRAL, seed=2))
+    with pytest.raises(NotImplementedError, match="KN"):
+        loader.convert_weight(srcm, str(tmp_path / "mkn"), quantization="q4f16_0", device="cpu")
+
+
 # ------------------------------------------------------------------------------ on the GPU
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("scheme", ["q4bf16_1", "q4f32_1", "q4f16_0", "q4f16_2"])
+def test_convert_weight_other_schemes_match_oracle(tmp_path, scheme):
+    """The schemes beyond q4f16_1 / q3f16_1 through the real GPU quantizer: packed words and scales of every
+    quantised parameter equal the oracle's for the scheme's model dtype and layout, bit for bit."""
+    from mlc_llm_amd.quantization import QUANTIZATION
+
+    quant = QUANTIZATION[scheme]
+    md = quant.model_dtype
+    tdt = {"float16": torch.float16, "float32": torch.float32, "bfloat16": torch.bfloat16}[md]
+    src, dst = str(tmp_path / "hf"), str(tmp_path / "mlc")
+    tensors = {k: t.float().mul(1.37).to(tdt) for k, t in _hf_tensors(LLAMA, seed=21).items()}
+    _write_checkpoint(src, LLAMA, tensors, shards=2)
+    loader.convert_weight(src, dst, quantization=scheme, device="cuda:0")
+    params, _ = tensor_cache.load_tensor_cache(dst, device="cpu", verify_md5=True)
+    mapping, quantized = loader.llama_huggingface(LLAMA)
+    np_t = {k: v.float().numpy() for k, v in tensors.items()}
+    s = o.SCHEMES["q4f16_1"]
+    for name in mapping.param_map:
+        full = mapping.map_func[name](*[np_t[n] for n in mapping.param_map[name]])
+        kind = loader.param_kind(name)
+        kept = name not in quantized or (kind == "embedding" and not quant.quantize_embedding) or \
+            (kind == "final_fc" and not quant.quantize_final_fc)
+        if kept:
+            assert params[name].dtype == tdt and np.array_equal(params[name].float().numpy(), full), name
+            continue
+        base = name[: -len(".weight")]
+        qw, qs = o.quantize_dt(full, s, md)
+        if quant.linear_weight_layout == "KN" and kind in ("linear", "final_fc"):
+            qw, qs = qw.T, qs.T
+        assert np.array_equal(params[f"{base}.q_weight"].numpy().view(np.uint32), qw), name
+        assert params[f"{base}.q_scale"].dtype == tdt
+        assert np.array_equal(params[f"{base}.q_scale"].float().numpy(), qs), name
+
+
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("scheme", ["q4f16_1", "q3f16_1"])
