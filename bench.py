@@ -142,15 +142,33 @@ def main() -> int:
     from oracle import gq_oracle as o
 
     s4 = o.SCHEMES["q4f16_1"]
-    qw0, qs0 = layers[0]["o_proj"]
-    qw0_h, qs0_h = qw0.cpu().numpy().view(np.uint32), qs0.cpu().numpy()
     x1_h = x_in[4096][:1].cpu().numpy()
-    run_linear("o_proj", qw0, qs0, 1, outs["o_proj"])
-    err, bound, rel = o.check_linear(outs["o_proj"][:1].float().cpu().numpy(),
-                                     o.linear_fp32(x1_h, qw0_h, qs0_h, s4), x1_h, 4096)
-    if not (err <= bound and rel <= 2e-3):
-        sys.stderr.write(f"parity check failed before timing: err {err} bound {bound} rel {rel}\n")
-        return 1
+
+    def sampled_parity(what, y, x, qw, qs, scheme, cols=384, rows=12):
+        """y [M, N] against the oracle on sampled weight rows (first, last, tile edges, random) and sampled
+        activation rows; the packed words and scales are copied from the tensors the kernel read."""
+        rng = np.random.default_rng(len(what) + qw.shape[0])
+        n, m = qw.shape[0], x.shape[0]
+        ci = np.unique(np.concatenate([[0, 1, 127, 128, 255, 256, n // 2, n - 2, n - 1], rng.integers(0, n, cols)]))
+        ri = np.arange(m) if m <= rows else np.unique(np.concatenate([[0, 1, 31, 32, 127, 128, 255, 256, m - 1],
+                                                                      rng.integers(0, m, rows)]))
+        ri = ri[ri < m]
+        ct, rt = torch.from_numpy(ci).to(dev), torch.from_numpy(ri).to(dev)
+        x_h = x[rt].cpu().numpy()
+        ref = o.linear_fp32(x_h, qw[ct].cpu().numpy().view(np.uint32), qs[ct].cpu().numpy(), scheme)
+        err, bound, rel = o.check_linear(y[rt][:, ct].float().cpu().numpy(), ref, x_h, x.shape[1])
+        if not (err <= bound and rel <= 2e-3):
+            raise SystemExit(f"parity check failed before timing ({what}): err {err} bound {bound} rel {rel}")
+
+    # every shape the step runs, at every batch the extras time, before anything is timed
+    for name, (n, k) in list(SHAPES.items()) + [("lm_head", LM_HEAD)]:
+        qw_, qs_ = lm_head if name == "lm_head" else layers[0][name]
+        out_ = out_lm if name == "lm_head" else outs[name]
+        for b in (1, 4, 8):
+            run_linear(name, qw_, qs_, b, out_)
+            sampled_parity(f"{name} B={b}", out_[:b], x_in[k][:b], qw_, qs_, s4)
+    run_linear("gate_up", *layers[0]["gate_up"], 1, outs["gate_up"])
+    dominant_kernel = gq._lib.last_kernel()  # the instantiation the dispatcher picked in this run
 
     # ---------------------------------------------------------------- timed region: K decode steps
     def timed(fn, iters, warmup, use_graph):
@@ -214,9 +232,11 @@ def main() -> int:
     us_read = timed(read_sweep, max(5, args.steps), 2, use_graph) * 1e3 / LAYERS
     read_bytes = layers[0]["gate_up"][0].numel() * 4 + layers[0]["gate_up"][1].numel() * 2
     roofline = {
-        "bound": "hbm", "kernel": "gq::gemv_reg_kernel<4,1,2,2,0,false> (gate_up 28672x4096, batch 1)",
+        "bound": "hbm", "kernel": f"{dominant_kernel} (gate_up 28672x4096, batch 1)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+        "traffic_source": "profiles/gemv_gate_up_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
+                          "command, scaled by a 256 MiB device copy in the same runs)",
         "bytes_per_launch": gu_bytes, "us_per_launch": round(us_gate_up, 3),
         "read_only_probe": {"what": "plain 128-bit streaming read of the same weight and scale tensors, one launch each",
                             "us_per_launch": round(us_read, 3),
@@ -255,6 +275,8 @@ def main() -> int:
 
             def call(qw=qw, qs=qs, k=k, ym=ym):
                 ops.linear(xm[k], qw, qs, BITS, G, None, torch.float16, ym)
+            call()
+            sampled_parity(f"{name} M={m}", ym, xm[k], qw, qs, s4, cols=256, rows=16)
             ms = timed(call, 20, 8, False)  # (the first launches of a process run 5-30 % slow while clocks settle)
             tf = 2.0 * m * n * k / (ms * 1e-3) / 1e12
             gemm[f"{name}_m{m}"] = {"us": round(ms * 1e3, 1), "TFLOP/s": round(tf, 1),

@@ -126,6 +126,20 @@ MI355GQ_API int mi355gq_linear(const void* x, const void* q_weight, const void* 
                    void* y, void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream);
 
 /*
+ * mi355gq_linear for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose VM allocates workspaces
+ * itself.  Same arguments and results as mi355gq_linear without the workspace: the split-K partial sums of the
+ * few-row GEMM go to a device array inside the library (mi355gq_linear_static_scratch_max_bytes() = 32 MiB, held
+ * by every GPU the library runs on until the process ends), so the call allocates nothing.  Shapes whose split
+ * would want more return MI355GQ_ERR_WORKSPACE (nothing is launched).  All calls on one GPU share the array:
+ * calls that overlap on one GPU (different streams, different threads) race on it; stream-ordered calls do not.
+ */
+MI355GQ_API int64_t mi355gq_linear_static_scratch_max_bytes(void);
+MI355GQ_API int mi355gq_linear_static_scratch(const void* x, const void* q_weight, const void* q_scale,
+                                  const void* bias, int64_t M, int64_t N, int64_t K, int bits, int group_size,
+                                  int out_dtype, void* y, mi355gq_stream_t stream);
+
+/*
  * The same linear with the element-wise tail the reference folds into the matmul kernel:
  * FuseDequantizeMatmulEwise (compiler_pass/fuse_dequantize_matmul_ewise.py:19-32) fuses the
  * dequantize + matmul pair together with up to three element-wise operands that operator fusion

@@ -18,6 +18,15 @@ Options& options() {
   return o;
 }
 
+static thread_local char g_last_kernel[160] = "";
+
+void note_kernel(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_kernel, sizeof(g_last_kernel), fmt, ap);
+  va_end(ap);
+}
+
 hipError_t allow_large_lds(const void* kernel) {
   constexpr int kMaxDevices = 64, kSlots = 512;
   static std::mutex mu;
@@ -131,6 +140,8 @@ int mi355gq_check_device(void) {
                 prop.gcnArchName);
   return MI355GQ_OK;
 }
+
+const char* mi355gq_testing_last_kernel(void) { return gq::g_last_kernel; }
 
 int mi355gq_testing_set_option(const char* name, int value) {
   GQ_REQUIRE(name != nullptr, "option name is null");
@@ -428,6 +439,49 @@ int mi355gq_linear(const void* x, const void* q_weight, const void* q_scale, con
                    void* y, void* workspace, int64_t workspace_bytes, mi355gq_stream_t stream) {
   return linear_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, out_dtype, y,
                      workspace, workspace_bytes, stream);
+}
+
+// ---- the linear for callers that cannot allocate: split-K partial sums in a device array of the library's own
+constexpr int64_t kStaticScratchBytes = int64_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// The array's device address on the current device (each GPU holds its own copy at its own address), looked up
+// once per device.  In host code `scratch` is only a handle for this lookup, never an address.
+static int static_scratch_ptr(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* ptrs[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_result(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(MI355GQ_ERR_UNSUPPORTED, "linear_static_scratch: device %d", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_result(e, "hipGetSymbolAddress(scratch)");
+    if (p == nullptr) return fail(MI355GQ_ERR_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return MI355GQ_OK;
+}
+
+int64_t mi355gq_linear_static_scratch_max_bytes(void) { return kStaticScratchBytes; }
+
+int mi355gq_linear_static_scratch(const void* x, const void* q_weight, const void* q_scale, const void* bias,
+                                  int64_t M, int64_t N, int64_t K, int bits, int group_size, int out_dtype,
+                                  void* y, mi355gq_stream_t stream) {
+  const int64_t need = mi355gq_linear_workspace_bytes(M, N, K, bits, group_size);
+  if (need > kStaticScratchBytes)
+    return fail(MI355GQ_ERR_WORKSPACE,
+                "linear_static_scratch: M=%lld N=%lld K=%lld wants %lld bytes of split-K partial sums, the library's "
+                "array holds %lld; call mi355gq_linear with a workspace of the caller's",
+                (long long)M, (long long)N, (long long)K, (long long)need, (long long)kStaticScratchBytes);
+  void* ws = nullptr;
+  if (need > 0) GQ_CHECK(static_scratch_ptr(&ws));
+  return linear_impl(x, q_weight, q_scale, bias, nullptr, M, N, K, bits, group_size, out_dtype, y, ws,
+                     ws ? kStaticScratchBytes : 0, stream);
 }
 
 int mi355gq_linear_residual(const void* x, const void* q_weight, const void* q_scale,

@@ -193,6 +193,7 @@ static hipError_t launch_cfg(const GemmParams& p, hipStream_t s) {
   }
   const int m_tiles = p.indptr ? (p.rows + BM - 1) / BM + p.num_experts : (p.rows + BM - 1) / BM;
   const dim3 grid((p.N + BN - 1) / BN, m_tiles);
+  note_kernel("gq::gemm_kernel<%d,%d,%d,%d,%d>", BITS, BM, BN, WM, WN);
   hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
   return hipGetLastError();
 }

@@ -309,6 +309,7 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr int PB = ((WN / 32) % 2 == 0) ? 32 : 16;
   const int n_cols = p.paired ? ((p.N / 2 + PB - 1) / PB) * 2 * PB : p.N;
   const dim3 grid((n_cols + BN - 1) / BN, m_tiles, split);
+  note_kernel("gq::gemm_pipe_kernel<%d,%d,%d,%d,%d,%d,%s>", BITS, BM, BN, WM, WN, DEPTH, BF ? "true" : "false");
   hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
   return hipGetLastError();
 }

@@ -198,6 +198,7 @@ static hipError_t launch_one(const GemvParams& p, int slots, hipStream_t s) {
   using T = GemvTraits<BITS>;
   const size_t lds = static_cast<size_t>(NB) * p.gc * (T::CH * 16 + 4);
   const dim3 grid((p.N + 4 * R - 1) / (4 * R), slots);
+  note_kernel("gq::gemv_dot2_kernel<%d,%d,%d>", BITS, NB, R);
   hipLaunchKernelGGL((gemv_dot2_kernel<BITS, NB, R>), grid, dim3(256), lds, s, p);
   return hipGetLastError();
 }

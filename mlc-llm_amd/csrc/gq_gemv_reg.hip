@@ -242,6 +242,8 @@ static hipError_t launch_k(const GemvParams& p, int slots, int blocks, int nsets
   const int threads = 256;
   const size_t lds = static_cast<size_t>(NB) * p.ng * GemvTraits<BITS>::G * 2;
   const dim3 grid(blocks, slots);
+  note_kernel("gq::gemv_reg_kernel<%d,%d,%d,%d,%d,%s>", BITS, NB, R, ITERS,
+              p.paired ? 2 : ((p.bias != nullptr || p.residual != nullptr) ? 1 : 0), p.bf16 ? "true" : "false");
   if (p.bf16) {
     if (p.paired) {
       if constexpr (R % 2 == 0)

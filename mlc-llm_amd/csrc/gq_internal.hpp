@@ -19,6 +19,10 @@ struct Options {
 };
 Options& options();
 
+// Records which kernel instantiation the calling thread launched last (thread-local text, read back through the
+// test hook mi355gq_testing_last_kernel): measurement code names the kernel it timed from the run itself.
+void note_kernel(const char* fmt, ...);
+
 // hipFuncAttributeMaxDynamicSharedMemorySize = the CU's whole LDS, set once per (kernel, device) and remembered;
 // kernels whose dynamic LDS may exceed 64 KiB call it before launching.
 hipError_t allow_large_lds(const void* kernel);

@@ -408,6 +408,7 @@ static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads,
     const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF>));
     if (e != hipSuccess) return e;
   }
+  note_kernel("gq::quad_kernel<%d,%d,%d,%d,%s>", BITS, NBQ, U, MODE, BF ? "true" : "false");
   hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF>), grid, dim3(threads), lds, s, p);
   return hipGetLastError();
 }

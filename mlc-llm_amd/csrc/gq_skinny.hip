@@ -614,6 +614,7 @@ static hipError_t launch_skinny_cfg(const SkinnyParams& p, int experts, int mtil
   constexpr size_t lds = lds_x > lds_red ? lds_x : lds_red;
   static_assert(lds <= 65536, "LDS budget");
   const dim3 grid((p.N + 16 * RT - 1) / (16 * RT), experts, mtiles);
+  note_kernel(pipelined ? "gq::skinny_q4_kernel<%d,%d>" : "gq::skinny_q4_simple_kernel<%d,%d>", MR, RT);
   if (pipelined) hipLaunchKernelGGL((skinny_q4_kernel<MR, RT>), grid, dim3(256), lds, s, p);
   else hipLaunchKernelGGL((skinny_q4_simple_kernel<MR, RT>), grid, dim3(256), lds, s, p);
   return hipGetLastError();
@@ -661,6 +662,7 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s) {
           const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
           if (e != hipSuccess) return e;
         }
+        note_kernel("gq::skinny_q4_persist_kernel<%d>", mr);
         hipLaunchKernelGGL(kern, grid, dim3(64 * wpb), lds_p, s, p, ntiles, nblk);
         return hipGetLastError();
       };

@@ -17,6 +17,10 @@ extern "C" {
 
 __attribute__((visibility("default"))) int mi355gq_testing_set_option(const char* name, int value);
 
+/* Name and template arguments of the kernel the calling thread's last matmul call launched ("" before any),
+ * e.g. "gq::gemv_reg_kernel<4,1,2,2,0,false>": lets a benchmark label its timings from the run. */
+__attribute__((visibility("default"))) const char* mi355gq_testing_last_kernel(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,8 @@ SIGNATURES = {
     "mi355gq_embedding_take": (_I, [_P, _L, _P, _P, _L, _L, _I, _I, _P, _P]),
     "mi355gq_linear_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
     "mi355gq_linear": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
+    "mi355gq_linear_static_scratch_max_bytes": (_L, []),
+    "mi355gq_linear_static_scratch": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P]),
     "mi355gq_linear_residual": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_linear_silu_mul_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
     "mi355gq_linear_silu_mul": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P, _P, _L, _P]),
@@ -81,6 +83,7 @@ SIGNATURES = {
 # exported for tests and tuning sweeps only (csrc/gq_testing.h); not declared in the public header
 TEST_HOOKS = {
     "mi355gq_testing_set_option": (_I, [c_char_p, _I]),
+    "mi355gq_testing_last_kernel": (c_char_p, []),
 }
 
 
@@ -127,6 +130,11 @@ def call(name: str, *args) -> None:
     rc = getattr(handle, name)(*args)
     if rc != OK:
         raise Mi355gqError(name, rc, handle.mi355gq_last_error().decode("utf-8", "replace"))
+
+
+def last_kernel() -> str:
+    """Test / measurement hook: the kernel instantiation this thread's last matmul call launched."""
+    return lib().mi355gq_testing_last_kernel().decode()
 
 
 def set_option(name: str, value: int) -> None:

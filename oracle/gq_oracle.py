@@ -524,27 +524,32 @@ def mixtral_moe_dt(x, gate_logits, w13, s13, w2, s2, scheme: Scheme, model_dtype
     return out
 
 
-def mixtral_moe(x, gate_logits, w13, s13, w2, s2, scheme: Scheme, top_k: int = 2):
+def mixtral_moe(x, gate_logits, w13, s13, w2, s2, scheme: Scheme, top_k: int = 2, gemv=None, group_gemm=None):
     """MixtralMoE.forward (mixtral_model.py:64-117) given the router logits.
 
     Expert matmuls are evaluated exactly (float64) and rounded to fp16 where the
     reference stores fp16 tensors; elementwise glue is fp16.  Returns fp16 [T, H].
+    gemv / group_gemm: other evaluations of the two expert matmuls with the signatures of
+    moe_dequantize_gemv_fp32 / dequantize_group_gemm_fp32 (the C restatement, for shapes
+    numpy takes minutes on); the composition around them stays this one.
     """
+    gemv = moe_dequantize_gemv_fp32 if gemv is None else gemv
+    group_gemm = dequantize_group_gemm_fp32 if group_gemm is None else group_gemm
     t, hdim = x.shape
     ne = w13.shape[0]
     weights, ids = gating_softmax_topk(gate_logits, top_k)
     if t == 1:
-        y = moe_dequantize_gemv_fp32(x, w13, s13, ids, scheme).astype(F16)
+        y = gemv(x, w13, s13, ids, scheme).astype(F16)
         y = silu_mul_f16(y)
-        y = moe_dequantize_gemv_fp32(y, w2, s2, ids, scheme).astype(F16)
+        y = gemv(y, w2, s2, ids, scheme).astype(F16)
     else:
         cs = moe_cumsum(ids, ne)
         rev, tok = get_indices(cs, ids)
         indptr = get_indptr(cs, ne, t, inclusive=False)
         xs = x[tok]
-        y = dequantize_group_gemm_fp32(xs, w13, s13, indptr, scheme).astype(F16)
+        y = group_gemm(xs, w13, s13, indptr, scheme).astype(F16)
         y = silu_mul_f16(y)
-        y = dequantize_group_gemm_fp32(y, w2, s2, indptr, scheme).astype(F16)
+        y = group_gemm(y, w2, s2, indptr, scheme).astype(F16)
         y = scatter_output(y, rev)
     y = (y.reshape(t, top_k, hdim) * weights.reshape(t, top_k, 1)).astype(F16)
     out = y[:, 0]

@@ -573,28 +573,7 @@ def test_gemm_prefill_shape_and_gemv_agreement():
     assert_linear_ok(y32, o.linear_fp32(x, qw, qs, s), x, 4096, "gemm fp32 out")
 
 
-@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
-@pytest.mark.parametrize("n,k", [(28672, 4096), (4096, 14336)])
-def test_every_row_regime_agrees_at_full_size(name, n, k):
-    """gate_up and down_proj at their real sizes: the same activation row through every regime of the dispatcher
-    (1 .. 2048 rows) must give the product with the dequantised matrix (itself bit-exact against the oracle in
-    the tests above), within the matmul tolerance."""
-    s = SCHEMES[name]
-    g = torch.Generator(device=DEV).manual_seed(n + k)
-    w = (torch.randn((n, k), generator=g, device=DEV) * 0.02).half()
-    qw, qs = ops.quantize(w, s.bits, s.group_size)
-    del w
-    wd = ops.dequantize(qw, qs, k, s.bits, s.group_size).double()
-    x = torch.randn((2048, k), generator=g, device=DEV).half()
-    ref = x[:3].double() @ wd.t()  # rows 0, 1 and 2 of every batch below
-    del wd
-    tol = 1e-2 * float(x[:3].float().abs().max()) * np.sqrt(k) / 64
-    for m in (1, 2, 3, 4, 8, 9, 16, 17, 32, 64, 128, 256, 300, 1024, 2048):
-        y = ops.linear(x[:m].contiguous(), qw, qs, s.bits, s.group_size)
-        rows = min(m, 3)
-        err = (y[:rows].double() - ref[:rows]).abs().max().item()
-        rel = ((y[:rows].double() - ref[:rows]).norm() / ref[:rows].norm()).item()
-        assert err <= tol and rel <= 2e-3, f"{name} {n}x{k} M={m}: max err {err:.3e} (tol {tol:.3e}), rel-L2 {rel:.2e}"
+# (float16 models at full size, every row regime against the oracle: tests/test_gpu_baseline_configs.py)
 
 
 @pytest.mark.parametrize("n,k", [(28672, 4096), (4096, 14336)])
@@ -1704,3 +1683,81 @@ def test_c_abi_from_plain_c():
     r = subprocess.run([exe], capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, f"exit {r.returncode}\n{r.stdout}\n{r.stderr}"
     assert "c_abi_check ok" in r.stdout
+
+
+# ------------------------------------------------------------------ tiny K, gating_topk, norm_topk_prob=False
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("k", [1, 3, 7, 8, 9])
+@pytest.mark.parametrize("m", [1, 2, 5])
+def test_linear_tiny_k(name, k, m):
+    # fewer than 8 halves per activation row: the register GEMV (whole 16-byte loads of x) must decline
+    s = SCHEMES[name]
+    x, qw, qs, b = _linear_case(s, m, 24, k, 31 * k + m, bias=True)
+    xd = torch.empty(m * k + 64, dtype=torch.float16, device=DEV)[: m * k].view(m, k)  # no slack behind x
+    xd.copy_(dev(x))
+    y = ops.linear(xd, dev(qw), dev(qs), s.bits, s.group_size, dev(b))
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"tiny K {name} k={k} m={m}")
+
+
+def _ulp16(a, b):
+    def line(v):
+        u = np.asarray(v, np.float16).view(np.uint16).astype(np.int64)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(line(a) - line(b))
+
+
+@pytest.mark.parametrize("t,ne,k", [(1, 8, 2), (16, 8, 2), (512, 8, 2), (70, 64, 6), (33, 6, 3), (5, 200, 8)])
+def test_gating_topk_bit_exact(t, ne, k):
+    # moe_misc.py:63-132: scores pass through, ties keep the lower index
+    rng = np.random.default_rng(seed_of("topk", t, ne, k))
+    sc = rng.random((t, ne)).astype(np.float16)
+    sc[0, :] = 0.5
+    if t > 2:
+        sc[2, ne // 2:] = sc[2, : ne - ne // 2]
+    v_ref, i_ref = o.gating_topk(sc, k)
+    v, i = ops.gating_topk(dev(sc), k)
+    assert np.array_equal(i.cpu().numpy(), i_ref)
+    assert np.array_equal(host_f16_bits(v), v_ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("t,ne,k", [(1, 8, 2), (16, 8, 2), (512, 8, 2), (70, 64, 6), (257, 60, 4)])
+def test_gating_softmax_topk_without_renormalisation(t, ne, k):
+    """norm_topk_prob=False (moe_misc.py:234-235): softmax over all experts in fp32, cast, top-k of the rounded
+    scores.  The device's exp differs from numpy's in the last place of fp32, which can move a score across an
+    fp16 rounding boundary (one unit) and with it a near tie; so: weights within one unit of the oracle's score of
+    the chosen expert, the choice a valid top-k of scores within one unit, and, on rows whose k + 1 best scores
+    lie more than three units apart, exactly the oracle's experts in the oracle's order."""
+    rng = np.random.default_rng(seed_of("full", t, ne, k))
+    logits = rng.standard_normal((t, ne)).astype(np.float16)
+    logits[0, :] = 1.0          # exact ties are exact on both sides: 1 / ne each, experts 0 .. k-1
+    w_ref, i_ref = o.gating_softmax_topk_full(logits, k)
+    w, i = ops.gating_softmax_topk(dev(logits), k, norm_topk_prob=False)
+    w, i = w.cpu().numpy(), i.cpu().numpy()
+    assert i[0].tolist() == list(range(k)) and np.array_equal(w[0], w_ref[0])
+    p16 = o.softmax_fp32(logits.astype(np.float32)).astype(np.float16)
+    line = lambda v: int(np.float16(v).view(np.uint16))  # positive scores: the bit pattern is monotone
+    exact_rows = 0
+    for r in range(t):
+        chosen = i[r]
+        assert len(set(chosen.tolist())) == k
+        assert _ulp16(w[r], p16[r, chosen]).max() <= 1
+        rest = np.setdiff1d(np.arange(ne), chosen)
+        # nothing left out beats the last one chosen by more than the one-unit slack on either side
+        if rest.size:
+            assert max(line(p16[r, e]) for e in rest) <= line(w[r, -1]) + 2
+        assert all(line(w[r, j]) >= line(w[r, j + 1]) for j in range(k - 1))
+        top = np.sort(p16[r].astype(np.float64))[::-1][: k + 1]
+        bits = np.array([line(v) for v in top])
+        if (bits[:-1] - bits[1:] > 3).all():
+            exact_rows += 1
+            assert chosen.tolist() == i_ref[r].tolist(), r
+    assert exact_rows >= t // 2 or ne > 32
+    # the float32 / bfloat16 forms run the same kernel with their own rounding
+    for tdt, md in ((torch.float32, "float32"), (torch.bfloat16, "bfloat16")):
+        lg = torch.from_numpy(logits.astype(np.float32)).to(DEV).to(tdt)
+        w2, i2 = ops.gating_softmax_topk(lg, k, norm_topk_prob=False)
+        w2_ref, i2_ref = o.gating_softmax_topk_full(lg.float().cpu().numpy(), k, md)
+        same = (i2.cpu().numpy() == i2_ref).all(axis=1)
+        assert same.mean() >= (0.97 if md == "float32" else 0.8)
+        np.testing.assert_allclose(w2.float().cpu().numpy()[same], w2_ref[same], rtol=2.0 ** -7 if md == "bfloat16" else 1e-5)
