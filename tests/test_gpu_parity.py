@@ -1693,11 +1693,12 @@ def test_c_abi_from_plain_c():
 def test_linear_tiny_k(name, k, m):
     # fewer than 8 halves per activation row: the register GEMV (whole 16-byte loads of x) must decline
     s = SCHEMES[name]
-    x, qw, qs, b = _linear_case(s, m, 24, k, 31 * k + m, bias=True)
-    xd = torch.empty(m * k + 64, dtype=torch.float16, device=DEV)[: m * k].view(m, k)  # no slack behind x
+    # (no bias: the bound scales with sqrt(K) and would sit below the fp16 rounding of an O(1) output)
+    x, qw, qs, _ = _linear_case(s, m, 24, k, 31 * k + m)
+    xd = torch.empty(m * k + 64, dtype=torch.float16, device=DEV)[: m * k].view(m, k)
     xd.copy_(dev(x))
-    y = ops.linear(xd, dev(qw), dev(qs), s.bits, s.group_size, dev(b))
-    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"tiny K {name} k={k} m={m}")
+    y = ops.linear(xd, dev(qw), dev(qs), s.bits, s.group_size)
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s), x, k, f"tiny K {name} k={k} m={m}")
 
 
 def _ulp16(a, b):

@@ -371,13 +371,16 @@ def test_convert_weight_other_schemes_match_oracle(tmp_path, scheme):
     mapping, quantized = loader.llama_huggingface(LLAMA)
     np_t = {k: v.float().numpy() for k, v in tensors.items()}
     s = o.SCHEMES["q4f16_1"]
+    # float32 tensors are stored as their upper 16 bits ("f32-to-bf16", interface/convert_weight.py:182-196 of the
+    # reference): what comes back from the directory is that encoding of the exact value
+    on_disk = (lambda a: tensor_cache.bf16_to_f32(tensor_cache.f32_to_bf16(a))) if md == "float32" else (lambda a: a)
     for name in mapping.param_map:
         full = mapping.map_func[name](*[np_t[n] for n in mapping.param_map[name]])
         kind = loader.param_kind(name)
         kept = name not in quantized or (kind == "embedding" and not quant.quantize_embedding) or \
             (kind == "final_fc" and not quant.quantize_final_fc)
         if kept:
-            assert params[name].dtype == tdt and np.array_equal(params[name].float().numpy(), full), name
+            assert params[name].dtype == tdt and np.array_equal(params[name].float().numpy(), on_disk(full)), name
             continue
         base = name[: -len(".weight")]
         qw, qs = o.quantize_dt(full, s, md)
@@ -385,7 +388,7 @@ def test_convert_weight_other_schemes_match_oracle(tmp_path, scheme):
             qw, qs = qw.T, qs.T
         assert np.array_equal(params[f"{base}.q_weight"].numpy().view(np.uint32), qw), name
         assert params[f"{base}.q_scale"].dtype == tdt
-        assert np.array_equal(params[f"{base}.q_scale"].float().numpy(), qs), name
+        assert np.array_equal(params[f"{base}.q_scale"].float().numpy(), on_disk(qs)), name
 
 
 
