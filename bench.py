@@ -50,6 +50,79 @@ def gemv_bytes(n: int, k: int, b: int = 1) -> int:
     return n * 4 * ng * 4 + n * ng * 2 + b * k * 2 + b * n * 2
 
 
+def run_only(args, dev, gq, ops, torch, make_weight) -> int:
+    """One linear (or the Mixtral layer) over distinct weight copies: a short run for rocprofv3 counters."""
+    parts = args.only.split(":")
+    q3 = parts[0] == "q3"
+    if q3:
+        parts = parts[1:]
+    gx = torch.Generator(device=dev).manual_seed(1)
+
+    def timed_loop(fn, per_call):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (args.steps * per_call)
+
+    if parts[0] == "moe":
+        from mlc_llm_amd import QUANTIZATION
+        from mlc_llm_amd.nn import MixtralMoE
+
+        t = int(parts[1])
+        moe = MixtralMoE(4096, 14336, 8, 2, QUANTIZATION["q4f16_1"], device=dev)
+        for e in range(8):
+            g = torch.Generator(device=dev).manual_seed(7000 + e)
+            w13 = (torch.randn((28672, 4096), generator=g, device=dev) * 0.02).half()
+            moe.e1_e3.q_weight.data[e], moe.e1_e3.q_scale.data[e] = ops.quantize(w13, BITS, G)
+            w2 = (torch.randn((4096, 14336), generator=g, device=dev) * 0.02).half()
+            moe.e2.q_weight.data[e], moe.e2.q_scale.data[e] = ops.quantize(w2, BITS, G)
+            del w13, w2
+        xt = torch.randn((1, t, 4096), generator=gx, device=dev).half()
+        logits = torch.randn((t, 8), generator=torch.Generator(device=dev).manual_seed(2), device=dev).half()
+        us = timed_loop(lambda: moe(xt, logits), 1)
+        print(json.dumps({"only": args.only, "us_per_layer": round(us, 2), "steps": args.steps}))
+        return 0
+
+    name, rows = parts[0], int(parts[1])
+    shapes = dict(SHAPES, lm_head=LM_HEAD)
+    if q3:
+        shapes = {"qkv": (12288, 4096), "o_proj": (4096, 4096), "gate_up": (22016, 4096), "down": (4096, 11008)}
+    n, k = shapes[name]
+    bits, gsz = (3, 40) if q3 else (BITS, G)
+    ng = -(-k // gsz)
+    copies = max(2, min(32, int(1.2e9 // (n * ng * 18))))
+    ws = []
+    for c in range(copies):
+        g = torch.Generator(device=dev).manual_seed(100 + c)
+        w = (torch.randn((n, k), generator=g, device=dev) * 0.02).half()
+        ws.append(ops.quantize(w, bits, gsz))
+        del w
+    x = torch.randn((rows, k), generator=gx, device=dev).half()
+    y = torch.empty((rows, n), dtype=torch.float16, device=dev)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def sweep():
+        for qw, qs in ws:
+            ops.linear(x, qw, qs, bits, gsz, None, torch.float16, y)
+            if args.probe:
+                gq._lib.call("mi355gq_probe_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
+                             sink.data_ptr(), stream)
+
+    us = timed_loop(sweep, copies)
+    nbytes = n * 4 * ng * 4 + n * ng * 2 + rows * k * 2 + rows * n * 2
+    print(json.dumps({"only": args.only, "kernel": gq._lib.last_kernel(), "copies": copies,
+                      "us_per_launch" + ("_incl_probe" if args.probe else ""): round(us, 2),
+                      "algorithmic_bytes": nbytes, "flop": 2 * rows * n * k, "steps": args.steps}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -61,6 +134,12 @@ def main() -> int:
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the prefill GEMM (gate_up 28672x4096, M = 2048): the run the MFMA counters "
                          "under profiles/ are collected on")
+    ap.add_argument("--only", default=None, metavar="SHAPE:ROWS",
+                    help="time only one linear, e.g. gate_up:1, o_proj:8, down:2048 (SHAPE in qkv, o_proj, gate_up, "
+                         "down, lm_head; q3:SHAPE:ROWS for the q3f16_1 Llama-2-7B shapes; moe:T for the Mixtral layer) "
+                         "over distinct weight copies, plus the read-only probe on the same tensors with --probe: the "
+                         "runs the counter summaries under profiles/ are collected on")
+    ap.add_argument("--probe", action="store_true", help="with --only: also launch the read-only probe on each copy")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 256 MiB device copy (known bytes) so that a rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE run of this command can scale its counters")
@@ -91,6 +170,9 @@ def main() -> int:
         g = torch.Generator(device=dev).manual_seed(seed)
         w = (torch.randn((n, k), generator=g, device=dev, dtype=torch.float32) * 0.02).half()
         return ops.quantize(w, BITS, G)
+
+    if args.only:
+        return run_only(args, dev, gq, ops, torch, make_weight)
 
     if args.prefill_only:
         n, k, m = *SHAPES["gate_up"], 2048

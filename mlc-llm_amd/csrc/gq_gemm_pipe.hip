@@ -8,6 +8,8 @@
 //    flight instead of draining the queue at every join;
 //  * the MFMA fragments of k-step s+1 are read from LDS before the MFMAs of step s are issued.
 // Requires K % 8 == 0 (16-byte aligned activation rows); other K take the kernel in gq_gemm.hip.
+#include <type_traits>
+
 #include "gq_gemm_common.hpp"
 
 namespace gq {
@@ -15,7 +17,8 @@ namespace gq {
 // DEPTH: K tiles of global loads in flight (register stages); even, 2 for the large tiles, more
 // for few-row tiles whose MFMA work per tile is far shorter than a trip to memory
 // BF: bfloat16 model (operands and 16-bit outputs are bf16; see dequant_word4_bf16)
-template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false>
+// SKIP: waves leave out the 32-row blocks of their sub-tile that lie past the segment's last row
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(const GemmParams p) {
   using T = GemmTraits<BITS>;
   constexpr int G = T::G;
@@ -29,8 +32,11 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   constexpr int TM = WM / 32, TN = WN / 32;
   constexpr int A_CHUNKS = (BM * CPR + NT - 1) / NT;  // the last round may cover part of the threads only
   constexpr bool A_EXACT = BM * CPR % NT == 0;
-  constexpr int W_GROUPS = BN * 2 / NT;
-  static_assert(BN * 2 % NT == 0, "tile / thread mismatch");
+  // groups of W per thread and K tile; a tile with fewer groups than threads (256 x 128) leaves the upper waves
+  // without any (W_ALL false: a wave-uniform test, every SIMD still hosts one wave that dequantises)
+  constexpr int W_GROUPS = BN * 2 >= NT ? BN * 2 / NT : 1;
+  constexpr bool W_ALL = BN * 2 >= NT;
+  static_assert(BN * 2 % NT == 0 || BN * 2 * 2 == NT, "tile / thread mismatch");
 
   extern __shared__ uint4 smem[];
   uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
@@ -38,12 +44,16 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   auto w_tile = [&](int s) { return lds + s * (BM + BN) * LDA + BM * LDA; };
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
+  const bool w_active = W_ALL || tid < BN * 2;  // (wave-uniform)
 
   int seg_lo, seg_hi, mt, expert;
   if (!locate_tile<BM>(p, blockIdx.y, seg_lo, seg_hi, mt, expert)) return;  // uniform
   const int m0 = seg_lo + mt * BM;
+  // 32-row blocks of this wave that hold rows of the segment: the others are skipped by the matrix core
+  // (SKIP; a ragged expert segment or a last row tile leaves most of a tall tile empty)
+  const int live = SKIP ? min(TM, max(0, (seg_hi - (m0 + wm0) + 31) / 32)) : TM;
   const int n0 = blockIdx.x * BN;
   const uint32_t* qw = p.qw + expert * p.expert_w_stride;
   const uint16_t* qs = p.qs + expert * p.expert_s_stride;
@@ -71,7 +81,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   int w_dst[W_GROUPS];
 #pragma unroll
   for (int i = 0; i < W_GROUPS; ++i) {
-    const int idx = tid + NT * i;
+    const int idx = w_active ? tid + NT * i : 0;
     const int r = idx >> 1, gsel = idx & 1;
     int row = min(n0 + r, p.N - 1);  // rows past N are computed and dropped
     if (p.paired) row = gate_up_row_blk<(TN % 2 == 0) ? 32 : 16>(n0 + r, p.N);
@@ -104,12 +114,14 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
       const bool ok = k_base + a_k[i] < k_lim;  // K % 8 == 0: a chunk is entirely inside or outside
       st.a[i] = *reinterpret_cast<const uint4*>(ok ? a_src[i] + k_base : a_src[i]);
     }
+    if (w_active) {
 #pragma unroll
-    for (int i = 0; i < W_GROUPS; ++i) {
-      const int g = 2 * kt + w_g[i];
-      const int gc = g < p.ng ? g : 0;
-      st.w[i] = *reinterpret_cast<const uint4*>(w_src[i] + 4 * gc);
-      st.s[i] = s_src[i][gc];
+      for (int i = 0; i < W_GROUPS; ++i) {
+        const int g = 2 * kt + w_g[i];
+        const int gc = g < p.ng ? g : 0;
+        st.w[i] = *reinterpret_cast<const uint4*>(w_src[i] + 4 * gc);
+        st.s[i] = s_src[i][gc];
+      }
     }
   };
   // One of KSTEPS slices of "tile kt: registers -> LDS stage s".  The slices are issued between the
@@ -126,6 +138,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
       if (A_EXACT || a_in_tile[i])
         *reinterpret_cast<uint4*>(at + a_dst[i]) = ok ? st.a[i] : make_uint4(0, 0, 0, 0);
     }
+    if (!w_active) return;
 #pragma unroll
     for (int i = 0; i < W_GROUPS; ++i) {
       const bool ok = 2 * kt + w_g[i] < g_lim;
@@ -167,36 +180,47 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
 
   const int frag_row = lane & 31, frag_k = 8 * (lane >> 5);
   // MFMAs of the tile in stage s; slice ks of the next tile's store is issued after k-step ks
-  auto mfma_tile = [&](int s, int kt_store, const Stage& st_store) {
+  // full: every 32-row block of the wave is live (the straight-line form); otherwise blocks >= live are skipped by
+  // wave-uniform branches, fragments and all
+  auto mfma_tile = [&](auto full, int s, int kt_store, const Stage& st_store) {
+    constexpr bool FULL = decltype(full)::value;
     const uint16_t* at = a_tile(s) + (wm0 + frag_row) * LDA + frag_k;
     const uint16_t* wt = w_tile(s) + (wn0 + frag_row) * LDA + frag_k;
     {  // fragments of k-step s+1 are read while the MFMAs of step s run
       half8_t af[2][TM], bf[2][TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA);
+      for (int i = 0; i < TM; ++i)
+        if (FULL || i < live) af[0][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA);
+      if (FULL || live > 0) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA);
+        for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA);
+      }
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
         const int cur = ks & 1, nxt = cur ^ 1;
         if (ks + 1 < KSTEPS) {
 #pragma unroll
           for (int i = 0; i < TM; ++i)
-            af[nxt][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA + (ks + 1) * 16);
+            if (FULL || i < live) af[nxt][i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA + (ks + 1) * 16);
+          if (FULL || live > 0) {
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            bf[nxt][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA + (ks + 1) * 16);
+            for (int j = 0; j < TN; ++j)
+              bf[nxt][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA + (ks + 1) * 16);
+          }
         }
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i) {
+          if (FULL || i < live) {
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            if constexpr (BF)
-              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[cur][i]),
-                                                                  __builtin_bit_cast(bf16x8_t, bf[cur][j]), acc[i][j],
-                                                                  0, 0, 0);
-            else
-              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TN; ++j)
+              if constexpr (BF)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[cur][i]),
+                                                                    __builtin_bit_cast(bf16x8_t, bf[cur][j]), acc[i][j],
+                                                                    0, 0, 0);
+              else
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+          }
+        }
         store_part(kt_store, st_store, s ^ 1, ks);
         __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
       }
@@ -212,14 +236,18 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   __syncthreads();
   // (a register stage is refilled right after the MFMA/store block that drains it; a tile past
   //  the end is stored as zeros and adds nothing)
-  for (int kt = kt0; kt < kt1; kt += DEPTH) {
+  auto k_loop = [&](auto full) {
+    for (int kt = kt0; kt < kt1; kt += DEPTH) {
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      mfma_tile(d & 1, kt + d + 1, r[(d + 1) % DEPTH]);
-      load_tile(kt + d + 1 + DEPTH, r[(d + 1) % DEPTH]);
-      __syncthreads();
+      for (int d = 0; d < DEPTH; ++d) {
+        mfma_tile(full, d & 1, kt + d + 1, r[(d + 1) % DEPTH]);
+        load_tile(kt + d + 1 + DEPTH, r[(d + 1) % DEPTH]);
+        __syncthreads();
+      }
     }
-  }
+  };
+  if (!SKIP || live == TM) k_loop(std::true_type{});
+  else k_loop(std::false_type{});
 
   // ---- epilogue: D[i][j] of a 32x32 tile sits in lane (j + 32*((i/4)%2)), register 4*(i/8) + i%4
   if (p.paired && p.partial == nullptr) {
@@ -292,12 +320,12 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   }
 }
 
-template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false>
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false>
 static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr int BK = 2 * GemmTraits<BITS>::G;
   constexpr int LDA = BK + 8;
   constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
-  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH, BF>;
+  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP>;
   if (lds > 65536) {
     const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
     if (e != hipSuccess) return e;
@@ -309,7 +337,8 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr int PB = ((WN / 32) % 2 == 0) ? 32 : 16;
   const int n_cols = p.paired ? ((p.N / 2 + PB - 1) / PB) * 2 * PB : p.N;
   const dim3 grid((n_cols + BN - 1) / BN, m_tiles, split);
-  note_kernel("gq::gemm_pipe_kernel<%d,%d,%d,%d,%d,%d,%s>", BITS, BM, BN, WM, WN, DEPTH, BF ? "true" : "false");
+  note_kernel("gq::gemm_pipe_kernel<%d,%d,%d,%d,%d,%d,%s,%s>", BITS, BM, BN, WM, WN, DEPTH, BF ? "true" : "false",
+              SKIP ? "true" : "false");
   hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
   return hipGetLastError();
 }
@@ -494,9 +523,22 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     if (p.bm_hint == 64) return launch_pipe_cfg<3, 64, 128, 32, 64, 4>(p, s);
     return launch_pipe_cfg<3, 128, 128, 64, 64>(p, s);
   }
+  // Grouped, from about 64 rows per expert on: 256-row tiles whose waves skip the 32-row blocks past the end of
+  // the expert's segment.  A ragged segment then costs its rows rounded up to 32 in matrix work, and the expert's
+  // weights are dequantised once per 256 rows instead of once per (often nearly empty) 128-row tile.  256 columns
+  // per tile while that still makes two workgroups per CU, else 128 (e2 of a Mixtral layer: 32 column tiles).
+  if (p.indptr != nullptr && ((variant < 0 && p.rows > 48 * p.num_experts) || variant == 10 || variant == 11)) {
+    const int64_t mt = p.rows / 256 + p.num_experts;
+    const bool wide = variant == 10 || (variant != 11 && bits == 4 && mt * ((p.N + 255) / 256) >= 512);
+    if (bits == 4) {
+      if (wide) return launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true>(p, s);
+      return launch_pipe_cfg<4, 256, 128, 64, 64, 2, false, true>(p, s);
+    }
+    return launch_pipe_cfg<3, 256, 128, 64, 64, 2, false, true>(p, s);
+  }
   if (bits == 4) {
     // grouped, few rows per expert: the tile height follows them (Mixtral layer, 8 experts: 144-384 routed
-    // rows 18-20 % faster than on 128-row tiles; at 512 rows the 128-row tile is ahead again)
+    // rows 18-20 % faster than on 128-row tiles)
     if (p.indptr != nullptr && (variant < 0 || variant == 1)) {
       if (p.rows <= 16 * p.num_experts) return launch_pipe_cfg<4, 32, 128, 32, 32, 4>(p, s);
       if (p.rows <= 48 * p.num_experts) return launch_pipe_cfg<4, 64, 128, 32, 64, 4>(p, s);

@@ -795,6 +795,41 @@ def test_moe_group_gemm_wide_tile(name):
     assert bool((fused == ops.silu_mul(out)).all())
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("variant", [-1, 1, 10, 11])  # heuristic, 128-row tiles, 256 x 256 / 256 x 128 tiles that skip empty row blocks
+def test_moe_group_gemm_tall_tiles_on_ragged_segments(name, variant):
+    """Grouped matmul from about 64 rows per expert on: 256-row tiles whose waves skip the 32-row blocks past the
+    end of a segment.  Segments of 1, 31..33, 127..129 and 300 rows (two tiles), an empty expert, the gather index,
+    the folded activation and both indptr dtypes; every tile choice must give the same bits."""
+    s = SCHEMES[name]
+    if variant == 10 and s.bits == 3:
+        pytest.skip("q3 has no 256 x 256 tile (its K tile does not fit LDS)")
+    rng = np.random.default_rng(61)
+    counts = [300, 0, 129, 33, 1, 127, 32, 31]
+    ne, n, k = len(counts), 520, 512 if s.bits == 4 else 520
+    ip = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(ip[-1])
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    x = rng.standard_normal((rows, k)).astype(np.float16)
+    ref = o.dequantize_group_gemm_fp32(x, qw, qs, ip, s)
+    base = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
+    src = rng.standard_normal((rows + 7, k)).astype(np.float16)
+    idx = rng.integers(0, rows + 7, rows).astype(np.int32)
+    gq._lib.set_option("gemm_variant", variant)
+    try:
+        out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
+        out64 = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip.astype(np.int64)), s.bits, s.group_size)
+        fused = ops.moe_experts(dev(x), None, dev(qw), dev(qs), dev(ip), s.bits, s.group_size, silu_mul_halves=True)
+        gathered = ops.moe_experts(dev(src), dev(idx), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
+    finally:
+        gq._lib.set_option("gemm_variant", -1)
+    assert_linear_ok(out, ref, x, k, f"grouped tall tiles {name} variant {variant}")
+    assert torch.equal(out, base) and torch.equal(out64, out)
+    assert torch.equal(fused, ops.silu_mul(out))
+    assert_linear_ok(gathered, o.dequantize_group_gemm_fp32(src[idx], qw, qs, ip, s), src[idx], k, "gathered")
+
+
 def test_silu_mul_and_combine():
     rng = np.random.default_rng(47)
     x = (rng.standard_normal((5, 192)) * 3).astype(np.float16)
