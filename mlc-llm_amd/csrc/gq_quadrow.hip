@@ -83,7 +83,7 @@ __device__ __forceinline__ float4_t mfma4_bf16(uint32_t a0, uint32_t a1, uint32_
 // 128 + q, so every field is shifted down to bit 0 of its half instead of being rescaled afterwards, and all
 // operand classes share the offset 128 + m.
 template <int BITS, int NBQ, int U, int MODE, bool BF = false>
-__global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
+__global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadParams p) {
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;  // 2: fused gate/up form, quad = 2 (gate, up) pairs
   constexpr uint32_t kMagic = BF ? 0x43004300u : 0x64006400u;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
@@ -128,11 +128,12 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
   const uint32_t* qw = p.qw + expert * p.expert_w_stride;
   const uint16_t* qs = p.qs + expert * p.expert_s_stride;
 
-  // LDS: x of one phase [NBQ][niter][CH words][64 lanes] uint4, its offset terms [NBQ][niter][64]
-  // floats, then this workgroup's partial sums between phases [wave][quad of the walk][NBQ][16]
+  // LDS: x of one phase [NBQ][niter][CH words][64 lanes] uint4, its offset terms [NBQ][niter][64] as four
+  // copies of the negated term (the C operand the group's first matrix instruction starts from), then this
+  // workgroup's partial sums between phases [wave][quad of the walk][NBQ][16]
   const int niter = p.nsteps * U;  // staged iterations per phase (groups past ng hold zeros)
-  float* const corr_lds = reinterpret_cast<float*>(smem + static_cast<size_t>(NBQ) * niter * CH * 64);
-  float* const part_lds = corr_lds + NBQ * niter * 64 + (tid >> 6) * (p.rounds * NBQ * 16);
+  float4* const corr_lds = reinterpret_cast<float4*>(smem + static_cast<size_t>(NBQ) * niter * CH * 64);
+  float* const part_lds = reinterpret_cast<float*>(corr_lds + NBQ * niter * 64) + (tid >> 6) * (p.rounds * NBQ * 16);
 
   uint4 wa[U], wb[U];
   uint32_t sa[U], sb[U];  // fp16 bits, 32 bits wide so that in-flight values are never re-packed
@@ -231,6 +232,29 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
             }
             const float corr = permute_group<BITS, BF>(nat, xr);
             const int lp = q & 63, bi = q >> 6;
+            // The float16 unpack leaves the odd fields times 16 (q3: times 8 and times 64) in their operands.  Their
+            // activations are divided by the same power of two here, once per workgroup, so that all of a group's
+            // products can run through ONE accumulator (exact unless the quotient is subnormal, where it moves the
+            // product by at most 2^-25 times the field's weight: far below the rounding of the accumulation).
+            if constexpr (!BF) {
+              const half2_t r16 = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
+              const half2_t r8 = {static_cast<_Float16>(0.125f), static_cast<_Float16>(0.125f)};
+              const half2_t r64 = {static_cast<_Float16>(0.015625f), static_cast<_Float16>(0.015625f)};
+              if constexpr (BITS == 4) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                  xr[4 * c + 1] = as_u32(as_half2(xr[4 * c + 1]) * r16);
+                  xr[4 * c + 3] = as_u32(as_half2(xr[4 * c + 3]) * r16);
+                }
+              } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                  xr[5 * c + 1] = as_u32(as_half2(xr[5 * c + 1]) * r8);
+                  xr[5 * c + 4] = as_u32(as_half2(xr[5 * c + 4]) * r8);
+                  xr[5 * c + 2] = as_u32(as_half2(xr[5 * c + 2]) * r64);
+                }
+              }
+            }
             if constexpr (BITS == 4) {
 #pragma unroll
               for (int c = 0; c < 4; ++c)  // word c: (even fields: 2 pairs), (odd fields: 2 pairs)
@@ -245,7 +269,7 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
                     make_uint4(xr[5 * c + 0], xr[5 * c + 3], xr[5 * c + 1], xr[5 * c + 4]);
               smem[(bi * CH + 4) * 64 + lp] = make_uint4(xr[2], xr[7], xr[12], xr[17]);
             }
-            corr_lds[bi * 64 + lp] = corr;
+            corr_lds[bi * 64 + lp] = make_float4(-corr, -corr, -corr, -corr);
           }
         }
       }
@@ -296,39 +320,34 @@ __global__ __launch_bounds__(512) void quad_kernel(const QuadParams p) {
             }
           }
         }
-        // the four rows' scales of this block: lane 4b+i holds row i's
+        // the four rows' scales of this block: lane 4b+i holds row i's (converted once, then broadcast)
+        const uint32_t s32 = __builtin_bit_cast(uint32_t, to_f32(static_cast<uint16_t>(sc[u])));
         float sv[4];
-        sv[0] = to_f32(static_cast<uint16_t>(dpp_u<0x00>(sc[u])));
-        sv[1] = to_f32(static_cast<uint16_t>(dpp_u<0x55>(sc[u])));
-        sv[2] = to_f32(static_cast<uint16_t>(dpp_u<0xAA>(sc[u])));
-        sv[3] = to_f32(static_cast<uint16_t>(dpp_u<0xFF>(sc[u])));
+        sv[0] = __builtin_bit_cast(float, dpp_u<0x00>(s32));
+        sv[1] = __builtin_bit_cast(float, dpp_u<0x55>(s32));
+        sv[2] = __builtin_bit_cast(float, dpp_u<0xAA>(s32));
+        sv[3] = __builtin_bit_cast(float, dpp_u<0xFF>(s32));
 #pragma unroll
         for (int bq = 0; bq < NBQ; ++bq) {
           if (bq > 0 && 4 * bq >= m_valid) continue;  // uniform: this segment has no such rows
           const int bi = bq * niter + it;
-          float4_t tl = {0.f, 0.f, 0.f, 0.f}, th = {0.f, 0.f, 0.f, 0.f};
+          // one accumulator per group: it starts from minus the offset term and takes every operand class (the
+          // activations of the scaled classes were divided when they were staged)
+          const float4 c4 = corr_lds[bi * 64 + lane];
+          float4_t t = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             const uint4 xv = smem[(bi * CH + d) * 64 + lane];
-            tl = mm(lo[d][0], lo[d][1], xv.x, xv.y, tl);
-            th = mm(hi[d][0], hi[d][1], xv.z, xv.w, th);
+            t = mm(lo[d][0], lo[d][1], xv.x, xv.y, t);
+            t = mm(hi[d][0], hi[d][1], xv.z, xv.w, t);
           }
-          const float corr = corr_lds[bi * 64 + lane];
-          // (bfloat16: the classes were shifted, not scaled)
-          constexpr float kHi = BF ? 1.0f : (BITS == 4 ? 0.0625f : 0.125f), k64 = BF ? 1.0f : 0.015625f;
-          if constexpr (BITS == 4) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              acc[bq][i] = fmaf(sv[i], fmaf(th[i], kHi, tl[i]) - corr, acc[bq][i]);
-          } else {
+          if constexpr (BITS == 3) {
             const uint4 xv = smem[(bi * CH + 4) * 64 + lane];
-            float4_t t64 = {0.f, 0.f, 0.f, 0.f};
-            t64 = mm(a64[0][0], a64[0][1], xv.x, xv.y, t64);
-            t64 = mm(a64[1][0], a64[1][1], xv.z, xv.w, t64);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              acc[bq][i] = fmaf(sv[i], fmaf(t64[i], k64, fmaf(th[i], kHi, tl[i])) - corr, acc[bq][i]);
+            t = mm(a64[0][0], a64[0][1], xv.x, xv.y, t);
+            t = mm(a64[1][0], a64[1][1], xv.z, xv.w, t);
           }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[bq][i] = fmaf(sv[i], t[i], acc[bq][i]);
         }
       }
       if (step == nst - 1) {  // uniform: the quad's share of this phase is complete
@@ -455,23 +474,33 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   const int experts = a.indptr ? static_cast<int>(a.num_experts) : 1;
 
   // LDS per iteration (16 groups) and batch quad: x in operand order and the offset terms
-  constexpr size_t kLdsIter = CH * 1024 + 256;
+  constexpr size_t kLdsIter = CH * 1024 + 1024;
   const int niter = (p.ng + 15) / 16;
-  int U = options().gemv_rows_per_wave;  // tuning override
-  // measured: 4 KiB items pay off only on matrices large enough to run long (gate_up, lm_head)
-  if (U != 2 && U != 4 && U != 8)
-    U = (niter >= 4 && static_cast<int64_t>(a.N) * a.K * experts >= (100ll << 20)) ? 4 : 2;
-  p.steps_total = (niter + U - 1) / U;
-  // More than 4 rows: 8 per pass when their x fits LDS whole.  Otherwise a plain linear runs
-  // two concurrent 4-row passes (the second pass's weight reads hit the last-level cache, and
-  // the grid doubles), a grouped matmul walks K in phases (experts already fill the grid).
-  // Tuning overrides: gemv_variant 7 prefers phases, 8 prefers 4-row passes.
+  const int opt_u = options().gemv_rows_per_wave;  // tuning override (1: 2 KiB items and sixteen waves per workgroup)
   const int mode = options().gemv_variant;
-  int nbq = rows_max <= 4 ? 1 : 2;
-  if (nbq == 2) {
-    const size_t whole = static_cast<size_t>(p.steps_total) * U * 2 * kLdsIter;
-    const bool phases = mode == 7 || (mode != 8 && a.indptr != nullptr);
-    if (mode == 8 || (whole > 150 * 1024 && !phases)) nbq = 1;
+  // measured: 4 KiB items pay off only on matrices large enough to run long (gate_up, lm_head)
+  const bool large = niter >= 4 && static_cast<int64_t>(a.N) * a.K * experts >= (100ll << 20);
+  // ... except with two batch quads (5..8 rows) of a plain linear: there sixteen waves per workgroup (four per
+  // SIMD, one copy of x between them) on 2 KiB items and twice the waves are ahead (gate_up 28672 x 4096 at 8
+  // rows: 24.9 -> 22.2 us, lm_head 74.3 -> 72.0; slower everywhere else, 4 rows included)
+  bool big_wg = opt_u == 1 || (opt_u < 0 && large && rows_max > 4 && a.indptr == nullptr && mode != 8 &&
+                               options().gemv_waves <= 0);
+  int U = 0, nbq = 0;
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    U = (opt_u == 2 || opt_u == 4 || opt_u == 8) ? opt_u : (big_wg ? 2 : (large ? 4 : 2));
+    p.steps_total = (niter + U - 1) / U;
+    // More than 4 rows: 8 per pass when their x fits LDS whole.  Otherwise a plain linear runs
+    // two concurrent 4-row passes (the second pass's weight reads hit the last-level cache, and
+    // the grid doubles), a grouped matmul walks K in phases (experts already fill the grid).
+    // Tuning overrides: gemv_variant 7 prefers phases, 8 prefers 4-row passes.
+    nbq = rows_max <= 4 ? 1 : 2;
+    if (nbq == 2) {
+      const size_t whole = static_cast<size_t>(p.steps_total) * U * 2 * kLdsIter;
+      const bool phases = mode == 7 || (mode != 8 && a.indptr != nullptr);
+      if (mode == 8 || (whole > 150 * 1024 && !phases)) nbq = 1;
+    }
+    if (!big_wg || nbq == 2) break;
+    big_wg = false;  // x of 8 rows does not fit: the concurrent 4-row passes keep their own launch shape
   }
   const int mtiles = (rows_max + 4 * nbq - 1) / (4 * nbq);
   if (mtiles > 4 && a.indptr == nullptr) return hipErrorNotSupported;
@@ -480,7 +509,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   // faster than 1024 waves of two to four quads each at 2..8 rows); concurrent passes over the same weights
   // already multiply the grid, and there 1024 measured better (down_proj 8192 x 28672 at 8 rows: 48 vs 66 us).
   int waves = options().gemv_waves > 0 ? options().gemv_waves
-                                       : (a.indptr != nullptr || mtiles == 1 ? 2048 : 1024);
+                                       : (big_wg ? 4096 : (a.indptr != nullptr || mtiles == 1 ? 2048 : 1024));
   // workgroups of experts without rows leave at once: share the waves among those that can have rows
   const int busy = p.rows < experts ? p.rows : experts;
   waves = (waves + busy - 1) / busy;
@@ -506,6 +535,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
     const int64_t wgs = static_cast<int64_t>(((p.nquads + p.rounds - 1) / p.rounds + 7) / 8) * busy * mtiles;
     if (2 * wgs <= 256) threads = 256;  // (the doubled count must still be one round of workgroups)
   }
+  if (big_wg && p.nphases == 1) threads = 1024;  // four waves per SIMD share one copy of x
   const int wpb = threads / 64;
   const size_t lds = lds_x + (p.nphases > 1 ? static_cast<size_t>(wpb) * p.rounds * nbq * 64 : 0);
   const int blocks = ((p.nquads + p.rounds - 1) / p.rounds + wpb - 1) / wpb;
