@@ -343,7 +343,7 @@ def main() -> int:
                         for lw in layers:
                             run_linear(name, lw[name][0], lw[name][1], b, outs[name])
                     cnt = LAYERS
-                us = timed(sweep, 5, 1, use_graph) * 1e3 / cnt
+                us = timed(sweep, 5, 3, use_graph) * 1e3 / cnt  # (the first replays of a new graph run a few % slow)
                 gbs = gemv_bytes(n, k, b) / (us * 1e-6) / 1e9
                 per_shape[f"{name}_b{b}"] = {"us": round(us, 2), "GB/s": round(gbs, 1),
                                              "frac_hbm": round(gbs / HBM_PEAK_GBS, 3)}

@@ -128,12 +128,12 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
   const uint32_t* qw = p.qw + expert * p.expert_w_stride;
   const uint16_t* qs = p.qs + expert * p.expert_s_stride;
 
-  // LDS: x of one phase [NBQ][niter][CH words][64 lanes] uint4, its offset terms [NBQ][niter][64] as four
-  // copies of the negated term (the C operand the group's first matrix instruction starts from), then this
-  // workgroup's partial sums between phases [wave][quad of the walk][NBQ][16]
+  // LDS: x of one phase [NBQ][niter][CH words][64 lanes] uint4, its negated offset terms [NBQ][niter][64]
+  // floats (what the group's accumulator starts from), then this workgroup's partial sums between phases
+  // [wave][quad of the walk][NBQ][16]
   const int niter = p.nsteps * U;  // staged iterations per phase (groups past ng hold zeros)
-  float4* const corr_lds = reinterpret_cast<float4*>(smem + static_cast<size_t>(NBQ) * niter * CH * 64);
-  float* const part_lds = reinterpret_cast<float*>(corr_lds + NBQ * niter * 64) + (tid >> 6) * (p.rounds * NBQ * 16);
+  float* const corr_lds = reinterpret_cast<float*>(smem + static_cast<size_t>(NBQ) * niter * CH * 64);
+  float* const part_lds = corr_lds + NBQ * niter * 64 + (tid >> 6) * (p.rounds * NBQ * 16);
 
   uint4 wa[U], wb[U];
   uint32_t sa[U], sb[U];  // fp16 bits, 32 bits wide so that in-flight values are never re-packed
@@ -269,7 +269,7 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
                     make_uint4(xr[5 * c + 0], xr[5 * c + 3], xr[5 * c + 1], xr[5 * c + 4]);
               smem[(bi * CH + 4) * 64 + lp] = make_uint4(xr[2], xr[7], xr[12], xr[17]);
             }
-            corr_lds[bi * 64 + lp] = make_float4(-corr, -corr, -corr, -corr);
+            corr_lds[bi * 64 + lp] = -corr;
           }
         }
       }
@@ -333,8 +333,8 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
           const int bi = bq * niter + it;
           // one accumulator per group: it starts from minus the offset term and takes every operand class (the
           // activations of the scaled classes were divided when they were staged)
-          const float4 c4 = corr_lds[bi * 64 + lane];
-          float4_t t = {c4.x, c4.y, c4.z, c4.w};
+          const float c = corr_lds[bi * 64 + lane];
+          float4_t t = {c, c, c, c};
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             const uint4 xv = smem[(bi * CH + d) * 64 + lane];
@@ -474,7 +474,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   const int experts = a.indptr ? static_cast<int>(a.num_experts) : 1;
 
   // LDS per iteration (16 groups) and batch quad: x in operand order and the offset terms
-  constexpr size_t kLdsIter = CH * 1024 + 1024;
+  constexpr size_t kLdsIter = CH * 1024 + 256;
   const int niter = (p.ng + 15) / 16;
   const int opt_u = options().gemv_rows_per_wave;  // tuning override (1: 2 KiB items and sixteen waves per workgroup)
   const int mode = options().gemv_variant;
