@@ -12,6 +12,7 @@ namespace gq {
 // public header) ever sees anything else, so calls arriving on other threads cannot be steered by it.
 struct Options {
   int gemv_rows_per_wave = -1;  // -1: heuristic
+  int quad_pairs = -1;          // -1: heuristic, 1 | 2: quads per item of the quad-row kernel
   int gemv_variant = -1;        // -1: heuristic, 0: LDS GEMV, 1: register GEMV, 2..5 skinny forms, 6..8 quad-row forms
   int gemm_variant = -1;
   int gemv_waves = -1;          // total waves of a persistent GEMV / quad-row / skinny grid

@@ -42,10 +42,11 @@ struct QuadParams {
   int64_t expert_w_stride, expert_s_stride;
   int rows, N, K, ng, nw;
   int nquads;       // N / 4
+  int nsets;        // quad sets (QP consecutive quads share every read of x): ceil(nquads / QP)
   int nsteps;       // k steps per quad and phase; a step is U iterations of 16 groups
   int steps_total;  // k steps per quad over all phases
   int nphases;      // passes over K, each with its slice of x in LDS
-  int rounds;       // most quads any wave walks
+  int rounds;       // most quad sets any wave walks
   int indptr_i64, out_f32;
   int paired;       // fused gate/up form: y is [rows, N / 2] fp16
   const int32_t* x_rows;  // null, or the row of x each activation row reads (int32 [rows])
@@ -82,8 +83,11 @@ __device__ __forceinline__ float4_t mfma4_bf16(uint32_t a0, uint32_t a1, uint32_
 // BF: bfloat16 model (x, scales, bias, residual and a 16-bit result are bfloat16).  0x4300 | q is the bfloat16
 // 128 + q, so every field is shifted down to bit 0 of its half instead of being rescaled afterwards, and all
 // operand classes share the offset 128 + m.
-template <int BITS, int NBQ, int U, int MODE, bool BF = false>
-__global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadParams p) {
+// QP: quads per item.  The x operands of an iteration are read from LDS once and meet the weights of QP
+// consecutive quads, so the LDS bytes read per weight byte fall by that factor (a 4x4x4 block needs as many
+// operand bytes of x as of weights: with 8 activation rows that is 8 LDS bytes per packed weight byte at QP = 1).
+template <int BITS, int NBQ, int U, int MODE, bool BF = false, int QP = 1>
+__global__ __launch_bounds__((U * QP <= 2 && !(QP > 1 && MODE == 1)) ? 1024 : 512) void quad_kernel(const QuadParams p) {
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;  // 2: fused gate/up form, quad = 2 (gate, up) pairs
   constexpr uint32_t kMagic = BF ? 0x43004300u : 0x64006400u;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
@@ -133,13 +137,13 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
   // [wave][quad of the walk][NBQ][16]
   const int niter = p.nsteps * U;  // staged iterations per phase (groups past ng hold zeros)
   float* const corr_lds = reinterpret_cast<float*>(smem + static_cast<size_t>(NBQ) * niter * CH * 64);
-  float* const part_lds = corr_lds + NBQ * niter * 64 + (tid >> 6) * (p.rounds * NBQ * 16);
+  float* const part_lds = corr_lds + NBQ * niter * 64 + (tid >> 6) * (p.rounds * QP * NBQ * 16);
 
-  uint4 wa[U], wb[U];
-  uint32_t sa[U], sb[U];  // fp16 bits, 32 bits wide so that in-flight values are never re-packed
-  uint2 ba, bb;
-  uint2 ra[NBQ], rb[NBQ];  // residual of (activation row 4 * bq + lane, the quad's 4 weight rows), lanes 0..3
-  float4_t acc[NBQ];
+  uint4 wa[QP][U], wb[QP][U];
+  uint32_t sa[QP][U], sb[QP][U];  // fp16 bits, 32 bits wide so that in-flight values are never re-packed
+  uint2 ba[QP], bb[QP];
+  uint2 ra[QP][NBQ], rb[QP][NBQ];  // residual of (activation row 4 * bq + lane, the quad's 4 weight rows), lanes 0..3
+  float4_t acc[QP][NBQ];
 
   // K is walked in phases when x does not fit LDS whole: every phase stages its slice of x and
   // walks all of this wave's quads; partial sums wait in LDS for the last phase.
@@ -148,44 +152,51 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
     const int it0 = phase * niter;                                    // first iteration of the phase
     const bool last_phase = phase == p.nphases - 1;
 #pragma unroll
-    for (int bq = 0; bq < NBQ; ++bq) acc[bq] = float4_t{0.f, 0.f, 0.f, 0.f};  // drops what an item past the end left
+    for (int qp = 0; qp < QP; ++qp)
+#pragma unroll
+      for (int bq = 0; bq < NBQ; ++bq) acc[qp][bq] = float4_t{0.f, 0.f, 0.f, 0.f};  // drops what an item past the end left
 
     // ---- weight / scale / bias loads of one item.  Branch-free: every path issues the same
     //      loads, so the wait counts let the other buffer's loads stay in flight across the loop;
     //      an item past the end reads one cached line instead.
-    auto issue = [&](int quad, int step, uint4 (&wn)[U], uint32_t (&sn)[U], uint2& bn, uint2 (&rn)[NBQ]) {
-      const bool live = quad < p.nquads;
-      int row = min(quad * 4 + li, p.N - 1);
-      if (PAIRED) row = gate_up_row(row, p.N);
-      const uint32_t* wr = qw + static_cast<int64_t>(row) * p.nw;
-      const uint16_t* sr = qs + static_cast<int64_t>(row) * p.ng;
+    auto issue = [&](int qset, int step, uint4 (&wn)[QP][U], uint32_t (&sn)[QP][U], uint2 (&bn)[QP],
+                     uint2 (&rn)[QP][NBQ]) {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int g = min((it0 + step * U + u) * 16 + ks, p.ng - 1);
-        wn[u] = *reinterpret_cast<const uint4*>(live ? wr + 4 * g : qw);
-        sn[u] = *(live ? sr + g : qs);
-      }
-      // bias and residual ride along (at store time they would wait behind the next items' weights)
-      if constexpr (EXTRA) {
-        bn = *reinterpret_cast<const uint2*>(
-            (live && p.bias != nullptr) ? p.bias + quad * 4 : reinterpret_cast<const uint16_t*>(qw));
+      for (int qp = 0; qp < QP; ++qp) {
+        const int quad = qset * QP + qp;
+        const bool live = quad < p.nquads;
+        int row = min(quad * 4 + li, p.N - 1);
+        if (PAIRED) row = gate_up_row(row, p.N);
+        const uint32_t* wr = qw + static_cast<int64_t>(row) * p.nw;
+        const uint16_t* sr = qs + static_cast<int64_t>(row) * p.ng;
 #pragma unroll
-        for (int bq = 0; bq < NBQ; ++bq) {
-          const int b = min(4 * bq + (lane & 3), m_valid - 1);
-          rn[bq] = *reinterpret_cast<const uint2*>(
-              (live && p.residual != nullptr) ? p.residual + static_cast<int64_t>(m0 + b) * p.N + quad * 4
-                                              : reinterpret_cast<const uint16_t*>(qw));
+        for (int u = 0; u < U; ++u) {
+          const int g = min((it0 + step * U + u) * 16 + ks, p.ng - 1);
+          wn[qp][u] = *reinterpret_cast<const uint4*>(live ? wr + 4 * g : qw);
+          sn[qp][u] = *(live ? sr + g : qs);
+        }
+        // bias and residual ride along (at store time they would wait behind the next items' weights)
+        if constexpr (EXTRA) {
+          bn[qp] = *reinterpret_cast<const uint2*>(
+              (live && p.bias != nullptr) ? p.bias + quad * 4 : reinterpret_cast<const uint16_t*>(qw));
+#pragma unroll
+          for (int bq = 0; bq < NBQ; ++bq) {
+            const int b = min(4 * bq + (lane & 3), m_valid - 1);
+            rn[qp][bq] = *reinterpret_cast<const uint2*>(
+                (live && p.residual != nullptr) ? p.residual + static_cast<int64_t>(m0 + b) * p.N + quad * 4
+                                                : reinterpret_cast<const uint16_t*>(qw));
+          }
         }
       }
     };
-    auto advance = [&](int& quad, int& step) {  // two items on
+    auto advance = [&](int& qset, int& step) {  // two items on
       step += 2;
       if (step >= nst) {
         step -= nst;
-        quad += nwaves;
+        qset += nwaves;
         if (step >= nst) {
           step -= nst;
-          quad += nwaves;
+          qset += nwaves;
         }
       }
     };
@@ -281,52 +292,55 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
 
     // ---- persistent walk
     int done = 0;  // quads this wave has completed in this phase
-    auto compute = [&](int quad, int step, const uint4 (&wc)[U], const uint32_t (&sc)[U],
-                       uint2 bias_bits, const uint2 (&res_bits)[NBQ]) {
+    auto compute = [&](int qset, int step, const uint4 (&wc)[QP][U], const uint32_t (&sc)[QP][U],
+                       const uint2 (&bias_bits)[QP], const uint2 (&res_bits)[QP][NBQ]) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int it = step * U + u;
-        const uint32_t w[4] = {wc[u].x, wc[u].y, wc[u].z, wc[u].w};
         // A operands: q4 lo/hi = even / odd fields (x1, x16) of word d; q3 a1/a8 = the x1 / x8
         // fields of word d, a64 = the x64 field pairs of words (0,1) and (2,3)
-        uint32_t lo[4][2], hi[4][2], a64[2][2];
+        uint32_t lo[QP][4][2], hi[QP][4][2], a64[QP][2][2];
+        float sv[QP][4];
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          if constexpr (BITS == 4) {
-            const uint32_t w8 = w[d] >> 8;
-            lo[d][0] = and_or(w[d], 0x000f000fu, kMagic);
-            lo[d][1] = and_or(w8, 0x000f000fu, kMagic);
-            if constexpr (BF) {
-              hi[d][0] = and_or(w[d] >> 4, 0x000f000fu, kMagic);
-              hi[d][1] = and_or(w[d] >> 12, 0x000f000fu, kMagic);
+        for (int qp = 0; qp < QP; ++qp) {
+          const uint32_t w[4] = {wc[qp][u].x, wc[qp][u].y, wc[qp][u].z, wc[qp][u].w};
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            if constexpr (BITS == 4) {
+              const uint32_t w8 = w[d] >> 8;
+              lo[qp][d][0] = and_or(w[d], 0x000f000fu, kMagic);
+              lo[qp][d][1] = and_or(w8, 0x000f000fu, kMagic);
+              if constexpr (BF) {
+                hi[qp][d][0] = and_or(w[d] >> 4, 0x000f000fu, kMagic);
+                hi[qp][d][1] = and_or(w[d] >> 12, 0x000f000fu, kMagic);
+              } else {
+                hi[qp][d][0] = and_or(w[d], 0x00f000f0u, kMagic);
+                hi[qp][d][1] = and_or(w8, 0x00f000f0u, kMagic);
+              }
             } else {
-              hi[d][0] = and_or(w[d], 0x00f000f0u, kMagic);
-              hi[d][1] = and_or(w8, 0x00f000f0u, kMagic);
-            }
-          } else {
-            // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
-            const uint32_t t = (w[d] & 0x0000ffffu) | ((w[d] << 1) & 0xffff0000u);
-            const uint32_t t9 = t >> 9;
-            lo[d][0] = and_or(t, 0x00070007u, kMagic);   // fields (0,5)
-            lo[d][1] = and_or(t9, 0x00070007u, kMagic);  // fields (3,8)
-            if constexpr (BF) {
-              hi[d][0] = and_or(t >> 3, 0x00070007u, kMagic);   // fields (1,6)
-              hi[d][1] = and_or(t >> 12, 0x00070007u, kMagic);  // fields (4,9)
-              a64[d >> 1][d & 1] = and_or(t >> 6, 0x00070007u, kMagic);  // fields (2,7)
-            } else {
-              hi[d][0] = and_or(t, 0x00380038u, kMagic);   // fields (1,6) x 8
-              hi[d][1] = and_or(t9, 0x00380038u, kMagic);  // fields (4,9) x 8
-              a64[d >> 1][d & 1] = and_or(t, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+              // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
+              const uint32_t t = (w[d] & 0x0000ffffu) | ((w[d] << 1) & 0xffff0000u);
+              const uint32_t t9 = t >> 9;
+              lo[qp][d][0] = and_or(t, 0x00070007u, kMagic);   // fields (0,5)
+              lo[qp][d][1] = and_or(t9, 0x00070007u, kMagic);  // fields (3,8)
+              if constexpr (BF) {
+                hi[qp][d][0] = and_or(t >> 3, 0x00070007u, kMagic);   // fields (1,6)
+                hi[qp][d][1] = and_or(t >> 12, 0x00070007u, kMagic);  // fields (4,9)
+                a64[qp][d >> 1][d & 1] = and_or(t >> 6, 0x00070007u, kMagic);  // fields (2,7)
+              } else {
+                hi[qp][d][0] = and_or(t, 0x00380038u, kMagic);   // fields (1,6) x 8
+                hi[qp][d][1] = and_or(t9, 0x00380038u, kMagic);  // fields (4,9) x 8
+                a64[qp][d >> 1][d & 1] = and_or(t, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+              }
             }
           }
+          // the four rows' scales of this block: lane 4b+i holds row i's (converted once, then broadcast)
+          const uint32_t s32 = __builtin_bit_cast(uint32_t, to_f32(static_cast<uint16_t>(sc[qp][u])));
+          sv[qp][0] = __builtin_bit_cast(float, dpp_u<0x00>(s32));
+          sv[qp][1] = __builtin_bit_cast(float, dpp_u<0x55>(s32));
+          sv[qp][2] = __builtin_bit_cast(float, dpp_u<0xAA>(s32));
+          sv[qp][3] = __builtin_bit_cast(float, dpp_u<0xFF>(s32));
         }
-        // the four rows' scales of this block: lane 4b+i holds row i's (converted once, then broadcast)
-        const uint32_t s32 = __builtin_bit_cast(uint32_t, to_f32(static_cast<uint16_t>(sc[u])));
-        float sv[4];
-        sv[0] = __builtin_bit_cast(float, dpp_u<0x00>(s32));
-        sv[1] = __builtin_bit_cast(float, dpp_u<0x55>(s32));
-        sv[2] = __builtin_bit_cast(float, dpp_u<0xAA>(s32));
-        sv[3] = __builtin_bit_cast(float, dpp_u<0xFF>(s32));
 #pragma unroll
         for (int bq = 0; bq < NBQ; ++bq) {
           if (bq > 0 && 4 * bq >= m_valid) continue;  // uniform: this segment has no such rows
@@ -334,71 +348,79 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
           // one accumulator per group: it starts from minus the offset term and takes every operand class (the
           // activations of the scaled classes were divided when they were staged)
           const float c = corr_lds[bi * 64 + lane];
-          float4_t t = {c, c, c, c};
+          uint4 xv[CH];
 #pragma unroll
-          for (int d = 0; d < 4; ++d) {
-            const uint4 xv = smem[(bi * CH + d) * 64 + lane];
-            t = mm(lo[d][0], lo[d][1], xv.x, xv.y, t);
-            t = mm(hi[d][0], hi[d][1], xv.z, xv.w, t);
-          }
-          if constexpr (BITS == 3) {
-            const uint4 xv = smem[(bi * CH + 4) * 64 + lane];
-            t = mm(a64[0][0], a64[0][1], xv.x, xv.y, t);
-            t = mm(a64[1][0], a64[1][1], xv.z, xv.w, t);
-          }
+          for (int d = 0; d < CH; ++d) xv[d] = smem[(bi * CH + d) * 64 + lane];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[bq][i] = fmaf(sv[i], t[i], acc[bq][i]);
+          for (int qp = 0; qp < QP; ++qp) {
+            float4_t t = {c, c, c, c};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              t = mm(lo[qp][d][0], lo[qp][d][1], xv[d].x, xv[d].y, t);
+              t = mm(hi[qp][d][0], hi[qp][d][1], xv[d].z, xv[d].w, t);
+            }
+            if constexpr (BITS == 3) {
+              t = mm(a64[qp][0][0], a64[qp][0][1], xv[CH - 1].x, xv[CH - 1].y, t);
+              t = mm(a64[qp][1][0], a64[qp][1][1], xv[CH - 1].z, xv[CH - 1].w, t);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[qp][bq][i] = fmaf(sv[qp][i], t[i], acc[qp][bq][i]);
+          }
         }
       }
-      if (step == nst - 1) {  // uniform: the quad's share of this phase is complete
+      if (step == nst - 1) {  // uniform: the quads' share of this phase is complete
 #pragma unroll
-        for (int bq = 0; bq < NBQ; ++bq) {
-          float v[4];
+        for (int qp = 0; qp < QP; ++qp) {
+          const int quad = qset * QP + qp;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            float t = acc[bq][i];
-            t += dpp_f<0x124>(t);  // row_ror:4
-            t += dpp_f<0x128>(t);  // row_ror:8: every lane holds the sum over its row of 16 lanes
-            t += __shfl_xor(t, 16, kWave);
-            t += __shfl_xor(t, 32, kWave);
-            v[i] = t;
-            acc[bq][i] = 0.f;
-          }
-          const int b = 4 * bq + lane;  // lanes 0..3: one activation row each, 4 weight rows
-          if (lane < 4 && b < m_valid && quad < p.nquads) {
-            float4* part = reinterpret_cast<float4*>(part_lds) + (done * NBQ + bq) * 4 + lane;
-            if (phase > 0) {
-              const float4 pv = *part;
-              v[0] += pv.x; v[1] += pv.y; v[2] += pv.z; v[3] += pv.w;
+          for (int bq = 0; bq < NBQ; ++bq) {
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              float t = acc[qp][bq][i];
+              t += dpp_f<0x124>(t);  // row_ror:4
+              t += dpp_f<0x128>(t);  // row_ror:8: every lane holds the sum over its row of 16 lanes
+              t += __shfl_xor(t, 16, kWave);
+              t += __shfl_xor(t, 32, kWave);
+              v[i] = t;
+              acc[qp][bq][i] = 0.f;
             }
-            if (!last_phase) {
-              *part = make_float4(v[0], v[1], v[2], v[3]);
-            } else {
-              if (EXTRA && p.bias != nullptr) {
-                v[0] += to_f32(static_cast<uint16_t>(bias_bits.x & 0xffffu));
-                v[1] += to_f32(static_cast<uint16_t>(bias_bits.x >> 16));
-                v[2] += to_f32(static_cast<uint16_t>(bias_bits.y & 0xffffu));
-                v[3] += to_f32(static_cast<uint16_t>(bias_bits.y >> 16));
+            const int b = 4 * bq + lane;  // lanes 0..3: one activation row each, 4 weight rows
+            if (lane < 4 && b < m_valid && quad < p.nquads) {
+              float4* part = reinterpret_cast<float4*>(part_lds) + ((done * QP + qp) * NBQ + bq) * 4 + lane;
+              if (phase > 0) {
+                const float4 pv = *part;
+                v[0] += pv.x; v[1] += pv.y; v[2] += pv.z; v[3] += pv.w;
               }
-              if (EXTRA && p.residual != nullptr) {
-                v[0] += to_f32(static_cast<uint16_t>(res_bits[bq].x & 0xffffu));
-                v[1] += to_f32(static_cast<uint16_t>(res_bits[bq].x >> 16));
-                v[2] += to_f32(static_cast<uint16_t>(res_bits[bq].y & 0xffffu));
-                v[3] += to_f32(static_cast<uint16_t>(res_bits[bq].y >> 16));
-              }
-              const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
-              if constexpr (PAIRED) {
-                *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p.y) + (oi >> 1)) =
-                    static_cast<uint32_t>(silu_mul_t<BF>(v[0], v[1])) |
-                    (static_cast<uint32_t>(silu_mul_t<BF>(v[2], v[3])) << 16);
-              } else if (p.out_f32) {
-                *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) =
-                    make_float4(v[0], v[1], v[2], v[3]);
+              if (!last_phase) {
+                *part = make_float4(v[0], v[1], v[2], v[3]);
               } else {
-                uint2 o;
-                o.x = static_cast<uint32_t>(to_out(v[0])) | (static_cast<uint32_t>(to_out(v[1])) << 16);
-                o.y = static_cast<uint32_t>(to_out(v[2])) | (static_cast<uint32_t>(to_out(v[3])) << 16);
-                *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.y) + oi) = o;
+                if (EXTRA && p.bias != nullptr) {
+                  v[0] += to_f32(static_cast<uint16_t>(bias_bits[qp].x & 0xffffu));
+                  v[1] += to_f32(static_cast<uint16_t>(bias_bits[qp].x >> 16));
+                  v[2] += to_f32(static_cast<uint16_t>(bias_bits[qp].y & 0xffffu));
+                  v[3] += to_f32(static_cast<uint16_t>(bias_bits[qp].y >> 16));
+                }
+                if (EXTRA && p.residual != nullptr) {
+                  v[0] += to_f32(static_cast<uint16_t>(res_bits[qp][bq].x & 0xffffu));
+                  v[1] += to_f32(static_cast<uint16_t>(res_bits[qp][bq].x >> 16));
+                  v[2] += to_f32(static_cast<uint16_t>(res_bits[qp][bq].y & 0xffffu));
+                  v[3] += to_f32(static_cast<uint16_t>(res_bits[qp][bq].y >> 16));
+                }
+                const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
+                if constexpr (PAIRED) {
+                  *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p.y) + (oi >> 1)) =
+                      static_cast<uint32_t>(silu_mul_t<BF>(v[0], v[1])) |
+                      (static_cast<uint32_t>(silu_mul_t<BF>(v[2], v[3])) << 16);
+                } else if (p.out_f32) {
+                  *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) =
+                      make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+                  uint2 o;
+                  o.x = static_cast<uint32_t>(to_out(v[0])) | (static_cast<uint32_t>(to_out(v[1])) << 16);
+                  o.y = static_cast<uint32_t>(to_out(v[2])) | (static_cast<uint32_t>(to_out(v[3])) << 16);
+                  *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.y) + oi) = o;
+                }
               }
             }
           }
@@ -407,7 +429,7 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
       }
     };
 
-    while (qa < p.nquads) {
+    while (qa < p.nsets) {
       compute(qa, sta, wa, sa, ba, ra);
       advance(qa, sta);
       issue(qa, sta, wa, sa, ba, ra);
@@ -420,31 +442,35 @@ __global__ __launch_bounds__(U <= 2 ? 1024 : 512) void quad_kernel(const QuadPar
   }
 }
 
-template <int BITS, int NBQ, int U, int MODE, bool BF = false>
+template <int BITS, int NBQ, int U, int MODE, bool BF = false, int QP = 1>
 static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                     hipStream_t s) {
   if (lds > 65536) {
-    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF>));
+    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF, QP>));
     if (e != hipSuccess) return e;
   }
-  note_kernel("gq::quad_kernel<%d,%d,%d,%d,%s>", BITS, NBQ, U, MODE, BF ? "true" : "false");
-  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF>), grid, dim3(threads), lds, s, p);
+  note_kernel("gq::quad_kernel<%d,%d,%d,%d,%s,%d>", BITS, NBQ, U, MODE, BF ? "true" : "false", QP);
+  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF, QP>), grid, dim3(threads), lds, s, p);
   return hipGetLastError();
 }
 
-template <int BITS, int NBQ, int U>
+template <int BITS, int NBQ, int U, int QP = 1>
 static hipError_t launch_quad_cfg(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                   hipStream_t s) {
   if (p.bf16) {
-    if (p.paired) return launch_quad_extra<BITS, NBQ, U, 2, true>(p, grid, threads, lds, s);
-    return (p.bias != nullptr || p.residual != nullptr)
-               ? launch_quad_extra<BITS, NBQ, U, 1, true>(p, grid, threads, lds, s)
-               : launch_quad_extra<BITS, NBQ, U, 0, true>(p, grid, threads, lds, s);
+    if constexpr (QP == 1) {
+      if (p.paired) return launch_quad_extra<BITS, NBQ, U, 2, true>(p, grid, threads, lds, s);
+      return (p.bias != nullptr || p.residual != nullptr)
+                 ? launch_quad_extra<BITS, NBQ, U, 1, true>(p, grid, threads, lds, s)
+                 : launch_quad_extra<BITS, NBQ, U, 0, true>(p, grid, threads, lds, s);
+    } else {
+      return hipErrorNotSupported;
+    }
   }
-  if (p.paired) return launch_quad_extra<BITS, NBQ, U, 2>(p, grid, threads, lds, s);
+  if (p.paired) return launch_quad_extra<BITS, NBQ, U, 2, false, QP>(p, grid, threads, lds, s);
   return (p.bias != nullptr || p.residual != nullptr)
-             ? launch_quad_extra<BITS, NBQ, U, 1>(p, grid, threads, lds, s)
-             : launch_quad_extra<BITS, NBQ, U, 0>(p, grid, threads, lds, s);
+             ? launch_quad_extra<BITS, NBQ, U, 1, false, QP>(p, grid, threads, lds, s)
+             : launch_quad_extra<BITS, NBQ, U, 0, false, QP>(p, grid, threads, lds, s);
 }
 
 // hipErrorNotSupported when the shape does not fit (the caller falls back to its other kernels)
@@ -483,6 +509,12 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   // ... except with two batch quads (5..8 rows) of a plain linear: there sixteen waves per workgroup (four per
   // SIMD, one copy of x between them) on 2 KiB items and twice the waves are ahead (gate_up 28672 x 4096 at 8
   // rows: 24.9 -> 22.2 us, lm_head 74.3 -> 72.0; slower everywhere else, 4 rows included)
+  // quads per item (tuning override; float16 only)
+  // Quads per item: two where the 8-row form runs long (float16; measured on 28672 x 4096 at 8 rows 21.5 -> 20.5 us,
+  // 128256 x 4096 68.6 -> 67.0, Mixtral's expert layer at 16 tokens 197 -> 180 us; 4-row forms within 1.5 % either
+  // way, small matrices 5-25 % slower: half as many items to spread over the waves; four quads per item no better)
+  const int opt_qp = options().quad_pairs;
+  int QP = 1;
   bool big_wg = opt_u == 1 || (opt_u < 0 && large && rows_max > 4 && a.indptr == nullptr && mode != 8 &&
                                options().gemv_waves <= 0);
   int U = 0, nbq = 0;
@@ -502,6 +534,11 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
     if (!big_wg || nbq == 2) break;
     big_wg = false;  // x of 8 rows does not fit: the concurrent 4-row passes keep their own launch shape
   }
+  QP = a.bf16 ? 1 : ((opt_qp == 1 || opt_qp == 2) ? opt_qp : ((large && nbq == 2) ? 2 : 1));
+  if (QP == 2) {
+    U = U >= 4 ? 2 : 1;  // the same bytes per item
+    p.steps_total = (niter + U - 1) / U;
+  }
   const int mtiles = (rows_max + 4 * nbq - 1) / (4 * nbq);
   if (mtiles > 4 && a.indptr == nullptr) return hipErrorNotSupported;
 
@@ -513,13 +550,14 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   // workgroups of experts without rows leave at once: share the waves among those that can have rows
   const int busy = p.rows < experts ? p.rows : experts;
   waves = (waves + busy - 1) / busy;
-  if (waves > p.nquads) waves = p.nquads;
-  p.rounds = (p.nquads + waves - 1) / waves;
+  p.nsets = (p.nquads + QP - 1) / QP;
+  if (waves > p.nsets) waves = p.nsets;
+  p.rounds = (p.nsets + waves - 1) / waves;
 
   // per wave: the partial sums of its quads.  Phases share K evenly.
   const size_t lds_cap = 150 * 1024;
   const size_t lds_step = static_cast<size_t>(U) * nbq * kLdsIter;
-  const size_t lds_part = static_cast<size_t>(8) * p.rounds * nbq * 64;  // up to 8 waves
+  const size_t lds_part = static_cast<size_t>(8) * p.rounds * QP * nbq * 64;  // up to 8 waves
   if (lds_part + lds_step > lds_cap) return hipErrorNotSupported;
   const int steps_fit = static_cast<int>((lds_cap - lds_part) / lds_step);
   p.nphases = (p.steps_total + steps_fit - 1) / steps_fit;
@@ -532,18 +570,30 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   // halve that traffic (qkv 6144 x 4096 at 8 rows 11.4 -> 9.9 us, gate_up 24.3 -> 22.6; never slower)
   int threads = (lds_x > 76 * 1024 || a.indptr == nullptr) ? 512 : 256;
   if (threads == 512) {
-    const int64_t wgs = static_cast<int64_t>(((p.nquads + p.rounds - 1) / p.rounds + 7) / 8) * busy * mtiles;
+    const int64_t wgs = static_cast<int64_t>(((p.nsets + p.rounds - 1) / p.rounds + 7) / 8) * busy * mtiles;
     if (2 * wgs <= 256) threads = 256;  // (the doubled count must still be one round of workgroups)
   }
-  if (big_wg && p.nphases == 1) threads = 1024;  // four waves per SIMD share one copy of x
+  // four waves per SIMD share one copy of x (the instances that fit 128 registers: 2 KiB items without bias / residual loads
+  // when two quads share an item)
+  if (big_wg && p.nphases == 1 && U * QP <= 2 && !(QP > 1 && (a.bias != nullptr || a.residual != nullptr)))
+    threads = 1024;
   const int wpb = threads / 64;
-  const size_t lds = lds_x + (p.nphases > 1 ? static_cast<size_t>(wpb) * p.rounds * nbq * 64 : 0);
-  const int blocks = ((p.nquads + p.rounds - 1) / p.rounds + wpb - 1) / wpb;
+  const size_t lds = lds_x + (p.nphases > 1 ? static_cast<size_t>(wpb) * p.rounds * QP * nbq * 64 : 0);
+  const int blocks = ((p.nsets + p.rounds - 1) / p.rounds + wpb - 1) / wpb;
   const dim3 grid(blocks, experts, mtiles);
 #define GQ_QUAD_CASE(NBQ_, U_) \
   if (nbq == NBQ_ && U == U_) return launch_quad_cfg<BITS, NBQ_, U_>(p, grid, threads, lds, s);
-  GQ_QUAD_CASE(1, 2) GQ_QUAD_CASE(1, 4) GQ_QUAD_CASE(1, 8)
-  GQ_QUAD_CASE(2, 2) GQ_QUAD_CASE(2, 4) GQ_QUAD_CASE(2, 8)
+  if (QP == 1) {
+    GQ_QUAD_CASE(1, 2) GQ_QUAD_CASE(1, 4) GQ_QUAD_CASE(1, 8)
+    GQ_QUAD_CASE(2, 2) GQ_QUAD_CASE(2, 4) GQ_QUAD_CASE(2, 8)
+  }
+#undef GQ_QUAD_CASE
+#define GQ_QUAD_CASE(NBQ_, U_) \
+  if (nbq == NBQ_ && U == U_) return launch_quad_cfg<BITS, NBQ_, U_, 2>(p, grid, threads, lds, s);
+  if (QP == 2) {
+    GQ_QUAD_CASE(1, 1) GQ_QUAD_CASE(1, 2)
+    GQ_QUAD_CASE(2, 1) GQ_QUAD_CASE(2, 2)
+  }
 #undef GQ_QUAD_CASE
   return hipErrorNotSupported;
 }

@@ -328,42 +328,50 @@ def test_skinny_kernel_forms_grouped(mode):
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("u", [-1, 2, 8])  # iterations per item: heuristic, smallest, largest
+@pytest.mark.parametrize("qp", [1, 2])  # quads per item (two: each read of x meets the weights of two quads)
 @pytest.mark.parametrize("m", [3, 4, 5, 8])
-@pytest.mark.parametrize("n,k", [(520, 1024), (100, 4096), (2100, 72), (64, 6176)])
-def test_quadrow_kernel(name, u, m, n, k):
+@pytest.mark.parametrize("n,k", [(520, 1024), (100, 4096), (2100, 72), (64, 6176), (4, 256)])
+def test_quadrow_kernel(name, u, qp, m, n, k):
     # the 4x4x4-MFMA kernel, forced; it is also what 3 <= M <= 8 takes by default
     s = SCHEMES[name]
     if s.bits == 3:
-        k = {1024: 1000, 4096: 4000, 72: 80, 6176: 6200}[k]  # whole, partial and odd group counts of 40
+        k = {1024: 1000, 4096: 4000, 72: 80, 6176: 6200, 256: 240}[k]  # whole, partial and odd group counts of 40
     x, qw, qs, b = _linear_case(s, m, n, k, 77 * m + n + k, bias=True)
     gq._lib.set_option("gemv_variant", 6)
     gq._lib.set_option("gemv_rows_per_wave", u)
+    gq._lib.set_option("quad_pairs", qp)
     try:
         y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
+        assert gq._lib.last_kernel().endswith(f",{qp}>"), gq._lib.last_kernel()
         y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
     finally:
         gq._lib.set_option("gemv_variant", -1)
         gq._lib.set_option("gemv_rows_per_wave", -1)
+        gq._lib.set_option("quad_pairs", -1)
     ref = o.linear_fp32(x, qw, qs, s, b)
-    assert_linear_ok(y, ref, x, k, f"quad-row {name} u={u} {m}x{n}x{k}")
-    assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"quad-row u={u} fp32 out")
+    assert_linear_ok(y, ref, x, k, f"quad-row {name} u={u} qp={qp} {m}x{n}x{k}")
+    assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"quad-row u={u} qp={qp} fp32 out")
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("waves", [-1, 8])  # 8 waves in all: every wave walks many quads
-@pytest.mark.parametrize("m,n,k", [(8, 64, 14336), (5, 520, 20520), (3, 132, 20480), (8, 520, 8200)])
-def test_quadrow_kernel_k_phases(name, waves, m, n, k):
-    # x does not fit LDS whole: K is walked in 2-3 phases with partial sums parked in LDS
+@pytest.mark.parametrize("qp", [1, 2])
+@pytest.mark.parametrize("m,n,k", [(8, 64, 14336), (5, 520, 20520), (3, 132, 20480), (8, 520, 8200), (8, 36, 14336)])
+def test_quadrow_kernel_k_phases(name, waves, qp, m, n, k):
+    # x does not fit LDS whole: K is walked in 2-3 phases with partial sums parked in LDS (N = 36: an odd number of
+    # quads, so the last item of the two-quad form holds one quad only)
     s = SCHEMES[name]
     x, qw, qs, b = _linear_case(s, m, n, k, 5 * m + n + k, bias=True)
     gq._lib.set_option("gemv_variant", 7)
     gq._lib.set_option("gemv_waves", waves)
+    gq._lib.set_option("quad_pairs", qp)
     try:
         y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b))
     finally:
         gq._lib.set_option("gemv_variant", -1)
         gq._lib.set_option("gemv_waves", -1)
-    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"quad-row phases {name} {m}x{n}x{k} waves={waves}")
+        gq._lib.set_option("quad_pairs", -1)
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"quad-row phases {name} {m}x{n}x{k} waves={waves} qp={qp}")
 
 
 @pytest.mark.parametrize("m", [9, 12, 16])
@@ -404,8 +412,9 @@ def test_quadrow_kernel_declines_odd_shapes():
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("qp", [1, 2])
 @pytest.mark.parametrize("k", [1024, 14336])
-def test_quadrow_kernel_grouped(name, k):
+def test_quadrow_kernel_grouped(name, qp, k):
     s = SCHEMES[name]
     if s.bits == 3:
         k = k // 40 * 40
@@ -416,13 +425,15 @@ def test_quadrow_kernel_grouped(name, k):
     ip = np.array([0, 2, 2, 21, 22, 40], np.int32)  # an empty expert and one with 19 rows (3 passes)
     x = rng.standard_normal((40, k)).astype(np.float16)
     gq._lib.set_option("gemv_variant", 6)
+    gq._lib.set_option("quad_pairs", qp)
     try:
         out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
         out64 = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip.astype(np.int64)), s.bits, s.group_size)
     finally:
         gq._lib.set_option("gemv_variant", -1)
+        gq._lib.set_option("quad_pairs", -1)
     ref = o.dequantize_group_gemm_fp32(x, qw, qs, ip, s)
-    assert_linear_ok(out, ref, x, k, f"grouped quad-row {name} k={k}")
+    assert_linear_ok(out, ref, x, k, f"grouped quad-row {name} qp={qp} k={k}")
     assert_linear_ok(out64, ref, x, k, f"grouped quad-row k={k} int64 indptr")
 
 
