@@ -18,7 +18,11 @@ namespace gq {
 // for few-row tiles whose MFMA work per tile is far shorter than a trip to memory
 // BF: bfloat16 model (operands and 16-bit outputs are bf16; see dequant_word4_bf16)
 // SKIP: waves leave out the 32-row blocks of their sub-tile that lie past the segment's last row
-template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false>
+// WX: extra register stages for the weights alone.  Loads return in issue order, so each iteration issues its
+// activation loads first and the weight loads (WX tiles further ahead) after them: waiting for the activations of
+// the next tile then leaves the newer weight loads in flight.  For matmuls whose weights are read once and come
+// straight from HBM (grouped, one row tile per expert) while the activations come from L2.
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false, int WX = 0>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(const GemmParams p) {
   using T = GemmTraits<BITS>;
   constexpr int G = T::G;
@@ -98,22 +102,29 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   const int k_lim = min(p.K, kt1 * BK);  // k and groups from here on contribute nothing
   const int g_lim = min(p.ng, 2 * kt1);
 
-  struct Stage {
+  struct StageA {
     uint4 a[A_CHUNKS];
+  };
+  struct StageW {
     uint4 w[W_GROUPS];
     uint32_t s[W_GROUPS];  // fp16 scale bits (32 bits wide on purpose: in flight, never re-packed)
   };
   static_assert(DEPTH >= 2 && DEPTH % 2 == 0, "register stages pair up with the two LDS stages");
-  Stage r[DEPTH];
+  constexpr int WD = DEPTH + WX;
+  static_assert(WD % DEPTH == 0, "the unrolled loop walks whole rounds of both register rings");
+  StageA ra[DEPTH];
+  StageW rw[WD];
 
   // K tile kt into registers.  Always valid addresses; validity is re-derived at store time.
-  auto load_tile = [&](int kt, Stage& st) {
+  auto load_a = [&](int kt, StageA& st) {
     const int k_base = kt * BK;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const bool ok = k_base + a_k[i] < k_lim;  // K % 8 == 0: a chunk is entirely inside or outside
       st.a[i] = *reinterpret_cast<const uint4*>(ok ? a_src[i] + k_base : a_src[i]);
     }
+  };
+  auto load_w = [&](int kt, StageW& st) {
     if (w_active) {
 #pragma unroll
       for (int i = 0; i < W_GROUPS; ++i) {
@@ -127,7 +138,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // One of KSTEPS slices of "tile kt: registers -> LDS stage s".  The slices are issued between the
   // MFMA k-steps of the tile being multiplied, so that dequantisation (VALU) and the LDS stores
   // run in the shadow of the matrix pipe instead of after it.
-  auto store_part = [&](int kt, const Stage& st, int s, int part) {
+  auto store_part = [&](int kt, const StageA& sa, const StageW& st, int s, int part) {
     uint16_t* at = a_tile(s);
     uint16_t* wt = w_tile(s);
     const int k_base = kt * BK;
@@ -136,7 +147,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
       if (i % KSTEPS != part) continue;
       const bool ok = a_row_ok[i] && (k_base + a_k[i] < k_lim);
       if (A_EXACT || a_in_tile[i])
-        *reinterpret_cast<uint4*>(at + a_dst[i]) = ok ? st.a[i] : make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4*>(at + a_dst[i]) = ok ? sa.a[i] : make_uint4(0, 0, 0, 0);
     }
     if (!w_active) return;
 #pragma unroll
@@ -165,9 +176,9 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
       }
     }
   };
-  auto store_tile = [&](int kt, const Stage& st, int s) {
+  auto store_tile = [&](int kt, const StageA& sa, const StageW& st, int s) {
 #pragma unroll
-    for (int part = 0; part < KSTEPS; ++part) store_part(kt, st, s, part);
+    for (int part = 0; part < KSTEPS; ++part) store_part(kt, sa, st, s, part);
   };
 
   float16_t acc[TM][TN];
@@ -182,7 +193,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // MFMAs of the tile in stage s; slice ks of the next tile's store is issued after k-step ks
   // full: every 32-row block of the wave is live (the straight-line form); otherwise blocks >= live are skipped by
   // wave-uniform branches, fragments and all
-  auto mfma_tile = [&](auto full, int s, int kt_store, const Stage& st_store) {
+  auto mfma_tile = [&](auto full, int s, int kt_store, const StageA& sa_store, const StageW& st_store) {
     constexpr bool FULL = decltype(full)::value;
     const uint16_t* at = a_tile(s) + (wm0 + frag_row) * LDA + frag_k;
     const uint16_t* wt = w_tile(s) + (wn0 + frag_row) * LDA + frag_k;
@@ -221,7 +232,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
           }
         }
-        store_part(kt_store, st_store, s ^ 1, ks);
+        store_part(kt_store, sa_store, st_store, s ^ 1, ks);
         __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
       }
     }
@@ -230,18 +241,22 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // ---- pipeline: tile t in LDS stage t&1, tile t+1 in registers, tile t+2 in flight
   // ---- pipeline: tile t in LDS stage t&1, tiles t+1 .. t+DEPTH-1 in registers, tile t+DEPTH in flight
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d) load_tile(kt0 + d, r[d]);
-  store_tile(kt0, r[0], 0);
-  load_tile(kt0 + DEPTH, r[0]);
+  for (int d = 0; d < DEPTH; ++d) load_a(kt0 + d, ra[d]);
+#pragma unroll
+  for (int d = 0; d < WD; ++d) load_w(kt0 + d, rw[d]);
+  store_tile(kt0, ra[0], rw[0], 0);
+  load_a(kt0 + DEPTH, ra[0]);
+  load_w(kt0 + WD, rw[0]);
   __syncthreads();
   // (a register stage is refilled right after the MFMA/store block that drains it; a tile past
   //  the end is stored as zeros and adds nothing)
   auto k_loop = [&](auto full) {
-    for (int kt = kt0; kt < kt1; kt += DEPTH) {
+    for (int kt = kt0; kt < kt1; kt += WD) {
 #pragma unroll
-      for (int d = 0; d < DEPTH; ++d) {
-        mfma_tile(full, d & 1, kt + d + 1, r[(d + 1) % DEPTH]);
-        load_tile(kt + d + 1 + DEPTH, r[(d + 1) % DEPTH]);
+      for (int d = 0; d < WD; ++d) {
+        mfma_tile(full, d & 1, kt + d + 1, ra[(d + 1) % DEPTH], rw[(d + 1) % WD]);
+        load_a(kt + d + 1 + DEPTH, ra[(d + 1) % DEPTH]);
+        load_w(kt + d + 1 + WD, rw[(d + 1) % WD]);
         __syncthreads();
       }
     }
@@ -320,12 +335,12 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   }
 }
 
-template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false>
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false, int WX = 0>
 static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr int BK = 2 * GemmTraits<BITS>::G;
   constexpr int LDA = BK + 8;
   constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
-  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP>;
+  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP, WX>;
   if (lds > 65536) {
     const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
     if (e != hipSuccess) return e;
@@ -337,8 +352,8 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr int PB = ((WN / 32) % 2 == 0) ? 32 : 16;
   const int n_cols = p.paired ? ((p.N / 2 + PB - 1) / PB) * 2 * PB : p.N;
   const dim3 grid((n_cols + BN - 1) / BN, m_tiles, split);
-  note_kernel("gq::gemm_pipe_kernel<%d,%d,%d,%d,%d,%d,%s,%s>", BITS, BM, BN, WM, WN, DEPTH, BF ? "true" : "false",
-              SKIP ? "true" : "false");
+  note_kernel("gq::gemm_pipe_kernel<%d,%d,%d,%d,%d,%d,%s,%s,%d>", BITS, BM, BN, WM, WN, DEPTH, BF ? "true" : "false",
+              SKIP ? "true" : "false", WX);
   hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
   return hipGetLastError();
 }
@@ -532,7 +547,9 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     const bool wide = variant == 10 || (variant != 11 && bits == 4 && mt * ((p.N + 255) / 256) >= 512);
     if (bits == 4) {
       if (wide) return launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true>(p, s);
-      return launch_pipe_cfg<4, 256, 128, 64, 64, 2, false, true>(p, s);
+      // the narrow tile has registers to spare: its weight loads run two more K tiles ahead (Mixtral's e2 at 64 / 128 /
+      // 256 rows per expert: 201 -> 177, 236 -> 213, 320 -> 305 us; the wide tile spills with them and loses)
+      return launch_pipe_cfg<4, 256, 128, 64, 64, 2, false, true, 2>(p, s);
     }
     return launch_pipe_cfg<3, 256, 128, 64, 64, 2, false, true>(p, s);
   }
