@@ -43,6 +43,9 @@ struct GemmParams {
   const int32_t* x_rows;  // null, or the row of x each activation row reads (int32 [rows])
   int x_src_rows;         // rows of x when x_rows is set
   int bf16;               // x, q_scale, bias and a 16-bit y are bfloat16 (q4bf16_* models), not float16
+  // columns (in tile order) this launch covers: [n_begin, n_end), n_end = 0 for all; a launch can leave the columns
+  // of its last, partly filled round of workgroups to a second launch with another tile
+  int n_begin = 0, n_end = 0;
 };
 
 // column c of the block-interleaved order above -> stored weight row (clamped into its half).

@@ -58,7 +58,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // 32-row blocks of this wave that hold rows of the segment: the others are skipped by the matrix core
   // (SKIP; a ragged expert segment or a last row tile leaves most of a tall tile empty)
   const int live = SKIP ? min(TM, max(0, (seg_hi - (m0 + wm0) + 31) / 32)) : TM;
-  const int n0 = blockIdx.x * BN;
+  const int n0 = p.n_begin + blockIdx.x * BN;
   const uint32_t* qw = p.qw + expert * p.expert_w_stride;
   const uint16_t* qs = p.qs + expert * p.expert_s_stride;
 
@@ -351,7 +351,9 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   // the fused gate/up form walks whole 64-column blocks (32 gate + 32 up rows)
   constexpr int PB = ((WN / 32) % 2 == 0) ? 32 : 16;
   const int n_cols = p.paired ? ((p.N / 2 + PB - 1) / PB) * 2 * PB : p.N;
-  const dim3 grid((n_cols + BN - 1) / BN, m_tiles, split);
+  const int n_last = p.n_end > 0 ? p.n_end : n_cols;
+  if (n_last <= p.n_begin) return hipSuccess;
+  const dim3 grid((n_last - p.n_begin + BN - 1) / BN, m_tiles, split);
   note_kernel("gq::gemm_pipe_kernel<%d,%d,%d,%d,%d,%d,%s,%s,%d>", BITS, BM, BN, WM, WN, DEPTH, BF ? "true" : "false",
               SKIP ? "true" : "false", WX);
   hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
@@ -546,7 +548,25 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
     const int64_t mt = p.rows / 256 + p.num_experts;
     const bool wide = variant == 10 || (variant != 11 && bits == 4 && mt * ((p.N + 255) / 256) >= 512);
     if (bits == 4) {
-      if (wide) return launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true>(p, s);
+      if (wide) {
+        // A last round of workgroups that is at most about half full costs a whole round here (the kernel waits on
+        // memory, not on the matrix pipe): its columns go to a second launch on the narrow tile, whose workgroups take
+        // half as long.  (Mixtral's e1_e3, 112 column tiles x 8 experts = 3.5 rounds of 256.)
+        const int64_t tiles_x = (p.N + 255) / 256;
+        const int64_t live = p.num_experts > p.rows / 256 ? p.num_experts : p.rows / 256;  // row tiles that hold rows
+        const int64_t rounds = tiles_x * live / 256, rest = tiles_x * live % 256;
+        if (variant != 10 && rounds >= 1 && rest > 0 && rest <= 144 && p.n_end == 0 && p.n_begin == 0) {
+          GemmParams a = p, b = p;
+          a.n_end = static_cast<int>(rounds * 256 / live * 256);
+          b.n_begin = a.n_end;
+          if (a.n_end > 0 && a.n_end < p.N) {
+            const hipError_t e = launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true>(a, s);
+            if (e != hipSuccess) return e;
+            return launch_pipe_cfg<4, 256, 128, 64, 64, 2, false, true, 2>(b, s);
+          }
+        }
+        return launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true>(p, s);
+      }
       // the narrow tile has registers to spare: its weight loads run two more K tiles ahead (Mixtral's e2 at 64 / 128 /
       // 256 rows per expert: 201 -> 177, 236 -> 213, 320 -> 305 us; the wide tile spills with them and loses)
       return launch_pipe_cfg<4, 256, 128, 64, 64, 2, false, true, 2>(p, s);

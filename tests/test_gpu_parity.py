@@ -841,6 +841,37 @@ def test_moe_group_gemm_tall_tiles_on_ragged_segments(name, variant):
     assert_linear_ok(gathered, o.dequantize_group_gemm_fp32(src[idx], qw, qs, ip, s), src[idx], k, "gathered")
 
 
+def test_moe_group_gemm_last_round_on_the_narrow_tile():
+    """A grouped matmul wide enough for more than one round of 256 x 256 workgroups leaves the columns of a last round
+    that is at most about half full to a second launch on the 256 x 128 tile (8 experts x 36 column tiles = 288
+    workgroups: 32 full column tiles, then 4 x 2 narrow ones).  Same bits as the single launch, plain and with the
+    folded activation (whose column order interleaves gate and up blocks)."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(67)
+    counts = [70, 64, 100, 65, 90, 128, 66, 77]
+    ne, n, k = len(counts), 9216, 64
+    ip = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(ip[-1])
+    qw = rng.integers(0, 2**32, (ne, n, k // 8), dtype=np.uint64).astype(np.uint32)
+    qs = (rng.random((ne, n, k // 32)) * 0.01 + 0.001).astype(np.float16)
+    x = rng.standard_normal((rows, k)).astype(np.float16)
+    out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), 4, 32)
+    assert gq._lib.last_kernel().startswith("gq::gemm_pipe_kernel<4,256,128,"), gq._lib.last_kernel()  # the second launch
+    fused = ops.moe_experts(dev(x), None, dev(qw), dev(qs), dev(ip), 4, 32, silu_mul_halves=True)
+    gq._lib.set_option("gemm_variant", 10)
+    try:
+        one = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), 4, 32)
+        assert gq._lib.last_kernel().startswith("gq::gemm_pipe_kernel<4,256,256,"), gq._lib.last_kernel()
+        fused_one = ops.moe_experts(dev(x), None, dev(qw), dev(qs), dev(ip), 4, 32, silu_mul_halves=True)
+    finally:
+        gq._lib.set_option("gemm_variant", -1)
+    assert torch.equal(out, one) and torch.equal(fused, fused_one)
+    sel = rng.choice(n, 96, replace=False)
+    sel[:4] = [0, 8191, 8192, n - 1]  # both sides of the seam
+    ref = o.dequantize_group_gemm_fp32(x, qw[:, sel], qs[:, sel], ip, s)
+    assert_linear_ok(out[:, torch.from_numpy(sel).to(out.device)], ref, x, k, "grouped, last round on the narrow tile")
+
+
 def test_silu_mul_and_combine():
     rng = np.random.default_rng(47)
     x = (rng.standard_normal((5, 192)) * 3).astype(np.float16)
