@@ -150,6 +150,9 @@ int mi355gq_testing_set_option(const char* name, int value) {
   if (!strcmp(name, "gemv_rows_per_wave")) {
     GQ_REQUIRE(value == -1 || value == 1 || value == 2 || value == 4 || value == 8, "gemv_rows_per_wave=%d (1, 2, 4, 8)", value);
     o.gemv_rows_per_wave = value;
+  } else if (!strcmp(name, "gemm_fast_loop")) {
+    GQ_REQUIRE(value == -1 || value == 0, "gemm_fast_loop=%d (0)", value);
+    o.gemm_fast_loop = value;
   } else if (!strcmp(name, "quad_pairs")) {
     GQ_REQUIRE(value == -1 || value == 1 || value == 2, "quad_pairs=%d (1, 2)", value);
     o.quad_pairs = value;

@@ -215,6 +215,12 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   p.paired = a.paired;
   p.x_rows = a.x_rows; p.x_src_rows = static_cast<int>(a.x_src_rows);
   p.bf16 = a.bf16;
+  {
+    const int64_t x_rows_total = a.x_rows != nullptr ? a.x_src_rows : a.rows;
+    const int64_t limit = int64_t(1) << 32;
+    p.fast_ok = a.K % (2 * a.group_size) == 0 && x_rows_total * a.K * 2 < limit && a.N * p.nw * 4 < limit &&
+                options().gemm_fast_loop != 0;  // (tuning / test override: general loop only)
+  }
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int variant = options().gemm_variant;
   if (variant < 0 || a.bf16) {

@@ -46,6 +46,9 @@ struct GemmParams {
   // columns (in tile order) this launch covers: [n_begin, n_end), n_end = 0 for all; a launch can leave the columns
   // of its last, partly filled round of workgroups to a second launch with another tile
   int n_begin = 0, n_end = 0;
+  // every byte offset into x, one expert's q_weight and q_scale fits 32 bits, and K is whole K tiles of two groups
+  // (set by the launcher; lets interior workgroups address with a uniform base plus a 32-bit lane offset)
+  int fast_ok = 0;
 };
 
 // column c of the block-interleaved order above -> stored weight row (clamped into its half).

@@ -438,16 +438,43 @@ def test_quadrow_kernel_grouped(name, qp, k):
 
 
 @pytest.mark.parametrize("variant", [3, 4, 6, 7, 9])  # plain 128/256 tiles, pipelined 128/256 tiles, pipelined 128x256
-@pytest.mark.parametrize("m,n,k", [(300, 512, 1024), (17, 260, 4096), (513, 300, 192)])
-def test_gemm_kernel_variants(variant, m, n, k):
+@pytest.mark.parametrize("fast_loop", [-1, 0])  # the K loop without zero-selects where K allows it / the general loop always
+@pytest.mark.parametrize("m,n,k", [(300, 512, 1024), (17, 260, 4096), (513, 300, 192), (130, 100, 128), (257, 129, 64)])
+def test_gemm_kernel_variants(variant, fast_loop, m, n, k):
+    # ragged rows and columns on every tile, K of whole K tiles (both loops apply) and the general loop forced
     s = SCHEMES["q4f16_1"]
     x, qw, qs, b = _linear_case(s, m, n, k, variant * 1000 + m + n + k, bias=True)
     gq._lib.set_option("gemm_variant", variant)
+    gq._lib.set_option("gemm_fast_loop", fast_loop)
     try:
         y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b))
     finally:
         gq._lib.set_option("gemm_variant", -1)
-    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"gemm variant {variant} {m}x{n}x{k}")
+        gq._lib.set_option("gemm_fast_loop", -1)
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"gemm variant {variant} fast_loop {fast_loop} {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("m", [17, 64, 100, 300, 1100])
+def test_gemm_fast_and_general_loop_agree_bit_for_bit(name, m):
+    """The K loop without zero-selects (K of whole K tiles) against the general loop on the same launch shape: identical
+    bits, on ragged rows and columns, with bias + residual, float32 output, the folded activation and split K."""
+    s = SCHEMES[name]
+    n, k = 1060, 16 * s.group_size
+    x, qw, qs, b = _linear_case(s, m, n, k, 31 * m + n, bias=True)
+    res = np.random.default_rng(m).standard_normal((m, n)).astype(np.float16)
+    outs = []
+    for fast_loop in (-1, 0):
+        gq._lib.set_option("gemm_fast_loop", fast_loop)
+        try:
+            outs.append((ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b), residual=dev(res)),
+                         ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32),
+                         ops.linear_silu_mul(dev(x), dev(qw), dev(qs), s.bits, s.group_size)))
+        finally:
+            gq._lib.set_option("gemm_fast_loop", -1)
+    for a, c in zip(*outs):
+        assert torch.equal(a, c)
+    assert_linear_ok(outs[0][1], o.linear_fp32(x, qw, qs, s), x, k, f"fast loop {name} m={m}")
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
@@ -817,7 +844,7 @@ def test_moe_group_gemm_tall_tiles_on_ragged_segments(name, variant):
         pytest.skip("q3 has no 256 x 256 tile (its K tile does not fit LDS)")
     rng = np.random.default_rng(61)
     counts = [300, 0, 129, 33, 1, 127, 32, 31]
-    ne, n, k = len(counts), 520, 512 if s.bits == 4 else 520
+    ne, n, k = len(counts), 520, 512 if s.bits == 4 else 480
     ip = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
     rows = int(ip[-1])
     w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
@@ -833,10 +860,13 @@ def test_moe_group_gemm_tall_tiles_on_ragged_segments(name, variant):
         out64 = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip.astype(np.int64)), s.bits, s.group_size)
         fused = ops.moe_experts(dev(x), None, dev(qw), dev(qs), dev(ip), s.bits, s.group_size, silu_mul_halves=True)
         gathered = ops.moe_experts(dev(src), dev(idx), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
+        gq._lib.set_option("gemm_fast_loop", 0)  # the general K loop (this K is whole K tiles: the other one ran above)
+        general = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
     finally:
         gq._lib.set_option("gemm_variant", -1)
+        gq._lib.set_option("gemm_fast_loop", -1)
     assert_linear_ok(out, ref, x, k, f"grouped tall tiles {name} variant {variant}")
-    assert torch.equal(out, base) and torch.equal(out64, out)
+    assert torch.equal(out, base) and torch.equal(out64, out) and torch.equal(general, out)
     assert torch.equal(fused, ops.silu_mul(out))
     assert_linear_ok(gathered, o.dequantize_group_gemm_fp32(src[idx], qw, qs, ip, s), src[idx], k, "gathered")
 
