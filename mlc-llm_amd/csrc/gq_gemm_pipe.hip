@@ -44,8 +44,10 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
 
   extern __shared__ uint4 smem[];
   uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
-  auto a_tile = [&](int s) { return lds + s * (BM + BN) * LDA; };
-  auto w_tile = [&](int s) { return lds + s * (BM + BN) * LDA + BM * LDA; };
+  // [A stage 0][A stage 1][W stage 0][W stage 1]: the two stages of an operand lie less than 64 KiB apart, so a
+  // stage is an immediate offset of the LDS instruction and both share one address register
+  auto a_tile = [&](int s) { return lds + s * BM * LDA; };
+  auto w_tile = [&](int s) { return lds + 2 * BM * LDA + s * BN * LDA; };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -73,7 +75,11 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     const int idx_raw = tid + NT * i;
     a_in_tile[i] = A_EXACT || idx_raw < BM * CPR;
     const int idx = a_in_tile[i] ? idx_raw : 0;
-    const int r = idx / CPR, c = idx - r * CPR;
+    // (q4: a thread's chunks sit NT / CPR rows apart in the same column, written out so that their LDS addresses
+    //  become one register plus constants instead of a register each)
+    constexpr bool AFFINE = A_EXACT && NT % CPR == 0;
+    const int r = AFFINE ? tid / CPR + i * (NT / CPR) : idx / CPR;
+    const int c = AFFINE ? tid % CPR : idx - r * CPR;
     a_row_ok[i] = m0 + r < seg_hi;
     a_k[i] = 8 * c;
     a_src[i] = p.x + x_row(p.x_rows, p.x_src_rows, a_row_ok[i] ? m0 + r : m0) * p.K + 8 * c;
@@ -92,7 +98,10 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     w_src[i] = qw + static_cast<int64_t>(row) * p.nw;
     s_src[i] = qs + static_cast<int64_t>(row) * p.ng;
     w_g[i] = gsel;
-    w_dst[i] = r * LDA + gsel * G;
+    // (offset from the start of LDS, made opaque: left to itself the compiler folds the W region's 72 KiB into the
+    //  constants, finds them past the 64 KiB an LDS instruction's immediate holds, and keeps a register per store)
+    w_dst[i] = 2 * BM * LDA + r * LDA + gsel * G;
+    asm volatile("" : "+v"(w_dst[i]));
   }
 
   // When K is whole K tiles and whole rounds of the register rings, and all byte offsets are below 4 GiB (`fast_ok` from
@@ -109,9 +118,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     w_off[i] = static_cast<uint32_t>(reinterpret_cast<const char*>(w_src[i] + 4 * w_g[i]) - reinterpret_cast<const char*>(qw));
     s_off[i] = static_cast<uint32_t>(reinterpret_cast<const char*>(s_src[i] + w_g[i]) - reinterpret_cast<const char*>(qs));
   }
-  // (not on the 256 x 256 tile, which is out of registers: measured 5-10 % slower there, against 8-37 % faster on the
-  //  smaller tiles)
-  constexpr bool FASTABLE = !(BM == 256 && BN == 256);
+  // (3-4 % on the 256 x 256 tile, 8-37 % on the smaller ones, which have fewer MFMAs per dequantised weight)
+  constexpr bool FASTABLE = true;
   const bool fast = FASTABLE && p.fast_ok;
 
   // this workgroup's share of K (all of it unless the launch splits K)
@@ -177,7 +185,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   auto store_part = [&](auto fast_path, int kt, const StageA& sa, const StageW& st, int s, int part) {
     constexpr bool FAST = decltype(fast_path)::value;
     uint16_t* at = a_tile(s);
-    uint16_t* wt = w_tile(s);
+    uint16_t* wt = lds + s * BN * LDA;  // (w_dst holds the offset of the W region)
     const int k_base = kt * BK;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
@@ -234,6 +242,13 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     constexpr bool FULL = decltype(full)::value;
     const uint16_t* at = a_tile(s) + (wm0 + frag_row) * LDA + frag_k;
     const uint16_t* wt = w_tile(s) + (wn0 + frag_row) * LDA + frag_k;
+    auto mma = [&](const half8_t& av, const half8_t& bv, float16_t& c) {
+      if constexpr (BF)
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, bv), c,
+                                                    0, 0, 0);
+      else
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c, 0, 0, 0);
+    };
     {  // fragments of k-step s+1 are read while the MFMAs of step s run
       half8_t af[2][TM], bf[2][TN];
 #pragma unroll
@@ -260,13 +275,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
         for (int i = 0; i < TM; ++i) {
           if (FULL || i < live) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-              if constexpr (BF)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, af[cur][i]),
-                                                                    __builtin_bit_cast(bf16x8_t, bf[cur][j]), acc[i][j],
-                                                                    0, 0, 0);
-              else
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[cur][i], bf[cur][j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < TN; ++j) mma(af[cur][i], bf[cur][j], acc[i][j]);
           }
         }
         store_part(fast_path, kt_store, sa_store, st_store, s ^ 1, ks);
