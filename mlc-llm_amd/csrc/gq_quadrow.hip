@@ -87,7 +87,9 @@ __device__ __forceinline__ float4_t mfma4_bf16(uint32_t a0, uint32_t a1, uint32_
 // consecutive quads, so the LDS bytes read per weight byte fall by that factor (a 4x4x4 block needs as many
 // operand bytes of x as of weights: with 8 activation rows that is 8 LDS bytes per packed weight byte at QP = 1).
 template <int BITS, int NBQ, int U, int MODE, bool BF = false, int QP = 1>
-__global__ __launch_bounds__((U * QP <= 2 && !(QP > 1 && MODE == 1)) ? 1024 : 512) void quad_kernel(const QuadParams p) {
+// (sixteen-wave workgroups exist for the forms that fit 128 registers: 2 KiB items without the bias / residual loads;
+//  with them the same bound forced spill reloads into the walk, and a reload waits for every weight load in flight)
+__global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_kernel(const QuadParams p) {
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;  // 2: fused gate/up form, quad = 2 (gate, up) pairs
   constexpr uint32_t kMagic = BF ? 0x43004300u : 0x64006400u;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
@@ -573,10 +575,8 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
     const int64_t wgs = static_cast<int64_t>(((p.nsets + p.rounds - 1) / p.rounds + 7) / 8) * busy * mtiles;
     if (2 * wgs <= 256) threads = 256;  // (the doubled count must still be one round of workgroups)
   }
-  // four waves per SIMD share one copy of x (the instances that fit 128 registers: 2 KiB items without bias / residual loads
-  // when two quads share an item)
-  if (big_wg && p.nphases == 1 && U * QP <= 2 && !(QP > 1 && (a.bias != nullptr || a.residual != nullptr)))
-    threads = 1024;
+  // four waves per SIMD share one copy of x (the instances that fit 128 registers: 2 KiB items without bias / residual loads)
+  if (big_wg && p.nphases == 1 && U * QP <= 2 && a.bias == nullptr && a.residual == nullptr) threads = 1024;
   const int wpb = threads / 64;
   const size_t lds = lds_x + (p.nphases > 1 ? static_cast<size_t>(wpb) * p.rounds * QP * nbq * 64 : 0);
   const int blocks = ((p.nsets + p.rounds - 1) / p.rounds + wpb - 1) / wpb;
