@@ -227,13 +227,17 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
       }
     }
   };
+  // (the scheduling barriers keep each refill ahead of the next set's arithmetic: left alone, the scheduler starts that
+  //  arithmetic first, and its wait for the set in flight then also holds back the refill: one set in flight, not two)
   while (set_a < nsets) {
     reduce(set_a, wa, sa, ba);
     set_a += 2 * nwaves;
     issue(set_a, wa, sa, ba);
+    __builtin_amdgcn_sched_barrier(0);
     reduce(set_b, wb, sb, bb);  // past the end: rows >= N, nothing is stored
     set_b += 2 * nwaves;
     issue(set_b, wb, sb, bb);
+    __builtin_amdgcn_sched_barrier(0);
   }
 }
 
