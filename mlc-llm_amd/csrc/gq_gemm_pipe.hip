@@ -22,7 +22,16 @@ namespace gq {
 // activation loads first and the weight loads (WX tiles further ahead) after them: waiting for the activations of
 // the next tile then leaves the newer weight loads in flight.  For matmuls whose weights are read once and come
 // straight from HBM (grouped, one row tile per expert) while the activations come from L2.
-template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false, int WX = 0>
+// FAST: K is whole K tiles and whole rounds of the register rings, and every byte offset is below 4 GiB (checked by the
+// launcher).  The K loop then has no zero-selects and no clamps, and loads through buffer descriptors (tensor in scalar
+// registers, K tile as the scalar offset, one 32-bit lane offset): 122 -> 62 VALU instructions per wave and K tile.  Rows
+// past the segment and columns past N need no zeros: their loads are clamped to valid rows when the offsets are set up, a
+// row of x or of W only ever reaches its own row or column of the result, and the epilogue drops those; only k past K
+// would reach live results, and in this form there is none.  A separate instantiation rather than a branch: the general
+// form's addresses and flags would otherwise stay in registers next to this one's, and the large tile has none to spare
+// (a spill reload inside the loop waits for every global load in flight).
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false, int WX = 0,
+          bool FAST = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(const GemmParams p) {
   using T = GemmTraits<BITS>;
   constexpr int G = T::G;
@@ -104,11 +113,6 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     asm volatile("" : "+v"(w_dst[i]));
   }
 
-  // When K is whole K tiles and whole rounds of the register rings, and all byte offsets are below 4 GiB (`fast_ok` from
-  // the host), the K loop runs a copy without the zero-selects and clamps of the general one, with addresses of the
-  // form uniform base + 32-bit lane offset (122 -> 74 VALU instructions per wave and K tile).  Rows past the segment and
-  // columns past N need no zeros: their loads are clamped to valid rows, a row of x or of W only ever reaches its own
-  // row or column of the result, and the epilogue drops those; only k past K would reach live results, and there is none.
   uint32_t a_off[A_CHUNKS], w_off[W_GROUPS], s_off[W_GROUPS];
 #pragma unroll
   for (int i = 0; i < A_CHUNKS; ++i)
@@ -118,9 +122,6 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     w_off[i] = static_cast<uint32_t>(reinterpret_cast<const char*>(w_src[i] + 4 * w_g[i]) - reinterpret_cast<const char*>(qw));
     s_off[i] = static_cast<uint32_t>(reinterpret_cast<const char*>(s_src[i] + w_g[i]) - reinterpret_cast<const char*>(qs));
   }
-  // (3-4 % on the 256 x 256 tile, 8-37 % on the smaller ones, which have fewer MFMAs per dequantised weight)
-  constexpr bool FASTABLE = true;
-  const bool fast = FASTABLE && p.fast_ok;
 
   // this workgroup's share of K (all of it unless the launch splits K)
   const int nk = (p.ng + 1) / 2;
@@ -143,24 +144,36 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   StageW rw[WD];
 
   // K tile kt into registers.  Always valid addresses; validity is re-derived at store time.
+  // (buffer loads: the descriptor of each tensor sits in scalar registers, the K tile is the scalar offset and the lane
+  //  offset one 32-bit register, so no 64-bit address is formed or kept per load)
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.x), short(0), -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(qw), short(0), -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(qs), short(0), -1, 0x00020000);
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   auto load_a_fast = [&](int kt, StageA& st) {  // (tiles past the end re-read the last one: never multiplied)
-    const char* base = reinterpret_cast<const char*>(p.x) + static_cast<int64_t>(min(kt, kt1 - 1)) * (BK * 2);
+    const int soff = min(kt, kt1 - 1) * (BK * 2);
 #pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) st.a[i] = *reinterpret_cast<const uint4*>(base + a_off[i]);
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, static_cast<int>(a_off[i]), soff, 0);
+      st.a[i] = make_uint4(v.x, v.y, v.z, v.w);
+    }
   };
   auto load_w_fast = [&](int kt, StageW& st) {
     if (w_active) {
       const int ktc = min(kt, kt1 - 1);
-      const char* wb = reinterpret_cast<const char*>(qw) + static_cast<int64_t>(ktc) * 32;
-      const char* sb = reinterpret_cast<const char*>(qs) + static_cast<int64_t>(ktc) * 4;
 #pragma unroll
       for (int i = 0; i < W_GROUPS; ++i) {
-        st.w[i] = *reinterpret_cast<const uint4*>(wb + w_off[i]);
-        st.s[i] = *reinterpret_cast<const uint16_t*>(sb + s_off[i]);
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, static_cast<int>(w_off[i]), ktc * 32, 0);
+        st.w[i] = make_uint4(v.x, v.y, v.z, v.w);
+        st.s[i] = __builtin_amdgcn_raw_buffer_load_b16(s_rsrc, static_cast<int>(s_off[i]), ktc * 4, 0);
       }
     }
   };
   auto load_a = [&](int kt, StageA& st) {
+    if constexpr (FAST) {
+      load_a_fast(kt, st);
+      return;
+    }
     const int k_base = kt * BK;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
@@ -169,6 +182,10 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     }
   };
   auto load_w = [&](int kt, StageW& st) {
+    if constexpr (FAST) {
+      load_w_fast(kt, st);
+      return;
+    }
     if (w_active) {
 #pragma unroll
       for (int i = 0; i < W_GROUPS; ++i) {
@@ -182,17 +199,20 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // One of KSTEPS slices of "tile kt: registers -> LDS stage s".  The slices are issued between the
   // MFMA k-steps of the tile being multiplied, so that dequantisation (VALU) and the LDS stores
   // run in the shadow of the matrix pipe instead of after it.
-  auto store_part = [&](auto fast_path, int kt, const StageA& sa, const StageW& st, int s, int part) {
-    constexpr bool FAST = decltype(fast_path)::value;
+  auto store_part = [&](int kt, const StageA& sa, const StageW& st, int s, int part) {
     uint16_t* at = a_tile(s);
     uint16_t* wt = lds + s * BN * LDA;  // (w_dst holds the offset of the W region)
     const int k_base = kt * BK;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       if (i % KSTEPS != part) continue;
-      const bool ok = FAST || (a_row_ok[i] && (k_base + a_k[i] < k_lim));
+      // (the zero for rows past the segment and k past K as an AND with a lane mask: written as a select of the four
+      //  words it becomes a branch around four moves, and control flow inside the loop makes the wait-count insertion
+      //  drain every load in flight at the loop header)
+      const uint32_t keep = (FAST || (a_row_ok[i] && (k_base + a_k[i] < k_lim))) ? 0xffffffffu : 0u;
       if (A_EXACT || a_in_tile[i])
-        *reinterpret_cast<uint4*>(at + a_dst[i]) = ok ? sa.a[i] : make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4*>(at + a_dst[i]) =
+            FAST ? sa.a[i] : make_uint4(sa.a[i].x & keep, sa.a[i].y & keep, sa.a[i].z & keep, sa.a[i].w & keep);
     }
     if (!w_active) return;
 #pragma unroll
@@ -223,7 +243,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   };
   auto store_tile = [&](int kt, const StageA& sa, const StageW& st, int s) {
 #pragma unroll
-    for (int part = 0; part < KSTEPS; ++part) store_part(std::false_type{}, kt, sa, st, s, part);
+    for (int part = 0; part < KSTEPS; ++part) store_part(kt, sa, st, s, part);
   };
 
   float16_t acc[TM][TN];
@@ -238,7 +258,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // MFMAs of the tile in stage s; slice ks of the next tile's store is issued after k-step ks
   // full: every 32-row block of the wave is live (the straight-line form); otherwise blocks >= live are skipped by
   // wave-uniform branches, fragments and all
-  auto mfma_tile = [&](auto full, auto fast_path, int s, int kt_store, const StageA& sa_store, const StageW& st_store) {
+  auto mfma_tile = [&](auto full, int s, int kt_store, const StageA& sa_store, const StageW& st_store) {
     constexpr bool FULL = decltype(full)::value;
     const uint16_t* at = a_tile(s) + (wm0 + frag_row) * LDA + frag_k;
     const uint16_t* wt = w_tile(s) + (wn0 + frag_row) * LDA + frag_k;
@@ -249,7 +269,39 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
       else
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c, 0, 0, 0);
     };
-    {  // fragments of k-step s+1 are read while the MFMAs of step s run
+    if constexpr (TM == 4) {
+      // Four row blocks per wave: the kernel runs close to the 256-register limit, and a spill reload inside this loop
+      // would wait for every global load in flight.  The activation fragments therefore live in ONE set of registers:
+      // block i of the next k-step is read right after the MFMAs that used block i of this one (six MFMAs ahead of its
+      // own use); only the weight fragments are double-buffered (same speed as two sets, 16 registers fewer).
+      half8_t af[TM], bf[2][TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        if (FULL || i < live) af[i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA);
+      if (FULL || live > 0) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA);
+      }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        if (ks + 1 < KSTEPS && (FULL || live > 0)) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            bf[nxt][j] = *reinterpret_cast<const half8_t*>(wt + j * 32 * LDA + (ks + 1) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          if (FULL || i < live) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j) mma(af[i], bf[cur][j], acc[i][j]);
+            if (ks + 1 < KSTEPS) af[i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA + (ks + 1) * 16);
+          }
+        }
+        store_part(kt_store, sa_store, st_store, s ^ 1, ks);
+        __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
+      }
+    } else {  // fragments of k-step s+1 are read while the MFMAs of step s run
       half8_t af[2][TM], bf[2][TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -278,7 +330,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
             for (int j = 0; j < TN; ++j) mma(af[cur][i], bf[cur][j], acc[i][j]);
           }
         }
-        store_part(fast_path, kt_store, sa_store, st_store, s ^ 1, ks);
+        store_part(kt_store, sa_store, st_store, s ^ 1, ks);
         __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
       }
     }
@@ -296,32 +348,19 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   __syncthreads();
   // (a register stage is refilled right after the MFMA/store block that drains it; a tile past
   //  the end is stored as zeros and adds nothing)
-  auto k_loop = [&](auto full, auto fast_path) {
-    constexpr bool FAST = decltype(fast_path)::value;
+  auto k_loop = [&](auto full) {
     for (int kt = kt0; kt < kt1; kt += WD) {
 #pragma unroll
       for (int d = 0; d < WD; ++d) {
-        mfma_tile(full, fast_path, d & 1, kt + d + 1, ra[(d + 1) % DEPTH], rw[(d + 1) % WD]);
-        if constexpr (FAST) {
-          load_a_fast(kt + d + 1 + DEPTH, ra[(d + 1) % DEPTH]);
-          load_w_fast(kt + d + 1 + WD, rw[(d + 1) % WD]);
-        } else {
-          load_a(kt + d + 1 + DEPTH, ra[(d + 1) % DEPTH]);
-          load_w(kt + d + 1 + WD, rw[(d + 1) % WD]);
-        }
+        mfma_tile(full, d & 1, kt + d + 1, ra[(d + 1) % DEPTH], rw[(d + 1) % WD]);
+        load_a(kt + d + 1 + DEPTH, ra[(d + 1) % DEPTH]);
+        load_w(kt + d + 1 + WD, rw[(d + 1) % WD]);
         __syncthreads();
       }
     }
   };
-  if (FASTABLE && fast && (kt1 - kt0) % WD == 0) {
-    if constexpr (FASTABLE) {
-      if (!SKIP || live == TM) k_loop(std::true_type{}, std::true_type{});
-      else k_loop(std::false_type{}, std::true_type{});
-    }
-  } else {
-    if (!SKIP || live == TM) k_loop(std::true_type{}, std::false_type{});
-    else k_loop(std::false_type{}, std::false_type{});
-  }
+  if (!SKIP || live == TM) k_loop(std::true_type{});
+  else k_loop(std::false_type{});
 
   // ---- epilogue: D[i][j] of a 32x32 tile sits in lane (j + 32*((i/4)%2)), register 4*(i/8) + i%4
   if (p.paired && p.partial == nullptr) {
@@ -394,12 +433,12 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   }
 }
 
-template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false, int WX = 0>
-static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH, bool BF, bool SKIP, int WX, bool FAST>
+static hipError_t launch_pipe_form(const GemmParams& p, hipStream_t s) {
   constexpr int BK = 2 * GemmTraits<BITS>::G;
   constexpr int LDA = BK + 8;
   constexpr size_t lds = size_t(2) * (BM + BN) * LDA * 2;
-  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP, WX>;
+  auto kern = gemm_pipe_kernel<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP, WX, FAST>;
   if (lds > 65536) {
     const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(kern));
     if (e != hipSuccess) return e;
@@ -413,10 +452,21 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   const int n_last = p.n_end > 0 ? p.n_end : n_cols;
   if (n_last <= p.n_begin) return hipSuccess;
   const dim3 grid((n_last - p.n_begin + BN - 1) / BN, m_tiles, split);
-  note_kernel("gq::gemm_pipe_kernel<%d,%d,%d,%d,%d,%d,%s,%s,%d>", BITS, BM, BN, WM, WN, DEPTH, BF ? "true" : "false",
-              SKIP ? "true" : "false", WX);
+  note_kernel("gq::gemm_pipe_kernel<%d,%d,%d,%d,%d,%d,%s,%s,%d,%s>", BITS, BM, BN, WM, WN, DEPTH, BF ? "true" : "false",
+              SKIP ? "true" : "false", WX, FAST ? "true" : "false");
   hipLaunchKernelGGL(kern, grid, dim3(64 * (BM / WM) * (BN / WN)), lds, s, p);
   return hipGetLastError();
+}
+
+template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false, int WX = 0>
+static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
+  // the form without zero-selects: K in whole K tiles (fast_ok), and every workgroup's share of them in whole rounds of
+  // the register rings (all of K, or the split's share; the last split gets what is left)
+  constexpr int WD = DEPTH + WX;
+  const int nk = (p.ng + 1) / 2;
+  const bool whole_rounds = nk % WD == 0 && (p.partial == nullptr || p.kt_per_split % WD == 0);
+  if (p.fast_ok && whole_rounds) return launch_pipe_form<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP, WX, true>(p, s);
+  return launch_pipe_form<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP, WX, false>(p, s);
 }
 
 // y = sum over splits of partial[s] + bias + residual, in the output type (y may be the residual
