@@ -669,15 +669,15 @@ hipError_t launch_gemm_pipe(const GemmParams& p, int bits, hipStream_t s) {
           a.n_end = static_cast<int>(rounds * 256 / live * 256);
           b.n_begin = a.n_end;
           if (a.n_end > 0 && a.n_end < p.N) {
-            const hipError_t e = launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true>(a, s);
+            const hipError_t e = launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true, 2>(a, s);
             if (e != hipSuccess) return e;
             return launch_pipe_cfg<4, 256, 128, 64, 64, 2, false, true, 2>(b, s);
           }
         }
-        return launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true>(p, s);
+        return launch_pipe_cfg<4, 256, 256, 128, 64, 2, false, true, 2>(p, s);
       }
-      // the narrow tile has registers to spare: its weight loads run two more K tiles ahead (Mixtral's e2 at 64 / 128 /
-      // 256 rows per expert: 201 -> 177, 236 -> 213, 320 -> 305 us; the wide tile spills with them and loses)
+      // both tiles' weight loads run two more K tiles ahead than their activation loads (Mixtral's e2 on the narrow tile
+      // at 64 / 128 / 256 rows per expert: 201 -> 177, 236 -> 213, 320 -> 305 us; e1_e3 on the wide one 1-2 %)
       return launch_pipe_cfg<4, 256, 128, 64, 64, 2, false, true, 2>(p, s);
     }
     return launch_pipe_cfg<3, 256, 128, 64, 64, 2, false, true>(p, s);
