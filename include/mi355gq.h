@@ -245,6 +245,20 @@ MI355GQ_API int mi355gq_moe_gemv_silu_mul(const void* x, int64_t x_rows, const v
                               const void* q_scale, const void* expert_ids, int64_t top_k,
                               int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,
                               void* out, mi355gq_stream_t stream);
+/*
+ * One token through the router and the e1_e3 expert matmul in one launch (MixtralMoE.forward with one token,
+ * mixtral_model.py:76-95: gating_softmax_topk of moe_misc.py:135-235, then dequantize_gemv of moe_matmul.py:77-176
+ * with silu(x1) * x3 folded in as above).  x [1, K] and gate_logits [num_experts] in the model dtype; every
+ * workgroup picks the top_k experts from the logits itself, so no routing kernel runs in front.  Writes
+ * expert_weights [top_k] (model dtype) and expert_ids int32 [top_k], bit for bit what mi355gq_gating_softmax_topk
+ * returns, for the operators that follow (the e2 matmul, the combine), and out [top_k, N / 2], bit for bit what
+ * mi355gq_moe_gemv_silu_mul_dt returns for those ids.  float16 / bfloat16 models, top_k <= 2, at most 64 experts;
+ * MI355GQ_ERR_UNSUPPORTED otherwise (the caller then runs the two operators).
+ */
+MI355GQ_API int mi355gq_moe_gemv_routed_silu_mul(const void* x, const void* gate_logits, int64_t num_experts,
+                                     int64_t top_k, const void* q_weight, const void* q_scale, int64_t N, int64_t K,
+                                     int bits, int group_size, int model_dtype, void* expert_weights,
+                                     void* expert_ids, void* out, mi355gq_stream_t stream);
 MI355GQ_API int mi355gq_moe_group_gemm_silu_mul(const void* x, int64_t rows, const void* q_weight,
                                     const void* q_scale, const void* indptr, int indptr_dtype,
                                     int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,

@@ -664,6 +664,49 @@ int mi355gq_moe_gemv_silu_mul(const void* x, int64_t x_rows, const void* q_weigh
                        out, stream, true);
 }
 
+int mi355gq_moe_gemv_routed_silu_mul(const void* x, const void* gate_logits, int64_t num_experts, int64_t top_k,
+                                     const void* q_weight, const void* q_scale, int64_t N, int64_t K, int bits,
+                                     int group_size, int model_dtype, void* expert_weights, void* expert_ids, void* out,
+                                     mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "moe_gemv_routed_silu_mul"));
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(top_k >= 1 && N >= 0 && K >= 1 && N < kMaxDim && K < kMaxDim && num_experts >= top_k &&
+                 num_experts < kMaxDim && (N & 1) == 0,
+             "moe_gemv_routed_silu_mul: bad shape (N=%lld even, K=%lld, %lld experts, top_k=%lld)", (long long)N,
+             (long long)K, (long long)num_experts, (long long)top_k);
+  GQ_REQUIRE(x && gate_logits && q_weight && q_scale && expert_weights && expert_ids && (out || N == 0),
+             "moe_gemv_routed_silu_mul: null pointer");
+  if (model_dtype == MI355GQ_F32 || top_k > 2 || num_experts > 64 || !aligned16(x) || !aligned16(q_weight) ||
+      !aligned2(gate_logits) || !aligned2(expert_weights) || !aligned4(expert_ids) || !aligned2(out))
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_gemv_routed_silu_mul: float16 / bfloat16 models, top_k <= 2, at most 64 "
+                                         "experts, 16-byte aligned x and q_weight");
+  if (N == 0) {  // nothing to multiply: the routing alone
+    return hip_result(gq::launch_topk_softmax(gate_logits, 1, static_cast<int>(num_experts), static_cast<int>(top_k),
+                                              expert_weights, static_cast<int32_t*>(expert_ids), model_dtype,
+                                              as_stream(stream)),
+                      "moe_gemv_routed_silu_mul routing launch");
+  }
+  gq::GemvArgs a{};
+  a.x = static_cast<const uint16_t*>(x);
+  a.q_weight = static_cast<const uint32_t*>(q_weight);
+  a.q_scale = static_cast<const uint16_t*>(q_scale);
+  a.bias = nullptr;
+  a.y = out;
+  a.expert_ids = nullptr;
+  a.M = 1; a.N = N; a.K = K; a.slots = top_k; a.x_slot_stride = 0;
+  a.num_experts = num_experts;
+  a.bits = bits; a.group_size = group_size; a.out_f32 = 0; a.paired = 1;
+  a.bf16 = model_dtype == MI355GQ_BF16;
+  a.gate = gate_logits;
+  a.route_w = expert_weights;
+  a.route_ids = static_cast<int32_t*>(expert_ids);
+  const hipError_t e = gq::launch_gemv(a, as_stream(stream));
+  if (e == hipErrorNotSupported)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_gemv_routed_silu_mul: no fused kernel for N=%lld K=%lld", (long long)N,
+                (long long)K);
+  return hip_result(e, "moe_gemv_routed_silu_mul launch");
+}
+
 // Expert-sorted rows, about one per expert: the register GEMV with one grid row per activation row streams an
 // expert's weights once per row, the quad-row kernel once per expert but at well under half the GEMV's rate, so up
 // to num_experts rows (about 1.5 rows per distinct expert under uniform routing) the GEMV is ahead or level.

@@ -44,6 +44,14 @@ struct GemvParams {
   int indptr_i64;
   const int32_t* x_row_index;
   int x_src_rows;
+  // The token routes itself (register kernel, expert_ids null): `gate` holds its num_experts router logits in the model
+  // dtype; every workgroup picks the top gate_k of them (the insertion of the routing kernels) and serves slot
+  // blockIdx.y's expert; the first workgroup of a slot also leaves that slot's id and softmax weight in route_ids /
+  // route_w for the operators that follow.
+  const void* gate = nullptr;
+  int gate_k = 0;
+  void* route_w = nullptr;
+  int32_t* route_ids = nullptr;
 };
 
 // sum_k x_k * (field_k - m) for one group, given the 4 storage words and the staged x pairs

@@ -13,6 +13,7 @@
 //  * the grid is sized to a few waves per SIMD (not one block per row block): fewer, longer
 //    lived waves stream HBM better than thousands of short ones.
 #include "gq_gemv_common.hpp"
+#include "gq_topk.hpp"
 
 namespace gq {
 
@@ -65,6 +66,20 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
       row = row < 0 ? 0 : (row >= p.x_src_rows ? p.x_src_rows - 1 : row);
     }
     x = p.x + static_cast<int64_t>(row) * p.K;
+  } else if (p.gate != nullptr) {
+    // every lane runs the same insertion over the token's logits (a few dozen instructions for 8 experts), so the expert
+    // of this slot is known without a routing kernel in front; same arithmetic as topk_softmax_slots
+    float val[2];
+    int idx[2];
+    if (BF) topk_insert<2, MODEL_BF16>(p.gate, 0, p.num_experts, p.gate_k, val, idx);
+    else topk_insert<2, MODEL_F16>(p.gate, 0, p.num_experts, p.gate_k, val, idx);
+    const int e = __builtin_amdgcn_readfirstlane(slot == 0 ? idx[0] : idx[1]);
+    qw += e * p.expert_w_stride;
+    qs += e * p.expert_s_stride;
+    if (blockIdx.x == 0 && threadIdx.x == 0 && slot == 0) {
+      if (BF) softmax_store<2, MODEL_BF16>(val, idx, p.gate_k, p.route_w, 0, p.route_ids);
+      else softmax_store<2, MODEL_F16>(val, idx, p.gate_k, p.route_w, 0, p.route_ids);
+    }
   } else if (p.expert_ids != nullptr) {
     int e = p.expert_ids[slot];
     e = e < 0 ? 0 : (e >= p.num_experts ? p.num_experts - 1 : e);
@@ -347,6 +362,8 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
 
 hipError_t launch_gemv_reg(const GemvParams& p, int bits, int nb, int slots, hipStream_t s) {
   if (p.ng == 0) return hipErrorNotSupported;
+  if (p.gate != nullptr && (p.gate_k < 1 || p.gate_k > 2 || slots != p.gate_k || p.num_experts > 64 || nb != 1))
+    return hipErrorNotSupported;
   // the x staging always issues whole 16-byte loads (from the base of x where a chunk is unusable): x must hold
   // at least 8 halves per row for that address to be readable
   if (p.K < 8) return hipErrorNotSupported;

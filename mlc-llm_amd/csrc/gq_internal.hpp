@@ -52,6 +52,11 @@ struct GemvArgs {
   int indptr_i64 = 0;
   const int32_t* x_row_index = nullptr;
   int64_t x_src_rows = 0;
+  // the token routes itself (expert_ids null, slots = top_k <= 2, num_experts <= 64): router logits in the model dtype,
+  // and where the chosen ids / softmax weights go
+  const void* gate = nullptr;
+  void* route_w = nullptr;
+  int32_t* route_ids = nullptr;
 };
 hipError_t launch_gemv(const GemvArgs& a, hipStream_t s);
 

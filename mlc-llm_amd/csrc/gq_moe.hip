@@ -9,63 +9,11 @@
 
 #include "gq_common.hpp"
 #include "gq_internal.hpp"
+#include "gq_topk.hpp"
 
 namespace gq {
 
 constexpr int kMaxTopK = 8;
-
-// Elements of the model dtype (MODEL_F16 | MODEL_F32 | MODEL_BF16): load as float, round a float to
-// the dtype, store.  The float16 forms are the original kernels; the others follow the same rounding
-// points with their own rounding (every op in fp32, its result rounded to the dtype).
-template <int DT>
-struct Elem;
-template <>
-struct Elem<MODEL_F16> {
-  static __device__ __forceinline__ float load(const void* p, int64_t i) { return h2f(static_cast<const uint16_t*>(p)[i]); }
-  static __device__ __forceinline__ float rnd(float v) { return h2f(f2h(v)); }
-  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { static_cast<uint16_t*>(p)[i] = f2h(v); }
-  static constexpr float kLowest = -65504.0f;
-};
-template <>
-struct Elem<MODEL_F32> {
-  static __device__ __forceinline__ float load(const void* p, int64_t i) { return static_cast<const float*>(p)[i]; }
-  static __device__ __forceinline__ float rnd(float v) { return v; }
-  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { static_cast<float*>(p)[i] = v; }
-  static constexpr float kLowest = -3.402823466e38f;
-};
-template <>
-struct Elem<MODEL_BF16> {
-  static __device__ __forceinline__ float load(const void* p, int64_t i) { return bf2f(static_cast<const uint16_t*>(p)[i]); }
-  static __device__ __forceinline__ float rnd(float v) { return bf2f(f2bf(v)); }
-  static __device__ __forceinline__ void store(void* p, int64_t i, float v) { static_cast<uint16_t*>(p)[i] = f2bf(v); }
-  static constexpr float kLowest = -3.3895313892515355e38f;  // min_value(bfloat16)
-};
-
-// softmax over the k selected logits in fp32, in slot order, and the stores of one token's results
-template <int KMAX, int DT>
-__device__ __forceinline__ void softmax_store(const float (&val)[KMAX], const int (&idx)[KMAX], int k,
-                                              void* __restrict__ w, int64_t w0, int32_t* __restrict__ ids) {
-  float mx = val[0];
-#pragma unroll
-  for (int i = 1; i < KMAX; ++i)
-    if (i < k) mx = fmaxf(mx, val[i]);
-  float ex[KMAX];
-  float den = 0.f;
-#pragma unroll
-  for (int i = 0; i < KMAX; ++i) {
-    if (i < k) {
-      ex[i] = expf(val[i] - mx);
-      den = (i == 0) ? ex[0] : den + ex[i];
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < KMAX; ++i) {
-    if (i < k) {
-      Elem<DT>::store(w, w0 + i, ex[i] / den);
-      ids[i] = idx[i];
-    }
-  }
-}
 
 // One thread per token: insertion top-k with strict '>' (ties keep the lower expert index),
 // then softmax over the k selected logits in fp32.
@@ -74,33 +22,9 @@ __device__ __forceinline__ void softmax_store(const float (&val)[KMAX], const in
 template <int KMAX, int DT>
 __device__ __forceinline__ void topk_softmax_slots(const void* __restrict__ logits, int64_t row0, int ne, int k,
                                                    void* __restrict__ w, int64_t w0, int32_t* __restrict__ ids) {
-  constexpr int kMaxTopK = KMAX;
-  float val[kMaxTopK];
-  int idx[kMaxTopK];
-#pragma unroll
-  for (int i = 0; i < kMaxTopK; ++i) {
-    val[i] = Elem<DT>::kLowest;  // min_value(dtype)
-    idx[i] = 0;
-  }
-  for (int e = 0; e < ne; ++e) {
-    const float v = Elem<DT>::load(logits, row0 + e);
-    bool placed = false;
-#pragma unroll
-    for (int i = 0; i < kMaxTopK; ++i) {
-      if (i < k && !placed && v > val[i]) {
-#pragma unroll
-        for (int j = kMaxTopK - 1; j > 0; --j) {
-          if (j > i && j < k) {
-            val[j] = val[j - 1];
-            idx[j] = idx[j - 1];
-          }
-        }
-        val[i] = v;
-        idx[i] = e;
-        placed = true;
-      }
-    }
-  }
+  float val[KMAX];
+  int idx[KMAX];
+  topk_insert<KMAX, DT>(logits, row0, ne, k, val, idx);
   softmax_store<KMAX, DT>(val, idx, k, w, w0, ids);
 }
 

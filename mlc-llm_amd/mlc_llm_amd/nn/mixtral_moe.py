@@ -58,6 +58,19 @@ class MixtralMoE(nn.Module):
                                     self.e1_e3.group_size, silu_mul_halves=True)
                 y = self.e2(h, indptr)
                 return ops.moe_combine_sorted(y, slot_positions, weights).reshape(batch_size, seq_len, hidden_size)
+        if num_tokens == 1:
+            try:
+                # the token routes itself inside the e1_e3 kernel: one launch where the two operators take two
+                cfg = self.e1_e3.config
+                h, expert_weights, expert_indices = ops.moe_gemv_routed_silu_mul(
+                    x, gate, experts_per_tok, self.e1_e3.q_weight, self.e1_e3.q_scale, cfg.bits, self.e1_e3.group_size)
+            except _lib.Mi355gqError as err:
+                if err.code != _lib.ERR_UNSUPPORTED:
+                    raise
+            else:
+                x = self.e2(h, expert_indices)
+                x = ops.moe_combine(x.reshape(1, experts_per_tok, hidden_size), expert_weights)
+                return x.reshape(batch_size, seq_len, hidden_size)
         expert_weights, expert_indices = moe_misc.gating_softmax_topk(gate, experts_per_tok)
         if num_tokens == 1:
             x = self._expert_forward(x, expert_indices)

@@ -230,6 +230,34 @@ def linear_silu_mul(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tens
     return out
 
 
+def moe_gemv_routed_silu_mul(x: torch.Tensor, gate_logits: torch.Tensor, top_k: int, q_weight: torch.Tensor,
+                             q_scale: torch.Tensor, bits: int, group_size: int):
+    """One token: gating_softmax_topk and the e1_e3 expert matmul with silu(x1) * x3 folded in, in one launch.
+    x [1, K], gate_logits [1, num_experts] (model dtype), q_weight [E, N, nw], q_scale [E, N, ng].  Returns
+    (out [top_k, N / 2], expert_weights [1, top_k], expert_ids int32 [1, top_k]); raises Mi355gqError with
+    ERR_UNSUPPORTED where the fused kernel does not apply (float32 models, top_k > 2, more than 64 experts)."""
+    _chk(x, _FLOATS, "x")
+    _chk(gate_logits, x.dtype, "gate_logits")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, x.dtype, "q_scale")
+    if x.dim() != 2 or x.shape[0] != 1 or gate_logits.dim() != 2 or gate_logits.shape[0] != 1:
+        raise ValueError("moe_gemv_routed_silu_mul: x must be [1, K] and gate_logits [1, num_experts]")
+    ne, n, _ = q_weight.shape
+    k = x.shape[1]
+    if gate_logits.shape[1] != ne:
+        raise ValueError(f"moe_gemv_routed_silu_mul: {gate_logits.shape[1]} logits for {ne} experts")
+    if n % 2:
+        raise ValueError(f"moe_gemv_routed_silu_mul: {n} rows cannot be split into gate and up halves")
+    _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
+    out = torch.empty((top_k, n // 2), dtype=x.dtype, device=x.device)
+    weights = torch.empty((1, top_k), dtype=x.dtype, device=x.device)
+    ids = torch.empty((1, top_k), dtype=torch.int32, device=x.device)
+    _lib.call("mi355gq_moe_gemv_routed_silu_mul", x.data_ptr(), gate_logits.data_ptr(), ne, top_k, q_weight.data_ptr(),
+              q_scale.data_ptr(), n, k, bits, group_size, _MODEL_DTYPES[x.dtype], weights.data_ptr(), ids.data_ptr(),
+              out.data_ptr(), _stream())
+    return out, weights, ids
+
+
 def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
              expert_ids: torch.Tensor, bits: int, group_size: int, silu_mul_halves: bool = False
              ) -> torch.Tensor:

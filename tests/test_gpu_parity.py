@@ -747,6 +747,52 @@ def test_moe_gemv(name, x_rows):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("ne,top_k", [(8, 2), (8, 1), (64, 2), (3, 2)])
+def test_moe_gemv_routed_silu_mul(name, dtype, ne, top_k):
+    """One token routing itself inside the e1_e3 expert matmul: ids and weights bit for bit those of the routing
+    operator (ties included: two equal logits, the lower expert first), the output bit for bit that of the
+    operator pair it replaces, and the oracle's values."""
+    s = SCHEMES[name]
+    rng = np.random.default_rng(47 + ne + top_k)
+    n, k = 520, 1024 if s.bits == 4 else 1000
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    x = dev(rng.standard_normal((1, k)).astype(np.float16)).to(dtype)
+    logits = rng.standard_normal((1, ne)).astype(np.float16)
+    logits[0, ne - 1] = logits[0, 1] = logits.max() + 0.5  # a tie for the first place
+    gate = dev(logits).to(dtype)
+    qs_d = dev(qs).to(dtype)
+    out, weights, ids = ops.moe_gemv_routed_silu_mul(x, gate, top_k, dev(qw), qs_d, s.bits, s.group_size)
+    assert gq._lib.last_kernel().startswith("gq::gemv_reg_kernel"), gq._lib.last_kernel()
+    w_ref, ids_ref = ops.gating_softmax_topk(gate, top_k)
+    assert torch.equal(ids, ids_ref) and torch.equal(weights, w_ref)
+    assert ids[0, 0].item() == 1 and (top_k == 1 or ids[0, 1].item() == ne - 1)
+    pair = ops.moe_gemv(x, dev(qw), qs_d, ids_ref, s.bits, s.group_size, silu_mul_halves=True)
+    assert torch.equal(out, pair)
+    if dtype == torch.float16:
+        full = o.moe_dequantize_gemv_fp32(x.cpu().numpy(), qw, qs, ids.cpu().numpy(), s)
+        ref = o.silu_mul_f16(full.astype(np.float16)).astype(np.float64)
+        got = out.float().cpu().numpy()
+        assert np.abs(got - ref).max() <= 2e-2 * max(1.0, np.abs(ref).max()), np.abs(got - ref).max()
+
+
+def test_moe_gemv_routed_silu_mul_declines():
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(5)
+    ne, n, k = 8, 64, 256
+    qw, qs = o.quantize((rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16), s)
+    x = dev(rng.standard_normal((1, k)).astype(np.float16))
+    gate = dev(rng.standard_normal((1, ne)).astype(np.float16))
+    with pytest.raises(gq._lib.Mi355gqError) as err:  # three slots: the operator pair serves those
+        ops.moe_gemv_routed_silu_mul(x, gate, 3, dev(qw), dev(qs), 4, 32)
+    assert err.value.code == gq._lib.ERR_UNSUPPORTED
+    with pytest.raises(gq._lib.Mi355gqError) as err:  # float32 models
+        ops.moe_gemv_routed_silu_mul(x.float(), gate.float(), 2, dev(qw), dev(qs).float(), 4, 32)
+    assert err.value.code == gq._lib.ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("indptr", [[0, 3, 3, 40, 41], [0, 0, 0, 0, 130], [0, 1, 2, 3, 4], [0, 0, 0, 0, 0],
                                     [0, 33, 34, 60, 64], [0, 70, 70, 71, 200]])
 def test_moe_group_gemm(name, indptr):
