@@ -313,6 +313,21 @@ def main() -> int:
 
     us_read = timed(read_sweep, max(5, args.steps), 2, use_graph) * 1e3 / LAYERS
     read_bytes = layers[0]["gate_up"][0].numel() * 4 + layers[0]["gate_up"][1].numel() * 2
+
+    # ... and the whole step through the probe: the same 129 launches in the same order, each only reading the weight
+    # and scale tensors of its linear.  What separate launches over these tensors cost on this device when nothing is
+    # computed: the floor for any implementation behind an operator-per-linear boundary.
+    def probe_step():
+        stream = torch.cuda.current_stream().cuda_stream
+        for lw in layers:
+            for name in SHAPES:
+                qw, qs = lw[name]
+                gq._lib.call("mi355gq_probe_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
+                             sink.data_ptr(), stream)
+        gq._lib.call("mi355gq_probe_stream_read", lm_head[0].data_ptr(), lm_head[0].numel() * 4, lm_head[1].data_ptr(),
+                     lm_head[1].numel() * 2, sink.data_ptr(), stream)
+
+    ms_probe_step = timed(probe_step, max(5, args.steps), 2, use_graph)
     roofline = {
         "bound": "hbm", "kernel": f"{dominant_kernel} (gate_up 28672x4096, batch 1)",
         "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -323,7 +338,11 @@ def main() -> int:
         "read_only_probe": {"what": "plain 128-bit streaming read of the same weight and scale tensors, one launch each",
                             "us_per_launch": round(us_read, 3),
                             "GB/s": round(read_bytes / (us_read * 1e-6) / 1e9, 1),
-                            "gemv_time_over_probe_time": round(us_gate_up / us_read, 3)},
+                            "gemv_time_over_probe_time": round(us_gate_up / us_read, 3),
+                            "whole_step_ms": round(ms_probe_step, 4),
+                            "whole_step_what": "the decode step's 129 launches with each linear replaced by the probe "
+                                               "over its weight and scale tensors",
+                            "step_time_over_probe_step_time": round(ms_step / ms_probe_step, 3)},
     }
 
     # ---------------------------------------------------------------- extra: per shape, batch 1/4/8, prefill GEMM

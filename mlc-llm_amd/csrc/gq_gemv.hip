@@ -262,8 +262,13 @@ hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
   p.bf16 = a.bf16;
   p.indptr = a.indptr; p.indptr_i64 = a.indptr_i64; p.x_row_index = a.x_row_index;
   p.x_src_rows = static_cast<int>(a.x_src_rows);
-  p.gate = a.gate; p.gate_k = a.gate != nullptr ? static_cast<int>(a.slots) : 0;
-  p.route_w = a.route_w; p.route_ids = a.route_ids;
+  p.routed = a.gate != nullptr;
+  if (p.routed) {  // (see GemvParams: three fields carry the router's tensors in this form)
+    if (a.bias != nullptr || a.residual != nullptr || a.expert_ids != nullptr) return hipErrorNotSupported;
+    p.bias = static_cast<const uint16_t*>(a.gate);
+    p.residual = static_cast<const uint16_t*>(a.route_w);
+    p.expert_ids = a.route_ids;
+  }
   if (a.N == 0 || a.slots == 0) return hipSuccess;
   const int nb = static_cast<int>(a.M);
   const int slots = static_cast<int>(a.slots);
@@ -272,7 +277,7 @@ hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
     const hipError_t e = launch_gemv_reg(p, a.bits, nb, slots, s);
     if (e != hipErrorNotSupported) return e;
   }
-  if (p.paired || p.bf16 || p.indptr != nullptr || p.gate != nullptr) return hipErrorNotSupported;  // only the register kernel has these forms
+  if (p.paired || p.bf16 || p.indptr != nullptr || p.routed) return hipErrorNotSupported;  // only the register kernel has these forms
   return launch_gemv_lds(p, a.bits, nb, slots, s);
 }
 

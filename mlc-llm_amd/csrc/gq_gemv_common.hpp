@@ -37,6 +37,7 @@ struct GemvParams {
   int out_f32;
   int paired;  // fused gate/up form: y[.., N / 2] = silu(x . W[j]) * (x . W[N / 2 + j]), fp16
   int bf16;    // x, q_scale, bias, residual and a 16-bit y are bfloat16 (register kernel only)
+  int routed = 0;
   // rows sorted by expert instead of expert_ids (register kernel only): slot s belongs to the expert e with
   // indptr[e] <= s < indptr[e + 1] (slots outside every segment are left alone) and reads x row
   // x_row_index[s] (null: row s)
@@ -44,14 +45,12 @@ struct GemvParams {
   int indptr_i64;
   const int32_t* x_row_index;
   int x_src_rows;
-  // The token routes itself (register kernel, expert_ids null): `gate` holds its num_experts router logits in the model
-  // dtype; every workgroup picks the top gate_k of them (the insertion of the routing kernels) and serves slot
-  // blockIdx.y's expert; the first workgroup of a slot also leaves that slot's id and softmax weight in route_ids /
-  // route_w for the operators that follow.
-  const void* gate = nullptr;
-  int gate_k = 0;
-  void* route_w = nullptr;
-  int32_t* route_ids = nullptr;
+  // The token routes itself (register kernel, fused gate/up form of one row): `routed` is set and three fields change
+  // their meaning, because a larger argument block measurably slows every launch of these kernels (129 per decode step):
+  // `bias` holds the token's num_experts router logits in the model dtype, `residual` points at the top_k softmax weights
+  // to write and `expert_ids` at the top_k ids to write.  Every workgroup picks the top gridDim.y logits (the insertion
+  // of the routing kernels) and serves slot blockIdx.y's expert; the first workgroup leaves ids and weights for the
+  // operators that follow.
 };
 
 // sum_k x_k * (field_k - m) for one group, given the 4 storage words and the staged x pairs

@@ -20,13 +20,15 @@ namespace gq {
 // MODE 1: a bias or residual operand exists (a template flag rather than a run-time test: their loads are
 // two more memory instructions per set, measured at 4-6 % of the plain GEMV's time).
 // MODE 2: fused gate/up form; a set holds R / 2 (gate, up) row pairs and stores R / 2 products.
+// MODE 3: MODE 2 for one token that routes itself (the expert of a slot comes from the router logits, see below); its
+// own instantiation so that no other form carries the selection code.
 // BF: bfloat16 model (x, scales, bias, residual and a 16-bit result are bfloat16); the same walk with
 // group_dot_bf16.  Like the float16 form it multiplies x with the integer fields and applies the scale
 // to the group sum in fp32, so the dequantised weight is never rounded to the model dtype on its own.
 template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false>
 __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int nsets) {
   using T = GemvTraits<BITS>;
-  constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;
+  constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2 || MODE == 3, ROUTED = MODE == 3;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
   static_assert(!PAIRED || R % 2 == 0, "a set holds whole (gate, up) pairs");
   constexpr int G = T::G;
@@ -66,19 +68,23 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
       row = row < 0 ? 0 : (row >= p.x_src_rows ? p.x_src_rows - 1 : row);
     }
     x = p.x + static_cast<int64_t>(row) * p.K;
-  } else if (p.gate != nullptr) {
+  } else if (ROUTED) {
     // every lane runs the same insertion over the token's logits (a few dozen instructions for 8 experts), so the expert
     // of this slot is known without a routing kernel in front; same arithmetic as topk_softmax_slots
     float val[2];
     int idx[2];
-    if (BF) topk_insert<2, MODEL_BF16>(p.gate, 0, p.num_experts, p.gate_k, val, idx);
-    else topk_insert<2, MODEL_F16>(p.gate, 0, p.num_experts, p.gate_k, val, idx);
+    // (in this form `bias` holds the logits, `residual` / `expert_ids` point at the weights and ids to write)
+    const int top_k = static_cast<int>(gridDim.y);
+    if (BF) topk_insert<2, MODEL_BF16>(p.bias, 0, p.num_experts, top_k, val, idx);
+    else topk_insert<2, MODEL_F16>(p.bias, 0, p.num_experts, top_k, val, idx);
     const int e = __builtin_amdgcn_readfirstlane(slot == 0 ? idx[0] : idx[1]);
     qw += e * p.expert_w_stride;
     qs += e * p.expert_s_stride;
     if (blockIdx.x == 0 && threadIdx.x == 0 && slot == 0) {
-      if (BF) softmax_store<2, MODEL_BF16>(val, idx, p.gate_k, p.route_w, 0, p.route_ids);
-      else softmax_store<2, MODEL_F16>(val, idx, p.gate_k, p.route_w, 0, p.route_ids);
+      void* route_w = const_cast<uint16_t*>(p.residual);
+      int32_t* route_ids = const_cast<int32_t*>(p.expert_ids);
+      if (BF) softmax_store<2, MODEL_BF16>(val, idx, top_k, route_w, 0, route_ids);
+      else softmax_store<2, MODEL_F16>(val, idx, top_k, route_w, 0, route_ids);
     }
   } else if (p.expert_ids != nullptr) {
     int e = p.expert_ids[slot];
@@ -262,7 +268,18 @@ static hipError_t launch_k(const GemvParams& p, int slots, int blocks, int nsets
   const size_t lds = static_cast<size_t>(NB) * p.ng * GemvTraits<BITS>::G * 2;
   const dim3 grid(blocks, slots);
   note_kernel("gq::gemv_reg_kernel<%d,%d,%d,%d,%d,%s>", BITS, NB, R, ITERS,
-              p.paired ? 2 : ((p.bias != nullptr || p.residual != nullptr) ? 1 : 0), p.bf16 ? "true" : "false");
+              p.paired ? (p.routed ? 3 : 2) : ((p.bias != nullptr || p.residual != nullptr) ? 1 : 0),
+              p.bf16 ? "true" : "false");
+  if (p.routed) {  // (the launcher admits the routed form only as the fused gate/up form of one row)
+    if constexpr (R % 2 == 0 && NB == 1) {
+      if (!p.paired) return hipErrorNotSupported;
+      if (p.bf16) hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 3, true>), grid, dim3(threads), lds, s, p, nsets);
+      else hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 3>), grid, dim3(threads), lds, s, p, nsets);
+      return hipGetLastError();
+    } else {
+      return hipErrorNotSupported;
+    }
+  }
   if (p.bf16) {
     if (p.paired) {
       if constexpr (R % 2 == 0)
@@ -362,8 +379,7 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
 
 hipError_t launch_gemv_reg(const GemvParams& p, int bits, int nb, int slots, hipStream_t s) {
   if (p.ng == 0) return hipErrorNotSupported;
-  if (p.gate != nullptr && (p.gate_k < 1 || p.gate_k > 2 || slots != p.gate_k || p.num_experts > 64 || nb != 1))
-    return hipErrorNotSupported;
+  if (p.routed && (slots < 1 || slots > 2 || p.num_experts > 64 || nb != 1 || !p.paired)) return hipErrorNotSupported;
   // the x staging always issues whole 16-byte loads (from the base of x where a chunk is unusable): x must hold
   // at least 8 halves per row for that address to be readable
   if (p.K < 8) return hipErrorNotSupported;
