@@ -2,6 +2,8 @@
 // per-group fused unpack + dot product.
 #pragma once
 
+#include <cstddef>
+
 #include "gq_common.hpp"
 #include "gq_internal.hpp"
 
@@ -20,38 +22,49 @@ struct GemvTraits<3> {
   static constexpr int CH = 5;
 };
 
+// Field order matters: a kernel's arguments sit in memory that every launch reads cold, 64 bytes per line, and each
+// line a kernel touches costs it about a quarter of a microsecond (measured: 32 more bytes of arguments, which pushed the
+// launch dimensions the kernel also read into one more line, took the decode step from 1.177 to 1.204 ms).  What the
+// plain batch-1 linear reads comes first and fills one line; the grid size rides along (nwaves) so that the register
+// kernel never reads the launch dimensions; the expert forms' fields follow and are only read by their instantiations.
 struct GemvParams {
+  // ---- line 0: every form
   const uint16_t* x;
   const uint32_t* qw;
   const uint16_t* qs;
+  void* y;
+  int N, K, ng, nw;
+  int nsets = 0;   // row sets the launch walks (register kernel; set by its launcher)
+  int nwaves = 0;  // waves of one grid row (register kernel; set by its launcher)
+  int out_f32;
+  int num_experts;
+  int paired;  // fused gate/up form: y[.., N / 2] = silu(x . W[j]) * (x . W[N / 2 + j]), fp16
+  int bf16;    // x, q_scale, bias, residual and a 16-bit y are bfloat16 (register kernel only)
+  int routed = 0;
+  int gc;  // groups staged per LDS chunk (multiple of 64; LDS kernel)
+  // ---- line 1: bias / residual forms and expert forms
   const uint16_t* bias;
   const uint16_t* residual;  // [M, N] or null
-  void* y;
   const int32_t* expert_ids;
   int64_t x_slot_stride;
   int64_t expert_w_stride;  // N * nw
   int64_t expert_s_stride;  // N * ng
-  int N, K, ng, nw;
-  int num_experts;
-  int gc;  // groups staged per LDS chunk (multiple of 64)
-  int out_f32;
-  int paired;  // fused gate/up form: y[.., N / 2] = silu(x . W[j]) * (x . W[N / 2 + j]), fp16
-  int bf16;    // x, q_scale, bias, residual and a 16-bit y are bfloat16 (register kernel only)
-  int routed = 0;
   // rows sorted by expert instead of expert_ids (register kernel only): slot s belongs to the expert e with
   // indptr[e] <= s < indptr[e + 1] (slots outside every segment are left alone) and reads x row
   // x_row_index[s] (null: row s)
   const void* indptr;
-  int indptr_i64;
   const int32_t* x_row_index;
+  int indptr_i64;
   int x_src_rows;
   // The token routes itself (register kernel, fused gate/up form of one row): `routed` is set and three fields change
-  // their meaning, because a larger argument block measurably slows every launch of these kernels (129 per decode step):
-  // `bias` holds the token's num_experts router logits in the model dtype, `residual` points at the top_k softmax weights
-  // to write and `expert_ids` at the top_k ids to write.  Every workgroup picks the top gridDim.y logits (the insertion
-  // of the routing kernels) and serves slot blockIdx.y's expert; the first workgroup leaves ids and weights for the
-  // operators that follow.
+  // their meaning (a larger argument block would slow every launch of these kernels, see above): `bias` holds the
+  // token's num_experts router logits in the model dtype, `residual` points at the top_k softmax weights to write and
+  // `expert_ids` at the top_k ids to write.  Every workgroup picks the top gridDim.y logits (the insertion of the
+  // routing kernels) and serves slot blockIdx.y's expert; the first workgroup leaves ids and weights for the operators
+  // that follow.
 };
+static_assert(offsetof(GemvParams, bias) == 80, "the fields of the plain linear fill the first argument lines");
+
 
 // sum_k x_k * (field_k - m) for one group, given the 4 storage words and the staged x pairs
 template <int BITS>

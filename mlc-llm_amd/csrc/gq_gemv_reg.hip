@@ -25,8 +25,11 @@ namespace gq {
 // BF: bfloat16 model (x, scales, bias, residual and a 16-bit result are bfloat16); the same walk with
 // group_dot_bf16.  Like the float16 form it multiplies x with the integer fields and applies the scale
 // to the group sum in fp32, so the dequantised weight is never rounded to the model dtype on its own.
-template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false>
-__global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int nsets) {
+// MOE: an expert form (expert ids, expert-sorted rows, one grid row per slot).  The plain linear's instantiation reads
+// none of those fields: its arguments are the first 64 bytes of GemvParams.
+template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false, bool MOE = true>
+__global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p) {
+  const int nsets = p.nsets;
   using T = GemvTraits<BITS>;
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2 || MODE == 3, ROUTED = MODE == 3;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
@@ -41,13 +44,15 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
 
   const int lane = threadIdx.x & 63;
   const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int nwaves = gridDim.x * 4;
-  const int slot = blockIdx.y;
+  const int nwaves = p.nwaves;
+  const int slot = MOE ? blockIdx.y : 0;
 
-  const uint16_t* x = p.x + slot * p.x_slot_stride;
+  const uint16_t* x = MOE ? p.x + slot * p.x_slot_stride : p.x;
   const uint32_t* qw = p.qw;
   const uint16_t* qs = p.qs;
-  if (p.indptr != nullptr) {
+  if constexpr (!MOE) {
+    static_assert(MODE != 3, "a token that routes itself is an expert form");
+  } else if (p.indptr != nullptr) {
     // expert-sorted rows: the segment ends at or before this row number its expert (each wave counts for itself)
     int e = 0;
     for (int e0 = 0; e0 < p.num_experts; e0 += 64) {
@@ -262,49 +267,42 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p, int n
   }
 }
 
+template <int BITS, int NB, int R, int ITERS, int MODE, bool MOE>
+static hipError_t launch_mode(const GemvParams& p, dim3 grid, size_t lds, hipStream_t s) {
+  if (p.bf16) hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, MODE, true, MOE>), grid, dim3(256), lds, s, p);
+  else hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, MODE, false, MOE>), grid, dim3(256), lds, s, p);
+  return hipGetLastError();
+}
+
 template <int BITS, int NB, int R, int ITERS>
-static hipError_t launch_k(const GemvParams& p, int slots, int blocks, int nsets, hipStream_t s) {
-  const int threads = 256;
-  const size_t lds = static_cast<size_t>(NB) * p.ng * GemvTraits<BITS>::G * 2;
+static hipError_t launch_k(const GemvParams& p0, int slots, int blocks, int nsets, hipStream_t s) {
+  const size_t lds = static_cast<size_t>(NB) * p0.ng * GemvTraits<BITS>::G * 2;
   const dim3 grid(blocks, slots);
-  note_kernel("gq::gemv_reg_kernel<%d,%d,%d,%d,%d,%s>", BITS, NB, R, ITERS,
-              p.paired ? (p.routed ? 3 : 2) : ((p.bias != nullptr || p.residual != nullptr) ? 1 : 0),
-              p.bf16 ? "true" : "false");
-  if (p.routed) {  // (the launcher admits the routed form only as the fused gate/up form of one row)
-    if constexpr (R % 2 == 0 && NB == 1) {
-      if (!p.paired) return hipErrorNotSupported;
-      if (p.bf16) hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 3, true>), grid, dim3(threads), lds, s, p, nsets);
-      else hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 3>), grid, dim3(threads), lds, s, p, nsets);
-      return hipGetLastError();
+  GemvParams p = p0;
+  p.nsets = nsets;
+  p.nwaves = blocks * 4;
+  const int mode = p.paired ? (p.routed ? 3 : 2) : ((p.bias != nullptr || p.residual != nullptr) ? 1 : 0);
+  // the plain linear (one grid row, no expert ids, no expert-sorted rows) has an instantiation of its own
+  const bool moe = slots != 1 || p.routed || p.indptr != nullptr || p.expert_ids != nullptr;
+  note_kernel("gq::gemv_reg_kernel<%d,%d,%d,%d,%d,%s,%s>", BITS, NB, R, ITERS, mode, p.bf16 ? "true" : "false",
+              moe ? "true" : "false");
+  if (mode >= 2) {
+    if constexpr (R % 2 == 0) {
+      if (mode == 3) {  // (the launcher admits the routed form only as the fused gate/up form of one row)
+        if constexpr (NB == 1) return launch_mode<BITS, NB, R, ITERS, 3, true>(p, grid, lds, s);
+        else return hipErrorNotSupported;
+      }
+      return moe ? launch_mode<BITS, NB, R, ITERS, 2, true>(p, grid, lds, s)
+                 : launch_mode<BITS, NB, R, ITERS, 2, false>(p, grid, lds, s);
     } else {
       return hipErrorNotSupported;
     }
   }
-  if (p.bf16) {
-    if (p.paired) {
-      if constexpr (R % 2 == 0)
-        hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 2, true>), grid, dim3(threads), lds, s, p, nsets);
-      else
-        return hipErrorNotSupported;
-      return hipGetLastError();
-    }
-    if (p.bias != nullptr || p.residual != nullptr)
-      hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 1, true>), grid, dim3(threads), lds, s, p, nsets);
-    else
-      hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 0, true>), grid, dim3(threads), lds, s, p, nsets);
-    return hipGetLastError();
-  }
-  if (p.paired) {
-    if constexpr (R % 2 == 0)
-      hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 2>), grid, dim3(threads), lds, s, p, nsets);
-    else
-      return hipErrorNotSupported;
-  } else if (p.bias != nullptr || p.residual != nullptr) {
-    hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 1>), grid, dim3(threads), lds, s, p, nsets);
-  } else {
-    hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, 0>), grid, dim3(threads), lds, s, p, nsets);
-  }
-  return hipGetLastError();
+  if (mode == 1)
+    return moe ? launch_mode<BITS, NB, R, ITERS, 1, true>(p, grid, lds, s)
+               : launch_mode<BITS, NB, R, ITERS, 1, false>(p, grid, lds, s);
+  return moe ? launch_mode<BITS, NB, R, ITERS, 0, true>(p, grid, lds, s)
+             : launch_mode<BITS, NB, R, ITERS, 0, false>(p, grid, lds, s);
 }
 
 template <int BITS, int NB, int R>
