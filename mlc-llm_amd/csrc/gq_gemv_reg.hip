@@ -28,8 +28,16 @@ namespace gq {
 // MOE: an expert form (expert ids, expert-sorted rows, one grid row per slot).  The plain linear's instantiation reads
 // none of those fields: its arguments are the first 64 bytes of GemvParams.
 template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false, bool MOE = true>
-__global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p) {
-  const int nsets = p.nsets;
+__global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const uint32_t* qw_, const uint16_t* qs_,
+                                                        void* y_, int N_, int K_, int ng_, int nsets, int nwaves_,
+                                                        int out_f32_, const GemvParams rest) {
+  // The ten leading arguments (14 dwords) arrive in scalar registers with the wave (the file is compiled with kernel
+  // argument preloading): the plain linear starts its x loads without a memory read for its own arguments.  `rest`
+  // carries the fields of the other forms; its copies of the leading ones are never read.
+  GemvParams p = rest;
+  p.x = x_; p.qw = qw_; p.qs = qs_; p.y = y_;
+  p.N = N_; p.K = K_; p.ng = ng_; p.nw = 4 * ng_;
+  p.nsets = nsets; p.nwaves = nwaves_; p.out_f32 = out_f32_;
   using T = GemvTraits<BITS>;
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2 || MODE == 3, ROUTED = MODE == 3;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
@@ -269,8 +277,10 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const GemvParams p) {
 
 template <int BITS, int NB, int R, int ITERS, int MODE, bool MOE>
 static hipError_t launch_mode(const GemvParams& p, dim3 grid, size_t lds, hipStream_t s) {
-  if (p.bf16) hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, MODE, true, MOE>), grid, dim3(256), lds, s, p);
-  else hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, MODE, false, MOE>), grid, dim3(256), lds, s, p);
+  if (p.bf16) hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, MODE, true, MOE>), grid, dim3(256), lds, s,
+                                    p.x, p.qw, p.qs, p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, p);
+  else hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, MODE, false, MOE>), grid, dim3(256), lds, s,
+                          p.x, p.qw, p.qs, p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, p);
   return hipGetLastError();
 }
 
