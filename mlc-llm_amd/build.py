@@ -34,17 +34,13 @@ FLAGS = [
     "-fhip-fp32-correctly-rounded-divide-sqrt",
     # packed-FP32 VALU forms are kept out of every code object
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the leading scalar arguments of a kernel (up to 14 dwords on gfx950) arrive in SGPRs with the wave instead of
+    # through a memory read at its start; firmware without the feature enters a prologue that loads them
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wall",
     "-Wno-unused-function",
     "-Wno-unknown-attributes",
 ]
-
-
-# Kernels whose leading scalar arguments should arrive in SGPRs with the wave (up to 14 dwords on gfx950; a kernel
-# entered by firmware without the feature runs a prologue that loads them instead).
-PER_FILE = {
-    "gq_gemv_reg.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=14"],
-}
 
 
 def _tvm_ffi_include() -> str | None:
@@ -77,7 +73,7 @@ def build(verbose: bool = True) -> str:
     link_extra: list[str] = []
     ffi_inc = _tvm_ffi_include()
     adapter = os.path.join(CSRC, "tvm_ffi_adapter.cc")
-    jobs = [(s, extra + PER_FILE.get(os.path.basename(s), [])) for s in srcs]
+    jobs = [(s, extra) for s in srcs]
     if ffi_inc and os.path.exists(adapter):
         jobs.append((adapter, ["-x", "hip", f"-I{ffi_inc}"]))
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(jobs))) as ex:

@@ -25,19 +25,35 @@ namespace gq {
 // BF: bfloat16 model (x, scales, bias, residual and a 16-bit result are bfloat16); the same walk with
 // group_dot_bf16.  Like the float16 form it multiplies x with the integer fields and applies the scale
 // to the group sum in fp32, so the dequantised weight is never rounded to the model dtype on its own.
+// The arguments behind the 56 bytes of leading ones, in the order of use: an expert form without sorted rows reads
+// 48 bytes of them, the plain linear none.
+struct GemvTail {
+  const int32_t* expert_ids;
+  int64_t expert_w_stride, expert_s_stride, x_slot_stride;
+  const uint16_t* bias;
+  const uint16_t* residual;
+  int num_experts;
+  int indptr_i64;
+  const void* indptr;
+  const int32_t* x_row_index;
+  int x_src_rows;
+};
+
 // MOE: an expert form (expert ids, expert-sorted rows, one grid row per slot).  The plain linear's instantiation reads
-// none of those fields: its arguments are the first 64 bytes of GemvParams.
+// none of those fields.
 template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false, bool MOE = true>
 __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const uint32_t* qw_, const uint16_t* qs_,
                                                         void* y_, int N_, int K_, int ng_, int nsets, int nwaves_,
-                                                        int out_f32_, const GemvParams rest) {
-  // The ten leading arguments (14 dwords) arrive in scalar registers with the wave (the file is compiled with kernel
-  // argument preloading): the plain linear starts its x loads without a memory read for its own arguments.  `rest`
-  // carries the fields of the other forms; its copies of the leading ones are never read.
-  GemvParams p = rest;
+                                                        int out_f32_, const GemvTail t) {
+  // The ten leading arguments (14 dwords) arrive in scalar registers with the wave (the library is compiled with
+  // kernel argument preloading): the plain linear starts its x loads without a memory read for its own arguments.
+  GemvParams p;
   p.x = x_; p.qw = qw_; p.qs = qs_; p.y = y_;
   p.N = N_; p.K = K_; p.ng = ng_; p.nw = 4 * ng_;
   p.nsets = nsets; p.nwaves = nwaves_; p.out_f32 = out_f32_;
+  p.expert_ids = t.expert_ids; p.expert_w_stride = t.expert_w_stride; p.expert_s_stride = t.expert_s_stride;
+  p.x_slot_stride = t.x_slot_stride; p.bias = t.bias; p.residual = t.residual; p.num_experts = t.num_experts;
+  p.indptr_i64 = t.indptr_i64; p.indptr = t.indptr; p.x_row_index = t.x_row_index; p.x_src_rows = t.x_src_rows;
   using T = GemvTraits<BITS>;
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2 || MODE == 3, ROUTED = MODE == 3;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
@@ -277,10 +293,12 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
 
 template <int BITS, int NB, int R, int ITERS, int MODE, bool MOE>
 static hipError_t launch_mode(const GemvParams& p, dim3 grid, size_t lds, hipStream_t s) {
+  const GemvTail t{p.expert_ids, p.expert_w_stride, p.expert_s_stride, p.x_slot_stride, p.bias, p.residual,
+                   p.num_experts, p.indptr_i64, p.indptr, p.x_row_index, p.x_src_rows};
   if (p.bf16) hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, MODE, true, MOE>), grid, dim3(256), lds, s,
-                                    p.x, p.qw, p.qs, p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, p);
+                                    p.x, p.qw, p.qs, p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, t);
   else hipLaunchKernelGGL((gemv_reg_kernel<BITS, NB, R, ITERS, MODE, false, MOE>), grid, dim3(256), lds, s,
-                          p.x, p.qw, p.qs, p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, p);
+                          p.x, p.qw, p.qs, p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, t);
   return hipGetLastError();
 }
 

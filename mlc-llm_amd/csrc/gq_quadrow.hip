@@ -54,6 +54,23 @@ struct QuadParams {
   int bf16;               // x, scales, bias, residual and a 16-bit y are bfloat16
 };
 
+// The kernel's ten leading arguments (14 dwords) arrive in scalar registers with the wave: x, qw, qs, y, rows, N, K and three
+// packed words (below); ng, nw, nquads and nsets follow from them.  A plain linear reads nothing else, so it starts its
+// loads without a memory read for its own arguments (about 0.4 us per launch, measured on the batch-1 kernel); the
+// launch dimensions, which would sit in one more 64-byte line of the argument block, are not read by any form.
+// QuadTail holds what the other forms add and is only read when kQuadHasTail is set.
+struct QuadTail {
+  const void* indptr;
+  const int32_t* x_rows;
+  int64_t expert_w_stride, expert_s_stride;
+  const uint16_t* bias;
+  const uint16_t* residual;
+  int x_src_rows;
+};
+// packed words: w0 = nsteps | steps_total << 16, w1 = rounds | nwaves << 16,
+// w2 = nphases | flags << 16 | waves per workgroup << 24
+constexpr uint32_t kQuadOutF32 = 1u << 16, kQuadIndptrI64 = 1u << 17, kQuadHasTail = 1u << 18;
+
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_u(uint32_t v) {
   return static_cast<uint32_t>(
@@ -89,7 +106,21 @@ __device__ __forceinline__ float4_t mfma4_bf16(uint32_t a0, uint32_t a1, uint32_
 template <int BITS, int NBQ, int U, int MODE, bool BF = false, int QP = 1>
 // (sixteen-wave workgroups exist for the forms that fit 128 registers: 2 KiB items without the bias / residual loads;
 //  with them the same bound forced spill reloads into the walk, and a reload waits for every weight load in flight)
-__global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_kernel(const QuadParams p) {
+__global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_kernel(const uint16_t* x_, const uint32_t* qw_, const uint16_t* qs_, void* y_, int rows_, int N_, int K_,
+                 uint32_t w0, uint32_t w1, uint32_t w2, const QuadTail t) {
+  QuadParams p;
+  p.x = x_; p.qw = qw_; p.qs = qs_; p.y = y_;
+  p.rows = rows_; p.N = N_; p.K = K_;
+  p.ng = (K_ + GemvTraits<BITS>::G - 1) / GemvTraits<BITS>::G; p.nw = 4 * p.ng;
+  p.nquads = N_ >> 2; p.nsets = (p.nquads + QP - 1) / QP;
+  p.nsteps = w0 & 0xffffu; p.steps_total = w0 >> 16; p.rounds = w1 & 0xffffu; p.nphases = w2 & 0xffffu;
+  p.out_f32 = (w2 & kQuadOutF32) != 0; p.indptr_i64 = (w2 & kQuadIndptrI64) != 0;
+  p.indptr = nullptr; p.x_rows = nullptr; p.expert_w_stride = 0; p.expert_s_stride = 0;
+  p.bias = nullptr; p.residual = nullptr; p.x_src_rows = 0;
+  if (MODE == 1 || (w2 & kQuadHasTail) != 0) {
+    p.indptr = t.indptr; p.x_rows = t.x_rows; p.expert_w_stride = t.expert_w_stride;
+    p.expert_s_stride = t.expert_s_stride; p.bias = t.bias; p.residual = t.residual; p.x_src_rows = t.x_src_rows;
+  }
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;  // 2: fused gate/up form, quad = 2 (gate, up) pairs
   constexpr uint32_t kMagic = BF ? 0x43004300u : 0x64006400u;
   auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
@@ -103,11 +134,11 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
 
   extern __shared__ uint4 smem[];
 
-  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int tid = threadIdx.x, nthreads = static_cast<int>(w2 >> 24) << 6;
   const int lane = tid & 63;
   const int wpb = nthreads >> 6;
   const int gw = blockIdx.x * wpb + (tid >> 6);
-  const int nwaves = gridDim.x * wpb;
+  const int nwaves = static_cast<int>(w1 >> 16);
   const int li = lane & 3;   // weight row of the quad (A), activation row of the batch quad (B, D)
   const int ks = lane >> 2;  // block: group 16 * iteration + ks
 
@@ -452,7 +483,19 @@ static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads,
     if (e != hipSuccess) return e;
   }
   note_kernel("gq::quad_kernel<%d,%d,%d,%d,%s,%d>", BITS, NBQ, U, MODE, BF ? "true" : "false", QP);
-  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF, QP>), grid, dim3(threads), lds, s, p);
+  const int nwaves = static_cast<int>(grid.x) * (threads >> 6);
+  if (threads % 64 != 0 || threads > 1024 || p.nsteps > 0xffff || p.steps_total > 0xffff || p.rounds > 0xffff ||
+      nwaves > 0xffff || p.nphases > 0xffff || p.nquads != p.N / 4 || p.nsets != (p.nquads + QP - 1) / QP)
+    return hipErrorNotSupported;
+  const bool tail = p.indptr != nullptr || p.x_rows != nullptr || p.bias != nullptr || p.residual != nullptr;
+  const QuadTail t{p.indptr, p.x_rows, p.expert_w_stride, p.expert_s_stride, p.bias, p.residual, p.x_src_rows};
+  const uint32_t w0 = static_cast<uint32_t>(p.nsteps) | static_cast<uint32_t>(p.steps_total) << 16;
+  const uint32_t w1 = static_cast<uint32_t>(p.rounds) | static_cast<uint32_t>(nwaves) << 16;
+  const uint32_t w2 = static_cast<uint32_t>(p.nphases) | (p.out_f32 ? kQuadOutF32 : 0u) |
+                      (p.indptr_i64 ? kQuadIndptrI64 : 0u) | (tail ? kQuadHasTail : 0u) |
+                      static_cast<uint32_t>(threads >> 6) << 24;
+  hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF, QP>), grid, dim3(threads), lds, s,
+                     p.x, p.qw, p.qs, p.y, p.rows, p.N, p.K, w0, w1, w2, t);
   return hipGetLastError();
 }
 
