@@ -2,8 +2,6 @@
 // per-group fused unpack + dot product.
 #pragma once
 
-#include <cstddef>
-
 #include "gq_common.hpp"
 #include "gq_internal.hpp"
 
@@ -22,13 +20,15 @@ struct GemvTraits<3> {
   static constexpr int CH = 5;
 };
 
-// Field order matters: a kernel's arguments sit in memory that every launch reads cold, 64 bytes per line, and each
-// line a kernel touches costs it about a quarter of a microsecond (measured: 32 more bytes of arguments, which pushed the
-// launch dimensions the kernel also read into one more line, took the decode step from 1.177 to 1.204 ms).  What the
-// plain batch-1 linear reads comes first and fills one line; the grid size rides along (nwaves) so that the register
-// kernel never reads the launch dimensions; the expert forms' fields follow and are only read by their instantiations.
+// What a launcher knows about one GEMV.  The LDS-staged kernel takes the struct as its argument; the register kernel
+// takes the fields of the first block as ten scalar arguments, which arrive in scalar registers with the wave, and the
+// rest as a struct of its own behind them.  Why the split: a kernel's arguments sit in memory that every launch reads
+// cold, 64 bytes per line; the read at the start of the batch-1 linear cost 0.4 us per launch, and each further line a
+// kernel touched another 0.1-0.25 us (measured: 32 more bytes of arguments, which pushed the launch dimensions the
+// kernel also read into one more line, took a 129-launch decode step from 1.177 to 1.204 ms; the first block alone in
+// one line 1.179 -> 1.160; no read at all 1.161 -> 1.108).
 struct GemvParams {
-  // ---- line 0: every form
+  // ---- every form (the register kernel's leading arguments, with nw = 4 * ng)
   const uint16_t* x;
   const uint32_t* qw;
   const uint16_t* qs;
@@ -42,7 +42,7 @@ struct GemvParams {
   int bf16;    // x, q_scale, bias, residual and a 16-bit y are bfloat16 (register kernel only)
   int routed = 0;
   int gc;  // groups staged per LDS chunk (multiple of 64; LDS kernel)
-  // ---- line 1: bias / residual forms and expert forms
+  // ---- bias / residual forms and expert forms
   const uint16_t* bias;
   const uint16_t* residual;  // [M, N] or null
   const int32_t* expert_ids;
@@ -57,13 +57,12 @@ struct GemvParams {
   int indptr_i64;
   int x_src_rows;
   // The token routes itself (register kernel, fused gate/up form of one row): `routed` is set and three fields change
-  // their meaning (a larger argument block would slow every launch of these kernels, see above): `bias` holds the
+  // their meaning: `bias` holds the
   // token's num_experts router logits in the model dtype, `residual` points at the top_k softmax weights to write and
   // `expert_ids` at the top_k ids to write.  Every workgroup picks the top gridDim.y logits (the insertion of the
   // routing kernels) and serves slot blockIdx.y's expert; the first workgroup leaves ids and weights for the operators
   // that follow.
 };
-static_assert(offsetof(GemvParams, bias) == 80, "the fields of the plain linear fill the first argument lines");
 
 
 // sum_k x_k * (field_k - m) for one group, given the 4 storage words and the staged x pairs

@@ -283,16 +283,19 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const void* __restrict_
 // table in (expert, chunk) order turns the counts into offsets.  Three barriers in all, where the
 // kernel above takes one per expert and round and re-reads k ids per token and expert.
 // do_topk 0: ids (and w) were produced by an earlier launch.  wave_topk: one wave per token.
+// flags = out_i64 | do_topk << 1 | wave_topk << 2 | waves of the workgroup << 8: with them in one word, everything the
+// kernel needs before its first loads is among the arguments that arrive in scalar registers.
 template <int DT>
 __global__ __launch_bounds__(1024) void moe_route_slots_kernel(const void* __restrict__ logits, int T, int ne, int k,
-                                                               void* __restrict__ w, int32_t* __restrict__ ids,
-                                                               int32_t* __restrict__ tok, int32_t* __restrict__ rev,
-                                                               int32_t* __restrict__ pos_of_slot, int out_i64,
-                                                               void* indptr, int do_topk, int wave_topk) {
+                                                               int flags, void* __restrict__ w,
+                                                               int32_t* __restrict__ ids, int32_t* __restrict__ tok,
+                                                               int32_t* __restrict__ rev,
+                                                               int32_t* __restrict__ pos_of_slot, void* indptr) {
   constexpr int kSlotsPerThread = 8;
   __shared__ int wave_tot[16];
   extern __shared__ int32_t cnt[];  // [ne, nchunks]: counts, then exclusive offsets
-  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int out_i64 = flags & 1, do_topk = flags & 2, wave_topk = flags & 4;
+  const int tid = threadIdx.x, nthreads = (flags >> 8) << 6;
   const int lane = tid & 63, wave = tid >> 6, nwaves = nthreads >> 6;
   const int S = T * k, nchunks = (S + 63) >> 6, N = ne * nchunks;
   if (do_topk) {
@@ -538,6 +541,39 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const void* __restrict
   Elem<DT>::store(out, i, acc);
 }
 
+// The same for 16-bit model dtypes with H a multiple of VEC (4 | 8) and 2 * VEC-byte aligned tensors: a thread owns VEC
+// consecutive h of one token, so every access is 8 or 16 bytes (per element the arithmetic above, in the same order).
+template <int DT, int VEC>
+__global__ __launch_bounds__(256) void moe_combine_vec_kernel(const void* __restrict__ y, const void* __restrict__ w,
+                                                              const int32_t* __restrict__ pos, int64_t T, int k,
+                                                              int64_t H, void* __restrict__ out) {
+  static_assert(DT != MODEL_F32, "16-bit elements");
+  struct alignas(2 * VEC) Pack { uint16_t v[VEC]; };
+  const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
+  if (i >= T * H) return;
+  const int64_t t = i / H, h = i - t * H;
+  float acc[VEC];
+  for (int j = 0; j < k; ++j) {
+    int64_t row = t * k + j;
+    if (pos != nullptr) {
+      row = pos[row];
+      row = row < 0 ? 0 : (row >= T * k ? T * k - 1 : row);
+    }
+    const Pack yv = *reinterpret_cast<const Pack*>(static_cast<const uint16_t*>(y) + row * H + h);
+    const float wj = Elem<DT>::load(w, t * k + j);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float ye = DT == MODEL_BF16 ? bf2f(yv.v[e]) : h2f(yv.v[e]);
+      const float prod = Elem<DT>::rnd(ye * wj);
+      acc[e] = (j == 0) ? prod : Elem<DT>::rnd(acc[e] + prod);
+    }
+  }
+  Pack o;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) o.v[e] = k > 0 ? (DT == MODEL_BF16 ? f2bf(acc[e]) : f2h(acc[e])) : uint16_t(0);
+  *reinterpret_cast<Pack*>(static_cast<uint16_t*>(out) + i) = o;
+}
+
 static inline unsigned blocks_for(int64_t n, int per) { return static_cast<unsigned>((n + per - 1) / per); }
 
 // dispatch on the model dtype: fn(std::integral_constant<int, DT>)
@@ -626,6 +662,25 @@ hipError_t launch_silu_mul(const void* x, int64_t R, int64_t I, void* out, int m
 hipError_t launch_moe_combine(const void* y, const void* w, const int32_t* pos, int64_t T, int k, int64_t H,
                               void* out, int model_dtype, hipStream_t s) {
   if (T * H == 0) return hipSuccess;
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(out);
+  if (model_dtype != MODEL_F32 && H % 4 == 0 && addr % 8 == 0) {
+    // 16 bytes per access once that still leaves a workgroup per CU, 8 below
+    const bool wide = H % 8 == 0 && addr % 16 == 0 && T * H >= 8 * 256 * 256;
+    auto go = [&](auto dt, auto vec) {
+      hipLaunchKernelGGL((moe_combine_vec_kernel<decltype(dt)::value, decltype(vec)::value>),
+                         dim3(blocks_for(T * H, 256 * decltype(vec)::value)), dim3(256), 0, s, y, w, pos, T, k, H, out);
+    };
+    if (model_dtype == MODEL_F16) {
+      if (wide) go(std::integral_constant<int, MODEL_F16>{}, std::integral_constant<int, 8>{});
+      else go(std::integral_constant<int, MODEL_F16>{}, std::integral_constant<int, 4>{});
+    } else if (model_dtype == MODEL_BF16) {
+      if (wide) go(std::integral_constant<int, MODEL_BF16>{}, std::integral_constant<int, 8>{});
+      else go(std::integral_constant<int, MODEL_BF16>{}, std::integral_constant<int, 4>{});
+    } else {
+      return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+  }
   return by_dtype(model_dtype, [&](auto dt) {
     hipLaunchKernelGGL(moe_combine_kernel<decltype(dt)::value>, dim3(blocks_for(T * H, 256)), dim3(256), 0, s, y, w,
                        pos, T, k, H, out);
@@ -658,8 +713,9 @@ hipError_t launch_moe_route(const void* logits, int64_t T, int ne, int k, void* 
     const size_t lds = static_cast<size_t>(ne) * ((slots + 63) / 64) * sizeof(int32_t);
     return by_dtype(model_dtype, [&](auto dt) {
       hipLaunchKernelGGL(moe_route_slots_kernel<decltype(dt)::value>, dim3(1), dim3(threads), lds, s, logits,
-                         static_cast<int>(T), ne, k, w, ids, tok, rev, pos_of_slot, out_i64, indptr,
-                         topk_first ? 0 : 1, by_wave ? 1 : 0);
+                         static_cast<int>(T), ne, k,
+                         (out_i64 ? 1 : 0) | (topk_first ? 0 : 2) | (by_wave ? 4 : 0) | (threads >> 6) << 8, w, ids, tok,
+                         rev, pos_of_slot, indptr);
     });
   }
   int threads = static_cast<int>((T + 63) / 64) * 64;
