@@ -218,8 +218,11 @@ hipError_t launch_gemm(const GemmArgs& a, hipStream_t s) {
   {
     const int64_t x_rows_total = a.x_rows != nullptr ? a.x_src_rows : a.rows;
     const int64_t limit = int64_t(1) << 32;
-    p.fast_ok = a.K % (2 * a.group_size) == 0 && x_rows_total * a.K * 2 < limit && a.N * p.nw * 4 < limit &&
+    // (q3f16_1 handles a last K tile that reaches past K inside that form: 80-wide tiles divide no power of two)
+    const bool k_ok = a.bits == 3 ? a.K % 8 == 0 : a.K % (2 * a.group_size) == 0;
+    p.fast_ok = k_ok && x_rows_total * a.K * 2 < limit && a.N * p.nw * 4 < limit &&
                 options().gemm_fast_loop != 0;  // (tuning / test override: general loop only)
+    p.x_bytes = p.fast_ok ? static_cast<uint32_t>(x_rows_total * a.K * 2) : 0u;
   }
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   const int variant = options().gemm_variant;

@@ -49,6 +49,7 @@ struct GemmParams {
   // every byte offset into x, one expert's q_weight and q_scale fits 32 bits, and K is whole K tiles of two groups
   // (set by the launcher; lets interior workgroups address with a uniform base plus a 32-bit lane offset)
   int fast_ok = 0;
+  uint32_t x_bytes = 0;  // size of x (the form without zero-selects, whose offsets fit 32 bits)
 };
 
 // column c of the block-interleaved order above -> stored weight row (clamped into its half).

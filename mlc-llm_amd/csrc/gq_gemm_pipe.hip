@@ -27,7 +27,10 @@ namespace gq {
 // registers, K tile as the scalar offset, one 32-bit lane offset): 122 -> 62 VALU instructions per wave and K tile.  Rows
 // past the segment and columns past N need no zeros: their loads are clamped to valid rows when the offsets are set up, a
 // row of x or of W only ever reaches its own row or column of the result, and the epilogue drops those; only k past K
-// would reach live results, and in this form there is none.  A separate instantiation rather than a branch: the general
+// would reach live results: q4 runs this form only when there is none; q3f16_1, whose 80-wide K tiles divide no power of two
+// (K = 4096 is 51.2 tiles), masks the activation chunks at k >= K and gives a group past the last one scale 0 (one AND per
+// chunk word, one select per group), and its descriptors carry the tensors' sizes, so that the last row's overrun reads
+// zeros instead of the bytes behind the tensor.  A separate instantiation rather than a branch: the general
 // form's addresses and flags would otherwise stay in registers next to this one's, and the large tile has none to spare
 // (a spill reload inside the loop waits for every global load in flight).
 template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false, int WX = 0,
@@ -146,9 +149,13 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // K tile kt into registers.  Always valid addresses; validity is re-derived at store time.
   // (buffer loads: the descriptor of each tensor sits in scalar registers, the K tile is the scalar offset and the lane
   //  offset one 32-bit register, so no 64-bit address is formed or kept per load)
-  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.x), short(0), -1, 0x00020000);
-  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(qw), short(0), -1, 0x00020000);
-  const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(qs), short(0), -1, 0x00020000);
+  constexpr bool KTAIL = FAST && BITS == 3;  // the last K tile may reach past K
+  const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(p.x), short(0), KTAIL ? static_cast<int>(p.x_bytes) : -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint32_t*>(qw), short(0), KTAIL ? static_cast<int>(static_cast<uint32_t>(p.N) * static_cast<uint32_t>(p.nw) * 4u) : -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint16_t*>(qs), short(0), KTAIL ? static_cast<int>(static_cast<uint32_t>(p.N) * static_cast<uint32_t>(p.ng) * 2u) : -1, 0x00020000);
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   auto load_a_fast = [&](int kt, StageA& st) {  // (tiles past the end re-read the last one: never multiplied)
     const int soff = min(kt, kt1 - 1) * (BK * 2);
@@ -209,15 +216,16 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
       // (the zero for rows past the segment and k past K as an AND with a lane mask: written as a select of the four
       //  words it becomes a branch around four moves, and control flow inside the loop makes the wait-count insertion
       //  drain every load in flight at the loop header)
-      const uint32_t keep = (FAST || (a_row_ok[i] && (k_base + a_k[i] < k_lim))) ? 0xffffffffu : 0u;
+      const bool kept = KTAIL ? k_base + a_k[i] < p.K : (FAST || (a_row_ok[i] && (k_base + a_k[i] < k_lim)));
+      const uint32_t keep = kept ? 0xffffffffu : 0u;
       if (A_EXACT || a_in_tile[i])
         *reinterpret_cast<uint4*>(at + a_dst[i]) =
-            FAST ? sa.a[i] : make_uint4(sa.a[i].x & keep, sa.a[i].y & keep, sa.a[i].z & keep, sa.a[i].w & keep);
+            (FAST && !KTAIL) ? sa.a[i] : make_uint4(sa.a[i].x & keep, sa.a[i].y & keep, sa.a[i].z & keep, sa.a[i].w & keep);
     }
     if (!w_active) return;
 #pragma unroll
     for (int i = 0; i < W_GROUPS; ++i) {
-      const bool ok = FAST || 2 * kt + w_g[i] < g_lim;
+      const bool ok = KTAIL ? 2 * kt + w_g[i] < p.ng : (FAST || 2 * kt + w_g[i] < g_lim);
       // a group past the end gets scale +0.0: every value becomes (q - m) * 0 = +-0
       const uint16_t sb = ok ? static_cast<uint16_t>(st.s[i]) : uint16_t(0);
       uint4* dst = reinterpret_cast<uint4*>(wt + w_dst[i]);

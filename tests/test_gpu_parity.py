@@ -477,6 +477,40 @@ def test_gemm_fast_and_general_loop_agree_bit_for_bit(name, m):
     assert_linear_ok(outs[0][1], o.linear_fp32(x, qw, qs, s), x, k, f"fast loop {name} m={m}")
 
 
+@pytest.mark.parametrize("m", [17, 100, 300, 1100, 2048])
+@pytest.mark.parametrize("k", [4096, 1000, 11008, 200, 88])
+def test_gemm_q3_fast_loop_with_a_k_tail(m, k):
+    """q3f16_1: K is rarely whole 80-wide K tiles (4096 = 51.2 of them), so its K loop without zero-selects masks the
+    activation chunks at k >= K and zeroes the scale of a group past the last.  Against the general loop: identical bits,
+    also when the values a masked chunk reads (the head of the next row of x) are NaN; against the oracle on the rest."""
+    s = SCHEMES["q3f16_1"]
+    n = 1060 if k <= 4096 else 300
+    x, qw, qs, b = _linear_case(s, m, n, k, 7 * m + k, bias=True)
+    x = x.copy()
+    bad = min(5, m - 1)
+    x[bad, : min(64, k)] = np.nan  # what the last K tile of row bad - 1 reads past its end
+    outs = []
+    for fast_loop in (-1, 0):
+        gq._lib.set_option("gemm_fast_loop", fast_loop)
+        try:
+            outs.append((ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b)),
+                         ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32),
+                         ops.linear_silu_mul(dev(x), dev(qw), dev(qs), s.bits, s.group_size)))
+            if fast_loop == -1 and m == 2048 and k == 4096:  # (the shape of the benchmark's q3f16_1 prefill)
+                assert gq._lib.last_kernel().startswith("gq::gemm_pipe_kernel<3,") and \
+                    gq._lib.last_kernel().endswith("true>"), gq._lib.last_kernel()
+        finally:
+            gq._lib.set_option("gemm_fast_loop", -1)
+    keep = np.arange(m) != bad
+    for a, c in zip(*outs):
+        a, c = a.cpu().numpy(), c.cpu().numpy()
+        assert np.isnan(a[bad]).all() and np.isnan(c[bad]).all()
+        assert np.array_equal(a[keep], c[keep])
+    y32 = outs[0][1].cpu().numpy()[keep]
+    assert np.isfinite(y32).all()
+    assert_linear_ok(torch.from_numpy(y32), o.linear_fp32(x[keep], qw, qs, s), x[keep], k, f"q3 fast loop k tail m={m} k={k}")
+
+
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("m", [17, 32, 33, 64, 100, 129, 256, 300, 700, 1024])
 @pytest.mark.parametrize("n,k", [(520, 4096), (130, 14336), (384, 1000)])
