@@ -52,6 +52,7 @@ struct QuadParams {
   const int32_t* x_rows;  // null, or the row of x each activation row reads (int32 [rows])
   int x_src_rows;         // rows of x when x_rows is set
   int bf16;               // x, scales, bias, residual and a 16-bit y are bfloat16
+  int kw_log2 = 0;        // log2 of the waves that share a quad set's K range (launcher: one phase, one round)
 };
 
 // The kernel's ten leading arguments (14 dwords) arrive in scalar registers with the wave: x, qw, qs, y, rows, N, K and three
@@ -68,7 +69,7 @@ struct QuadTail {
   int x_src_rows;
 };
 // packed words: w0 = nsteps | steps_total << 16, w1 = rounds | nwaves << 16,
-// w2 = nphases | flags << 16 | waves per workgroup << 24
+// w2 = nphases | flags << 16 | log2(waves that share a quad set) << 20 | waves per workgroup << 24
 constexpr uint32_t kQuadOutF32 = 1u << 16, kQuadIndptrI64 = 1u << 17, kQuadHasTail = 1u << 18;
 
 template <int CTRL>
@@ -103,10 +104,12 @@ __device__ __forceinline__ float4_t mfma4_bf16(uint32_t a0, uint32_t a1, uint32_
 // QP: quads per item.  The x operands of an iteration are read from LDS once and meet the weights of QP
 // consecutive quads, so the LDS bytes read per weight byte fall by that factor (a 4x4x4 block needs as many
 // operand bytes of x as of weights: with 8 activation rows that is 8 LDS bytes per packed weight byte at QP = 1).
-template <int BITS, int NBQ, int U, int MODE, bool BF = false, int QP = 1>
+// KS: neighbouring waves may share the K range of a quad set (see kw_log2 below).  An instantiation of its own: with the
+// split's bookkeeping the forms that run sixteen-wave workgroups no longer fit their 128 registers.
+template <int BITS, int NBQ, int U, int MODE, bool BF = false, int QP = 1, bool KS = false>
 // (sixteen-wave workgroups exist for the forms that fit 128 registers: 2 KiB items without the bias / residual loads;
 //  with them the same bound forced spill reloads into the walk, and a reload waits for every weight load in flight)
-__global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_kernel(const uint16_t* x_, const uint32_t* qw_, const uint16_t* qs_, void* y_, int rows_, int N_, int K_,
+__global__ __launch_bounds__((U * QP <= 2 && MODE != 1 && !KS) ? 1024 : 512) void quad_kernel(const uint16_t* x_, const uint32_t* qw_, const uint16_t* qs_, void* y_, int rows_, int N_, int K_,
                  uint32_t w0, uint32_t w1, uint32_t w2, const QuadTail t) {
   QuadParams p;
   p.x = x_; p.qw = qw_; p.qs = qs_; p.y = y_;
@@ -138,7 +141,14 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
   const int lane = tid & 63;
   const int wpb = nthreads >> 6;
   const int gw = blockIdx.x * wpb + (tid >> 6);
-  const int nwaves = static_cast<int>(w1 >> 16);
+  // K shared among neighbouring waves (matrices with few quads, where every wave has one quad set at most: a wave is
+  // one dependent chain of loads, LDS reads and matrix instructions over its K range, and on such launches a SIMD hosts
+  // a single wave, so nothing overlaps the chain): 2^kw_log2 consecutive waves of a workgroup take equal shares of the
+  // steps of the same quad set, leave their sums in LDS, and the first of them adds the shares up after the walk.
+  const int kw_log2 = KS ? static_cast<int>(w2 >> 20) & 3 : 0;
+  const int ksub = gw & ((1 << kw_log2) - 1);
+  const int gwq = gw >> kw_log2;
+  const int nwaves = static_cast<int>(w1 >> 16) >> kw_log2;  // stride of the walk over quad sets
   const int li = lane & 3;   // weight row of the quad (A), activation row of the batch quad (B, D)
   const int ks = lane >> 2;  // block: group 16 * iteration + ks
 
@@ -181,8 +191,12 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
   // K is walked in phases when x does not fit LDS whole: every phase stages its slice of x and
   // walks all of this wave's quads; partial sums wait in LDS for the last phase.
   for (int phase = 0; phase < p.nphases; ++phase) {
-    const int nst = min(p.nsteps, p.steps_total - phase * p.nsteps);  // steps of this phase
-    const int it0 = phase * niter;                                    // first iteration of the phase
+    const int nst_all = min(p.nsteps, p.steps_total - phase * p.nsteps);  // steps of this phase
+    const int spw = (nst_all + (1 << kw_log2) - 1) >> kw_log2;            // ... per wave of a quad set
+    const int step0 = ksub * spw;
+    const int nst = max(0, min(spw, nst_all - step0));                    // ... of this wave (all of them unless K is shared)
+    const int it0 = phase * niter;                                        // first iteration of the phase
+    const int itw = step0 * U;                                            // ... of this wave inside the phase
     const bool last_phase = phase == p.nphases - 1;
 #pragma unroll
     for (int qp = 0; qp < QP; ++qp)
@@ -204,7 +218,7 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
         const uint16_t* sr = qs + static_cast<int64_t>(row) * p.ng;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          const int g = min((it0 + step * U + u) * 16 + ks, p.ng - 1);
+          const int g = min((it0 + itw + step * U + u) * 16 + ks, p.ng - 1);
           wn[qp][u] = *reinterpret_cast<const uint4*>(live ? wr + 4 * g : qw);
           sn[qp][u] = *(live ? sr + g : qs);
         }
@@ -233,7 +247,8 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
         }
       }
     };
-    int qa = gw, sta = 0, qb = gw, stb = 1;
+    const int q_first = nst > 0 ? gwq : p.nsets;  // (a wave whose share of the steps is empty has no quad set)
+    int qa = q_first, sta = 0, qb = q_first, stb = 1;
     if (stb >= nst) {
       stb = 0;
       qb += nwaves;
@@ -324,12 +339,27 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
     __syncthreads();
 
     // ---- persistent walk
+    // the four results of (activation row m0 + b, quad) leave in the output's type
+    auto put = [&](int quad, int b, const float (&v)[4]) {
+      const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
+      if constexpr (PAIRED) {
+        *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p.y) + (oi >> 1)) =
+            static_cast<uint32_t>(silu_mul_t<BF>(v[0], v[1])) | (static_cast<uint32_t>(silu_mul_t<BF>(v[2], v[3])) << 16);
+      } else if (p.out_f32) {
+        *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+        uint2 o;
+        o.x = static_cast<uint32_t>(to_out(v[0])) | (static_cast<uint32_t>(to_out(v[1])) << 16);
+        o.y = static_cast<uint32_t>(to_out(v[2])) | (static_cast<uint32_t>(to_out(v[3])) << 16);
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.y) + oi) = o;
+      }
+    };
     int done = 0;  // quads this wave has completed in this phase
     auto compute = [&](int qset, int step, const uint4 (&wc)[QP][U], const uint32_t (&sc)[QP][U],
                        const uint2 (&bias_bits)[QP], const uint2 (&res_bits)[QP][NBQ]) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int it = step * U + u;
+        const int it = itw + step * U + u;
         // A operands: q4 lo/hi = even / odd fields (x1, x16) of word d; q3 a1/a8 = the x1 / x8
         // fields of word d, a64 = the x64 field pairs of words (0,1) and (2,3)
         uint32_t lo[QP][4][2], hi[QP][4][2], a64[QP][2][2];
@@ -421,6 +451,10 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
             const int b = 4 * bq + lane;  // lanes 0..3: one activation row each, 4 weight rows
             if (lane < 4 && b < m_valid && quad < p.nquads) {
               float4* part = reinterpret_cast<float4*>(part_lds) + ((done * QP + qp) * NBQ + bq) * 4 + lane;
+              if (kw_log2 != 0) {  // (uniform) this wave's share of K: the shares meet after the walk
+                *part = make_float4(v[0], v[1], v[2], v[3]);
+                continue;
+              }
               if (phase > 0) {
                 const float4 pv = *part;
                 v[0] += pv.x; v[1] += pv.y; v[2] += pv.z; v[3] += pv.w;
@@ -440,20 +474,7 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
                   v[2] += to_f32(static_cast<uint16_t>(res_bits[qp][bq].y & 0xffffu));
                   v[3] += to_f32(static_cast<uint16_t>(res_bits[qp][bq].y >> 16));
                 }
-                const int64_t oi = static_cast<int64_t>(m0 + b) * p.N + quad * 4;
-                if constexpr (PAIRED) {
-                  *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(p.y) + (oi >> 1)) =
-                      static_cast<uint32_t>(silu_mul_t<BF>(v[0], v[1])) |
-                      (static_cast<uint32_t>(silu_mul_t<BF>(v[2], v[3])) << 16);
-                } else if (p.out_f32) {
-                  *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) =
-                      make_float4(v[0], v[1], v[2], v[3]);
-                } else {
-                  uint2 o;
-                  o.x = static_cast<uint32_t>(to_out(v[0])) | (static_cast<uint32_t>(to_out(v[1])) << 16);
-                  o.y = static_cast<uint32_t>(to_out(v[2])) | (static_cast<uint32_t>(to_out(v[3])) << 16);
-                  *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.y) + oi) = o;
-                }
+                put(quad, b, v);
               }
             }
           }
@@ -472,20 +493,52 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1) ? 1024 : 512) void quad_
       issue(qb, stb, wb, sb, bb, rb);
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (kw_log2 != 0) {  // (uniform over the launch; one phase, one quad set per group of waves: see the launcher)
+      __syncthreads();
+      if (ksub == 0 && gwq < p.nsets && lane < 4) {
+        const int stride = p.rounds * QP * NBQ * 16;  // floats between the slots of consecutive waves
+#pragma unroll
+        for (int qp = 0; qp < QP; ++qp) {
+          const int quad = gwq * QP + qp;
+#pragma unroll
+          for (int bq = 0; bq < NBQ; ++bq) {
+            const int b = 4 * bq + lane;
+            if (b < m_valid && quad < p.nquads) {
+              float v[4] = {0.f, 0.f, 0.f, 0.f};
+              for (int j = 0; j < (1 << kw_log2) && j * spw < nst_all; ++j) {  // in wave order, whatever finished first
+                const float4 pv = reinterpret_cast<const float4*>(part_lds + j * stride)[(qp * NBQ + bq) * 4 + lane];
+                v[0] += pv.x; v[1] += pv.y; v[2] += pv.z; v[3] += pv.w;
+              }
+              put(quad, b, v);
+            }
+          }
+        }
+      }
+    }
   }
 }
 
 template <int BITS, int NBQ, int U, int MODE, bool BF = false, int QP = 1>
 static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads, size_t lds,
                                     hipStream_t s) {
+  constexpr bool KS_OK = MODE != 1 && U * QP <= 2;  // the forms that exist with K shared between waves
+  const bool ks = p.kw_log2 != 0;
+  if (ks && !KS_OK) return hipErrorNotSupported;
   if (lds > 65536) {
-    const hipError_t e = allow_large_lds(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF, QP>));
+    hipError_t e = hipSuccess;
+    if constexpr (KS_OK) {
+      if (ks) e = allow_large_lds(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF, QP, true>));
+    }
+    if (!ks) e = allow_large_lds(reinterpret_cast<const void*>(&quad_kernel<BITS, NBQ, U, MODE, BF, QP>));
     if (e != hipSuccess) return e;
   }
-  note_kernel("gq::quad_kernel<%d,%d,%d,%d,%s,%d>", BITS, NBQ, U, MODE, BF ? "true" : "false", QP);
+  note_kernel("gq::quad_kernel<%d,%d,%d,%d,%s,%d%s>", BITS, NBQ, U, MODE, BF ? "true" : "false", QP, ks ? ",true" : "");
   const int nwaves = static_cast<int>(grid.x) * (threads >> 6);
-  if (threads % 64 != 0 || threads > 1024 || p.nsteps > 0xffff || p.steps_total > 0xffff || p.rounds > 0xffff ||
-      nwaves > 0xffff || p.nphases > 0xffff || p.nquads != p.N / 4 || p.nsets != (p.nquads + QP - 1) / QP)
+  if (threads % 64 != 0 || threads > (ks ? 512 : 1024) || p.nsteps > 0xffff || p.steps_total > 0xffff || p.rounds > 0xffff ||
+      nwaves > 0xffff || p.nphases > 0xffff || p.nquads != p.N / 4 || p.nsets != (p.nquads + QP - 1) / QP ||
+      p.kw_log2 < 0 || p.kw_log2 > 2 ||
+      (p.kw_log2 != 0 && (p.nphases != 1 || p.rounds != 1 || MODE == 1 || (threads >> 6) % (1 << p.kw_log2) != 0 ||
+                          (nwaves >> p.kw_log2) < p.nsets)))
     return hipErrorNotSupported;
   const bool tail = p.indptr != nullptr || p.x_rows != nullptr || p.bias != nullptr || p.residual != nullptr;
   const QuadTail t{p.indptr, p.x_rows, p.expert_w_stride, p.expert_s_stride, p.bias, p.residual, p.x_src_rows};
@@ -493,7 +546,14 @@ static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads,
   const uint32_t w1 = static_cast<uint32_t>(p.rounds) | static_cast<uint32_t>(nwaves) << 16;
   const uint32_t w2 = static_cast<uint32_t>(p.nphases) | (p.out_f32 ? kQuadOutF32 : 0u) |
                       (p.indptr_i64 ? kQuadIndptrI64 : 0u) | (tail ? kQuadHasTail : 0u) |
-                      static_cast<uint32_t>(threads >> 6) << 24;
+                      static_cast<uint32_t>(p.kw_log2) << 20 | static_cast<uint32_t>(threads >> 6) << 24;
+  if constexpr (KS_OK) {
+    if (ks) {
+      hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF, QP, true>), grid, dim3(threads), lds, s,
+                         p.x, p.qw, p.qs, p.y, p.rows, p.N, p.K, w0, w1, w2, t);
+      return hipGetLastError();
+    }
+  }
   hipLaunchKernelGGL((quad_kernel<BITS, NBQ, U, MODE, BF, QP>), grid, dim3(threads), lds, s,
                      p.x, p.qw, p.qs, p.y, p.rows, p.N, p.K, w0, w1, w2, t);
   return hipGetLastError();
@@ -613,16 +673,32 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   // of 8 waves): then 4 waves per workgroup and twice the workgroups
   // ... and for a plain linear in general: every workgroup stages all of x, so eight waves sharing one copy
   // halve that traffic (qkv 6144 x 4096 at 8 rows 11.4 -> 9.9 us, gate_up 24.3 -> 22.6; never slower)
+  // K shared among 2 neighbouring waves: a plain linear whose waves have one quad set at most, on a long K (every wave
+  // keeps five steps or more) and while the launch stays within two waves per SIMD.  Measured at 4 rows: 4096 x 14336
+  // 15.7 -> 14.0 us, 4096 x 11008 12.7 -> 11.6; with four steps per wave to share (K = 4096) the meeting of the shares costs
+  // more than the shorter chains return (o_proj 6.5 -> 7.1 us), past two waves per SIMD it loses outright (6144 x 4096:
+  // 8.0 -> 12.4), and so do four waves per quad set (14.5 -> 19.6).
+  // Tuning override: quad_ksplit 0 | 1 | 2.
+  p.kw_log2 = 0;
+  if (a.indptr == nullptr && p.nphases == 1 && p.rounds == 1 && a.bias == nullptr && a.residual == nullptr &&
+      U * QP <= 2 && !big_wg) {
+    const int opt_kw = options().quad_ksplit;
+    const int want = opt_kw >= 0 ? opt_kw : 1;
+    while (p.kw_log2 < want && p.kw_log2 < 2 && (p.steps_total >> (p.kw_log2 + 1)) >= (opt_kw >= 0 ? 1 : 5) &&
+           (static_cast<int64_t>(p.nsets) * mtiles << (p.kw_log2 + 1)) <= (opt_kw >= 0 ? 4096 : 2048))
+      ++p.kw_log2;
+  }
+  const int sets_w = ((p.nsets + p.rounds - 1) / p.rounds) << p.kw_log2;  // waves of one grid row that have work
   int threads = (lds_x > 76 * 1024 || a.indptr == nullptr) ? 512 : 256;
   if (threads == 512) {
-    const int64_t wgs = static_cast<int64_t>(((p.nsets + p.rounds - 1) / p.rounds + 7) / 8) * busy * mtiles;
+    const int64_t wgs = static_cast<int64_t>((sets_w + 7) / 8) * busy * mtiles;
     if (2 * wgs <= 256) threads = 256;  // (the doubled count must still be one round of workgroups)
   }
   // four waves per SIMD share one copy of x (the instances that fit 128 registers: 2 KiB items without bias / residual loads)
   if (big_wg && p.nphases == 1 && U * QP <= 2 && a.bias == nullptr && a.residual == nullptr) threads = 1024;
   const int wpb = threads / 64;
-  const size_t lds = lds_x + (p.nphases > 1 ? static_cast<size_t>(wpb) * p.rounds * QP * nbq * 64 : 0);
-  const int blocks = ((p.nsets + p.rounds - 1) / p.rounds + wpb - 1) / wpb;
+  const size_t lds = lds_x + ((p.nphases > 1 || p.kw_log2 != 0) ? static_cast<size_t>(wpb) * p.rounds * QP * nbq * 64 : 0);
+  const int blocks = (sets_w + wpb - 1) / wpb;
   const dim3 grid(blocks, experts, mtiles);
 #define GQ_QUAD_CASE(NBQ_, U_) \
   if (nbq == NBQ_ && U == U_) return launch_quad_cfg<BITS, NBQ_, U_>(p, grid, threads, lds, s);

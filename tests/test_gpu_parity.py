@@ -354,6 +354,37 @@ def test_quadrow_kernel(name, u, qp, m, n, k):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("ksplit", [0, 1, 2])  # 1, 2, 4 neighbouring waves share the K range of a quad set
+@pytest.mark.parametrize("qp", [1, 2])
+@pytest.mark.parametrize("m", [3, 4, 8])
+@pytest.mark.parametrize("n,k", [(520, 1024), (100, 4096), (1024, 4096), (64, 6176), (4, 256), (36, 2080)])
+def test_quadrow_kernel_k_shared_between_waves(name, ksplit, qp, m, n, k):
+    """Matrices with few quads: the waves of a workgroup split the K range of a quad set and the first of them adds the
+    shares up after the walk (step counts that do not divide, shares that come out empty, an odd number of quads with two
+    quads per item); plain, float32 and folded-activation outputs against the oracle."""
+    s = SCHEMES[name]
+    if s.bits == 3:
+        k = {1024: 1000, 4096: 4000, 6176: 6200, 256: 240, 2080: 2080}[k]
+    x, qw, qs, _ = _linear_case(s, m, n, k, 3 * m + n + k + ksplit, bias=False)
+    gq._lib.set_option("gemv_variant", 6)
+    gq._lib.set_option("quad_pairs", qp)
+    gq._lib.set_option("quad_ksplit", ksplit)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None)
+        assert gq._lib.last_kernel().startswith("gq::quad_kernel"), gq._lib.last_kernel()
+        y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
+        if n % 8 == 0:  # the folded activation shares the K range the same way: same bits as the two steps
+            assert torch.equal(ops.linear_silu_mul(dev(x), dev(qw), dev(qs), s.bits, s.group_size), ops.silu_mul(y))
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+        gq._lib.set_option("quad_pairs", -1)
+        gq._lib.set_option("quad_ksplit", -1)
+    ref = o.linear_fp32(x, qw, qs, s)
+    assert_linear_ok(y, ref, x, k, f"quad-row k shared {name} ksplit={ksplit} qp={qp} {m}x{n}x{k}")
+    assert_linear_ok(y32, ref, x, k, f"quad-row k shared ksplit={ksplit} qp={qp} fp32 out")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("waves", [-1, 8])  # 8 waves in all: every wave walks many quads
 @pytest.mark.parametrize("qp", [1, 2])
 @pytest.mark.parametrize("m,n,k", [(8, 64, 14336), (5, 520, 20520), (3, 132, 20480), (8, 520, 8200), (8, 36, 14336)])
