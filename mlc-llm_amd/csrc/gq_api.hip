@@ -153,6 +153,9 @@ int mi355gq_testing_set_option(const char* name, int value) {
   } else if (!strcmp(name, "gemm_fast_loop")) {
     GQ_REQUIRE(value == -1 || value == 0, "gemm_fast_loop=%d (0)", value);
     o.gemm_fast_loop = value;
+  } else if (!strcmp(name, "gemv_ksplit")) {
+    GQ_REQUIRE(value >= -1 && value <= 1, "gemv_ksplit=%d (-1, 0, 1)", value);
+    o.gemv_ksplit = value;
   } else if (!strcmp(name, "quad_ksplit")) {
     GQ_REQUIRE(value >= -1 && value <= 2, "quad_ksplit=%d (-1, 0, 1, 2)", value);
     o.quad_ksplit = value;

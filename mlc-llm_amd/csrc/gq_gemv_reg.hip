@@ -41,7 +41,10 @@ struct GemvTail {
 
 // MOE: an expert form (expert ids, expert-sorted rows, one grid row per slot).  The plain linear's instantiation reads
 // none of those fields.
-template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false, bool MOE = true>
+// KW = 2 (long K, one row per set, plain epilogue): two neighbouring waves share every row, each with ITERS groups per
+// lane of its half of K; the halves' sums wait in LDS and meet after the walk (one barrier in all).  A wave then holds
+// half of x in registers, so two waves fit a SIMD where the whole-K form runs one.
+template <int BITS, int NB, int R, int ITERS, int MODE, bool BF = false, bool MOE = true, int KW = 1>
 __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const uint32_t* qw_, const uint16_t* qs_,
                                                         void* y_, int N_, int K_, int ng_, int nsets, int nwaves_,
                                                         int out_f32_, const GemvTail t) {
@@ -61,14 +64,17 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
   constexpr int G = T::G;
   constexpr int HP = G / 2;  // half pairs of x per group
   // 16-byte x chunks each of the 256 threads stages: NB * ITERS * 64 groups * G/8 chunks / 256
-  constexpr int XS = (NB * ITERS * 64 * (G / 8) + 255) / 256;
+  constexpr int XS = (NB * ITERS * KW * 64 * (G / 8) + 255) / 256;
 
   extern __shared__ uint4 smem[];  // x as [NB][ng * G] halves, zero beyond K
   const int kpad = p.ng * G;
 
   const int lane = threadIdx.x & 63;
-  const int gw = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int nwaves = p.nwaves;
+  static_assert(KW == 1 || (KW == 2 && R == 1 && NB == 1 && MODE == 0), "shared K: one row per set, plain epilogue");
+  const int wave_all = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int ksub = KW == 2 ? (wave_all & 1) : 0;           // which half of K
+  const int gw = KW == 2 ? (wave_all >> 1) : wave_all;     // walker of row sets
+  const int nwaves = KW == 2 ? (p.nwaves >> 1) : p.nwaves;
   const int slot = MOE ? blockIdx.y : 0;
 
   const uint16_t* x = MOE ? p.x + slot * p.x_slot_stride : p.x;
@@ -144,7 +150,7 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
   bool gok[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
-    const int g = it * 64 + lane;
+    const int g = (ksub * ITERS + it) * 64 + lane;
     gok[it] = g < p.ng;
     gidx[it] = gok[it] ? g : p.ng - 1;
   }
@@ -219,6 +225,10 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
     }
   }
 
+  // (shared K) the halves' row sums: [4 waves][kPartSlots] floats behind x
+  constexpr int kPartSlots = 64;
+  float* const part = reinterpret_cast<float*>(smem) + NB * kpad / 2;
+  int part_n = 0;
   // ---- persistent walk: reduce one set, then refill its registers with the set two strides on
   auto reduce = [&](int cur, const uint4 (&wc)[R][ITERS], const uint32_t (&sc)[R][ITERS],
                     uint32_t bias_bits) {
@@ -237,6 +247,12 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
         }
         acc[r][b] = wave_sum_last(a);
       }
+    if constexpr (KW == 2) {
+      // this half's sum of row `cur` waits in LDS: slot [wave of the workgroup][sets this wave has reduced so far]
+      if (lane == 63 && cur < nsets) part[(threadIdx.x >> 6) * kPartSlots + part_n] = acc[0][0];
+      ++part_n;
+      return;
+    }
     if constexpr (PAIRED) {
       if (lane == 63) {
 #pragma unroll
@@ -289,6 +305,19 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
     issue(set_b, wb, sb, bb);
     __builtin_amdgcn_sched_barrier(0);
   }
+  if constexpr (KW == 2) {
+    // the halves meet: lane i of the first wave of a pair owns the i-th set the pair walked (the launcher keeps that
+    // count within kPartSlots)
+    __syncthreads();
+    const int set = gw + lane * nwaves;
+    if (ksub == 0 && lane < kPartSlots && set < nsets) {
+      const int w = threadIdx.x >> 6;
+      const float v = part[w * kPartSlots + lane] + part[(w + 1) * kPartSlots + lane];
+      const int64_t oi = static_cast<int64_t>(slot) * p.N + set;
+      if (p.out_f32) static_cast<float*>(p.y)[oi] = v;
+      else static_cast<uint16_t*>(p.y)[oi] = BF ? f2bf(v) : f2h(v);
+    }
+  }
 }
 
 template <int BITS, int NB, int R, int ITERS, int MODE, bool MOE>
@@ -331,6 +360,32 @@ static hipError_t launch_k(const GemvParams& p0, int slots, int blocks, int nset
                : launch_mode<BITS, NB, R, ITERS, 1, false>(p, grid, lds, s);
   return moe ? launch_mode<BITS, NB, R, ITERS, 0, true>(p, grid, lds, s)
              : launch_mode<BITS, NB, R, ITERS, 0, false>(p, grid, lds, s);
+}
+
+// Long K shared between two neighbouring waves (KW = 2): HALF groups per lane and wave.
+template <int BITS, int HALF>
+static hipError_t launch_shared_k(const GemvParams& p0, int slots, int blocks, int nsets, hipStream_t s) {
+  const size_t lds = static_cast<size_t>(p0.ng) * GemvTraits<BITS>::G * 2 + 4 * 64 * sizeof(float);
+  const dim3 grid(blocks, slots);
+  GemvParams p = p0;
+  p.nsets = nsets;
+  p.nwaves = blocks * 4;
+  const bool moe = slots != 1 || p.indptr != nullptr || p.expert_ids != nullptr;
+  note_kernel("gq::gemv_reg_kernel<%d,1,1,%d,0,%s,%s,2>", BITS, HALF, p.bf16 ? "true" : "false", moe ? "true" : "false");
+  const GemvTail t{p.expert_ids, p.expert_w_stride, p.expert_s_stride, p.x_slot_stride, p.bias, p.residual,
+                   p.num_experts, p.indptr_i64, p.indptr, p.x_row_index, p.x_src_rows};
+#define GQ_SHARED_K(BF_, MOE_)                                                                                      \
+  hipLaunchKernelGGL((gemv_reg_kernel<BITS, 1, 1, HALF, 0, BF_, MOE_, 2>), grid, dim3(256), lds, s, p.x, p.qw, p.qs, \
+                     p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, t)
+  if (p.bf16) {
+    if (moe) GQ_SHARED_K(true, true);
+    else GQ_SHARED_K(true, false);
+  } else {
+    if (moe) GQ_SHARED_K(false, true);
+    else GQ_SHARED_K(false, false);
+  }
+#undef GQ_SHARED_K
+  return hipGetLastError();
 }
 
 template <int BITS, int NB, int R>
@@ -393,6 +448,21 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
   if (slots > 1) waves = waves / (4 * slots) * 4;
   if (waves < 4) waves = 4;
   const int rounds = (nsets + waves - 1) / waves;
+  // Long K (5 to 12 groups per lane), one row, plain epilogue: two neighbouring waves share every row's K (3 to 6 groups
+  // per lane each, so that two waves fit a SIMD where the whole-K form runs one), twice the waves.
+  // Tuning override: gemv_ksplit 0 | 1.
+  const bool plain = !p.paired && !p.routed && p.bias == nullptr && p.residual == nullptr;
+  if (iters >= 5 && nb == 1 && R == 1 && plain && rounds <= 64 && options().gemv_ksplit != 0) {
+    const int half = (iters + 1) / 2;
+    const int blocks2 = (2 * ((nsets + rounds - 1) / rounds) + 3) / 4;
+    switch (half) {
+      case 3: return launch_shared_k<BITS, 3>(p, slots, blocks2, nsets, s);
+      case 4: return launch_shared_k<BITS, 4>(p, slots, blocks2, nsets, s);
+      case 5: return launch_shared_k<BITS, 5>(p, slots, blocks2, nsets, s);
+      case 6: return launch_shared_k<BITS, 6>(p, slots, blocks2, nsets, s);
+      default: break;
+    }
+  }
   const int blocks = ((nsets + rounds - 1) / rounds + 3) / 4;  // even share of sets per wave
   if (nb == 1) {
     if (R == 4) return launch_iters<BITS, 1, 4>(p, slots, iters, blocks, nsets, s);

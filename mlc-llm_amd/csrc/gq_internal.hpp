@@ -14,6 +14,7 @@ struct Options {
   int gemv_rows_per_wave = -1;  // -1: heuristic
   int gemm_fast_loop = -1;      // 0: the pipelined GEMM always runs its general K loop (with the zero-selects and clamps)
   int quad_pairs = -1;          // -1: heuristic, 1 | 2: quads per item of the quad-row kernel
+  int gemv_ksplit = -1;         // -1: heuristic, 0: never, 1: wherever it applies (register GEMV: two waves share a row's K)
   int quad_ksplit = -1;         // -1: heuristic, 0 | 1 | 2: log2 of the waves that share a quad set's K range
   int gemv_variant = -1;        // -1: heuristic, 0: LDS GEMV, 1: register GEMV, 2..5 skinny forms, 6..8 quad-row forms
   int gemm_variant = -1;

@@ -234,6 +234,36 @@ def test_one_and_two_rows_of_a_long_k(name, m, n, k):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("ksplit", [0, 1])
+@pytest.mark.parametrize("n,k", [(130, 8200), (1000, 11008), (4100, 14336), (66, 18944), (64, 24576), (40, 10240),
+                                 (9000, 8192)])
+def test_gemv_long_k_shared_between_two_waves(name, ksplit, n, k):
+    """One row, 5 to 12 groups per lane: two neighbouring waves take half of K each and their row sums meet in LDS after
+    the walk (odd group counts per lane, a last group that is partly filled, more row sets than waves, float32 output,
+    expert ids with their own rows of x); against the oracle, and forced off for the whole-K form next to it."""
+    s = SCHEMES[name]
+    x, qw, qs, _ = _linear_case(s, 1, n, k, n + k + ksplit, bias=False)
+    gq._lib.set_option("gemv_ksplit", ksplit)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None)
+        kern = gq._lib.last_kernel()
+        y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
+        # two expert slots reading rows 0 and 1 of x (the same matrix as both experts' weights, stacked)
+        x2 = np.concatenate([x, x[:, ::-1]], axis=0).copy()
+        qw2, qs2 = np.stack([qw, qw]), np.stack([qs, qs])
+        ids = np.array([[1, 0]], np.int32)
+        ym = ops.moe_gemv(dev(x2), dev(qw2), dev(qs2), dev(ids), s.bits, s.group_size)
+    finally:
+        gq._lib.set_option("gemv_ksplit", -1)
+    groups_per_lane = -(-(-(-k // s.group_size)) // 64)
+    assert kern.startswith("gq::gemv_reg_kernel") and kern.endswith(",2>") == (ksplit == 1 and groups_per_lane >= 5), kern
+    ref = o.linear_fp32(x, qw, qs, s)
+    assert_linear_ok(y, ref, x, k, f"gemv long K {name} ksplit={ksplit} {n}x{k}")
+    assert_linear_ok(y32, ref, x, k, f"gemv long K ksplit={ksplit} fp32 out")
+    assert_linear_ok(ym, o.moe_dequantize_gemv_fp32(x2, qw2, qs2, ids, s), x2, k, f"moe gemv long K ksplit={ksplit}")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_gemv_all_batches(name, m):
     s = SCHEMES[name]
