@@ -259,6 +259,19 @@ MI355GQ_API int mi355gq_moe_gemv_routed_silu_mul(const void* x, const void* gate
                                      int64_t top_k, const void* q_weight, const void* q_scale, int64_t N, int64_t K,
                                      int bits, int group_size, int model_dtype, void* expert_weights,
                                      void* expert_ids, void* out, mi355gq_stream_t stream);
+/*
+ * One token's e2 expert matmul and the weighted sum over its experts in one launch (MixtralMoE.forward with one token,
+ * mixtral_model.py:96-117: dequantize_gemv of moe_matmul.py:77-176 on the top_k rows of x, each against its expert,
+ * then x * expert_weights and moe_sum of moe_misc.py:14-32).  x [top_k, K], expert_ids int32 [top_k], expert_weights
+ * [top_k] and out [1, N] in the model dtype; out equals, bit for bit in its roundings (matmul result, product, sum, each
+ * rounded to the model dtype), mi355gq_moe_gemv_dt followed by mi355gq_moe_combine_dt up to the order in which a row's
+ * K is summed (two halves).  float16 / bfloat16 models, top_k = 2, K of 3 to 12 groups per lane (q4: 4097..24576 while
+ * both rows of x fit 63 KiB of LDS); MI355GQ_ERR_UNSUPPORTED otherwise (the caller then runs the two operators).
+ */
+MI355GQ_API int mi355gq_moe_gemv_combine(const void* x, const void* q_weight, const void* q_scale, int64_t N, int64_t K,
+                             int bits, int group_size, int model_dtype, int64_t num_experts,
+                             const void* expert_ids, const void* expert_weights, int64_t top_k, void* out,
+                             mi355gq_stream_t stream);
 MI355GQ_API int mi355gq_moe_group_gemm_silu_mul(const void* x, int64_t rows, const void* q_weight,
                                     const void* q_scale, const void* indptr, int indptr_dtype,
                                     int64_t num_experts, int64_t N, int64_t K, int bits, int group_size,

@@ -713,6 +713,38 @@ int mi355gq_moe_gemv_routed_silu_mul(const void* x, const void* gate_logits, int
   return hip_result(e, "moe_gemv_routed_silu_mul launch");
 }
 
+int mi355gq_moe_gemv_combine(const void* x, const void* q_weight, const void* q_scale, int64_t N, int64_t K, int bits,
+                             int group_size, int model_dtype, int64_t num_experts, const void* expert_ids,
+                             const void* expert_weights, int64_t top_k, void* out, mi355gq_stream_t stream) {
+  GQ_CHECK(check_model_dtype(model_dtype, "moe_gemv_combine"));
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(top_k >= 1 && N >= 0 && K >= 1 && N < kMaxDim && K < kMaxDim && num_experts >= 1 && num_experts < kMaxDim,
+             "moe_gemv_combine: bad shape (N=%lld, K=%lld, %lld experts, top_k=%lld)", (long long)N, (long long)K,
+             (long long)num_experts, (long long)top_k);
+  GQ_REQUIRE(x && q_weight && q_scale && expert_ids && expert_weights && (out || N == 0), "moe_gemv_combine: null pointer");
+  if (model_dtype == MI355GQ_F32 || top_k != 2 || (K & 7) != 0 || !aligned16(x) || !aligned16(q_weight) ||
+      !aligned2(q_scale) || !aligned4(expert_ids) || !aligned2(expert_weights) || !aligned2(out))
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_gemv_combine: float16 / bfloat16 models, top_k = 2, K a multiple of 8, "
+                                         "16-byte aligned x and q_weight");
+  if (N == 0) return MI355GQ_OK;
+  gq::GemvArgs a{};
+  a.x = static_cast<const uint16_t*>(x);
+  a.q_weight = static_cast<const uint32_t*>(q_weight);
+  a.q_scale = static_cast<const uint16_t*>(q_scale);
+  a.bias = nullptr;
+  a.y = out;
+  a.expert_ids = static_cast<const int32_t*>(expert_ids);
+  a.M = 1; a.N = N; a.K = K; a.slots = top_k; a.x_slot_stride = K;
+  a.num_experts = num_experts;
+  a.bits = bits; a.group_size = group_size; a.out_f32 = 0; a.paired = 0;
+  a.bf16 = model_dtype == MI355GQ_BF16;
+  a.sum_weights = expert_weights;
+  const hipError_t e = gq::launch_gemv(a, as_stream(stream));
+  if (e == hipErrorNotSupported)
+    return fail(MI355GQ_ERR_UNSUPPORTED, "moe_gemv_combine: no fused kernel for N=%lld K=%lld", (long long)N, (long long)K);
+  return hip_result(e, "moe_gemv_combine launch");
+}
+
 // Expert-sorted rows, about one per expert: the register GEMV with one grid row per activation row streams an
 // expert's weights once per row, the quad-row kernel once per expert but at well under half the GEMV's rate, so up
 // to num_experts rows (about 1.5 rows per distinct expert under uniform routing) the GEMV is ahead or level.

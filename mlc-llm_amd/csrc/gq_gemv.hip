@@ -269,6 +269,13 @@ hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
     p.residual = static_cast<const uint16_t*>(a.route_w);
     p.expert_ids = a.route_ids;
   }
+  if (a.sum_weights != nullptr) {
+    if (p.routed || a.bias != nullptr || a.residual != nullptr || a.expert_ids == nullptr || a.slots != 2 || a.M != 1 ||
+        a.paired || a.out_f32 || a.indptr != nullptr)
+      return hipErrorNotSupported;
+    p.sum2 = 1;
+    p.residual = static_cast<const uint16_t*>(a.sum_weights);
+  }
   if (a.N == 0 || a.slots == 0) return hipSuccess;
   const int nb = static_cast<int>(a.M);
   const int slots = static_cast<int>(a.slots);
@@ -277,7 +284,7 @@ hipError_t launch_gemv(const GemvArgs& a, hipStream_t s) {
     const hipError_t e = launch_gemv_reg(p, a.bits, nb, slots, s);
     if (e != hipErrorNotSupported) return e;
   }
-  if (p.paired || p.bf16 || p.indptr != nullptr || p.routed) return hipErrorNotSupported;  // only the register kernel has these forms
+  if (p.paired || p.bf16 || p.indptr != nullptr || p.routed || p.sum2) return hipErrorNotSupported;  // only the register kernel has these forms
   return launch_gemv_lds(p, a.bits, nb, slots, s);
 }
 

@@ -41,6 +41,7 @@ struct GemvParams {
   int paired;  // fused gate/up form: y[.., N / 2] = silu(x . W[j]) * (x . W[N / 2 + j]), fp16
   int bf16;    // x, q_scale, bias, residual and a 16-bit y are bfloat16 (register kernel only)
   int routed = 0;
+  int sum2 = 0;  // the two slots' results are weighted and summed in the launch (`residual` points at the two weights)
   int gc;  // groups staged per LDS chunk (multiple of 64; LDS kernel)
   // ---- bias / residual forms and expert forms
   const uint16_t* bias;

@@ -22,6 +22,12 @@ namespace gq {
 // MODE 2: fused gate/up form; a set holds R / 2 (gate, up) row pairs and stores R / 2 products.
 // MODE 3: MODE 2 for one token that routes itself (the expert of a slot comes from the router logits, see below); its
 // own instantiation so that no other form carries the selection code.
+// MODE 4 (with KW = 2): one token's second expert matmul and the weighted sum over its two experts in one launch.  The
+// four waves of a workgroup are (expert slot 0 | 1) x (half of K 0 | 1) and walk the same rows; each slot has its own row
+// of x (both staged in LDS) and its own expert; after the walk the first wave forms
+// out[n] = rnd(rnd(y0[n]) * w0) + rnd(rnd(y1[n]) * w1), rounded once more: what the matmul's store, the multiplication by the
+// routing weights and the sum over the slots do in the model dtype.  `expert_ids` holds the two ids, `residual` points at
+// the two routing weights.
 // BF: bfloat16 model (x, scales, bias, residual and a 16-bit result are bfloat16); the same walk with
 // group_dot_bf16.  Like the float16 form it multiplies x with the integer fields and applies the scale
 // to the group sum in fp32, so the dequantised weight is never rounded to the model dtype on its own.
@@ -64,18 +70,21 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
   constexpr int G = T::G;
   constexpr int HP = G / 2;  // half pairs of x per group
   // 16-byte x chunks each of the 256 threads stages: NB * ITERS * 64 groups * G/8 chunks / 256
-  constexpr int XS = (NB * ITERS * KW * 64 * (G / 8) + 255) / 256;
+  constexpr int XS = ((MODE == 4 ? 2 : NB) * ITERS * KW * 64 * (G / 8) + 255) / 256;
 
   extern __shared__ uint4 smem[];  // x as [NB][ng * G] halves, zero beyond K
   const int kpad = p.ng * G;
 
   const int lane = threadIdx.x & 63;
-  static_assert(KW == 1 || (KW == 2 && R == 1 && NB == 1 && MODE == 0), "shared K: one row per set, plain epilogue");
+  constexpr bool SUM2 = MODE == 4;
+  static_assert(KW == 1 || (KW == 2 && R == 1 && NB == 1 && (MODE == 0 || SUM2)), "shared K: one row per set, plain epilogue");
+  static_assert(!SUM2 || (KW == 2 && MOE), "the sum over two experts is a form of the shared-K expert GEMV");
   const int wave_all = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int ksub = KW == 2 ? (wave_all & 1) : 0;           // which half of K
-  const int gw = KW == 2 ? (wave_all >> 1) : wave_all;     // walker of row sets
-  const int nwaves = KW == 2 ? (p.nwaves >> 1) : p.nwaves;
-  const int slot = MOE ? blockIdx.y : 0;
+  const int ksub = KW == 2 ? (wave_all & 1) : 0;                                     // which half of K
+  const int gw = SUM2 ? static_cast<int>(blockIdx.x) : (KW == 2 ? (wave_all >> 1) : wave_all);  // walker of row sets
+  const int nwaves = SUM2 ? (p.nwaves >> 2) : (KW == 2 ? (p.nwaves >> 1) : p.nwaves);
+  const int slot = SUM2 ? static_cast<int>((threadIdx.x >> 7) & 1) : (MOE ? static_cast<int>(blockIdx.y) : 0);
+  constexpr int NBX = SUM2 ? 2 : NB;  // rows of x a workgroup stages
 
   const uint16_t* x = MOE ? p.x + slot * p.x_slot_stride : p.x;
   const uint32_t* qw = p.qw;
@@ -130,7 +139,10 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
 
   // ---- x chunks go out first: waiting for them later must not wait for the weight loads,
   //      and the load counter retires in issue order
-  const int chunks = NB * (kpad / 8);
+  const int chunks = NBX * (kpad / 8);
+  // (the sum over two experts stages both slots' rows: row b of the staging is slot b's)
+  const uint16_t* xs_base = SUM2 ? p.x : x;
+  const int64_t xs_stride = SUM2 ? p.x_slot_stride : p.K;
   const bool vec = (p.K & 7) == 0;
   uint4 xv[XS];
   bool xok[XS];
@@ -141,7 +153,7 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
     const int k = (c - b * (kpad / 8)) * 8;
     xok[i] = vec && c < chunks && k + 8 <= p.K;
     // always a valid 16-byte load (x itself when the chunk is out of range); zeroed at store time
-    const uint16_t* src = xok[i] ? x + static_cast<int64_t>(b) * p.K + k : x;
+    const uint16_t* src = xok[i] ? xs_base + static_cast<int64_t>(b) * xs_stride + k : xs_base;
     xv[i] = *reinterpret_cast<const uint4*>(src);
   }
 
@@ -200,9 +212,9 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
     }
   } else {  // K not a multiple of 8: rows of x are not 16-byte aligned, copy element-wise
     uint16_t* xs16 = reinterpret_cast<uint16_t*>(smem);
-    for (int i = threadIdx.x; i < NB * kpad; i += 256) {
+    for (int i = threadIdx.x; i < NBX * kpad; i += 256) {
       const int b = i / kpad, k = i - b * kpad;
-      xs16[i] = k < p.K ? x[static_cast<int64_t>(b) * p.K + k] : uint16_t(0);
+      xs16[i] = k < p.K ? xs_base[static_cast<int64_t>(b) * xs_stride + k] : uint16_t(0);
     }
   }
   __syncthreads();
@@ -217,7 +229,7 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
       uint32_t nat[HP];
 #pragma unroll
       for (int c = 0; c < G / 8; ++c) {
-        uint4 raw = smem[(b * kpad + gidx[it] * G) / 8 + c];
+        uint4 raw = smem[((SUM2 ? slot : b) * kpad + gidx[it] * G) / 8 + c];
         if (!gok[it]) raw = make_uint4(0, 0, 0, 0);
         nat[4 * c + 0] = raw.x; nat[4 * c + 1] = raw.y; nat[4 * c + 2] = raw.z; nat[4 * c + 3] = raw.w;
       }
@@ -227,7 +239,7 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
 
   // (shared K) the halves' row sums: [4 waves][kPartSlots] floats behind x
   constexpr int kPartSlots = 64;
-  float* const part = reinterpret_cast<float*>(smem) + NB * kpad / 2;
+  float* const part = reinterpret_cast<float*>(smem) + NBX * kpad / 2;
   int part_n = 0;
   // ---- persistent walk: reduce one set, then refill its registers with the set two strides on
   auto reduce = [&](int cur, const uint4 (&wc)[R][ITERS], const uint32_t (&sc)[R][ITERS],
@@ -310,7 +322,16 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
     // count within kPartSlots)
     __syncthreads();
     const int set = gw + lane * nwaves;
-    if (ksub == 0 && lane < kPartSlots && set < nsets) {
+    if constexpr (SUM2) {
+      if (threadIdx.x < kPartSlots && set < nsets) {
+        auto rnd = [](float v) { return BF ? bf2f(f2bf(v)) : h2f(f2h(v)); };
+        const float y0 = rnd(part[lane] + part[kPartSlots + lane]);
+        const float y1 = rnd(part[2 * kPartSlots + lane] + part[3 * kPartSlots + lane]);
+        const float w0 = to_f32(p.residual[0]), w1 = to_f32(p.residual[1]);
+        const float v = rnd(y0 * w0) + rnd(y1 * w1);
+        static_cast<uint16_t*>(p.y)[set] = BF ? f2bf(v) : f2h(v);
+      }
+    } else if (ksub == 0 && lane < kPartSlots && set < nsets) {
       const int w = threadIdx.x >> 6;
       const float v = part[w * kPartSlots + lane] + part[(w + 1) * kPartSlots + lane];
       const int64_t oi = static_cast<int64_t>(slot) * p.N + set;
@@ -365,8 +386,8 @@ static hipError_t launch_k(const GemvParams& p0, int slots, int blocks, int nset
 // Long K shared between two neighbouring waves (KW = 2): HALF groups per lane and wave.
 template <int BITS, int HALF>
 static hipError_t launch_shared_k(const GemvParams& p0, int slots, int blocks, int nsets, hipStream_t s) {
-  const size_t lds = static_cast<size_t>(p0.ng) * GemvTraits<BITS>::G * 2 + 4 * 64 * sizeof(float);
-  const dim3 grid(blocks, slots);
+  const size_t lds = static_cast<size_t>(p0.sum2 ? 2 : 1) * p0.ng * GemvTraits<BITS>::G * 2 + 4 * 64 * sizeof(float);
+  const dim3 grid(blocks, p0.sum2 ? 1 : slots);
   GemvParams p = p0;
   p.nsets = nsets;
   p.nwaves = blocks * 4;
@@ -377,6 +398,16 @@ static hipError_t launch_shared_k(const GemvParams& p0, int slots, int blocks, i
 #define GQ_SHARED_K(BF_, MOE_)                                                                                      \
   hipLaunchKernelGGL((gemv_reg_kernel<BITS, 1, 1, HALF, 0, BF_, MOE_, 2>), grid, dim3(256), lds, s, p.x, p.qw, p.qs, \
                      p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, t)
+  if (p.sum2) {  // both expert slots in every workgroup, their results weighted and summed at the end
+    note_kernel("gq::gemv_reg_kernel<%d,1,1,%d,4,%s,true,2>", BITS, HALF, p.bf16 ? "true" : "false");
+    if (p.bf16)
+      hipLaunchKernelGGL((gemv_reg_kernel<BITS, 1, 1, HALF, 4, true, true, 2>), grid, dim3(256), lds, s, p.x, p.qw, p.qs,
+                         p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, t);
+    else
+      hipLaunchKernelGGL((gemv_reg_kernel<BITS, 1, 1, HALF, 4, false, true, 2>), grid, dim3(256), lds, s, p.x, p.qw, p.qs,
+                         p.y, p.N, p.K, p.ng, p.nsets, p.nwaves, p.out_f32, t);
+    return hipGetLastError();
+  }
   if (p.bf16) {
     if (moe) GQ_SHARED_K(true, true);
     else GQ_SHARED_K(true, false);
@@ -451,6 +482,24 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
   // Long K (5 to 12 groups per lane), one row, plain epilogue: two neighbouring waves share every row's K (3 to 6 groups
   // per lane each, so that two waves fit a SIMD where the whole-K form runs one), twice the waves.
   // Tuning override: gemv_ksplit 0 | 1.
+  if (p.sum2) {
+    // one token's e2 and the weighted sum over its two experts: four waves per row walker (2 slots x 2 halves of K),
+    // 512 walkers; 2 to 6 groups per lane and wave, both rows of x in LDS
+    const int half = (iters + 1) / 2;
+    const int walkers = 512;
+    const int rounds2 = (p.N + walkers - 1) / walkers;
+    const int64_t lds2 = 2ll * p.ng * GemvTraits<BITS>::G * 2 + 1024;
+    if (nb != 1 || slots != 2 || iters < 3 || rounds2 > 64 || lds2 > 65536) return hipErrorNotSupported;
+    const int blocks2 = (p.N + rounds2 - 1) / rounds2;
+    switch (half) {
+      case 2: return launch_shared_k<BITS, 2>(p, slots, blocks2, p.N, s);
+      case 3: return launch_shared_k<BITS, 3>(p, slots, blocks2, p.N, s);
+      case 4: return launch_shared_k<BITS, 4>(p, slots, blocks2, p.N, s);
+      case 5: return launch_shared_k<BITS, 5>(p, slots, blocks2, p.N, s);
+      case 6: return launch_shared_k<BITS, 6>(p, slots, blocks2, p.N, s);
+      default: return hipErrorNotSupported;
+    }
+  }
   const bool plain = !p.paired && !p.routed && p.bias == nullptr && p.residual == nullptr;
   if (iters >= 5 && nb == 1 && R == 1 && plain && rounds <= 64 && options().gemv_ksplit != 0) {
     const int half = (iters + 1) / 2;

@@ -59,6 +59,9 @@ struct GemvArgs {
   const void* gate = nullptr;
   void* route_w = nullptr;
   int32_t* route_ids = nullptr;
+  // one token's two expert slots summed with their routing weights in the same launch (slots = 2, expert_ids set, y is
+  // [1, N] in the model dtype): the two weights, model dtype
+  const void* sum_weights = nullptr;
 };
 hipError_t launch_gemv(const GemvArgs& a, hipStream_t s);
 

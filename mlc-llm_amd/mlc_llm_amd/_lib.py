@@ -49,6 +49,7 @@ SIGNATURES = {
     "mi355gq_linear_silu_mul": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P, _P, _L, _P]),
     "mi355gq_moe_gemv_silu_mul": (_I, [_P, _L, _P, _P, _P, _L, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_moe_gemv_routed_silu_mul": (_I, [_P, _P, _L, _L, _P, _P, _L, _L, _I, _I, _I, _P, _P, _P, _P]),
+    "mi355gq_moe_gemv_combine": (_I, [_P, _P, _P, _L, _L, _I, _I, _I, _L, _P, _P, _L, _P, _P]),
     "mi355gq_moe_group_gemm_silu_mul": (_I, [_P, _L, _P, _P, _P, _I, _L, _L, _L, _I, _I, _P, _P]),
     "mi355gq_linear_silu_mul_dt_workspace_bytes": (_L, [_L, _L, _L, _I, _I, _I]),
     "mi355gq_linear_silu_mul_dt": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),

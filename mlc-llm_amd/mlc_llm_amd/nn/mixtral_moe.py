@@ -68,8 +68,16 @@ class MixtralMoE(nn.Module):
                 if err.code != _lib.ERR_UNSUPPORTED:
                     raise
             else:
-                x = self.e2(h, expert_indices)
-                x = ops.moe_combine(x.reshape(1, experts_per_tok, hidden_size), expert_weights)
+                try:
+                    # e2 and the weighted sum over the experts in one launch as well
+                    cfg2 = self.e2.config
+                    x = ops.moe_gemv_combine(h, self.e2.q_weight, self.e2.q_scale, expert_indices, expert_weights,
+                                             cfg2.bits, self.e2.group_size)
+                except _lib.Mi355gqError as err:
+                    if err.code != _lib.ERR_UNSUPPORTED:
+                        raise
+                    x = self.e2(h, expert_indices)
+                    x = ops.moe_combine(x.reshape(1, experts_per_tok, hidden_size), expert_weights)
                 return x.reshape(batch_size, seq_len, hidden_size)
         expert_weights, expert_indices = moe_misc.gating_softmax_topk(gate, experts_per_tok)
         if num_tokens == 1:

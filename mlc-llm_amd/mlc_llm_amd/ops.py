@@ -258,6 +258,32 @@ def moe_gemv_routed_silu_mul(x: torch.Tensor, gate_logits: torch.Tensor, top_k: 
     return out, weights, ids
 
 
+def moe_gemv_combine(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, expert_ids: torch.Tensor,
+                     expert_weights: torch.Tensor, bits: int, group_size: int) -> torch.Tensor:
+    """One token: the e2 expert matmul on its top_k rows and the weighted sum over them, in one launch.
+    x [top_k, K], expert_ids int32 [1, top_k], expert_weights [1, top_k] (model dtype), q_weight [E, N, nw],
+    q_scale [E, N, ng].  Returns out [1, N]; raises Mi355gqError with ERR_UNSUPPORTED where the fused kernel does not
+    apply (float32 models, top_k other than 2, short or very long K)."""
+    _chk(x, _FLOATS, "x")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, x.dtype, "q_scale")
+    _chk(expert_ids, torch.int32, "expert_ids")
+    _chk(expert_weights, x.dtype, "expert_weights")
+    if x.dim() != 2 or expert_ids.dim() != 2 or expert_ids.shape[0] != 1 or tuple(expert_weights.shape) != tuple(expert_ids.shape):
+        raise ValueError("moe_gemv_combine: x must be [top_k, K], expert_ids and expert_weights [1, top_k]")
+    top_k = expert_ids.shape[1]
+    if x.shape[0] != top_k:
+        raise ValueError(f"moe_gemv_combine: {x.shape[0]} rows of x for {top_k} experts")
+    ne, n, _ = q_weight.shape
+    k = x.shape[1]
+    _check_qshapes(q_weight, q_scale, (ne, n), k, bits, group_size)
+    out = torch.empty((1, n), dtype=x.dtype, device=x.device)
+    _lib.call("mi355gq_moe_gemv_combine", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(), n, k, bits, group_size,
+              _MODEL_DTYPES[x.dtype], ne, expert_ids.data_ptr(), expert_weights.data_ptr(), top_k, out.data_ptr(),
+              _stream())
+    return out
+
+
 def moe_gemv(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor,
              expert_ids: torch.Tensor, bits: int, group_size: int, silu_mul_halves: bool = False
              ) -> torch.Tensor:

@@ -872,6 +872,57 @@ def test_moe_gemv_routed_silu_mul(name, dtype, ne, top_k):
         assert np.abs(got - ref).max() <= 2e-2 * max(1.0, np.abs(ref).max()), np.abs(got - ref).max()
 
 
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k", [(520, 14336), (4100, 14336), (100, 8200), (64, 5200), (36, 15360), (1000, 11008)])
+def test_moe_gemv_combine(name, dtype, n, k):
+    """One token's e2 expert matmul and the weighted sum over its two experts in one launch, against the operator pair it
+    replaces (bit for bit wherever the pair's matmul splits K the same way, i.e. from 5 groups per lane on; a last place
+    of the model dtype otherwise, where the pair adds a row's K in one run) and against the oracle's values."""
+    s = SCHEMES[name]
+    rng = np.random.default_rng(n + k)
+    ne = 4
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    x = dev(rng.standard_normal((2, k)).astype(np.float16)).to(dtype)
+    ids = dev(np.array([[3, 1]], np.int32))
+    weights = dev(np.array([[0.625, 0.375]], np.float16)).to(dtype)
+    qs_d = dev(qs).to(dtype)
+    out = ops.moe_gemv_combine(x, dev(qw), qs_d, ids, weights, s.bits, s.group_size)
+    assert gq._lib.last_kernel().startswith("gq::gemv_reg_kernel") and ",4," in gq._lib.last_kernel(), gq._lib.last_kernel()
+    y = ops.moe_gemv(x, dev(qw), qs_d, ids, s.bits, s.group_size)
+    pair = ops.moe_combine(y.reshape(1, 2, n), weights)
+    assert out.shape == pair.shape == (1, n)
+    groups_per_lane = -(-(-(-k // s.group_size)) // 64)
+    if groups_per_lane >= 5:
+        assert torch.equal(out, pair)
+    else:
+        err = (out.float() - pair.float()).abs().max().item()
+        assert err <= (2 ** -7 if dtype == torch.bfloat16 else 2 ** -10) * max(1.0, pair.float().abs().max().item()), err
+    if dtype == torch.float16:
+        full = o.moe_dequantize_gemv_fp32(x.cpu().numpy(), qw, qs, ids.cpu().numpy(), s)  # [2, n] float64
+        ref = 0.625 * full[0] + 0.375 * full[1]
+        got = out.float().cpu().numpy()[0]
+        assert np.abs(got - ref).max() <= 1e-2 * max(1.0, np.abs(ref).max()), np.abs(got - ref).max()
+
+
+def test_moe_gemv_combine_declines():
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(6)
+    ne, n = 4, 64
+    for k, top_k, f32 in [(14336, 3, False), (14336, 2, True), (1024, 2, False)]:  # three slots; float32; a short K
+        qw, qs = o.quantize((rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16), s)
+        x = dev(rng.standard_normal((top_k, k)).astype(np.float16))
+        ids = dev(np.arange(top_k, dtype=np.int32).reshape(1, top_k))
+        wts = dev(np.full((1, top_k), 0.25, np.float16))
+        qs_d = dev(qs)
+        if f32:
+            x, wts, qs_d = x.float(), wts.float(), qs_d.float()
+        with pytest.raises(gq._lib.Mi355gqError) as err:
+            ops.moe_gemv_combine(x, dev(qw), qs_d, ids, wts, 4, 32)
+        assert err.value.code == gq._lib.ERR_UNSUPPORTED
+
+
 def test_moe_gemv_routed_silu_mul_declines():
     s = SCHEMES["q4f16_1"]
     rng = np.random.default_rng(5)
