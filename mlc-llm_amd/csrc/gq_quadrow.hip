@@ -109,7 +109,7 @@ __device__ __forceinline__ float4_t mfma4_bf16(uint32_t a0, uint32_t a1, uint32_
 template <int BITS, int NBQ, int U, int MODE, bool BF = false, int QP = 1, bool KS = false>
 // (sixteen-wave workgroups exist for the forms that fit 128 registers: 2 KiB items without the bias / residual loads;
 //  with them the same bound forced spill reloads into the walk, and a reload waits for every weight load in flight)
-__global__ __launch_bounds__((U * QP <= 2 && MODE != 1 && !KS) ? 1024 : 512) void quad_kernel(const uint16_t* x_, const uint32_t* qw_, const uint16_t* qs_, void* y_, int rows_, int N_, int K_,
+__global__ __launch_bounds__((NBQ == 2 && U * QP <= 2 && MODE != 1 && !KS) ? 1024 : 512) void quad_kernel(const uint16_t* x_, const uint32_t* qw_, const uint16_t* qs_, void* y_, int rows_, int N_, int K_,
                  uint32_t w0, uint32_t w1, uint32_t w2, const QuadTail t) {
   QuadParams p;
   p.x = x_; p.qw = qw_; p.qs = qs_; p.y = y_;
@@ -357,6 +357,23 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1 && !KS) ? 1024 : 512) voi
     int done = 0;  // quads this wave has completed in this phase
     auto compute = [&](int qset, int step, const uint4 (&wc)[QP][U], const uint32_t (&sc)[QP][U],
                        const uint2 (&bias_bits)[QP], const uint2 (&res_bits)[QP][NBQ]) {
+      // One batch quad: every LDS read of the item goes out before the first matrix instruction.  Left to the compiler
+      // each read is issued one ahead of its use, so a wave waits out most of an LDS round trip ten times per item, and
+      // on the launches this form serves a SIMD often hosts a single wave.  (q3 with two quads per item keeps its reads
+      // where they are used: hoisted, that one instantiation returned wrong sums for the first quad of every pair on the
+      // GPU while its assembly read correct; the cause was not found, so it stays as it was.)
+      constexpr bool HOIST = NBQ == 1 && U <= 4 && !(BITS == 3 && QP == 2);
+      uint4 xh[HOIST ? U : 1][CH];
+      float ch[HOIST ? U : 1];
+      if constexpr (HOIST) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int bi = itw + step * U + u;
+          ch[u] = corr_lds[bi * 64 + lane];
+#pragma unroll
+          for (int d = 0; d < CH; ++d) xh[u][d] = smem[(bi * CH + d) * 64 + lane];
+        }
+      }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int it = itw + step * U + u;
@@ -410,10 +427,17 @@ __global__ __launch_bounds__((U * QP <= 2 && MODE != 1 && !KS) ? 1024 : 512) voi
           const int bi = bq * niter + it;
           // one accumulator per group: it starts from minus the offset term and takes every operand class (the
           // activations of the scaled classes were divided when they were staged)
-          const float c = corr_lds[bi * 64 + lane];
+          float c;
           uint4 xv[CH];
+          if constexpr (HOIST) {
+            c = ch[u];
 #pragma unroll
-          for (int d = 0; d < CH; ++d) xv[d] = smem[(bi * CH + d) * 64 + lane];
+            for (int d = 0; d < CH; ++d) xv[d] = xh[u][d];
+          } else {
+            c = corr_lds[bi * 64 + lane];
+#pragma unroll
+            for (int d = 0; d < CH; ++d) xv[d] = smem[(bi * CH + d) * 64 + lane];
+          }
 #pragma unroll
           for (int qp = 0; qp < QP; ++qp) {
             float4_t t = {c, c, c, c};
@@ -534,7 +558,7 @@ static hipError_t launch_quad_extra(const QuadParams& p, dim3 grid, int threads,
   }
   note_kernel("gq::quad_kernel<%d,%d,%d,%d,%s,%d%s>", BITS, NBQ, U, MODE, BF ? "true" : "false", QP, ks ? ",true" : "");
   const int nwaves = static_cast<int>(grid.x) * (threads >> 6);
-  if (threads % 64 != 0 || threads > (ks ? 512 : 1024) || p.nsteps > 0xffff || p.steps_total > 0xffff || p.rounds > 0xffff ||
+  if (threads % 64 != 0 || threads > ((ks || NBQ != 2 || U * QP > 2 || MODE == 1) ? 512 : 1024) || p.nsteps > 0xffff || p.steps_total > 0xffff || p.rounds > 0xffff ||
       nwaves > 0xffff || p.nphases > 0xffff || p.nquads != p.N / 4 || p.nsets != (p.nquads + QP - 1) / QP ||
       p.kw_log2 < 0 || p.kw_log2 > 2 ||
       (p.kw_log2 != 0 && (p.nphases != 1 || p.rounds != 1 || MODE == 1 || (threads >> 6) % (1 << p.kw_log2) != 0 ||
@@ -695,7 +719,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
     if (2 * wgs <= 256) threads = 256;  // (the doubled count must still be one round of workgroups)
   }
   // four waves per SIMD share one copy of x (the instances that fit 128 registers: 2 KiB items without bias / residual loads)
-  if (big_wg && p.nphases == 1 && U * QP <= 2 && a.bias == nullptr && a.residual == nullptr) threads = 1024;
+  if (big_wg && nbq == 2 && p.nphases == 1 && U * QP <= 2 && a.bias == nullptr && a.residual == nullptr) threads = 1024;
   const int wpb = threads / 64;
   const size_t lds = lds_x + ((p.nphases > 1 || p.kw_log2 != 0) ? static_cast<size_t>(wpb) * p.rounds * QP * nbq * 64 : 0);
   const int blocks = (sets_w + wpb - 1) / wpb;
