@@ -448,12 +448,14 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
   if (nb == 2) rmax = iters <= 2 ? 2 : (iters <= 4 ? 1 : 0);
   if (nb > 2 || rmax == 0) return hipErrorNotSupported;
   // Measured on MI355X (q4, batch 1): short K wants one row per set until the matrix is large
-  // (fine-grained sets hide the pipeline fill of a 5 us kernel), large matrices want 4 rows per
-  // set; long K is register-bound and runs one wave per SIMD.
+  // (fine-grained sets hide the pipeline fill of a 5 us kernel), large matrices want 2 rows per
+  // set; long K is register-bound (one wave per SIMD, or two that share every row's K).
   const int64_t rows_total = static_cast<int64_t>(p.N) * slots;
   int R = options().gemv_rows_per_wave;
   if (R != 1 && R != 2 && R != 4) {
-    if (iters <= 2) R = rows_total >= 65536 ? 4 : (rows_total >= 16384 ? 2 : 1);
+    // (four rows per set, once the choice for 65536 rows and more, measures 2 % behind two on 128256 x 4096 since the
+    //  kernel's arguments arrive in registers: 47.1 -> 46.1 us)
+    if (iters <= 2) R = rows_total >= 16384 ? 2 : 1;
     else R = 1;  // K of 5120 / 8192 (13B, 70B projections): 8-17 % faster than two rows per set
   }
   if (R > rmax) R = rmax;
