@@ -362,7 +362,7 @@ static hipError_t launch_k(const GemvParams& p0, int slots, int blocks, int nset
   const int mode = p.paired ? (p.routed ? 3 : 2) : ((p.bias != nullptr || p.residual != nullptr) ? 1 : 0);
   // the plain linear (one grid row, no expert ids, no expert-sorted rows) has an instantiation of its own
   const bool moe = slots != 1 || p.routed || p.indptr != nullptr || p.expert_ids != nullptr;
-  note_kernel("gq::gemv_reg_kernel<%d,%d,%d,%d,%d,%s,%s>", BITS, NB, R, ITERS, mode, p.bf16 ? "true" : "false",
+  note_kernel("gq::gemv_reg_kernel<%d,%d,%d,%d,%d,%s,%s,1>", BITS, NB, R, ITERS, mode, p.bf16 ? "true" : "false",
               moe ? "true" : "false");
   if (mode >= 2) {
     if constexpr (R % 2 == 0) {
