@@ -17,7 +17,9 @@
  * PARITY UNPINNED (depends on TVM's lowering, which the checkout does not hold):
  * the tie rule of round() in _quantize (round_mode 0 = half away from zero, the
  * llvm/rocm lowering; 1 = half to even) and the code emitted for an all-zero
- * group (0/0 -> NaN -> compare+select max -> 0).
+ * group (0/0 -> NaN -> compare+select max -> 0).  The rounding points themselves
+ * (fp16 divide, fp16 add, then round) are pinned: tests/ compares the codes with
+ * exact integer arithmetic on a million values.
  *
  * fp16 values travel as uint16_t bit patterns.  Each fp16 operation is done in
  * float and rounded to nearest-even half straight away; for + - * / that equals

@@ -33,8 +33,14 @@ cumsum or indptr in it (tests/test_oracle.py).  What stays PARITY UNPINNED
 there is the summation order of TVM's fp32 softmax over all experts
 (norm_topk_prob=False) and any rounding TVM's legalisation puts inside silu.
 
-Everything else (field order, offset, scale indexing, padded K) is pinned in
-tests/ against the reference's own numpy test twins and hand-derived vectors.
+Everything else is pinned in tests/: field order, offset, scale indexing and
+padded K against the reference's own numpy test twins and hand-derived
+vectors; the rounding points of _quantize (a float16 divide, then a float16
+add, then round: two roundings, group_quantization.py:278-282) against exact
+rational arithmetic with an explicit round-to-nearest-even, element for element
+on a million values of the first baseline configuration, with hand-derived
+vectors on which one rounding and two give different codes (the same for the
+bfloat16 and float32 forms of quantize_dt).
 """
 
 from __future__ import annotations

@@ -20,6 +20,8 @@ import pytest
 from oracle import c_oracle
 from oracle import gq_oracle as o
 
+import exact_fp
+
 Q4, Q3 = o.SCHEMES["q4f16_1"], o.SCHEMES["q3f16_1"]
 REF_SHAPES = [("q3f16_1", (2, 13)), ("q3f16_1", (16, 120)), ("q4f16_1", (2, 13)), ("q4f16_1", (16, 128))]
 
@@ -201,6 +203,180 @@ def test_quantize_within_reference_test_tolerance(name, shape):
     want = (q_ref - s.max_int) * np.repeat(scale_ref, s.group_size, axis=1)[:, : shape[1]]
     np.testing.assert_allclose(got, want, rtol=1e-2 if s.bits == 3 else 1e-3,
                                atol=0.4 if s.bits == 3 else 0.2)
+
+
+# --------------------------------------------------------------------------- the two roundings of _quantize
+#
+# group_quantization.py:274-287 rounds twice in the model dtype before `round`: the quotient w / scale, then
+# its sum with max_int.  The checks below pin both rounding points with arithmetic that shares nothing with
+# numpy's float16 operators or with the oracle (tests/exact_fp.py: exact rationals, and long division in
+# int64), so that a quantizer which divides and adds in float32 and rounds once does not pass.
+
+
+def _config1_weights(rows, k):
+    """Rows of the baseline's first configuration: seed 0, N(0, 0.02), float16 [4096, 4096]."""
+    w = (np.random.default_rng(0).standard_normal((4096, 4096)) * 0.02).astype(np.float16)
+    return w[:rows, :k]
+
+
+def _single_rounding_float32(w, s, mode="half_away"):
+    """The plausible mistake: float32 divide and add, no rounding to the model dtype in between."""
+    _, scale = o.quantize_values(w, s, mode)
+    sf = np.repeat(scale.astype(np.float32), s.group_size, axis=-1)[..., : w.shape[-1]]
+    t = w.astype(np.float32) / sf + np.float32(s.max_int)
+    return np.clip(o._round(t, mode), 0, 2 * s.max_int).astype(np.uint32)
+
+
+@pytest.mark.parametrize("s", [Q4, Q3])
+@pytest.mark.parametrize("mode", ["half_away", "half_even"])
+def test_quantize_equals_exact_rational_arithmetic(s, mode):
+    # every code of 8 rows (32 768 values) against fractions.Fraction with an explicit round-to-nearest-even
+    # to binary16 after the divide and again after the add; scales as well
+    k = 4096 if s.bits == 4 else 4080
+    w = _config1_weights(8, k)
+    q, scale = o.quantize_values(w, s, mode)
+    for r in range(w.shape[0]):
+        for g in range(k // s.group_size):
+            sl = slice(g * s.group_size, (g + 1) * s.group_size)
+            codes, sc = exact_fp.quantize_group_fraction(exact_fp.to_fraction(w[r, sl]), s.max_int, "float16", mode)
+            assert codes == q[r, sl].tolist(), (r, g)
+            assert float(sc) == float(scale[r, g])
+
+
+@pytest.mark.parametrize("s", [Q4, Q3])
+def test_quantize_equals_exact_integer_arithmetic_on_a_million_values(s):
+    # the same two roundings by long division in int64, on 256 rows of the configuration-1 matrix (1 048 576
+    # values for q4; 1 044 480 for q3 with K = 102 whole groups of 40), both tie modes
+    k = 4096 if s.bits == 4 else 4080
+    w = _config1_weights(256, k)
+    for mode in ("half_away", "half_even"):
+        q, _ = o.quantize_values(w, s, mode)
+        exact = exact_fp.quantize_codes_int(w.view(np.uint16), s.group_size, s.max_int, "float16", mode)
+        assert np.array_equal(q, exact), int((q != exact).sum())
+        cw, _ = c_oracle.quantize(w, s.bits, s.group_size, 0 if mode == "half_away" else 1)  # the C twin, directly
+        assert np.array_equal(o.unpack(cw, s, k), exact)
+    # the check cannot go vacuous: on this data the one-rounding variants differ from the reference's order,
+    # the float32 one on more than 0.1 % of the values (0.30 % q4, 0.11 % q3), and the integer checker tells
+    # one rounding from two as well
+    q, _ = o.quantize_values(w, s)
+    wrong = _single_rounding_float32(w, s)
+    assert (wrong != q).mean() > 1e-3
+    once = exact_fp.quantize_codes_int(w.view(np.uint16), s.group_size, s.max_int, "float16", roundings=1)
+    assert (once != q).mean() > 2e-4
+    # and the integer form of "one rounding" is the rational one (so the integer checker is itself pinned)
+    for g in range(0, 8 * s.group_size, s.group_size):
+        c1, _ = exact_fp.quantize_group_fraction(exact_fp.to_fraction(w[0, g: g + s.group_size]), s.max_int, "float16",
+                                                 roundings=1)
+        assert c1 == once[0, g: g + s.group_size].tolist()
+
+
+def test_exact_rounding_helper_known_values():
+    # the checker's own rounding against values that can be read off the binary16 grid by hand
+    F = exact_fp.Fraction
+    rne = lambda x: exact_fp.rne(F(x), "float16")
+    assert rne(F(1) + F(1, 2048)) == 1  # tie between 1 and 1 + 2^-10: even significand
+    assert rne(F(1) + F(3, 2048)) == F(1) + F(2, 1024)  # tie between 1+2^-10 (odd) and 1+2^-9 (even)
+    assert rne(F(1, 3)) == F(1365, 4096)  # 0.333..: grid 2^-12 in [0.25, 0.5): 1365.33 -> 1365
+    assert rne(F(2) ** -25) == 0 and rne(F(3, 2) * F(2) ** -25) == F(2) ** -24  # subnormal ties / rounding
+    assert rne(F(65519)) == 65504 and rne(F(65520)) == exact_fp.INF  # overflow threshold
+    assert rne(F(-7) * F(1025, 1024)) == F(-1794, 256)
+    # and against numpy's conversion on random doubles (float64 -> float16 is one correctly rounded step)
+    rng = np.random.default_rng(23)
+    xs = rng.standard_normal(3000) * 10.0 ** rng.integers(-8, 5, 3000)
+    with np.errstate(over="ignore"):
+        want = xs.astype(np.float16)
+    for x, h in zip(xs, want):
+        got = exact_fp.rne(F(float(x)), "float16")
+        assert (got == exact_fp.INF and np.isinf(h) and h > 0) or (got == -exact_fp.INF and np.isinf(h) and h < 0) \
+            or got == F(float(h))
+    b = lambda x: exact_fp.rne(F(x), "bfloat16")
+    assert b(F(1) + F(1, 256)) == 1 and b(F(1) + F(3, 256)) == F(1) + F(2, 128)  # bf16 ties (8-bit significand)
+
+
+def _codes(values, s, mode="half_away"):
+    w = np.zeros((1, s.group_size), np.float16)
+    w[0, : len(values)] = values
+    return o.unpack(o.quantize(w, s, mode)[0], s, s.group_size)[0, : len(values)].tolist()
+
+
+def test_quantize_hand_derived_double_rounding_vectors():
+    # (1) the ADD rounds.  q4, group maximum 7 -> scale = 7 / 7 = 1 exactly.  w = 0.5 - 2^-12 = 0.499755859375
+    # (binary16 0x37FF).  Quotient = w, exact.  w + 7 = 7.499755859375 lies in [4, 8), where binary16 steps by
+    # 2^-8: the neighbours are 7.49609375 (distance 0.00366) and 7.5 (distance 0.00024) -> 7.5, and round() of
+    # 7.5 is 8 (both tie rules: 8 is even).  Rounding once, 7.4997... goes to 7.
+    assert _codes([7.0, 0.499755859375], Q4) == [14, 8]
+    assert _codes([7.0, 0.499755859375], Q4, "half_even") == [14, 8]
+    assert _single_rounding_float32(np.array([[7.0, 0.499755859375] + [0] * 30], np.float16), Q4)[0, 1] == 7
+    # the mirror image: w = -(0.5 + 2^-11), quotient exact, 7 - 0.50048828125 = 6.49951171875 -> neighbours
+    # 6.49609375 / 6.5 -> 6.5 -> half away: 7, half even: 6; rounding once gives 6 under either rule
+    assert _codes([7.0, -0.50048828125], Q4) == [14, 7]
+    assert _codes([7.0, -0.50048828125], Q4, "half_even") == [14, 6]
+    # q3: maximum 3 -> scale 1; 3 + 0.499755859375 = 3.499755859375 in [2, 4), step 2^-9: neighbours 3.498046875
+    # (0.0017) and 3.5 (0.00024) -> 3.5 -> 4 (even too); rounding once: 3
+    assert _codes([3.0, 0.499755859375], Q3) == [6, 4]
+    assert _codes([3.0, 0.499755859375], Q3, "half_even") == [6, 4]
+    # (2) the DIVIDE rounds, with a scale that is not a power of two.  q4, maximum 7.0078125 = 1794 / 256:
+    # 7.0078125 / 7 = 1.0011160..., binary16 steps by 2^-10 in [1, 2): 1025.14 / 1024 -> scale = 1025 / 1024.
+    # w = -6.5078125 = -1666 / 256.  w / scale = -1666 * 4 / 1025 = -6664 / 1025 = -6.501463..., step 2^-8 in
+    # [4, 8): -1664.37 / 256 -> -1664 / 256 = -6.5 exactly.  -6.5 + 7 = 0.5 (exact) -> half away: 1, half even: 0.
+    # Rounding once: 7 - 6.501463... = 0.498536... -> 0 under either rule.
+    assert _codes([7.0078125, -6.5078125], Q4) == [14, 1]
+    assert _codes([7.0078125, -6.5078125], Q4, "half_even") == [14, 0]
+    assert _single_rounding_float32(np.array([[7.0078125, -6.5078125] + [0] * 30], np.float16), Q4)[0, 1] == 0
+    # q3, maximum 3.0078125 = 1540 / 512: / 3 = 1.0026041..., * 1024 = 1026.67 -> scale = 1027 / 1024.
+    # w = -2.5078125 = -1284 / 512.  w / scale = -1284 * 2 / 1027 = -2568 / 1027 = -2.500486..., step 2^-9 in
+    # [2, 4): -1280.25 / 512 -> -1280 / 512 = -2.5.  -2.5 + 3 = 0.5 -> half away: 1, half even: 0; once: 0.
+    assert _codes([3.0078125, -2.5078125], Q3) == [6, 1]
+    assert _codes([3.0078125, -2.5078125], Q3, "half_even") == [6, 0]
+    assert _single_rounding_float32(np.array([[3.0078125, -2.5078125] + [0] * 38], np.float16), Q3)[0, 1] == 0
+    # (3) a scale that was rounded DOWN makes the most negative weight overshoot: maximum 7.01953125 = 1797 / 256,
+    # / 7 = 1.00279..., * 1024 = 1026.86 -> scale = 1027 / 1024 (rounded up, no overshoot); maximum 7.0078125 above
+    # has scale 1025 / 1024 < 7.0078125 / 7, so -7.0078125 / scale = -7.00097 -> -7.0 after the divide's rounding
+    # (step 2^-8) and the sum is 0, never negative; code 0.  Its positive twin: 7.0 + 7 = 14.
+    assert _codes([7.0078125, -7.0078125], Q4) == [14, 0]
+
+
+@pytest.mark.parametrize("md", ["bfloat16", "float16"])
+@pytest.mark.parametrize("s", [Q4, Q3])
+def test_quantize_dt_equals_exact_arithmetic(md, s):
+    # the generic-dtype quantizer (float32 carrier arrays rounded to the model dtype after each operation)
+    # against the same exact checkers: rationals on 4 rows, int64 on 128 rows (half a million values)
+    import torch
+
+    k = 4096 if s.bits == 4 else 4080
+    w16 = _config1_weights(128, k)
+    if md == "bfloat16":
+        wf = torch.from_numpy(w16.astype(np.float32)).bfloat16().float().numpy()
+        bits = (wf.view(np.uint32) >> 16).astype(np.uint16)
+    else:
+        wf = w16.astype(np.float32)
+        bits = w16.view(np.uint16)
+    for mode in ("half_away", "half_even"):
+        qw, scale = o.quantize_dt(wf, s, md, mode)
+        q = o.unpack(qw, s, k)
+        exact = exact_fp.quantize_codes_int(bits, s.group_size, s.max_int, md, mode)
+        assert np.array_equal(q, exact), int((q != exact).sum())
+    qw, scale = o.quantize_dt(wf, s, md)
+    q = o.unpack(qw, s, k)
+    for r in range(4):
+        for g in range(k // s.group_size):
+            sl = slice(g * s.group_size, (g + 1) * s.group_size)
+            codes, sc = exact_fp.quantize_group_fraction(exact_fp.to_fraction(wf[r, sl]), s.max_int, md)
+            assert codes == q[r, sl].tolist() and float(sc) == float(scale[r, g])
+    once = exact_fp.quantize_codes_int(bits, s.group_size, s.max_int, md, roundings=1)
+    assert (once != q).mean() > 2e-4  # bf16: 0.54 % (q4), 0.20 % (q3)
+
+
+def test_quantize_dt_float32_equals_exact_rational_arithmetic():
+    # q4f32_1: every operation is an IEEE single operation; 2 rows of 4096 against rationals rounded to binary32
+    w = _config1_weights(2, 4096).astype(np.float32) * np.float32(1.0009766)  # off the binary16 grid
+    qw, scale = o.quantize_dt(w, Q4, "float32")
+    q = o.unpack(qw, Q4, 4096)
+    for r in range(2):
+        for g in range(128):
+            sl = slice(g * 32, g * 32 + 32)
+            codes, sc = exact_fp.quantize_group_fraction(exact_fp.to_fraction(w[r, sl]), 7, "float32")
+            assert codes == q[r, sl].tolist() and float(sc) == float(scale[r, g])
 
 
 @pytest.mark.parametrize("s", [Q4, Q3])
