@@ -216,7 +216,7 @@ def test_quantize_within_reference_test_tolerance(name, shape):
 def _config1_weights(rows, k):
     """Rows of the baseline's first configuration: seed 0, N(0, 0.02), float16 [4096, 4096]."""
     w = (np.random.default_rng(0).standard_normal((4096, 4096)) * 0.02).astype(np.float16)
-    return w[:rows, :k]
+    return np.ascontiguousarray(w[:rows, :k])
 
 
 def _single_rounding_float32(w, s, mode="half_away"):
