@@ -112,7 +112,7 @@ def run_only(args, dev, gq, ops, torch, make_weight) -> int:
         for qw, qs in ws:
             ops.linear(x, qw, qs, bits, gsz, None, torch.float16, y)
             if args.probe:
-                gq._lib.call("mi355gq_probe_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
+                gq._lib.call("mi355gq_testing_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
                              sink.data_ptr(), stream)
 
     us = timed_loop(sweep, copies)
@@ -308,7 +308,7 @@ def main() -> int:
     def read_sweep():
         for lw in layers:
             qw, qs = lw["gate_up"]
-            gq._lib.call("mi355gq_probe_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
+            gq._lib.call("mi355gq_testing_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
                       sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
 
     us_read = timed(read_sweep, max(5, args.steps), 2, use_graph) * 1e3 / LAYERS
@@ -322,9 +322,9 @@ def main() -> int:
         for lw in layers:
             for name in SHAPES:
                 qw, qs = lw[name]
-                gq._lib.call("mi355gq_probe_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
+                gq._lib.call("mi355gq_testing_stream_read", qw.data_ptr(), qw.numel() * 4, qs.data_ptr(), qs.numel() * 2,
                              sink.data_ptr(), stream)
-        gq._lib.call("mi355gq_probe_stream_read", lm_head[0].data_ptr(), lm_head[0].numel() * 4, lm_head[1].data_ptr(),
+        gq._lib.call("mi355gq_testing_stream_read", lm_head[0].data_ptr(), lm_head[0].numel() * 4, lm_head[1].data_ptr(),
                      lm_head[1].numel() * 2, sink.data_ptr(), stream)
 
     ms_probe_step = timed(probe_step, max(5, args.steps), 2, use_graph)

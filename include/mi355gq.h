@@ -56,13 +56,6 @@ MI355GQ_API const char* mi355gq_last_error(void);
 /* 0 when the current HIP device is gfx950, MI355GQ_ERR_UNSUPPORTED otherwise. */
 MI355GQ_API int mi355gq_check_device(void);
 
-/* Measurement aid, no counterpart in the reference: one launch that only reads the byte ranges
- * a and b (sizes multiples of 16, pointers 16-byte aligned) with 128-bit loads and discards
- * them; sink is 4 bytes of device memory or NULL.  bench.py times it on a GEMV's weight and
- * scale tensors to quote what the device delivers for those bytes without any arithmetic. */
-MI355GQ_API int mi355gq_probe_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,
-                              void* sink, mi355gq_stream_t stream);
-
 /*
  * GroupQuantize.quantize_weight, NK layout (replaces the Relax function built at
  * python/mlc_llm/quantization/group_quantization.py:188-306 and utils.py:136-188).
@@ -133,8 +126,12 @@ MI355GQ_API int mi355gq_linear(const void* x, const void* q_weight, const void* 
  * by every GPU the library runs on until the process ends), so the call allocates nothing.  Shapes whose split
  * would want more return MI355GQ_ERR_WORKSPACE (nothing is launched).  All calls on one GPU share the array:
  * calls that overlap on one GPU (different streams, different threads) race on it; stream-ordered calls do not.
+ * The first use on a device looks the array's address up (and may load it with the code object): call
+ * mi355gq_linear_static_scratch_init() once per device, with that device current, before a region that must not
+ * allocate or that is being captured; later calls only read the kept address.
  */
 MI355GQ_API int64_t mi355gq_linear_static_scratch_max_bytes(void);
+MI355GQ_API int mi355gq_linear_static_scratch_init(void);
 MI355GQ_API int mi355gq_linear_static_scratch(const void* x, const void* q_weight, const void* q_scale,
                                   const void* bias, int64_t M, int64_t N, int64_t K, int bits, int group_size,
                                   int out_dtype, void* y, mi355gq_stream_t stream);
@@ -325,6 +322,8 @@ MI355GQ_API int mi355gq_gating_topk(const void* scores, int64_t T, int64_t num_e
  * mi355gq_gating_softmax_topk(_dt).  norm_topk_prob == 0 is the branch of :234-235: softmax over ALL experts in
  * fp32, cast to the model dtype, then gating_topk of those rounded scores; the weights are the selected scores,
  * not renormalised. */
+/* (The reference leaves the order of the fp32 sum over all experts to TVM's reduction; this entry sums left to right,
+ * so a score may differ from the reference's in the last place of the model dtype and, with it, a near-tie's winner.) */
 MI355GQ_API int mi355gq_gating_softmax_topk_ex(const void* logits, int64_t T, int64_t num_experts, int64_t top_k,
                                    int norm_topk_prob, int model_dtype, void* weights, void* ids,
                                    mi355gq_stream_t stream);

@@ -5,8 +5,8 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <atomic>
 #include <cstring>
-#include <mutex>
 
 #include "../../include/mi355gq.h"
 #include "gq_internal.hpp"
@@ -27,23 +27,36 @@ void note_kernel(const char* fmt, ...) {
   va_end(ap);
 }
 
+// Raises a kernel's dynamic-LDS limit to the CU's 160 KiB, once per (kernel, device).  Called on every launch that
+// wants more than 64 KiB, from any thread: a lock-free table (open addressing on the kernel's address, a device bit mask
+// per entry) answers the repeat calls with two atomic loads.  A race on a new entry at worst sets the attribute twice.
 hipError_t allow_large_lds(const void* kernel) {
-  constexpr int kMaxDevices = 64, kSlots = 512;
-  static std::mutex mu;
-  static const void* seen[kMaxDevices][kSlots];  // kernels already set, per device (a few dozen instantiations exist)
-  static int count[kMaxDevices];
+  constexpr int kSlots = 1024;  // a few dozen instantiations exist
+  static std::atomic<const void*> keys[kSlots];
+  static std::atomic<uint64_t> masks[kSlots];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
-  if (dev >= 0 && dev < kMaxDevices) {
-    std::lock_guard<std::mutex> lock(mu);
-    for (int i = 0; i < count[dev]; ++i)
-      if (seen[dev][i] == kernel) return hipSuccess;
-    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e == hipSuccess && count[dev] < kSlots) seen[dev][count[dev]++] = kernel;
-    return e;
+  int slot = -1;
+  if (dev >= 0 && dev < 64) {
+    unsigned h = static_cast<unsigned>((reinterpret_cast<uintptr_t>(kernel) >> 4) * 2654435761u) % kSlots;
+    for (int probe = 0; probe < kSlots; ++probe, h = (h + 1) % kSlots) {
+      const void* k = keys[h].load(std::memory_order_acquire);
+      if (k == nullptr) {
+        const void* expected = nullptr;
+        if (keys[h].compare_exchange_strong(expected, kernel, std::memory_order_acq_rel)) k = kernel;
+        else k = expected;
+      }
+      if (k == kernel) {
+        slot = static_cast<int>(h);
+        break;
+      }
+    }
+    if (slot >= 0 && (masks[slot].load(std::memory_order_acquire) >> dev) & 1u) return hipSuccess;
   }
-  return hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+  if (e == hipSuccess && slot >= 0) masks[slot].fetch_or(uint64_t(1) << dev, std::memory_order_release);
+  return e;
 }
 }  // namespace gq
 
@@ -180,12 +193,12 @@ int mi355gq_testing_set_option(const char* name, int value) {
   return MI355GQ_OK;
 }
 
-int mi355gq_probe_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,
-                              void* sink, mi355gq_stream_t stream) {
+int mi355gq_testing_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes, void* sink,
+                                void* stream) {
   GQ_REQUIRE(a_bytes >= 0 && b_bytes >= 0 && (a_bytes % 16) == 0 && (b_bytes % 16) == 0,
-             "probe_stream_read: sizes must be non-negative multiples of 16");
-  GQ_REQUIRE((a_bytes == 0 || a) && (b_bytes == 0 || b), "probe_stream_read: null pointer");
-  GQ_REQUIRE(aligned16(a) && aligned16(b) && aligned4(sink), "probe_stream_read: 16-byte alignment");
+             "testing_stream_read: sizes must be non-negative multiples of 16");
+  GQ_REQUIRE((a_bytes == 0 || a) && (b_bytes == 0 || b), "testing_stream_read: null pointer");
+  GQ_REQUIRE(aligned16(a) && aligned16(b) && aligned4(sink), "testing_stream_read: 16-byte alignment");
   return hip_result(gq::launch_stream_read(a, a_bytes, b, b_bytes, sink, as_stream(stream)),
                     "stream read launch");
 }
@@ -461,25 +474,28 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 // once per device.  In host code `scratch` is only a handle for this lookup, never an address.
 static int static_scratch_ptr(void** out) {
   constexpr int kMaxDevices = 64;
-  static std::mutex mu;
-  static void* ptrs[kMaxDevices];
+  static std::atomic<void*> ptrs[kMaxDevices];
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return hip_result(e, "hipGetDevice");
   if (dev < 0 || dev >= kMaxDevices) return fail(MI355GQ_ERR_UNSUPPORTED, "linear_static_scratch: device %d", dev);
-  std::lock_guard<std::mutex> lock(mu);
-  if (ptrs[dev] == nullptr) {
-    void* p = nullptr;
+  void* p = ptrs[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {  // (two threads that race here look the same address up twice)
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess) return hip_result(e, "hipGetSymbolAddress(scratch)");
     if (p == nullptr) return fail(MI355GQ_ERR_HIP, "hipGetSymbolAddress(scratch) returned a null address");
-    ptrs[dev] = p;
+    ptrs[dev].store(p, std::memory_order_release);
   }
-  *out = ptrs[dev];
+  *out = p;
   return MI355GQ_OK;
 }
 
 int64_t mi355gq_linear_static_scratch_max_bytes(void) { return kStaticScratchBytes; }
+
+int mi355gq_linear_static_scratch_init(void) {
+  void* p = nullptr;
+  return static_scratch_ptr(&p);
+}
 
 int mi355gq_linear_static_scratch(const void* x, const void* q_weight, const void* q_scale, const void* bias,
                                   int64_t M, int64_t N, int64_t K, int bits, int group_size, int out_dtype,
@@ -526,7 +542,6 @@ static int moe_gemv_impl(const void* x, int64_t x_rows, const void* q_weight, co
   GQ_REQUIRE(out && (K == 0 || (x && q_weight && q_scale && expert_ids)), "moe_gemv: null pointer");
   GQ_REQUIRE(aligned16(x) && aligned16(q_weight) && aligned4(expert_ids) && aligned2(out),
              "moe_gemv: x and q_weight must be 16-byte aligned");
-  GQ_REQUIRE(x_rows == 1 || (K % 8) == 0, "moe_gemv: K must be a multiple of 8 when x has top_k rows");
   GQ_REQUIRE(!paired || (N & 1) == 0, "moe_gemv_silu_mul: N=%lld must be even", (long long)N);
   if (K == 0) return launch_empty_k(nullptr, nullptr, out, top_k, paired ? N / 2 : N, 0, as_stream(stream));
   gq::GemvArgs a{};

@@ -152,8 +152,9 @@ __global__ __launch_bounds__(256) void gemv_reg_kernel(const uint16_t* x_, const
     const int b = c / (kpad / 8);
     const int k = (c - b * (kpad / 8)) * 8;
     xok[i] = vec && c < chunks && k + 8 <= p.K;
-    // always a valid 16-byte load (x itself when the chunk is out of range); zeroed at store time
-    const uint16_t* src = xok[i] ? xs_base + static_cast<int64_t>(b) * xs_stride + k : xs_base;
+    // always a valid, aligned 16-byte load (the base of x when the chunk is out of range or rows of x are not
+    // 16-byte aligned, as an expert slot's row is when K is not a multiple of 8); zeroed at store time
+    const uint16_t* src = xok[i] ? xs_base + static_cast<int64_t>(b) * xs_stride + k : p.x;
     xv[i] = *reinterpret_cast<const uint4*>(src);
   }
 

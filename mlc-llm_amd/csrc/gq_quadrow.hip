@@ -289,12 +289,15 @@ __global__ __launch_bounds__((NBQ == 2 && U * QP <= 2 && MODE != 1 && !KS) ? 102
               const uint4 r = ok[i][c] ? raw[i][c] : make_uint4(0, 0, 0, 0);
               nat[4 * c + 0] = r.x; nat[4 * c + 1] = r.y; nat[4 * c + 2] = r.z; nat[4 * c + 3] = r.w;
             }
-            const float corr = permute_group<BITS, BF>(nat, xr);
+            float corr = permute_group<BITS, BF>(nat, xr);
             const int lp = q & 63, bi = q >> 6;
             // The float16 unpack leaves the odd fields times 16 (q3: times 8 and times 64) in their operands.  Their
             // activations are divided by the same power of two here, once per workgroup, so that all of a group's
-            // products can run through ONE accumulator (exact unless the quotient is subnormal, where it moves the
-            // product by at most 2^-25 times the field's weight: far below the rounding of the accumulation).
+            // products can run through ONE accumulator.  The division is exact unless the quotient is subnormal
+            // (|x| < 2^-10 for the x16 class, 2^-8 for x64).  The offset term is therefore formed from the divided
+            // values (times 16 x 71, 8 x 131, 64 x 19: the same real numbers, so the same bits, wherever the division
+            // was exact): what a rounded quotient adds to the products then cancels against it up to
+            // 2^-25 * 16 * (q - m) per weight, instead of 2^-25 * 16 * (64 + q) with the offset taken from x itself.
             if constexpr (!BF) {
               const half2_t r16 = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
               const half2_t r8 = {static_cast<_Float16>(0.125f), static_cast<_Float16>(0.125f)};
@@ -311,6 +314,25 @@ __global__ __launch_bounds__((NBQ == 2 && U * QP <= 2 && MODE != 1 && !KS) ? 102
                   xr[5 * c + 1] = as_u32(as_half2(xr[5 * c + 1]) * r8);
                   xr[5 * c + 4] = as_u32(as_half2(xr[5 * c + 4]) * r8);
                   xr[5 * c + 2] = as_u32(as_half2(xr[5 * c + 2]) * r64);
+                }
+              }
+              corr = 0.f;  // same order of accumulation as permute_group
+              if constexpr (BITS == 4) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                  corr = dot2(xr[4 * c + 0], 0x64076407u /* (1031, 1031) */, corr);
+                  corr = dot2(xr[4 * c + 1], 0x64706470u /* (16 * 71, ..) */, corr);
+                  corr = dot2(xr[4 * c + 2], 0x64076407u, corr);
+                  corr = dot2(xr[4 * c + 3], 0x64706470u, corr);
+                }
+              } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                  corr = dot2(xr[5 * c + 0], 0x64036403u /* (1027, 1027) */, corr);
+                  corr = dot2(xr[5 * c + 1], 0x64186418u /* (8 * 131, ..) */, corr);
+                  corr = dot2(xr[5 * c + 2], 0x64c064c0u /* (64 * 19, ..) */, corr);
+                  corr = dot2(xr[5 * c + 3], 0x64036403u, corr);
+                  corr = dot2(xr[5 * c + 4], 0x64186418u, corr);
                 }
               }
             }
@@ -359,10 +381,11 @@ __global__ __launch_bounds__((NBQ == 2 && U * QP <= 2 && MODE != 1 && !KS) ? 102
                        const uint2 (&bias_bits)[QP], const uint2 (&res_bits)[QP][NBQ]) {
       // One batch quad: every LDS read of the item goes out before the first matrix instruction.  Left to the compiler
       // each read is issued one ahead of its use, so a wave waits out most of an LDS round trip ten times per item, and
-      // on the launches this form serves a SIMD often hosts a single wave.  (q3 with two quads per item keeps its reads
-      // where they are used: hoisted, that one instantiation returned wrong sums for the first quad of every pair on the
-      // GPU while its assembly read correct; the cause was not found, so it stays as it was.)
-      constexpr bool HOIST = NBQ == 1 && U <= 4 && !(BITS == 3 && QP == 2);
+      // on the launches this form serves a SIMD often hosts a single wave.  Only with one quad per item: with two, the
+      // q3 instantiation returned wrong sums for the first quad of every pair with its reads hoisted while its assembly
+      // read correct, and the cause was not found, so no two-quad form hoists (the heuristic picks two quads per item
+      // only with two batch quads, which never hoisted; one batch quad with two quads per item is a tuning override).
+      constexpr bool HOIST = NBQ == 1 && U <= 4 && QP == 1;
       uint4 xh[HOIST ? U : 1][CH];
       float ch[HOIST ? U : 1];
       if constexpr (HOIST) {

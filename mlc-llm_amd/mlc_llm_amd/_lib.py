@@ -38,11 +38,11 @@ SIGNATURES = {
     "mi355gq_linear_residual_dt": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_linear_dt_workspace_bytes": (_L, [_L, _L, _L, _I, _I, _I]),
     "mi355gq_linear_dt": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _I, _P, _P, _L, _P]),
-    "mi355gq_probe_stream_read": (_I, [_P, _L, _P, _L, _P, _P]),
     "mi355gq_embedding_take": (_I, [_P, _L, _P, _P, _L, _L, _I, _I, _P, _P]),
     "mi355gq_linear_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
     "mi355gq_linear": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_linear_static_scratch_max_bytes": (_L, []),
+    "mi355gq_linear_static_scratch_init": (_I, []),
     "mi355gq_linear_static_scratch": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P]),
     "mi355gq_linear_residual": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_linear_silu_mul_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
@@ -86,6 +86,7 @@ SIGNATURES = {
 TEST_HOOKS = {
     "mi355gq_testing_set_option": (_I, [c_char_p, _I]),
     "mi355gq_testing_last_kernel": (c_char_p, []),
+    "mi355gq_testing_stream_read": (_I, [_P, _L, _P, _L, _P, _P]),
 }
 
 

@@ -28,6 +28,31 @@ class MixtralMoE(nn.Module):
                                                  2 * intermediate_size, config, device=device)
         self.e2 = GroupQuantizeMixtralExperts(num_local_experts, intermediate_size, hidden_size,
                                               config, device=device)
+        # Which fused forms the library has for this module is a property of its dtype, expert count, top-k and
+        # shapes: each is tried until the library first answers "unsupported", then never again (a failing call
+        # formats a message and raises on every forward otherwise).
+        self._fused = {"route": True, "routed_gemv": True, "gemv_combine": True}
+
+    def _try(self, name, fn, *args, **kwargs):
+        """fn(*args) if the fused form `name` is (still) believed to exist, else None; a first ERR_UNSUPPORTED
+        switches the form off for this module."""
+        if not self._fused[name]:
+            return None
+        try:
+            return fn(*args, **kwargs)
+        except _lib.Mi355gqError as err:
+            if err.code != _lib.ERR_UNSUPPORTED:
+                raise
+            self._fused[name] = False
+            return None
+
+    def _route_fits(self, num_tokens: int) -> bool:
+        """The batch sizes mi355gq_moe_route scans in one workgroup (it answers "unsupported" beyond them, which says
+        nothing about smaller batches, so that answer is not remembered)."""
+        slots, experts = num_tokens * self.num_experts_per_tok, self.num_local_experts
+        if slots <= 8192 and experts * -(-slots // 64) <= 8192:
+            return True
+        return experts <= 64 and num_tokens <= 8192 and experts * -(-num_tokens // 1024) <= 64
 
     def _expert_forward(self, x: torch.Tensor, indptr: torch.Tensor) -> torch.Tensor:
         # x1, x3 = split(e1_e3(x)); e2(silu(x1) * x3): the activation rides in the e1_e3 kernel
@@ -41,14 +66,11 @@ class MixtralMoE(nn.Module):
         num_tokens = batch_size * seq_len
         x = x.reshape(num_tokens, hidden_size).contiguous()
         if num_tokens > 1:
-            try:
-                # routing in one launch; the gather rides in e1_e3's row addressing, the scatter in the
-                # combine's: four launches where the op-by-op sequence below takes nine
-                weights, _, token_indices, _, slot_positions, indptr = ops.moe_route(gate, experts_per_tok)
-            except _lib.Mi355gqError as err:
-                if err.code != _lib.ERR_UNSUPPORTED:
-                    raise
-            else:
+            # routing in one launch; the gather rides in e1_e3's row addressing, the scatter in the
+            # combine's: four launches where the op-by-op sequence below takes nine
+            routed = self._try("route", ops.moe_route, gate, experts_per_tok) if self._route_fits(num_tokens) else None
+            if routed is not None:
+                weights, _, token_indices, _, slot_positions, indptr = routed
                 cfg = self.e1_e3.config
                 if num_tokens * experts_per_tok > 128:
                     # the GEMM's workgroups would each start with one more dependent load (index, then
@@ -59,26 +81,20 @@ class MixtralMoE(nn.Module):
                 y = self.e2(h, indptr)
                 return ops.moe_combine_sorted(y, slot_positions, weights).reshape(batch_size, seq_len, hidden_size)
         if num_tokens == 1:
-            try:
-                # the token routes itself inside the e1_e3 kernel: one launch where the two operators take two
-                cfg = self.e1_e3.config
-                h, expert_weights, expert_indices = ops.moe_gemv_routed_silu_mul(
-                    x, gate, experts_per_tok, self.e1_e3.q_weight, self.e1_e3.q_scale, cfg.bits, self.e1_e3.group_size)
-            except _lib.Mi355gqError as err:
-                if err.code != _lib.ERR_UNSUPPORTED:
-                    raise
-            else:
-                try:
-                    # e2 and the weighted sum over the experts in one launch as well
-                    cfg2 = self.e2.config
-                    x = ops.moe_gemv_combine(h, self.e2.q_weight, self.e2.q_scale, expert_indices, expert_weights,
-                                             cfg2.bits, self.e2.group_size)
-                except _lib.Mi355gqError as err:
-                    if err.code != _lib.ERR_UNSUPPORTED:
-                        raise
-                    x = self.e2(h, expert_indices)
-                    x = ops.moe_combine(x.reshape(1, experts_per_tok, hidden_size), expert_weights)
-                return x.reshape(batch_size, seq_len, hidden_size)
+            # the token routes itself inside the e1_e3 kernel: one launch where the two operators take two
+            cfg = self.e1_e3.config
+            first = self._try("routed_gemv", ops.moe_gemv_routed_silu_mul, x, gate, experts_per_tok, self.e1_e3.q_weight,
+                              self.e1_e3.q_scale, cfg.bits, self.e1_e3.group_size)
+            if first is not None:
+                h, expert_weights, expert_indices = first
+                # e2 and the weighted sum over the experts in one launch as well
+                cfg2 = self.e2.config
+                out = self._try("gemv_combine", ops.moe_gemv_combine, h, self.e2.q_weight, self.e2.q_scale, expert_indices,
+                                expert_weights, cfg2.bits, self.e2.group_size)
+                if out is None:
+                    out = self.e2(h, expert_indices)
+                    out = ops.moe_combine(out.reshape(1, experts_per_tok, hidden_size), expert_weights)
+                return out.reshape(batch_size, seq_len, hidden_size)
         expert_weights, expert_indices = moe_misc.gating_softmax_topk(gate, experts_per_tok)
         if num_tokens == 1:
             x = self._expert_forward(x, expert_indices)

@@ -384,6 +384,65 @@ def test_quadrow_kernel(name, u, qp, m, n, k):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("m", [1, 3, 4, 8, 16, 40])
+@pytest.mark.parametrize("log2_scale", [-6, -10, -13])
+def test_linear_small_activations(name, m, log2_scale):
+    """Activations far below 1 (N(0, 1) * 2^-6, 2^-10, 2^-13; the last are float16 subnormals in part): the bound
+    scales with max|x|, so a kernel that loses bits of small activations fails it.  The few-row kernel divides the
+    activations of its scaled operand classes by 16 (q3: 8, 64) in float16, which is exact down to |x| = 2^-10 (2^-8);
+    below that a product moves by at most 2^-25 * 16 (64) * (q - m) * scale: at 2^-13 the relative L2 error may reach
+    4e-3 there (q3), which the test allows for that kernel and that scale only."""
+    s = SCHEMES[name]
+    n, k = 520, 4096 if s.bits == 4 else 4000
+    rng = np.random.default_rng(seed_of("small", name, m, log2_scale))
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    x = (rng.standard_normal((m, k)) * 2.0**log2_scale).astype(np.float16)
+    y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
+    kern = gq._lib.last_kernel()
+    ref = o.linear_fp32(x, qw, qs, s)
+    err, bound, rel = o.check_linear(y.cpu().numpy(), ref, x, k)
+    loose = log2_scale == -13 and kern.startswith("gq::quad_kernel")
+    assert err <= bound, (kern, err, bound)
+    assert rel <= (6e-3 if loose else REL_L2), (kern, rel)
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("u", [-1, 2, 4, 8])
+@pytest.mark.parametrize("qp", [1, 2])
+@pytest.mark.parametrize("m", [3, 4, 7])
+@pytest.mark.parametrize("n,k", [(520, 1024), (2100, 200), (72, 6176)])
+def test_quadrow_kernel_many_quads_per_wave(name, u, qp, m, n, k):
+    """Sixteen waves in all, so that every wave walks many quad sets and items of different quads follow each other in its
+    register ring (with the default launch shape a wave has one quad set): every item size and quads-per-item form, with
+    bias + residual, plain with float32 output, and the folded activation, against the oracle."""
+    s = SCHEMES[name]
+    if s.bits == 3:
+        k = {1024: 1000, 200: 200, 6176: 6200}[k]
+    x, qw, qs, b = _linear_case(s, m, n, k, 11 * m + n + k + u, bias=True)
+    res = np.random.default_rng(n + k).standard_normal((m, n)).astype(np.float16)
+    gq._lib.set_option("gemv_variant", 6)
+    gq._lib.set_option("gemv_rows_per_wave", u)
+    gq._lib.set_option("quad_pairs", qp)
+    gq._lib.set_option("gemv_waves", 16)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b), residual=dev(res))
+        assert gq._lib.last_kernel().startswith("gq::quad_kernel") and gq._lib.last_kernel().endswith(f",{qp}>")
+        y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
+        y16 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None)
+        if n % 8 == 0:
+            assert torch.equal(ops.linear_silu_mul(dev(x), dev(qw), dev(qs), s.bits, s.group_size), ops.silu_mul(y16))
+            assert gq._lib.last_kernel().startswith("gq::quad_kernel")
+    finally:
+        for opt in ("gemv_variant", "gemv_rows_per_wave", "quad_pairs", "gemv_waves"):
+            gq._lib.set_option(opt, -1)
+    ref = o.linear_fp32(x, qw, qs, s)
+    assert_linear_ok(y, ref + b.astype(np.float64) + res.astype(np.float64), x, k, f"quad-row walk {name} u={u} qp={qp} {m}x{n}x{k}")
+    assert_linear_ok(y32, ref, x, k, f"quad-row walk u={u} qp={qp} fp32 out")
+    assert_linear_ok(y16, ref, x, k, f"quad-row walk u={u} qp={qp}")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("ksplit", [0, 1, 2])  # 1, 2, 4 neighbouring waves share the K range of a quad set
 @pytest.mark.parametrize("qp", [1, 2])
 @pytest.mark.parametrize("m", [3, 4, 8])
@@ -830,8 +889,6 @@ def test_moe_gemv(name, x_rows):
     s = SCHEMES[name]
     rng = np.random.default_rng(41)
     ne, n, k = 8, 520, 1024 if s.bits == 4 else 1000
-    if x_rows == 2 and k % 8:
-        pytest.skip("x rows must stay 16-byte aligned")
     w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
     qw, qs = o.quantize(w, s)
     x = rng.standard_normal((x_rows, k)).astype(np.float16)
@@ -839,6 +896,28 @@ def test_moe_gemv(name, x_rows):
     out = ops.moe_gemv(dev(x), dev(qw), dev(qs), dev(ids), s.bits, s.group_size)
     ref = o.moe_dequantize_gemv_fp32(x, qw, qs, ids, s)
     assert_linear_ok(out, ref, x, k, f"moe_gemv {name}")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("k", [1004, 1001, 37])
+@pytest.mark.parametrize("variant", [-1, 0])
+def test_moe_gemv_unaligned_rows_of_x(name, k, variant):
+    """x with top_k rows and K not a multiple of 8 (op/moe_matmul.py:147-176 has no such restriction): the second
+    slot's row of x then starts off a 16-byte boundary; both GEMV kernels (register, LDS-staged) against the oracle."""
+    s = SCHEMES[name]
+    rng = np.random.default_rng(43)
+    ne, n = 4, 72
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    x = rng.standard_normal((2, k)).astype(np.float16)
+    ids = np.array([[3, 1]], np.int32)
+    gq._lib.set_option("gemv_variant", variant)
+    try:
+        out = ops.moe_gemv(dev(x), dev(qw), dev(qs), dev(ids), s.bits, s.group_size)
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+    ref = o.moe_dequantize_gemv_fp32(x, qw, qs, ids, s)
+    assert_linear_ok(out, ref, x, k, f"moe_gemv {name} K={k}")
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
@@ -1177,12 +1256,12 @@ def test_stream_read_probe_runs_and_validates():
     a = torch.arange(4096 + 8, dtype=torch.int32, device="cuda:0")  # sizes that exercise the tail loop
     b = torch.ones(64, dtype=torch.int32, device="cuda:0")
     sink = torch.zeros(1, dtype=torch.int32, device="cuda:0")
-    gq._lib.call("mi355gq_probe_stream_read", a.data_ptr(), a.numel() * 4, b.data_ptr(), b.numel() * 4,
+    gq._lib.call("mi355gq_testing_stream_read", a.data_ptr(), a.numel() * 4, b.data_ptr(), b.numel() * 4,
                  sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
-    gq._lib.call("mi355gq_probe_stream_read", a.data_ptr(), a.numel() * 4, None, 0, None,
+    gq._lib.call("mi355gq_testing_stream_read", a.data_ptr(), a.numel() * 4, None, 0, None,
                  torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
-    assert gq._lib.lib().mi355gq_probe_stream_read(a.data_ptr(), 24, None, 0, None, None) == -1  # not a multiple of 16
+    assert gq._lib.lib().mi355gq_testing_stream_read(a.data_ptr(), 24, None, 0, None, None) == -1  # not a multiple of 16
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
