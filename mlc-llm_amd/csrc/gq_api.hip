@@ -170,7 +170,7 @@ int mi355gq_testing_set_option(const char* name, int value) {
     GQ_REQUIRE(value >= -1 && value <= 1, "gemv_ksplit=%d (-1, 0, 1)", value);
     o.gemv_ksplit = value;
   } else if (!strcmp(name, "quad_ksplit")) {
-    GQ_REQUIRE(value >= -1 && value <= 2, "quad_ksplit=%d (-1, 0, 1, 2)", value);
+    GQ_REQUIRE(value >= -1 && value <= 3, "quad_ksplit=%d (-1, 0, 1, 2, 3)", value);
     o.quad_ksplit = value;
   } else if (!strcmp(name, "quad_pairs")) {
     GQ_REQUIRE(value == -1 || value == 1 || value == 2, "quad_pairs=%d (1, 2)", value);
@@ -402,7 +402,9 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
       a.bits = bits; a.group_size = group_size; a.out_f32 = 0; a.paired = 1;
       e = gq::launch_gemv(a, as_stream(stream));
     } else if (M <= (bits == 3 ? 16 : 8) && !q3_passes_lose) {
-      e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
+      const int gvp = gq::options().gemv_variant;
+      if (M <= 8 && (gvp < 0 || gvp == 9)) e = gq::launch_quadreg(g, static_cast<int>(M), as_stream(stream));
+      if (e == hipErrorNotSupported) e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     }
     // (one or two rows never reach the matrix-core kernels in the plain linear either: without a fused form
     //  the caller runs the two steps, and the result stays the same bit for bit)
@@ -419,6 +421,11 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // (q3 has no 16x16x32 skinny kernel: 9..16 rows run as two concurrent 8-row passes of the quad-row kernel)
   // (... on the smaller matrices: from about 40 M weights on, the GEMM's 32-row tile is ahead of them: gate_up 38
   //  against 42-46 us, down 25.6 against 27-29.5, while qkv stays at 14.7 against 17.1 and o_proj at 10.3 against 15.2)
+  // 3..8 rows: the 4x4x4 kernel with x resident in registers, where it applies
+  if (M >= 3 && M <= 8 && gm < 0 && (gv < 0 || gv == 9)) {
+    const hipError_t q = gq::launch_quadreg(g, static_cast<int>(M), as_stream(stream));
+    if (q != hipErrorNotSupported) return hip_result(q, "quad-row (registers) launch");
+  }
   if (bits == 3 && M >= 3 && M <= 16 && gm != 1 && (M > 8 || gm != 2) && (gv < 0 || (gv >= 6 && gv <= 8)) &&
       !q3_passes_lose) {
     const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));

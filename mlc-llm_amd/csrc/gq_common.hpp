@@ -57,6 +57,19 @@ __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t b
   return r;
 }
 
+// The same instruction, emitted by the compiler: the mask is laundered into a VGPR through an EMPTY asm statement
+// (so that it is not folded back into a second literal) and the expression is left to instruction selection.
+// This is the form for results that feed a matrix instruction directly.  An instruction inside an asm statement is
+// invisible to the compiler's hazard handling and to its scheduler's latencies: with the asm form above, a
+// v_and_or_b32 landed one instruction in front of the v_mfma_f32_4x4x4 that reads its result, and that matrix
+// instruction used the register's old value (deterministic wrong sums in the first of two accumulator chains, q3
+// forms with two chains per item); the compiler's own placement keeps seven or more instructions between them.
+__device__ __forceinline__ uint32_t and_or_c(uint32_t a, uint32_t mask, uint32_t bits) {
+  uint32_t m = mask;
+  asm("" : "+v"(m));
+  return (a & m) | bits;
+}
+
 __device__ __forceinline__ float h2f(uint16_t h) {
   return static_cast<float>(__builtin_bit_cast(_Float16, h));
 }

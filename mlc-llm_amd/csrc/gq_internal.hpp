@@ -16,7 +16,7 @@ struct Options {
   int quad_pairs = -1;          // -1: heuristic, 1 | 2: quads per item of the quad-row kernel
   int gemv_ksplit = -1;         // -1: heuristic, 0: never, 1: wherever it applies (register GEMV: two waves share a row's K)
   int quad_ksplit = -1;         // -1: heuristic, 0 | 1 | 2: log2 of the waves that share a quad set's K range
-  int gemv_variant = -1;        // -1: heuristic, 0: LDS GEMV, 1: register GEMV, 2..5 skinny forms, 6..8 quad-row forms
+  int gemv_variant = -1;        // -1: heuristic, 0: LDS GEMV, 1: register GEMV, 2..5 skinny forms, 6..8 quad-row forms (x in LDS), 9: quad-row with x in registers
   int gemm_variant = -1;
   int gemv_waves = -1;          // total waves of a persistent GEMV / quad-row / skinny grid
   int gemm_split_k = -1;        // wanted workgroups of the few-row GEMM's split along K
@@ -92,6 +92,10 @@ hipError_t launch_skinny(const GemmArgs& a, int rows_max, hipStream_t s);
 // 4x4x4-MFMA kernel with GEMV-like weight streaming (q4, activations resident in LDS);
 // hipErrorNotSupported when the shape does not fit.
 hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s);
+
+// the same matrix instruction with the activations resident in registers (plain linears of up to 8 float16 rows);
+// hipErrorNotSupported when the shape does not fit.
+hipError_t launch_quadreg(const GemmArgs& a, int rows_max, hipStream_t s);
 
 // plain streaming read of two byte ranges (multiples of 16 bytes, 16-byte aligned)
 hipError_t launch_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,

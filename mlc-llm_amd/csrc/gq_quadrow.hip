@@ -381,11 +381,11 @@ __global__ __launch_bounds__((NBQ == 2 && U * QP <= 2 && MODE != 1 && !KS) ? 102
                        const uint2 (&bias_bits)[QP], const uint2 (&res_bits)[QP][NBQ]) {
       // One batch quad: every LDS read of the item goes out before the first matrix instruction.  Left to the compiler
       // each read is issued one ahead of its use, so a wave waits out most of an LDS round trip ten times per item, and
-      // on the launches this form serves a SIMD often hosts a single wave.  Only with one quad per item: with two, the
-      // q3 instantiation returned wrong sums for the first quad of every pair with its reads hoisted while its assembly
-      // read correct, and the cause was not found, so no two-quad form hoists (the heuristic picks two quads per item
-      // only with two batch quads, which never hoisted; one batch quad with two quads per item is a tuning override).
-      constexpr bool HOIST = NBQ == 1 && U <= 4 && QP == 1;
+      // on the launches this form serves a SIMD often hosts a single wave.  (One instantiation, q3 with two quads per
+      // item, once returned wrong sums for the first quad of every pair in this form.  The cause was the unpack's
+      // v_and_or_b32 sitting in an asm statement, where the compiler cannot keep its distance to the matrix
+      // instruction that reads the result: see and_or_c.)
+      constexpr bool HOIST = NBQ == 1 && U <= 4;
       uint4 xh[HOIST ? U : 1][CH];
       float ch[HOIST ? U : 1];
       if constexpr (HOIST) {
@@ -411,29 +411,29 @@ __global__ __launch_bounds__((NBQ == 2 && U * QP <= 2 && MODE != 1 && !KS) ? 102
           for (int d = 0; d < 4; ++d) {
             if constexpr (BITS == 4) {
               const uint32_t w8 = w[d] >> 8;
-              lo[qp][d][0] = and_or(w[d], 0x000f000fu, kMagic);
-              lo[qp][d][1] = and_or(w8, 0x000f000fu, kMagic);
+              lo[qp][d][0] = and_or_c(w[d], 0x000f000fu, kMagic);
+              lo[qp][d][1] = and_or_c(w8, 0x000f000fu, kMagic);
               if constexpr (BF) {
-                hi[qp][d][0] = and_or(w[d] >> 4, 0x000f000fu, kMagic);
-                hi[qp][d][1] = and_or(w[d] >> 12, 0x000f000fu, kMagic);
+                hi[qp][d][0] = and_or_c(w[d] >> 4, 0x000f000fu, kMagic);
+                hi[qp][d][1] = and_or_c(w[d] >> 12, 0x000f000fu, kMagic);
               } else {
-                hi[qp][d][0] = and_or(w[d], 0x00f000f0u, kMagic);
-                hi[qp][d][1] = and_or(w8, 0x00f000f0u, kMagic);
+                hi[qp][d][0] = and_or_c(w[d], 0x00f000f0u, kMagic);
+                hi[qp][d][1] = and_or_c(w8, 0x00f000f0u, kMagic);
               }
             } else {
               // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
               const uint32_t t = (w[d] & 0x0000ffffu) | ((w[d] << 1) & 0xffff0000u);
               const uint32_t t9 = t >> 9;
-              lo[qp][d][0] = and_or(t, 0x00070007u, kMagic);   // fields (0,5)
-              lo[qp][d][1] = and_or(t9, 0x00070007u, kMagic);  // fields (3,8)
+              lo[qp][d][0] = and_or_c(t, 0x00070007u, kMagic);   // fields (0,5)
+              lo[qp][d][1] = and_or_c(t9, 0x00070007u, kMagic);  // fields (3,8)
               if constexpr (BF) {
-                hi[qp][d][0] = and_or(t >> 3, 0x00070007u, kMagic);   // fields (1,6)
-                hi[qp][d][1] = and_or(t >> 12, 0x00070007u, kMagic);  // fields (4,9)
-                a64[qp][d >> 1][d & 1] = and_or(t >> 6, 0x00070007u, kMagic);  // fields (2,7)
+                hi[qp][d][0] = and_or_c(t >> 3, 0x00070007u, kMagic);   // fields (1,6)
+                hi[qp][d][1] = and_or_c(t >> 12, 0x00070007u, kMagic);  // fields (4,9)
+                a64[qp][d >> 1][d & 1] = and_or_c(t >> 6, 0x00070007u, kMagic);  // fields (2,7)
               } else {
-                hi[qp][d][0] = and_or(t, 0x00380038u, kMagic);   // fields (1,6) x 8
-                hi[qp][d][1] = and_or(t9, 0x00380038u, kMagic);  // fields (4,9) x 8
-                a64[qp][d >> 1][d & 1] = and_or(t, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+                hi[qp][d][0] = and_or_c(t, 0x00380038u, kMagic);   // fields (1,6) x 8
+                hi[qp][d][1] = and_or_c(t9, 0x00380038u, kMagic);  // fields (4,9) x 8
+                a64[qp][d >> 1][d & 1] = and_or_c(t, 0x01c001c0u, kMagic);  // fields (2,7) x 64
               }
             }
           }
@@ -729,7 +729,7 @@ static hipError_t launch_quadrow_bits(const GemmArgs& a, int rows_max, hipStream
   p.kw_log2 = 0;
   if (a.indptr == nullptr && p.nphases == 1 && p.rounds == 1 && a.bias == nullptr && a.residual == nullptr &&
       U * QP <= 2 && !big_wg) {
-    const int opt_kw = options().quad_ksplit;
+    const int opt_kw = options().quad_ksplit > 2 ? 2 : options().quad_ksplit;
     const int want = opt_kw >= 0 ? opt_kw : 1;
     while (p.kw_log2 < want && p.kw_log2 < 2 && (p.steps_total >> (p.kw_log2 + 1)) >= (opt_kw >= 0 ? 1 : 5) &&
            (static_cast<int64_t>(p.nsets) * mtiles << (p.kw_log2 + 1)) <= (opt_kw >= 0 ? 4096 : 2048))

@@ -6,10 +6,12 @@
  * the calling thread, and a thread that never calls it always gets the heuristics.  value < 0 restores the
  * heuristic.  Names and ranges:
  *   "gemv_rows_per_wave"  1, 2, 4, 8     rows per row set of the register GEMV
- *   "gemv_variant"        0..15          kernel family for up to 16 rows (2..5 a skinny form, 6..8 the quad-row kernel)
+ *   "gemv_variant"        0..15          kernel family for up to 16 rows (2..5 a skinny form, 6..8 the quad-row kernel, 9 its
+ *                                        form with x in registers)
  *   "gemv_waves"          4..16384       persistent waves of the register GEMV / quad-row kernel
  *   "gemv_ksplit"         0, 1           K of a row shared between two waves of the register GEMV (off / on)
- *   "quad_ksplit"         0, 1, 2        log2 of the waves of the quad-row kernel that share a quad set's K range
+ *   "quad_ksplit"         0, 1, 2, 3     log2 of the waves of a quad-row kernel that share a quad's K range (3: the form
+ *                                        with x in registers only)
  *   "quad_pairs"          1, 2           weight quads per item of the quad-row kernel
  *   "gemm_variant"        0..15          GEMM tile (1: GEMM only, 2: GEMV up to 8 rows, others pick a tile)
  *   "gemm_split_k"        1..4096        split of K in the few-row GEMM

@@ -384,6 +384,50 @@ def test_quadrow_kernel(name, u, qp, m, n, k):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("ksplit", [-1, 0, 1, 2, 3])  # log2 of the waves that share a quad's K range
+@pytest.mark.parametrize("waves", [-1, 16])  # 16 waves in all: every walker goes through many quads
+@pytest.mark.parametrize("m", [3, 4, 5, 8])
+@pytest.mark.parametrize("n,k", [(520, 1024), (100, 4096), (2100, 72), (64, 6176), (4, 256), (36, 14336), (1024, 4096)])
+def test_quadreg_kernel(name, ksplit, waves, m, n, k):
+    """The few-row kernel that keeps its slice of x in registers, forced: every split of K among 1..8 waves that the
+    shape admits (iterations per wave 1..4; the others must be declined), one quad per walker and many, bias + residual,
+    float32 output, and the folded activation bit for bit against the two steps."""
+    s = SCHEMES[name]
+    if s.bits == 3:
+        k = {1024: 1000, 4096: 4000, 72: 80, 6176: 6200, 256: 240, 14336: 11008}[k]
+    x, qw, qs, b = _linear_case(s, m, n, k, 13 * m + n + k + ksplit, bias=True)
+    res = np.random.default_rng(n + k).standard_normal((m, n)).astype(np.float16)
+    niter = -(-s.num_group(k) // 16)
+    umax = 2 if m > 4 else 4
+    gq._lib.set_option("gemv_variant", 9)
+    gq._lib.set_option("quad_ksplit", ksplit)
+    gq._lib.set_option("gemv_waves", waves)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, dev(b), residual=dev(res))
+        kern = gq._lib.last_kernel()
+        if ksplit >= 0 and waves < 0:  # (with 16 waves the partial sums of a long walk may not fit LDS: declined too)
+            u = -(-niter // (1 << ksplit))
+            fits = u <= umax and niter <= 16
+            assert kern.startswith("gq::quadreg_kernel") == fits, (kern, niter, ksplit)
+        y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
+        y16 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None)
+        kern16 = gq._lib.last_kernel()
+        if n % 8 == 0:
+            fused = ops.linear_silu_mul(dev(x), dev(qw), dev(qs), s.bits, s.group_size)
+            # (a declined shape falls back to different kernels for the two forms: equal bits only within a family)
+            if kern16.startswith("gq::quadreg_kernel") and gq._lib.last_kernel().startswith("gq::quadreg_kernel"):
+                assert torch.equal(fused, ops.silu_mul(y16))
+    finally:
+        for opt in ("gemv_variant", "quad_ksplit", "gemv_waves"):
+            gq._lib.set_option(opt, -1)
+    ref = o.linear_fp32(x, qw, qs, s)
+    what = f"quadreg {name} ksplit={ksplit} waves={waves} {m}x{n}x{k} [{kern}]"
+    assert_linear_ok(y, ref + b.astype(np.float64) + res.astype(np.float64), x, k, what)
+    assert_linear_ok(y32, ref, x, k, what + " fp32 out")
+    assert_linear_ok(y16, ref, x, k, what + " plain")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("m", [1, 3, 4, 8, 16, 40])
 @pytest.mark.parametrize("log2_scale", [-6, -10, -13])
 def test_linear_small_activations(name, m, log2_scale):
@@ -402,7 +446,7 @@ def test_linear_small_activations(name, m, log2_scale):
     kern = gq._lib.last_kernel()
     ref = o.linear_fp32(x, qw, qs, s)
     err, bound, rel = o.check_linear(y.cpu().numpy(), ref, x, k)
-    loose = log2_scale == -13 and kern.startswith("gq::quad_kernel")
+    loose = log2_scale == -13 and kern.startswith(("gq::quad_kernel", "gq::quadreg_kernel"))
     assert err <= bound, (kern, err, bound)
     assert rel <= (6e-3 if loose else REL_L2), (kern, rel)
 
