@@ -137,6 +137,30 @@ MI355GQ_API int mi355gq_linear_static_scratch(const void* x, const void* q_weigh
                                   int out_dtype, void* y, mi355gq_stream_t stream);
 
 /*
+ * KN-layout schemes (q4f16_0, q3f16_0, q4bf16_0 of quantization/quantization.py:47-57, 69-79): quantize_weight with
+ * output_transpose stores the transposed tensors (group_quantization.py:125-130, 299-305),
+ *   q_weight uint32 [nw, N],  q_scale fp16 [ng, N],
+ * and GroupQuantizeLinear.forward dequantises along axis 0 and multiplies without a transpose (:404-437).
+ * mi355gq_linear_kn is mi355gq_linear on those tensors as stored: up to 8 rows (N a multiple of 4) run a GEMV that
+ * streams them in place (its split along K keeps fp32 partial sums in the workspace; without one it runs unsplit,
+ * slower); every other shape runs the NK kernels on an NK copy made in the workspace, which must then hold
+ * mi355gq_linear_kn_workspace_bytes() bytes, 16-byte aligned (MI355GQ_ERR_WORKSPACE otherwise).
+ * mi355gq_kn_to_nk / mi355gq_nk_to_kn move both tensors between the layouts (bit moves: a caller that keeps converted
+ * q4f16_0 weights can make the NK tensors once and use every other entry point); mi355gq_dequantize_kn is
+ * GroupQuantize._dequantize with axis 0: out fp16 [K, N].  float16 models.
+ */
+MI355GQ_API int mi355gq_kn_to_nk(const void* q_weight_kn, const void* q_scale_kn, int64_t N, int64_t K, int bits,
+                     int group_size, void* q_weight_nk, void* q_scale_nk, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_nk_to_kn(const void* q_weight_nk, const void* q_scale_nk, int64_t N, int64_t K, int bits,
+                     int group_size, void* q_weight_kn, void* q_scale_kn, mi355gq_stream_t stream);
+MI355GQ_API int mi355gq_dequantize_kn(const void* q_weight, const void* q_scale, int64_t N, int64_t K, int bits,
+                          int group_size, void* out, mi355gq_stream_t stream);
+MI355GQ_API int64_t mi355gq_linear_kn_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size);
+MI355GQ_API int mi355gq_linear_kn(const void* x, const void* q_weight, const void* q_scale, const void* bias, int64_t M,
+                      int64_t N, int64_t K, int bits, int group_size, int out_dtype, void* y, void* workspace,
+                      int64_t workspace_bytes, mi355gq_stream_t stream);
+
+/*
  * The same linear with the element-wise tail the reference folds into the matmul kernel:
  * FuseDequantizeMatmulEwise (compiler_pass/fuse_dequantize_matmul_ewise.py:19-32) fuses the
  * dequantize + matmul pair together with up to three element-wise operands that operator fusion

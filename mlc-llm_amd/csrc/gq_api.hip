@@ -519,6 +519,101 @@ int mi355gq_linear_static_scratch(const void* x, const void* q_weight, const voi
                      ws ? kStaticScratchBytes : 0, stream);
 }
 
+// ---- KN layout (q4f16_0 / q3f16_0): tensors as convert_weight stores them
+static int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
+
+int mi355gq_kn_to_nk(const void* q_weight_kn, const void* q_scale_kn, int64_t N, int64_t K, int bits, int group_size,
+                     void* q_weight_nk, void* q_scale_nk, mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(N >= 0 && K >= 0 && N < kMaxDim && K < kMaxDim, "kn_to_nk: bad shape N=%lld K=%lld", (long long)N, (long long)K);
+  if (N == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(q_weight_kn && q_scale_kn && q_weight_nk && q_scale_nk, "kn_to_nk: null pointer");
+  GQ_REQUIRE(aligned4(q_weight_kn) && aligned4(q_weight_nk) && aligned2(q_scale_kn) && aligned2(q_scale_nk),
+             "kn_to_nk: misaligned tensor");
+  const int64_t ng = (K + group_size - 1) / group_size, nw = 4 * ng;
+  return hip_result(gq::launch_kn_transpose(static_cast<const uint32_t*>(q_weight_kn), static_cast<const uint16_t*>(q_scale_kn),
+                                            nw, ng, N, static_cast<uint32_t*>(q_weight_nk),
+                                            static_cast<uint16_t*>(q_scale_nk), as_stream(stream)),
+                    "kn_to_nk launch");
+}
+
+int mi355gq_nk_to_kn(const void* q_weight_nk, const void* q_scale_nk, int64_t N, int64_t K, int bits, int group_size,
+                     void* q_weight_kn, void* q_scale_kn, mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(N >= 0 && K >= 0 && N < kMaxDim && K < kMaxDim, "nk_to_kn: bad shape N=%lld K=%lld", (long long)N, (long long)K);
+  if (N == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(q_weight_kn && q_scale_kn && q_weight_nk && q_scale_nk, "nk_to_kn: null pointer");
+  GQ_REQUIRE(aligned4(q_weight_kn) && aligned4(q_weight_nk) && aligned2(q_scale_kn) && aligned2(q_scale_nk),
+             "nk_to_kn: misaligned tensor");
+  const int64_t ng = (K + group_size - 1) / group_size, nw = 4 * ng;
+  // both source tensors have N rows; their widths differ, so they go as two transposes
+  hipError_t e = gq::launch_kn_transpose(static_cast<const uint32_t*>(q_weight_nk), nullptr, N, 0, nw,
+                                         static_cast<uint32_t*>(q_weight_kn), nullptr, as_stream(stream));
+  if (e == hipSuccess)
+    e = gq::launch_kn_transpose(nullptr, static_cast<const uint16_t*>(q_scale_nk), 0, N, ng, nullptr,
+                                static_cast<uint16_t*>(q_scale_kn), as_stream(stream));
+  return hip_result(e, "nk_to_kn launch");
+}
+
+int mi355gq_dequantize_kn(const void* q_weight, const void* q_scale, int64_t N, int64_t K, int bits, int group_size,
+                          void* out, mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(N >= 0 && K >= 0 && N < kMaxDim && K < kMaxDim, "dequantize_kn: bad shape");
+  if (N == 0 || K == 0) return MI355GQ_OK;
+  GQ_REQUIRE(q_weight && q_scale && out, "dequantize_kn: null pointer");
+  GQ_REQUIRE(aligned4(q_weight) && aligned2(q_scale) && aligned2(out), "dequantize_kn: misaligned tensor");
+  return hip_result(gq::launch_dequantize_kn(static_cast<const uint32_t*>(q_weight), static_cast<const uint16_t*>(q_scale), N,
+                                             K, bits, static_cast<uint16_t*>(out), as_stream(stream)),
+                    "dequantize_kn launch");
+}
+
+// workspace of mi355gq_linear_kn: the GEMV's partial sums (M <= 8), or an NK copy of both tensors plus what mi355gq_linear
+// wants for the shape
+int64_t mi355gq_linear_kn_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
+  if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim || N >= kMaxDim || K >= kMaxDim)
+    return 0;
+  const int64_t ng = (K + group_size - 1) / group_size, nw = 4 * ng;
+  if (M >= 1 && M <= 8 && (N & 3) == 0) return gq::gemv_kn_workspace_bytes(M, N, K, bits);
+  return align256(N * nw * 4) + align256(N * ng * 2) + mi355gq_linear_workspace_bytes(M, N, K, bits, group_size);
+}
+
+int mi355gq_linear_kn(const void* x, const void* q_weight, const void* q_scale, const void* bias, int64_t M, int64_t N,
+                      int64_t K, int bits, int group_size, int out_dtype, void* y, void* workspace,
+                      int64_t workspace_bytes, mi355gq_stream_t stream) {
+  GQ_CHECK(check_scheme(bits, group_size));
+  GQ_REQUIRE(M >= 0 && N >= 0 && K >= 0 && M < kMaxDim && N < kMaxDim && K < kMaxDim,
+             "linear_kn: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  GQ_REQUIRE(out_dtype == MI355GQ_F16 || out_dtype == MI355GQ_F32, "linear_kn: out_dtype=%d", out_dtype);
+  GQ_REQUIRE(workspace_bytes >= 0, "linear_kn: negative workspace size");
+  if (M == 0 || N == 0) return MI355GQ_OK;
+  GQ_REQUIRE(y != nullptr, "linear_kn: y is null");
+  if (K == 0) return launch_empty_k(bias, nullptr, y, M, N, out_dtype == MI355GQ_F32, as_stream(stream));
+  GQ_REQUIRE(x && q_weight && q_scale, "linear_kn: null pointer");
+  GQ_REQUIRE(aligned2(x) && aligned4(q_weight) && aligned2(q_scale) && aligned4(y) && aligned2(bias),
+             "linear_kn: misaligned tensor");
+  if (workspace == nullptr) workspace_bytes = 0;
+  if (M <= 8) {
+    const hipError_t e = gq::launch_gemv_kn(static_cast<const uint16_t*>(x), static_cast<const uint32_t*>(q_weight),
+                                            static_cast<const uint16_t*>(q_scale), static_cast<const uint16_t*>(bias), M, N,
+                                            K, bits, out_dtype == MI355GQ_F32, y, workspace, workspace_bytes,
+                                            as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "linear_kn launch");
+  }
+  // every other shape: an NK copy in the workspace, then the NK kernels
+  const int64_t ng = (K + group_size - 1) / group_size, nw = 4 * ng;
+  const int64_t w_bytes = align256(N * nw * 4), s_bytes = align256(N * ng * 2);
+  if (workspace_bytes < w_bytes + s_bytes || !aligned16(workspace))
+    return fail(MI355GQ_ERR_WORKSPACE,
+                "linear_kn: M=%lld N=%lld K=%lld runs on an NK copy of the weights and needs a 16-byte aligned workspace of "
+                "%lld bytes (mi355gq_linear_kn_workspace_bytes); got %lld",
+                (long long)M, (long long)N, (long long)K,
+                (long long)mi355gq_linear_kn_workspace_bytes(M, N, K, bits, group_size), (long long)workspace_bytes);
+  char* const ws = static_cast<char*>(workspace);
+  GQ_CHECK(mi355gq_kn_to_nk(q_weight, q_scale, N, K, bits, group_size, ws, ws + w_bytes, stream));
+  return linear_impl(x, ws, ws + w_bytes, bias, nullptr, M, N, K, bits, group_size, out_dtype, y, ws + w_bytes + s_bytes,
+                     workspace_bytes - w_bytes - s_bytes, stream);
+}
+
 int mi355gq_linear_residual(const void* x, const void* q_weight, const void* q_scale,
                             const void* bias, const void* residual, int64_t M, int64_t N, int64_t K,
                             int bits, int group_size, int out_dtype, void* y, void* workspace,

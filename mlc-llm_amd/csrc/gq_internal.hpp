@@ -97,6 +97,17 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s);
 // hipErrorNotSupported when the shape does not fit.
 hipError_t launch_quadreg(const GemmArgs& a, int rows_max, hipStream_t s);
 
+// KN-layout tensors (q_weight [nw, N], q_scale [ng, N]): both tensors transposed in one call (src_rows_w / src_rows_s rows
+// of src_cols columns each), the dequantisation to [K, N], and the decode GEMV (M <= 8, N % 4 == 0) with its workspace
+hipError_t launch_kn_transpose(const uint32_t* qw_src, const uint16_t* qs_src, int64_t src_rows_w, int64_t src_rows_s,
+                               int64_t src_cols, uint32_t* qw_dst, uint16_t* qs_dst, hipStream_t s);
+hipError_t launch_dequantize_kn(const uint32_t* qw, const uint16_t* qs, int64_t N, int64_t K, int bits, uint16_t* out,
+                                hipStream_t s);
+int64_t gemv_kn_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits);
+hipError_t launch_gemv_kn(const uint16_t* x, const uint32_t* qw, const uint16_t* qs, const uint16_t* bias, int64_t M,
+                          int64_t N, int64_t K, int bits, int out_f32, void* y, void* workspace, int64_t workspace_bytes,
+                          hipStream_t s);
+
 // plain streaming read of two byte ranges (multiples of 16 bytes, 16-byte aligned)
 hipError_t launch_stream_read(const void* a, int64_t a_bytes, const void* b, int64_t b_bytes,
                               void* sink, hipStream_t s);

@@ -44,6 +44,11 @@ SIGNATURES = {
     "mi355gq_linear_static_scratch_max_bytes": (_L, []),
     "mi355gq_linear_static_scratch_init": (_I, []),
     "mi355gq_linear_static_scratch": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P]),
+    "mi355gq_kn_to_nk": (_I, [_P, _P, _L, _L, _I, _I, _P, _P, _P]),
+    "mi355gq_nk_to_kn": (_I, [_P, _P, _L, _L, _I, _I, _P, _P, _P]),
+    "mi355gq_dequantize_kn": (_I, [_P, _P, _L, _L, _I, _I, _P, _P]),
+    "mi355gq_linear_kn_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
+    "mi355gq_linear_kn": (_I, [_P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_linear_residual": (_I, [_P, _P, _P, _P, _P, _L, _L, _L, _I, _I, _I, _P, _P, _L, _P]),
     "mi355gq_linear_silu_mul_workspace_bytes": (_L, [_L, _L, _L, _I, _I]),
     "mi355gq_linear_silu_mul": (_I, [_P, _P, _P, _L, _L, _L, _I, _I, _P, _P, _L, _P]),

@@ -155,6 +155,82 @@ def linear(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits:
     return out
 
 
+def _check_kn_shapes(q_weight, q_scale, k, bits, group_size):
+    ng = -(-k // group_size)
+    nw = (group_size // (32 // bits)) * ng
+    if q_weight.dim() != 2 or q_scale.dim() != 2 or q_weight.shape[0] != nw or q_scale.shape[0] != ng or \
+            q_weight.shape[1] != q_scale.shape[1]:
+        raise ValueError(f"KN layout: q_weight {tuple(q_weight.shape)} / q_scale {tuple(q_scale.shape)}, expected "
+                         f"({nw}, N) / ({ng}, N) for K={k}")
+    if not (q_weight.is_contiguous() and q_scale.is_contiguous()):
+        raise ValueError("KN layout: q_weight and q_scale must be contiguous")
+    return q_weight.shape[1]
+
+
+def linear_kn(x: torch.Tensor, q_weight: torch.Tensor, q_scale: torch.Tensor, bits: int, group_size: int,
+              bias: Optional[torch.Tensor] = None, out_dtype=torch.float16) -> torch.Tensor:
+    """linear() on KN-layout tensors as a q4f16_0 / q3f16_0 model stores them: q_weight [nw, N], q_scale [ng, N]
+    (float16 models).  Up to 8 rows stream them in place; more rows run on an NK copy made in a workspace."""
+    _chk(x, torch.float16, "x")
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    k = x.shape[-1]
+    n = _check_kn_shapes(q_weight, q_scale, k, bits, group_size)
+    m = 1
+    for d in x.shape[:-1]:
+        m *= d
+    if bias is not None:
+        _chk(bias, torch.float16, "bias")
+        if tuple(bias.shape) != (n,):
+            raise ValueError(f"bias shape {tuple(bias.shape)}, expected {(n,)}")
+    if out_dtype not in (torch.float16, torch.float32):
+        raise TypeError(f"out_dtype {out_dtype}")
+    out = torch.empty((*x.shape[:-1], n), dtype=out_dtype, device=x.device)
+    ws_bytes = _lib.lib().mi355gq_linear_kn_workspace_bytes(m, n, k, bits, group_size)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    _lib.call("mi355gq_linear_kn", x.data_ptr(), q_weight.data_ptr(), q_scale.data_ptr(),
+              bias.data_ptr() if bias is not None else None, m, n, k, bits, group_size,
+              _lib.F32 if out_dtype == torch.float32 else _lib.F16, out.data_ptr(),
+              ws.data_ptr() if ws is not None else None, ws_bytes, _stream())
+    return out
+
+
+def kn_to_nk(q_weight: torch.Tensor, q_scale: torch.Tensor, k: int, bits: int, group_size: int):
+    """KN-layout tensors (q_weight [nw, N], q_scale [ng, N]) -> the NK tensors every other entry point takes."""
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    n = _check_kn_shapes(q_weight, q_scale, k, bits, group_size)
+    qw = torch.empty((n, q_weight.shape[0]), dtype=torch.int32, device=q_weight.device)
+    qs = torch.empty((n, q_scale.shape[0]), dtype=torch.float16, device=q_weight.device)
+    _lib.call("mi355gq_kn_to_nk", q_weight.data_ptr(), q_scale.data_ptr(), n, k, bits, group_size, qw.data_ptr(),
+              qs.data_ptr(), _stream())
+    return qw, qs
+
+
+def nk_to_kn(q_weight: torch.Tensor, q_scale: torch.Tensor, k: int, bits: int, group_size: int):
+    """NK tensors (q_weight [N, nw], q_scale [N, ng]) -> the KN layout of the `_0` schemes."""
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    n = q_weight.shape[0]
+    _check_qshapes(q_weight, q_scale, (n,), k, bits, group_size)
+    qw = torch.empty((q_weight.shape[1], n), dtype=torch.int32, device=q_weight.device)
+    qs = torch.empty((q_scale.shape[1], n), dtype=torch.float16, device=q_weight.device)
+    _lib.call("mi355gq_nk_to_kn", q_weight.data_ptr(), q_scale.data_ptr(), n, k, bits, group_size, qw.data_ptr(),
+              qs.data_ptr(), _stream())
+    return qw, qs
+
+
+def dequantize_kn(q_weight: torch.Tensor, q_scale: torch.Tensor, k: int, bits: int, group_size: int) -> torch.Tensor:
+    """GroupQuantize._dequantize along axis 0: KN tensors -> float16 [K, N]."""
+    _chk(q_weight, _STORAGE, "q_weight")
+    _chk(q_scale, torch.float16, "q_scale")
+    n = _check_kn_shapes(q_weight, q_scale, k, bits, group_size)
+    out = torch.empty((k, n), dtype=torch.float16, device=q_weight.device)
+    _lib.call("mi355gq_dequantize_kn", q_weight.data_ptr(), q_scale.data_ptr(), n, k, bits, group_size, out.data_ptr(),
+              _stream())
+    return out
+
+
 def _linear_other_dtype(x, q_weight, q_scale, bits, group_size, bias, out_dtype, out, residual):
     """linear() for float32 / bfloat16 models: x, q_scale and bias share the model dtype; the output is
     that dtype (the default here, whatever `out_dtype` defaults to for float16) or float32."""

@@ -234,7 +234,11 @@ class GroupQuantizeLinear(nn.Module):
             return self.q_weight, self.q_scale
         key = (self.q_weight.data_ptr(), self.q_scale.data_ptr())
         if getattr(self, "_nk_key", None) != key:
-            self._nk = (self.q_weight.detach().t().contiguous(), self.q_scale.detach().t().contiguous())
+            if self.q_scale.dtype == torch.float16 and self.q_weight.is_cuda:
+                self._nk = ops.kn_to_nk(self.q_weight.detach(), self.q_scale.detach(), self.in_features,
+                                        self.config.bits, self.config.group_size)
+            else:
+                self._nk = (self.q_weight.detach().t().contiguous(), self.q_scale.detach().t().contiguous())
             self._nk_key = key
         return self._nk
 
@@ -250,8 +254,13 @@ class GroupQuantizeLinear(nn.Module):
         self.config._require_built()
         model_dtype = _TORCH_DTYPE[self.config.model_dtype]
         out_dtype = model_dtype if self.out_dtype is None else _TORCH_DTYPE[self.out_dtype]
-        q_weight, q_scale = self._nk_tensors()
         bias = self.bias
+        rows = x.numel() // max(x.shape[-1], 1)
+        if (self.config.linear_weight_layout == "KN" and model_dtype == torch.float16 and rows <= 8
+                and self.out_features % 4 == 0 and (bias is None or bias.dtype == model_dtype)):
+            # decode batches of a KN-layout model: the stored tensors are streamed as they are
+            return ops.linear_kn(x, self.q_weight, self.q_scale, self.config.bits, self.config.group_size, bias, out_dtype)
+        q_weight, q_scale = self._nk_tensors()
         if bias is not None and bias.dtype != model_dtype:
             # fp32 bias with fp32 output: added after the kernel, as the reference's `x + bias`
             y = ops.linear(x, q_weight, q_scale, self.config.bits, self.config.group_size, None, out_dtype)

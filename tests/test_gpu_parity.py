@@ -869,8 +869,11 @@ def test_kn_layout_is_the_transposed_nk_tensors(kn_name, nk_name):
     lin_kn.q_weight.data, lin_kn.q_scale.data = qw, qs
     lin_nk.q_weight.data, lin_nk.q_scale.data = dev(qw_ref), dev(qs_ref)
     for m in (1, 5, 40):
-        x = dev(rng.standard_normal((m, k)).astype(np.float16))
-        assert torch.equal(lin_kn(x), lin_nk(x))
+        xh = rng.standard_normal((m, k)).astype(np.float16)
+        if m > 8:  # an NK copy and the NK kernels: the same bits
+            assert torch.equal(lin_kn(dev(xh)), lin_nk(dev(xh)))
+        else:  # decode batches stream the KN tensors as stored (another order of summation)
+            assert_linear_ok(lin_kn(dev(xh)), o.linear_fp32(xh, qw_ref, qs_ref, s), xh, k, f"KN module M={m}")
     # new parameters are picked up (the transposed copy is remade)
     w2 = (rng.standard_normal((96, k)) * 0.05).astype(np.float16)
     qw2, qs2 = kn.quantize_weight(dev(w2), output_transpose=True)
@@ -878,6 +881,69 @@ def test_kn_layout_is_the_transposed_nk_tensors(kn_name, nk_name):
     x = rng.standard_normal((3, k)).astype(np.float16)
     q2w, q2s = o.quantize(w2, s)
     assert_linear_ok(lin_kn(dev(x)), o.linear_fp32(x, q2w, q2s, s), x, k, "KN after update")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("n,k", [(96, 256), (4096, 4096), (130, 1000), (28672, 4096), (7, 72)])
+def test_kn_entry_points(name, n, k):
+    """The C ABI on KN-layout tensors (q_weight [nw, N], q_scale [ng, N], as quantize_weight(output_transpose=True)
+    stores them, group_quantization.py:299-305): both transposes bit for bit, the dequantisation along axis 0 bit for
+    bit (the oracle's NK dequantisation, transposed), and the linear against the oracle at decode batches (the GEMV that
+    streams the stored tensors, N % 4 == 0) and beyond (an NK copy in the workspace), with bias and float32 output."""
+    s = SCHEMES[name]
+    if s.bits == 3:
+        k = {256: 240, 4096: 4096, 1000: 1000, 72: 80}[k]
+    rng = np.random.default_rng(seed_of("kn", name, n, k))
+    rows = min(n, 520)  # (the oracle's float64 matmul on a sample of the output columns of the large shapes)
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    qw_kn, qs_kn = dev(np.ascontiguousarray(qw.T)), dev(np.ascontiguousarray(qs.T))
+    nk_w, nk_s = ops.kn_to_nk(qw_kn, qs_kn, k, s.bits, s.group_size)
+    assert np.array_equal(host_u32(nk_w), qw) and np.array_equal(host_f16_bits(nk_s), qs.view(np.uint16))
+    back_w, back_s = ops.nk_to_kn(nk_w, nk_s, k, s.bits, s.group_size)
+    assert torch.equal(back_w, qw_kn) and torch.equal(back_s, qs_kn)
+    cols = np.unique(np.concatenate([[0, 1, n // 2, n - 1], rng.integers(0, n, rows)]))
+    d = ops.dequantize_kn(qw_kn, qs_kn, k, s.bits, s.group_size)
+    assert tuple(d.shape) == (k, n)
+    want = o.dequantize(qw[cols], qs[cols], s, k)
+    assert np.array_equal(host_f16_bits(d[:, torch.from_numpy(cols).to(DEV)]), want.T.view(np.uint16))
+    b = rng.standard_normal(n).astype(np.float16)
+    for m in (1, 2, 4, 8, 19):
+        x = rng.standard_normal((m, k)).astype(np.float16)
+        ref = o.linear_fp32(x, qw[cols], qs[cols], s)
+        y = ops.linear_kn(dev(x), qw_kn, qs_kn, s.bits, s.group_size)
+        kern = gq._lib.last_kernel()
+        assert kern.startswith("gq::gemv_kn_kernel") == (m <= 8 and n % 4 == 0), (kern, m, n)
+        assert_linear_ok(y[:, torch.from_numpy(cols).to(DEV)], ref, x, k, f"linear_kn {name} {m}x{n}x{k} [{kern}]")
+        y32 = ops.linear_kn(dev(x), qw_kn, qs_kn, s.bits, s.group_size, dev(b), torch.float32)
+        assert_linear_ok(y32[:, torch.from_numpy(cols).to(DEV)], ref + b[cols].astype(np.float64), x, k,
+                         f"linear_kn bias fp32 {name} {m}x{n}x{k}")
+
+
+def test_linear_kn_workspace_contract():
+    """Without a workspace the decode GEMV runs unsplit (same tolerance); the other shapes need room for the NK copy
+    and say so (MI355GQ_ERR_WORKSPACE) before anything is launched."""
+    lib = gq._lib
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(77)
+    n, k = 512, 2048
+    w = (rng.standard_normal((n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    qw_kn, qs_kn = dev(np.ascontiguousarray(qw.T)), dev(np.ascontiguousarray(qs.T))
+    x = rng.standard_normal((3, k)).astype(np.float16)
+    xd = dev(x)
+    y = torch.empty((3, n), dtype=torch.float16, device=DEV)
+    assert lib.lib().mi355gq_linear_kn_workspace_bytes(3, n, k, 4, 32) > 0  # (few column blocks: K is split)
+    lib.call("mi355gq_linear_kn", xd.data_ptr(), qw_kn.data_ptr(), qs_kn.data_ptr(), None, 3, n, k, 4, 32, lib.F16,
+             y.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+    assert gq._lib.last_kernel().endswith("slices=1")
+    assert_linear_ok(y, o.linear_fp32(x, qw, qs, s), x, k, "linear_kn without a workspace")
+    x40 = dev(rng.standard_normal((40, k)).astype(np.float16))
+    y40 = torch.empty((40, n), dtype=torch.float16, device=DEV)
+    with pytest.raises(lib.Mi355gqError) as ei:
+        lib.call("mi355gq_linear_kn", x40.data_ptr(), qw_kn.data_ptr(), qs_kn.data_ptr(), None, 40, n, k, 4, 32, lib.F16,
+                 y40.data_ptr(), None, 0, torch.cuda.current_stream().cuda_stream)
+    assert ei.value.code == lib.ERR_WORKSPACE
 
 
 # ------------------------------------------------------------------ MoE
