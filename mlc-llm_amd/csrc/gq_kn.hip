@@ -72,6 +72,7 @@ struct KnParams {
   void* y;              // [M, N] (fp16 / fp32), or the fp32 partial sums [slices, M, N] when slices > 1
   int N, K, ng, slices, gps;  // gps: groups per slice
   int out_f32;
+  int x_vec;  // x rows are 16-byte aligned (K % 8 == 0, aligned base)
 };
 
 // grid (column blocks of 256, K slices); a workgroup's 4 waves take the groups of its slice round robin
@@ -91,12 +92,22 @@ __global__ __launch_bounds__(256) void gemv_kn_kernel(const KnParams p) {
     const int b = q / gcount, gl = q - b * gcount;
     const int k0 = (g0 + gl) * G;
     uint32_t nat[HP], xr[HP];
+    if (p.x_vec) {  // K % 8 == 0 and a 16-byte aligned x: whole 16-byte chunks, inside or outside K
 #pragma unroll
-    for (int h = 0; h < HP; ++h) {
-      const int k = k0 + 2 * h;
-      const uint32_t lo = k < p.K ? p.x[static_cast<int64_t>(b) * p.K + k] : 0u;
-      const uint32_t hi = k + 1 < p.K ? p.x[static_cast<int64_t>(b) * p.K + k + 1] : 0u;
-      nat[h] = lo | (hi << 16);
+      for (int c = 0; c < CH; ++c) {
+        const int k = k0 + 8 * c;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (k + 8 <= p.K) v = *reinterpret_cast<const uint4*>(p.x + static_cast<int64_t>(b) * p.K + k);
+        nat[4 * c] = v.x; nat[4 * c + 1] = v.y; nat[4 * c + 2] = v.z; nat[4 * c + 3] = v.w;
+      }
+    } else {
+#pragma unroll
+      for (int h = 0; h < HP; ++h) {
+        const int k = k0 + 2 * h;
+        const uint32_t lo = k < p.K ? p.x[static_cast<int64_t>(b) * p.K + k] : 0u;
+        const uint32_t hi = k + 1 < p.K ? p.x[static_cast<int64_t>(b) * p.K + k + 1] : 0u;
+        nat[h] = lo | (hi << 16);
+      }
     }
     corr_lds[b * p.gps + gl] = permute_group<BITS>(nat, xr);
 #pragma unroll
@@ -199,7 +210,7 @@ __global__ __launch_bounds__(256) void kn_reduce_kernel(const float* __restrict_
 // K slices for a shape: enough workgroups to cover the chip a few times over, whole groups, at most 64 per slice's x in LDS
 int kn_slices(int64_t M, int64_t N, int ng) {
   const int64_t colblocks = (N + 255) / 256;
-  int64_t slices = (1024 + colblocks - 1) / colblocks;
+  int64_t slices = (512 + colblocks - 1) / colblocks;
   if (slices > (ng + 3) / 4) slices = (ng + 3) / 4;  // every wave keeps at least one group
   if (slices < 1) slices = 1;
   // x of a slice must fit LDS next to the sums: 48 KiB for x
@@ -289,6 +300,7 @@ hipError_t launch_gemv_kn(const uint16_t* x, const uint32_t* qw, const uint16_t*
   p.x = x; p.qw = qw; p.qs = qs; p.bias = bias; p.y = y;
   p.N = static_cast<int>(N); p.K = static_cast<int>(K); p.ng = static_cast<int>((K + G - 1) / G);
   p.out_f32 = out_f32;
+  p.x_vec = (K & 7) == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0;
   if (bits == 4) return launch_gemv_kn_bits<4>(p, static_cast<int>(M), workspace, workspace_bytes, y, bias, s);
   return launch_gemv_kn_bits<3>(p, static_cast<int>(M), workspace, workspace_bytes, y, bias, s);
 }
