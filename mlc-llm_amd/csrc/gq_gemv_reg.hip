@@ -504,15 +504,30 @@ static hipError_t launch_bits(const GemvParams& p, int nb, int slots, hipStream_
     }
   }
   const bool plain = !p.paired && !p.routed && p.bias == nullptr && p.residual == nullptr;
-  if (iters >= 5 && nb == 1 && R == 1 && plain && rounds <= 64 && options().gemv_ksplit != 0) {
+  // ... and on K = 4096 (two groups per lane: one per wave of a pair) for the mid-sized matrices, one row per set whatever
+  // was chosen above: 28672 x 4096 14.8 -> 13.8 us on 4096 waves, 6144 x 4096 5.24 -> 5.03 on 6144; 4096 x 4096 and
+  // 128256 x 4096 unchanged (same-process A/B, graph replay over rotating weights), so they keep the whole-K form.
+  const bool short_pair = iters == 2 && slots == 1 && p.N >= 6144 && p.N < 65536 && options().gemv_waves <= 0 &&
+                          options().gemv_rows_per_wave < 0;
+  if ((iters >= 5 || short_pair || (options().gemv_ksplit == 1 && iters >= 2)) && nb == 1 && plain &&
+      options().gemv_ksplit != 0) {
+    const int nsets1 = p.N;
+    int walkers = waves;  // (long K: twice the waves of the whole-K form)
+    if (iters < 5) walkers = (options().gemv_waves > 0 ? options().gemv_waves : (p.N >= 16384 ? 4096 : 6144)) / 2;
+    if (walkers < 1) walkers = 1;
+    const int rounds1 = (nsets1 + walkers - 1) / walkers;
+    if (rounds1 <= 64 && (iters < 5 || R == 1)) {
     const int half = (iters + 1) / 2;
-    const int blocks2 = (2 * ((nsets + rounds - 1) / rounds) + 3) / 4;
+    const int blocks2 = (2 * ((nsets1 + rounds1 - 1) / rounds1) + 3) / 4;
     switch (half) {
-      case 3: return launch_shared_k<BITS, 3>(p, slots, blocks2, nsets, s);
-      case 4: return launch_shared_k<BITS, 4>(p, slots, blocks2, nsets, s);
-      case 5: return launch_shared_k<BITS, 5>(p, slots, blocks2, nsets, s);
-      case 6: return launch_shared_k<BITS, 6>(p, slots, blocks2, nsets, s);
+      case 1: return launch_shared_k<BITS, 1>(p, slots, blocks2, nsets1, s);
+      case 2: return launch_shared_k<BITS, 2>(p, slots, blocks2, nsets1, s);
+      case 3: return launch_shared_k<BITS, 3>(p, slots, blocks2, nsets1, s);
+      case 4: return launch_shared_k<BITS, 4>(p, slots, blocks2, nsets1, s);
+      case 5: return launch_shared_k<BITS, 5>(p, slots, blocks2, nsets1, s);
+      case 6: return launch_shared_k<BITS, 6>(p, slots, blocks2, nsets1, s);
       default: break;
+    }
     }
   }
   const int blocks = ((nsets + rounds - 1) / rounds + 3) / 4;  // even share of sets per wave

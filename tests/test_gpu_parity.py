@@ -256,11 +256,30 @@ def test_gemv_long_k_shared_between_two_waves(name, ksplit, n, k):
     finally:
         gq._lib.set_option("gemv_ksplit", -1)
     groups_per_lane = -(-(-(-k // s.group_size)) // 64)
-    assert kern.startswith("gq::gemv_reg_kernel") and kern.endswith(",2>") == (ksplit == 1 and groups_per_lane >= 5), kern
+    # (forced on, the pair form takes any K of two groups per lane or more; by itself it runs from five on, and on
+    #  K of exactly two for mid-sized matrices: test_gemv_short_k_pairs)
+    assert kern.startswith("gq::gemv_reg_kernel") and kern.endswith(",2>") == (ksplit == 1 and groups_per_lane >= 2), kern
     ref = o.linear_fp32(x, qw, qs, s)
     assert_linear_ok(y, ref, x, k, f"gemv long K {name} ksplit={ksplit} {n}x{k}")
     assert_linear_ok(y32, ref, x, k, f"gemv long K ksplit={ksplit} fp32 out")
     assert_linear_ok(ym, o.moe_dequantize_gemv_fp32(x2, qw2, qs2, ids, s), x2, k, f"moe gemv long K ksplit={ksplit}")
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+@pytest.mark.parametrize("n", [6144, 6150, 28672])
+def test_gemv_short_k_pairs(name, n):
+    """K of two groups per lane on a mid-sized matrix: by default two neighbouring waves take one group per lane each
+    (one row per set, the halves meet in LDS after the walk); against the oracle, float32 output too."""
+    s = SCHEMES[name]
+    k = 4096
+    x, qw, qs, _ = _linear_case(s, 1, n, k, n + 5, bias=False)
+    y = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None)
+    kern = gq._lib.last_kernel()
+    assert kern.startswith("gq::gemv_reg_kernel") and kern.endswith(",2>"), kern
+    y32 = ops.linear(dev(x), dev(qw), dev(qs), s.bits, s.group_size, None, torch.float32)
+    ref = o.linear_fp32(x, qw, qs, s)
+    assert_linear_ok(y, ref, x, k, f"gemv short K pairs {name} n={n}")
+    assert_linear_ok(y32, ref, x, k, f"gemv short K pairs {name} n={n} fp32")
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
