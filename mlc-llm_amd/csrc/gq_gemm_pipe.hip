@@ -33,6 +33,12 @@ namespace gq {
 // zeros instead of the bytes behind the tensor.  A separate instantiation rather than a branch: the general
 // form's addresses and flags would otherwise stay in registers next to this one's, and the large tile has none to spare
 // (a spill reload inside the loop waits for every global load in flight).
+// q4 in that form also reads its scales in bulk: the two lanes of a weight row load the row's 16 bytes of scales for FOUR
+// K tiles at once (one request: both lanes name the same address) instead of 2 bytes per lane and K tile.  A 2-byte load
+// costs the memory pipeline what a 16-byte one does (a wave's instruction touches 32 rows = 32 cache lines either way),
+// and those loads alone were 9 % of the plain 256 x 256 GEMM, 18 % of down_proj's and a third of a grouped GEMM with few
+// rows per expert (timing-only builds without them).  Needs K in whole blocks of four K tiles and 16-byte aligned scale
+// rows (checked by the launcher).
 template <int BITS, int BM, int BN, int WM, int WN, int DEPTH = 2, bool BF = false, bool SKIP = false, int WX = 0,
           bool FAST = false>
 __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(const GemmParams p) {
@@ -53,6 +59,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   constexpr int W_GROUPS = BN * 2 >= NT ? BN * 2 / NT : 1;
   constexpr bool W_ALL = BN * 2 >= NT;
   static_assert(BN * 2 % NT == 0 || BN * 2 * 2 == NT, "tile / thread mismatch");
+  constexpr bool SCV = FAST && BITS == 4;  // scales of four K tiles per load
 
   extern __shared__ uint4 smem[];
   uint16_t* lds = reinterpret_cast<uint16_t*>(smem);
@@ -117,13 +124,15 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   }
 
   uint32_t a_off[A_CHUNKS], w_off[W_GROUPS], s_off[W_GROUPS];
+  uint32_t sc_shift[W_GROUPS];  // (SCV) bit position of this lane's group inside a K tile's word of two scales
 #pragma unroll
   for (int i = 0; i < A_CHUNKS; ++i)
     a_off[i] = static_cast<uint32_t>(reinterpret_cast<const char*>(a_src[i]) - reinterpret_cast<const char*>(p.x));
 #pragma unroll
   for (int i = 0; i < W_GROUPS; ++i) {
     w_off[i] = static_cast<uint32_t>(reinterpret_cast<const char*>(w_src[i] + 4 * w_g[i]) - reinterpret_cast<const char*>(qw));
-    s_off[i] = static_cast<uint32_t>(reinterpret_cast<const char*>(s_src[i] + w_g[i]) - reinterpret_cast<const char*>(qs));
+    s_off[i] = static_cast<uint32_t>(reinterpret_cast<const char*>(s_src[i] + (SCV ? 0 : w_g[i])) - reinterpret_cast<const char*>(qs));
+    sc_shift[i] = 16u * static_cast<uint32_t>(w_g[i]);
   }
 
   // this workgroup's share of K (all of it unless the launch splits K)
@@ -172,9 +181,27 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
       for (int i = 0; i < W_GROUPS; ++i) {
         const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, static_cast<int>(w_off[i]), ktc * 32, 0);
         st.w[i] = make_uint4(v.x, v.y, v.z, v.w);
-        st.s[i] = __builtin_amdgcn_raw_buffer_load_b16(s_rsrc, static_cast<int>(s_off[i]), ktc * 4, 0);
+        if constexpr (!SCV) st.s[i] = __builtin_amdgcn_raw_buffer_load_b16(s_rsrc, static_cast<int>(s_off[i]), ktc * 4, 0);
       }
     }
+  };
+  // (SCV) the scales of K tiles kt0 + 4 blk .. + 3 of this lane's weight row: word c = the two groups of tile c
+  struct ScaleBlock {
+    uint4 v[W_GROUPS];
+  };
+  auto load_scales = [&](int blk, ScaleBlock& sb) {
+    if (w_active) {
+      const int t = min(kt0 + 4 * blk, kt1 - 4);
+#pragma unroll
+      for (int i = 0; i < W_GROUPS; ++i) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(s_rsrc, static_cast<int>(s_off[i]), t * 4, 0);
+        sb.v[i] = make_uint4(v.x, v.y, v.z, v.w);
+      }
+    }
+  };
+  auto scale_of = [&](const ScaleBlock& sb, int i, int c) -> uint32_t {  // c: K tile inside the block (compile-time)
+    const uint32_t word = c == 0 ? sb.v[i].x : (c == 1 ? sb.v[i].y : (c == 2 ? sb.v[i].z : sb.v[i].w));
+    return (word >> sc_shift[i]) & 0xffffu;
   };
   auto load_a = [&](int kt, StageA& st) {
     if constexpr (FAST) {
@@ -206,7 +233,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // One of KSTEPS slices of "tile kt: registers -> LDS stage s".  The slices are issued between the
   // MFMA k-steps of the tile being multiplied, so that dequantisation (VALU) and the LDS stores
   // run in the shadow of the matrix pipe instead of after it.
-  auto store_part = [&](int kt, const StageA& sa, const StageW& st, int s, int part) {
+  auto store_part = [&](int kt, const StageA& sa, const StageW& st, int s, int part, const ScaleBlock& scb, int sc_c) {
     uint16_t* at = a_tile(s);
     uint16_t* wt = lds + s * BN * LDA;  // (w_dst holds the offset of the W region)
     const int k_base = kt * BK;
@@ -227,7 +254,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
     for (int i = 0; i < W_GROUPS; ++i) {
       const bool ok = KTAIL ? 2 * kt + w_g[i] < p.ng : (FAST || 2 * kt + w_g[i] < g_lim);
       // a group past the end gets scale +0.0: every value becomes (q - m) * 0 = +-0
-      const uint16_t sb = ok ? static_cast<uint16_t>(st.s[i]) : uint16_t(0);
+      const uint16_t sb = SCV ? static_cast<uint16_t>(scale_of(scb, i, sc_c)) : (ok ? static_cast<uint16_t>(st.s[i]) : uint16_t(0));
       uint4* dst = reinterpret_cast<uint4*>(wt + w_dst[i]);
       if (BITS == 4) {
         // word `part` of the group -> 8 halves = one 16-byte chunk
@@ -249,9 +276,9 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
       }
     }
   };
-  auto store_tile = [&](int kt, const StageA& sa, const StageW& st, int s) {
+  auto store_tile = [&](int kt, const StageA& sa, const StageW& st, int s, const ScaleBlock& scb, int sc_c) {
 #pragma unroll
-    for (int part = 0; part < KSTEPS; ++part) store_part(kt, sa, st, s, part);
+    for (int part = 0; part < KSTEPS; ++part) store_part(kt, sa, st, s, part, scb, sc_c);
   };
 
   float16_t acc[TM][TN];
@@ -266,7 +293,8 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
   // MFMAs of the tile in stage s; slice ks of the next tile's store is issued after k-step ks
   // full: every 32-row block of the wave is live (the straight-line form); otherwise blocks >= live are skipped by
   // wave-uniform branches, fragments and all
-  auto mfma_tile = [&](auto full, int s, int kt_store, const StageA& sa_store, const StageW& st_store) {
+  auto mfma_tile = [&](auto full, int s, int kt_store, const StageA& sa_store, const StageW& st_store,
+                       const ScaleBlock& scb, int sc_c) {
     constexpr bool FULL = decltype(full)::value;
     const uint16_t* at = a_tile(s) + (wm0 + frag_row) * LDA + frag_k;
     const uint16_t* wt = w_tile(s) + (wn0 + frag_row) * LDA + frag_k;
@@ -306,7 +334,7 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
             if (ks + 1 < KSTEPS) af[i] = *reinterpret_cast<const half8_t*>(at + i * 32 * LDA + (ks + 1) * 16);
           }
         }
-        store_part(kt_store, sa_store, st_store, s ^ 1, ks);
+        store_part(kt_store, sa_store, st_store, s ^ 1, ks, scb, sc_c);
         __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
       }
     } else {  // fragments of k-step s+1 are read while the MFMAs of step s run
@@ -338,33 +366,58 @@ __global__ __launch_bounds__(64 * (BM / WM) * (BN / WN)) void gemm_pipe_kernel(c
             for (int j = 0; j < TN; ++j) mma(af[cur][i], bf[cur][j], acc[i][j]);
           }
         }
-        store_part(kt_store, sa_store, st_store, s ^ 1, ks);
+        store_part(kt_store, sa_store, st_store, s ^ 1, ks, scb, sc_c);
         __builtin_amdgcn_sched_barrier(0);  // keep the slices where they were written
       }
     }
   };
 
-  // ---- pipeline: tile t in LDS stage t&1, tile t+1 in registers, tile t+2 in flight
   // ---- pipeline: tile t in LDS stage t&1, tiles t+1 .. t+DEPTH-1 in registers, tile t+DEPTH in flight
+  ScaleBlock sc_cur{}, sc_nxt{};  // (SCV) scales of the block of four K tiles being stored, and of the block after it
+  if constexpr (SCV) {
+    load_scales(0, sc_cur);
+    load_scales(1, sc_nxt);
+  }
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) load_a(kt0 + d, ra[d]);
 #pragma unroll
   for (int d = 0; d < WD; ++d) load_w(kt0 + d, rw[d]);
-  store_tile(kt0, ra[0], rw[0], 0);
+  store_tile(kt0, ra[0], rw[0], 0, sc_cur, 0);
   load_a(kt0 + DEPTH, ra[0]);
   load_w(kt0 + WD, rw[0]);
   __syncthreads();
   // (a register stage is refilled right after the MFMA/store block that drains it; a tile past
   //  the end is stored as zeros and adds nothing)
-  auto k_loop = [&](auto full) {
-    for (int kt = kt0; kt < kt1; kt += WD) {
+  constexpr int TRIP = SCV ? 4 : WD;  // K tiles per trip: whole rounds of the register rings, and of a scale block
+  static_assert(TRIP % WD == 0, "a trip walks whole rounds of the register rings");
+  // one trip; SCV: the four tiles stored are 1..3 of block `cur` and the first of block `nxt`, after which `cur` is free
+  // and takes the block after `nxt` (consumed four K tiles from there)
+  auto trip = [&](auto full, int kt, ScaleBlock& cur, ScaleBlock& nxt) __attribute__((always_inline)) {
 #pragma unroll
-      for (int d = 0; d < WD; ++d) {
-        mfma_tile(full, d & 1, kt + d + 1, ra[(d + 1) % DEPTH], rw[(d + 1) % WD]);
-        load_a(kt + d + 1 + DEPTH, ra[(d + 1) % DEPTH]);
-        load_w(kt + d + 1 + WD, rw[(d + 1) % WD]);
-        __syncthreads();
+    for (int d = 0; d < TRIP; ++d) {
+      // the tile stored during this step is kt + d + 1
+      mfma_tile(full, d & 1, kt + d + 1, ra[(d + 1) % DEPTH], rw[(d + 1) % WD], (SCV && d == 3) ? nxt : cur, (d + 1) & 3);
+      load_a(kt + d + 1 + DEPTH, ra[(d + 1) % DEPTH]);
+      load_w(kt + d + 1 + WD, rw[(d + 1) % WD]);
+      if constexpr (SCV) {
+        if (d == 3) load_scales((kt - kt0) / 4 + 2, cur);
       }
+      __syncthreads();
+    }
+  };
+  auto k_loop = [&](auto full) {
+    if constexpr (SCV) {
+      // the two scale blocks swap roles from trip to trip: written out as two trips per round (no register copies, which
+      // the compiler would place right behind the load they wait for); an odd last trip follows the loop (an exit in
+      // the middle of the round would make the loop a join of two paths, where the wait-count insertion drains the queue)
+      int kt = kt0;
+      for (; kt + 2 * TRIP <= kt1; kt += 2 * TRIP) {
+        trip(full, kt, sc_cur, sc_nxt);
+        trip(full, kt + TRIP, sc_nxt, sc_cur);
+      }
+      if (kt < kt1) trip(full, kt, sc_cur, sc_nxt);
+    } else {
+      for (int kt = kt0; kt < kt1; kt += TRIP) trip(full, kt, sc_cur, sc_nxt);
     }
   };
   if (!SKIP || live == TM) k_loop(std::true_type{});
@@ -473,7 +526,11 @@ static hipError_t launch_pipe_cfg(const GemmParams& p, hipStream_t s) {
   constexpr int WD = DEPTH + WX;
   const int nk = (p.ng + 1) / 2;
   const bool whole_rounds = nk % WD == 0 && (p.partial == nullptr || p.kt_per_split % WD == 0);
-  if (p.fast_ok && whole_rounds) return launch_pipe_form<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP, WX, true>(p, s);
+  // q4 reads its scales 16 bytes (four K tiles) at a time there: whole blocks of four K tiles, 16-byte aligned scale rows
+  const bool scale_blocks = BITS != 4 || (nk % 4 == 0 && (p.partial == nullptr || p.kt_per_split % 4 == 0) &&
+                                          (reinterpret_cast<uintptr_t>(p.qs) & 15) == 0 && p.ng % 8 == 0);
+  if (p.fast_ok && whole_rounds && scale_blocks)
+    return launch_pipe_form<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP, WX, true>(p, s);
   return launch_pipe_form<BITS, BM, BN, WM, WN, DEPTH, BF, SKIP, WX, false>(p, s);
 }
 
