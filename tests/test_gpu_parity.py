@@ -660,6 +660,64 @@ def test_gemm_fast_and_general_loop_agree_bit_for_bit(name, m):
     assert_linear_ok(outs[0][1], o.linear_fp32(x, qw, qs, s), x, k, f"fast loop {name} m={m}")
 
 
+@pytest.mark.parametrize("m", [17, 100, 300, 1100])
+@pytest.mark.parametrize("k", [256, 768, 1280, 11008])
+def test_gemm_q4_scale_blocks_odd_and_even_trip_counts(m, k):
+    """q4f16_1, K loop without zero-selects: scales are read 16 bytes (four K tiles) at a time into two register blocks that
+    swap roles from trip to trip, two trips per loop round and a peeled last one.  K of one block (the peeled trip alone),
+    three, five and 43 blocks (odd counts), against the general loop bit for bit and against the oracle; the same launch
+    with a scale tensor that is not 16-byte aligned must take the per-tile scale loads and give the same bits."""
+    s = SCHEMES["q4f16_1"]
+    n = 520 if k <= 1280 else 300
+    x, qw, qs, b = _linear_case(s, m, n, k, 13 * m + k, bias=True)
+    outs = []
+    for fast_loop in (-1, 0):
+        gq._lib.set_option("gemm_fast_loop", fast_loop)
+        try:
+            outs.append((ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b)),
+                         ops.linear(dev(x), dev(qw), dev(qs), 4, 32, None, torch.float32),
+                         ops.linear_silu_mul(dev(x), dev(qw), dev(qs), 4, 32)))
+            if fast_loop == -1 and m > 16:
+                assert gq._lib.last_kernel().startswith("gq::gemm_pipe_kernel<4,") and \
+                    gq._lib.last_kernel().endswith("true>"), gq._lib.last_kernel()
+        finally:
+            gq._lib.set_option("gemm_fast_loop", -1)
+    for a, c in zip(*outs):
+        assert torch.equal(a, c)
+    assert_linear_ok(outs[0][1], o.linear_fp32(x, qw, qs, s), x, k, f"q4 scale blocks m={m} k={k}")
+    # scales at an address that is 2 bytes past a 16-byte boundary
+    flat = torch.zeros(qs.size + 8, dtype=torch.float16, device="cuda")
+    flat[1:1 + qs.size] = dev(qs).reshape(-1)
+    qs_odd = flat[1:1 + qs.size].view(qs.shape)
+    assert qs_odd.data_ptr() % 16 == 2
+    y_odd = ops.linear(dev(x), dev(qw), qs_odd, 4, 32, None, torch.float32)
+    assert gq._lib.last_kernel().endswith("false>"), gq._lib.last_kernel()
+    assert torch.equal(y_odd, outs[0][1])
+
+
+def test_grouped_gemm_q4_scale_blocks_on_ragged_segments():
+    """The grouped tiles with skipped row blocks and the deeper weight ring (four K tiles per trip), K of three scale blocks
+    (a loop round and the peeled trip): against the general loop bit for bit, and the oracle."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(77)
+    ne, n, k = 4, 300, 768
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    ip = np.array([0, 130, 131, 400, 520], np.int32)  # 130, 1, 269 and 120 rows
+    x = rng.standard_normal((520, k)).astype(np.float16)
+    outs = []
+    for fast_loop in (-1, 0):
+        gq._lib.set_option("gemm_fast_loop", fast_loop)
+        try:
+            outs.append(ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), 4, 32))
+            name = gq._lib.last_kernel()
+            assert name.startswith("gq::gemm_pipe_kernel<4,256,") and name.endswith("true>" if fast_loop else "false>"), name
+        finally:
+            gq._lib.set_option("gemm_fast_loop", -1)
+    assert torch.equal(outs[0], outs[1])
+    assert_linear_ok(outs[0], o.dequantize_group_gemm_fp32(x, qw, qs, ip, s), x, k, "grouped scale blocks")
+
+
 @pytest.mark.parametrize("m", [17, 100, 300, 1100, 2048])
 @pytest.mark.parametrize("k", [4096, 1000, 11008, 200, 88])
 def test_gemm_q3_fast_loop_with_a_k_tail(m, k):
