@@ -321,7 +321,8 @@ int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits
       N >= kMaxDim || K >= kMaxDim)
     return 0;
   // only the few-row GEMM (more rows than the GEMV / skinny kernels take, at most 256) splits K
-  if (M <= 16 && bits == 4) return 0;
+  // (q4 at 9..16 rows: the skinny kernel, except on matrices of 40 M to 256 M weights, see linear_impl)
+  if (M <= 16 && bits == 4 && !(M > 8 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return 0;
   if (M <= 8) return 0;
   return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
 }
@@ -340,7 +341,9 @@ int64_t mi355gq_linear_silu_mul_workspace_bytes(int64_t M, int64_t N, int64_t K,
   if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
       N >= kMaxDim || K >= kMaxDim)
     return 0;
-  if (M <= 16 || (N % 64) != 0) return 0;  // GEMV / few-row kernels, or a shape that never splits
+  // GEMV / few-row kernels, or a shape that never splits
+  if (M <= 8 || (N % 64) != 0) return 0;
+  if (M <= 16 && !(bits == 4 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return 0;
   return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
 }
 
@@ -386,6 +389,16 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // q3, 9..16 rows as passes of the quad-row kernel: only on the smaller matrices (see below)
   const bool q3_passes_lose = bits == 3 && M > 8 && gq::options().gemv_variant < 0 && N * K >= (40ll << 20) &&
                               (K & 7) == 0;
+  // q4, 9..16 rows: the skinny kernel on the small projections and on the largest one; in between (40 M to 256 M weights) the
+  // GEMM's 32-row tile is ahead of it since it reads its scales in bulk, provided its split of K has its scratch
+  // (28672 x 4096 at 9 / 12 / 16 rows 30.3 / 32.5 / 33.4 us against 27.5-28.3, 4096 x 14336 21.9-22.0 against 19.5-20.4; while
+  //  4096 x 4096 stays at 9.3 against 11.5, 6144 x 4096 at 12.4-13.2 against 13.1 and 128256 x 4096 at 85-92 against 99)
+  bool q4_skinny_loses = false;
+  if (bits == 4 && M > 8 && M <= 16 && gq::options().gemv_variant < 0 && (K & 7) == 0 && N * K >= (40ll << 20) &&
+      N * K < (256ll << 20)) {
+    const int64_t need = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+    q4_skinny_loses = need == 0 || (workspace != nullptr && workspace_bytes >= need);
+  }
   if (paired) {
     // the regimes of the plain linear: register GEMV up to 2 rows, quad-row kernel up to 8 (q3: 16),
     // skinny kernel up to 16 (q4), else the pipelined GEMM
@@ -408,7 +421,7 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     }
     // (one or two rows never reach the matrix-core kernels in the plain linear either: without a fused form
     //  the caller runs the two steps, and the result stays the same bit for bit)
-    if (e == hipErrorNotSupported && M > 2 && M <= 16 && bits == 4)
+    if (e == hipErrorNotSupported && M > 2 && M <= 16 && bits == 4 && !q4_skinny_loses)
       e = gq::launch_skinny(g, static_cast<int>(M), as_stream(stream));
     if (e == hipErrorNotSupported && M > 2) e = gq::launch_gemm(g, as_stream(stream));
     if (e == hipErrorNotSupported)
@@ -455,7 +468,7 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     a.bits = bits; a.group_size = group_size; a.out_f32 = out_dtype == MI355GQ_F32;
     return hip_result(gq::launch_gemv(a, as_stream(stream)), "gemv launch");
   }
-  if (M <= 16 && bits == 4 && gm != 1) {
+  if (M <= 16 && bits == 4 && gm != 1 && !q4_skinny_loses) {
     if ((gv < 0 && M <= 8) || (gv >= 6 && gv <= 8)) {
       const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
       if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
@@ -925,16 +938,16 @@ static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight
     if (paired) return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul: no fused GEMV for N=%lld K=%lld",
                             (long long)N, (long long)K);
   }
-  // (up to about six rows per expert: 8 experts, 40-48 rows 255-263 us for the whole layer against 285 with the
-  //  skinny kernel; from 64 rows on the order flips)
-  const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;
+  // (up to about seven rows per expert.  Mixtral layer, 8 experts, whole layer in us at 40 / 48 / 56 / 64 / 80 routed rows:
+  //  this kernel 249 / 258 / 262 / 300 / 319, the GEMM's 32-row tiles 270 / 266 / 276 / 272 / 272, the skinny kernel
+  //  282 / 292 / 301 / 307 / 343: the skinny kernel, once the step between the two, is behind both since the GEMM reads
+  //  its scales in bulk, and only a forced variant runs it on expert segments)
+  const int64_t quad_rows = 7 * num_experts > 32 ? 7 * num_experts : 32;
   if (rows <= 128 && gq::options().gemm_variant != 1 && ((gv < 0 && rows <= quad_rows) || (gv >= 6 && gv <= 8))) {
     const hipError_t q = gq::launch_quadrow(g, static_cast<int>(rows), as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "moe quad-row launch");
   }
-  // up to about ten rows per expert; beyond, the GEMM's 32-row tiles are ahead (8 experts: 128 rows 323 vs 401 us
-  // for the whole layer, 96 rows equal)
-  if (rows <= 128 && rows <= 10 * num_experts && bits == 4 && gq::options().gemm_variant != 1) {
+  if (rows <= 128 && rows <= 10 * num_experts && bits == 4 && gq::options().gemm_variant != 1 && gv >= 2 && gv <= 5) {
     const hipError_t e = gq::launch_skinny(g, static_cast<int>(rows), as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "moe skinny launch");
   }
