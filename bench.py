@@ -530,6 +530,23 @@ def main() -> int:
         pk["embedding_take_8192_tokens"] = {"us": round(ms * 1e3, 1), "GB/s": round(8192 * row_bytes / ms / 1e6, 1)}
         extra["packing"] = pk
 
+        # KN-layout tensors (q4f16_0: q_weight [nw, N], q_scale [ng, N]) through mi355gq_linear_kn: the GEMV that streams them
+        # as stored, on rotating copies of the transposed gate_up / o_proj tensors of the first layers
+        kn = {}
+        for name in ("o_proj", "gate_up"):
+            n, k = SHAPES[name]
+            cnt = min(LAYERS, 16)
+            kn_w = [ops.nk_to_kn(layers[i][name][0], layers[i][name][1], k, BITS, G) for i in range(cnt)]
+            for b in (1, 4, 8):
+                xb = torch.randn((b, k), generator=gx, device=dev).half()
+                def sweep(xb=xb, kn_w=kn_w):
+                    for qw_kn, qs_kn in kn_w:
+                        ops.linear_kn(xb, qw_kn, qs_kn, BITS, G)
+                us = timed(sweep, 5, 3, use_graph) * 1e3 / cnt
+                kn[f"{name}_b{b}"] = {"us": round(us, 2), "GB/s": round(gemv_bytes(n, k, b) / (us * 1e-6) / 1e9, 1)}
+            del kn_w
+        extra["kn_layout_gemv"] = kn
+
         # the other model dtypes of the registry (q4bf16_1, q4f32_1) on the gate_up shape: packing,
         # batch-1 GEMV (weight bytes per second) and the M = 2048 GEMM
         other = {}
