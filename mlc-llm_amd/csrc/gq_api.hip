@@ -403,7 +403,10 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     // the regimes of the plain linear: register GEMV up to 2 rows, quad-row kernel up to 8 (q3: 16),
     // skinny kernel up to 16 (q4), else the pipelined GEMM
     hipError_t e = hipErrorNotSupported;
-    if ((M == 2 && (K > 8192 || N * K >= (1ll << 28))) || (M <= 2 && K > 24576))  // as the plain linear
+    const int gvp2 = gq::options().gemv_variant;
+    if (M == 2 && bits == 4 && gq::options().gemm_variant < 0 && (gvp2 < 0 || gvp2 == 9))  // as the plain linear
+      e = gq::launch_quadreg(g, static_cast<int>(M), as_stream(stream));
+    if (e == hipErrorNotSupported && ((M == 2 && (K > 8192 || N * K >= (1ll << 28))) || (M <= 2 && K > 24576)))
       e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     if (e != hipErrorNotSupported) {
       // served above
@@ -435,7 +438,9 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // (... on the smaller matrices: from about 40 M weights on, the GEMM's 32-row tile is ahead of them: gate_up 38
   //  against 42-46 us, down 25.6 against 27-29.5, while qkv stays at 14.7 against 17.1 and o_proj at 10.3 against 15.2)
   // 3..8 rows: the 4x4x4 kernel with x resident in registers, where it applies
-  if (M >= 3 && M <= 8 && gm < 0 && (gv < 0 || gv == 9)) {
+  // (q4 also at 2 rows: 28672 x 4096 13.9 us against 17.1 for the two-row GEMV, 6144 x 4096 5.8 / 6.2, 4096 x 4096 4.9 / 5.2,
+  //  128256 x 4096 52 against 56 for the kernel with x in LDS)
+  if (M >= (bits == 4 ? 2 : 3) && M <= 8 && gm < 0 && (gv < 0 || gv == 9)) {
     const hipError_t q = gq::launch_quadreg(g, static_cast<int>(M), as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "quad-row (registers) launch");
   }

@@ -594,6 +594,34 @@ def test_quadrow_kernel_declines_odd_shapes():
     assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, 256, "quad-row declined")
 
 
+@pytest.mark.parametrize("n,k", [(512, 4096), (1000, 1024), (260, 8192)])
+def test_two_rows_of_q4_take_the_register_fewrow_kernel(n, k):
+    """Two activation rows of a q4f16_1 linear run on the few-row kernel with x in registers (it is ahead of the two-row
+    GEMV on every decode shape); a long K, which that kernel declines, and q3f16_1 keep their kernels.  Plain, with bias and
+    residual, float32 output, and the fused gate/up form against the two steps."""
+    s = SCHEMES["q4f16_1"]
+    x, qw, qs, b = _linear_case(s, 2, n, k, 5 * n + k, bias=True)
+    res = np.random.default_rng(n).standard_normal((2, n)).astype(np.float16)
+    y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32)
+    assert gq._lib.last_kernel().startswith("gq::quadreg_kernel<4,1,"), gq._lib.last_kernel()
+    yb = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b), residual=dev(res))
+    assert gq._lib.last_kernel().startswith("gq::quadreg_kernel<4,1,"), gq._lib.last_kernel()
+    y32 = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, None, torch.float32)
+    ref = o.linear_fp32(x, qw, qs, s)
+    assert_linear_ok(y, ref, x, k, f"two rows {n}x{k}")
+    assert_linear_ok(y32, ref, x, k, f"two rows f32 {n}x{k}")
+    assert_linear_ok(yb, o.linear_fp32(x, qw, qs, s, b) + res.astype(np.float64), x, k, f"two rows bias+residual {n}x{k}")
+    fused = ops.linear_silu_mul(dev(x), dev(qw), dev(qs), 4, 32)
+    assert gq._lib.last_kernel().startswith("gq::quadreg_kernel<4,1,"), gq._lib.last_kernel()
+    assert torch.equal(fused, ops.silu_mul(y))
+    s3 = SCHEMES["q3f16_1"]
+    k3 = k // 40 * 40
+    x3, qw3, qs3, _ = _linear_case(s3, 2, n, k3, n + k3, bias=False)
+    y3 = ops.linear(dev(x3), dev(qw3), dev(qs3), 3, 40)
+    assert "quadreg" not in gq._lib.last_kernel(), gq._lib.last_kernel()
+    assert_linear_ok(y3, o.linear_fp32(x3, qw3, qs3, s3), x3, k3, f"two rows q3 {n}x{k3}")
+
+
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("qp", [1, 2])
 @pytest.mark.parametrize("k", [1024, 14336])
