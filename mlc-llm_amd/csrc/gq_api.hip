@@ -406,7 +406,8 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     const int gvp2 = gq::options().gemv_variant;
     if (M == 2 && bits == 4 && gq::options().gemm_variant < 0 && (gvp2 < 0 || gvp2 == 9))  // as the plain linear
       e = gq::launch_quadreg(g, static_cast<int>(M), as_stream(stream));
-    if (e == hipErrorNotSupported && ((M == 2 && (K > 8192 || N * K >= (1ll << 28))) || (M <= 2 && K > 24576)))
+    if (e == hipErrorNotSupported &&
+        ((M == 2 && (K > 8192 || N * K >= (bits == 3 ? (80ll << 20) : (1ll << 28)))) || (M <= 2 && K > 24576)))
       e = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     if (e != hipErrorNotSupported) {
       // served above
@@ -454,7 +455,8 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // (beyond K = 24 Ki the register GEMV does not apply at all and the quad-row kernel also takes single rows)
   const bool long_k = (M == 2 && K > 8192) || K > 24576;
   // ... and two rows of a very large matrix (lm_head 128256 x 4096: 56 us against 70; 70B gate_up 58 against 66)
-  const bool huge2 = M == 2 && N * K >= (1ll << 28);
+  // (q3f16_1 from about 80 M weights: 22016 x 4096 13.4 us against 14.9, while 12288 x 4096 stays at 9.8 against 10.2)
+  const bool huge2 = M == 2 && N * K >= (bits == 3 ? (80ll << 20) : (1ll << 28));
   if (M <= 2 && gm < 0 && ((gv < 0 && (long_k || huge2)) || (gv >= 6 && gv <= 8))) {
     const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "quad-row launch");
