@@ -948,9 +948,12 @@ static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight
   // (up to about seven rows per expert.  Mixtral layer, 8 experts, whole layer in us at 40 / 48 / 56 / 64 / 80 routed rows:
   //  this kernel 249 / 258 / 262 / 300 / 319, the GEMM's 32-row tiles 270 / 266 / 276 / 272 / 272, the skinny kernel
   //  282 / 292 / 301 / 307 / 343: the skinny kernel, once the step between the two, is behind both since the GEMM reads
-  //  its scales in bulk, and only a forced variant runs it on expert segments)
+  //  its scales in bulk, and only a forced variant runs it on expert segments.  The same rows per expert hold for many
+  //  experts: 64 experts x top-6 (2048 x 1408 projections), whole layer at 144 / 192 / 288 / 384 / 432 routed rows
+  //  112 / 115 / 117 / 127 / 142 us against 137 / 141 / 146 / 143 / 144 on the GEMM's tiles)
   const int64_t quad_rows = 7 * num_experts > 32 ? 7 * num_experts : 32;
-  if (rows <= 128 && gq::options().gemm_variant != 1 && ((gv < 0 && rows <= quad_rows) || (gv >= 6 && gv <= 8))) {
+  if ((rows <= 128 || rows <= 8 * num_experts) && gq::options().gemm_variant != 1 &&
+      ((gv < 0 && rows <= quad_rows) || (gv >= 6 && gv <= 8))) {
     const hipError_t q = gq::launch_quadrow(g, static_cast<int>(rows), as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "moe quad-row launch");
   }

@@ -623,6 +623,30 @@ def test_two_rows_of_q4_take_the_register_fewrow_kernel(n, k):
 
 
 @pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
+def test_grouped_many_experts_more_than_128_rows(name):
+    """Many experts with a few rows each: the few-row kernel serves up to seven rows per expert whatever the total (200 rows
+    over 40 experts here: segments of 0 to 19 rows, i.e. up to three passes), where a cap of 128 rows once sent such calls to
+    the GEMM's mostly empty tiles.  Against the oracle, int32 and int64 indptr."""
+    s = SCHEMES[name]
+    rng = np.random.default_rng(91)
+    ne, n, k = 40, 132, 640 if s.bits == 4 else 640
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    sizes = rng.integers(0, 9, ne)
+    sizes[7] = 19
+    sizes[-1] += 200 - sizes.sum()
+    assert sizes.min() >= 0 and sizes.sum() == 200
+    ip = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    x = rng.standard_normal((200, k)).astype(np.float16)
+    out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip), s.bits, s.group_size)
+    assert gq._lib.last_kernel().startswith("gq::quad_kernel<"), gq._lib.last_kernel()
+    out64 = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ip.astype(np.int64)), s.bits, s.group_size)
+    ref = o.dequantize_group_gemm_fp32(x, qw, qs, ip, s)
+    assert_linear_ok(out, ref, x, k, f"grouped, 40 experts, 200 rows {name}")
+    assert torch.equal(out, out64)
+
+
+@pytest.mark.parametrize("name", ["q4f16_1", "q3f16_1"])
 @pytest.mark.parametrize("qp", [1, 2])
 @pytest.mark.parametrize("k", [1024, 14336])
 def test_quadrow_kernel_grouped(name, qp, k):
