@@ -709,6 +709,25 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
                                          : aligned2(x) && aligned2(q_scale) && aligned2(bias) && aligned2(residual)) &&
                  (out_dtype == MI355GQ_F32 ? aligned4(y) : aligned2(y)),
              "linear_dt: q_weight must be 16-byte aligned, the other tensors naturally aligned");
+  if (model_dtype == MI355GQ_BF16 && M == 2 && bits == 4 && (K & 7) == 0 && aligned16(x) && gq::options().gemm_variant < 0 &&
+      (gq::options().gemv_variant < 0 || gq::options().gemv_variant == 9)) {
+    // two rows of q4: the few-row kernel with x in registers, as in the float16 linear (28672 x 4096 14.6 us against 17.4
+    // for the two-row GEMV, 6144 x 4096 6.1 / 6.4, 4096 x 4096 4.9 / 5.2, 128256 x 4096 51 / 62)
+    gq::GemmArgs g2{};
+    g2.x = static_cast<const uint16_t*>(x);
+    g2.q_weight = static_cast<const uint32_t*>(q_weight);
+    g2.q_scale = static_cast<const uint16_t*>(q_scale);
+    g2.bias = static_cast<const uint16_t*>(bias);
+    g2.residual = static_cast<const uint16_t*>(residual);
+    g2.y = y;
+    g2.indptr = nullptr; g2.indptr_i64 = 0;
+    g2.rows = M; g2.N = N; g2.K = K; g2.num_experts = 1;
+    g2.bits = bits; g2.group_size = group_size; g2.out_f32 = out_dtype == MI355GQ_F32;
+    g2.bf16 = 1;
+    g2.paired = paired;
+    const hipError_t qr = gq::launch_quadreg(g2, static_cast<int>(M), as_stream(stream));
+    if (qr != hipErrorNotSupported) return hip_result(qr, "linear_dt quad-row (registers) launch");
+  }
   if (model_dtype == MI355GQ_BF16 && M <= 2 && aligned16(x)) {
     // one or two rows: the float16 path's register-resident GEMV on v_dot2_f32_bf16
     gq::GemvArgs a{};
@@ -746,8 +765,14 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
     g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
     g.bf16 = 1;
     g.paired = paired;
-    // up to 8 rows: the float16 path's quad-row kernel on the bf16 4x4x4 matrix instruction
+    // up to 8 rows: the float16 path's quad-row kernels on the bf16 4x4x4 matrix instruction (x in registers where that
+    // form applies, as in the float16 linear)
     if (M <= 8) {
+      const int gvq = gq::options().gemv_variant;
+      if (gq::options().gemm_variant < 0 && (gvq < 0 || gvq == 9)) {
+        const hipError_t qr = gq::launch_quadreg(g, static_cast<int>(M), as_stream(stream));
+        if (qr != hipErrorNotSupported) return hip_result(qr, "linear_dt quad-row (registers) launch");
+      }
       const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
       if (q != hipErrorNotSupported) return hip_result(q, "linear_dt quad-row launch");
     }

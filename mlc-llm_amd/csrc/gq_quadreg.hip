@@ -37,6 +37,15 @@ __device__ __forceinline__ float4_t qr_mfma4(uint32_t a0, uint32_t a1, uint32_t 
   return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), c, 0, 0, 0);
 }
 
+// the same blocks on bfloat16 operands (v_mfma_f32_4x4x4_16b_bf16)
+__device__ __forceinline__ float4_t qr_mfma4_bf16(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
+  typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+  typedef short short4_t __attribute__((ext_vector_type(4)));
+  const u2 a = {a0, a1}, b = {b0, b1};
+  return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(short4_t, a), __builtin_bit_cast(short4_t, b), c, 0,
+                                                0, 0);
+}
+
 struct QuadRegTail {
   const uint16_t* bias;      // [N] or null
   const uint16_t* residual;  // [rows, N] or null
@@ -46,8 +55,10 @@ constexpr uint32_t kQrOutF32 = 1u;
 
 // NBQ: batch quads (rows <= 4 * NBQ); U: iterations (of 16 groups) a wave owns; KWL: log2 of the waves that share a quad;
 // MODE 0: plain, 1: bias / residual, 2: fused gate/up form (y is [rows, N / 2]).
+// BF: bfloat16 model (x, scales, bias, residual and the 16-bit result are bfloat16): the unpack shifts every field down to
+// the low bits (a bfloat16 has no room for the x16 trick), every field carries the offset 128 + m, x is not rescaled.
 // The eleven leading arguments (13 dwords) arrive in scalar registers with the wave.
-template <int BITS, int NBQ, int U, int KWL, int MODE>
+template <int BITS, int NBQ, int U, int KWL, int MODE, bool BF = false>
 __global__ __launch_bounds__(KWL == 3 ? 512 : 256) void quadreg_kernel(const uint16_t* x, const uint32_t* qw,
                                                                         const uint16_t* qs, void* y, int rows, int N, int K,
                                                                         uint32_t w0, uint32_t flags, const QuadRegTail t) {
@@ -56,7 +67,12 @@ __global__ __launch_bounds__(KWL == 3 ? 512 : 256) void quadreg_kernel(const uin
   constexpr int KW = 1 << KWL;
   constexpr int WPB = KWL == 3 ? 8 : 4;
   constexpr bool EXTRA = MODE == 1, PAIRED = MODE == 2;
-  constexpr uint32_t kMagic = 0x64006400u;
+  constexpr uint32_t kMagic = BF ? 0x43004300u : 0x64006400u;
+  auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
+  auto to_out = [](float v) { return BF ? f2bf(v) : f2h(v); };
+  auto mm = [](uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
+    return BF ? qr_mfma4_bf16(a0, a1, b0, b1, c) : qr_mfma4(a0, a1, b0, b1, c);
+  };
 
   extern __shared__ float4 part_lds[];  // [wave][round][batch quad][4 lanes]
 
@@ -140,12 +156,20 @@ __global__ __launch_bounds__(KWL == 3 ? 512 : 256) void quadreg_kernel(const uin
         nat[4 * c + 0] = v.x; nat[4 * c + 1] = v.y; nat[4 * c + 2] = v.z; nat[4 * c + 3] = v.w;
       }
       __builtin_amdgcn_wave_barrier();
-      permute_group<BITS, false>(nat, xr);
+      float corr = permute_group<BITS, BF>(nat, xr);
       const half2_t r16 = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
       const half2_t r8 = {static_cast<_Float16>(0.125f), static_cast<_Float16>(0.125f)};
       const half2_t r64 = {static_cast<_Float16>(0.015625f), static_cast<_Float16>(0.015625f)};
-      float corr = 0.f;
-      if constexpr (BITS == 4) {
+      if constexpr (BF) {
+        // (no rescaling: every field was shifted down to the low bits, the offset term is permute_group's)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          if constexpr (BITS == 4) xo[bq][u][c] = make_uint4(xr[4 * c + 0], xr[4 * c + 2], xr[4 * c + 1], xr[4 * c + 3]);
+          else xo[bq][u][c] = make_uint4(xr[5 * c + 0], xr[5 * c + 3], xr[5 * c + 1], xr[5 * c + 4]);
+        }
+        if constexpr (BITS == 3) xo[bq][u][CH - 1] = make_uint4(xr[2], xr[7], xr[12], xr[17]);
+      } else if constexpr (BITS == 4) {
+        corr = 0.f;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           xr[4 * c + 1] = as_u32(as_half2(xr[4 * c + 1]) * r16);
@@ -157,6 +181,7 @@ __global__ __launch_bounds__(KWL == 3 ? 512 : 256) void quadreg_kernel(const uin
           xo[bq][u][c] = make_uint4(xr[4 * c + 0], xr[4 * c + 2], xr[4 * c + 1], xr[4 * c + 3]);
         }
       } else {
+        corr = 0.f;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           xr[5 * c + 1] = as_u32(as_half2(xr[5 * c + 1]) * r8);
@@ -182,24 +207,24 @@ __global__ __launch_bounds__(KWL == 3 ? 512 : 256) void quadreg_kernel(const uin
     if constexpr (EXTRA) {
       if (t.bias != nullptr) {
         const uint2 bb = *reinterpret_cast<const uint2*>(t.bias + quad * 4);
-        v[0] += h2f(static_cast<uint16_t>(bb.x & 0xffffu)); v[1] += h2f(static_cast<uint16_t>(bb.x >> 16));
-        v[2] += h2f(static_cast<uint16_t>(bb.y & 0xffffu)); v[3] += h2f(static_cast<uint16_t>(bb.y >> 16));
+        v[0] += to_f32(static_cast<uint16_t>(bb.x & 0xffffu)); v[1] += to_f32(static_cast<uint16_t>(bb.x >> 16));
+        v[2] += to_f32(static_cast<uint16_t>(bb.y & 0xffffu)); v[3] += to_f32(static_cast<uint16_t>(bb.y >> 16));
       }
       if (t.residual != nullptr) {
         const uint2 rr = *reinterpret_cast<const uint2*>(t.residual + oi);
-        v[0] += h2f(static_cast<uint16_t>(rr.x & 0xffffu)); v[1] += h2f(static_cast<uint16_t>(rr.x >> 16));
-        v[2] += h2f(static_cast<uint16_t>(rr.y & 0xffffu)); v[3] += h2f(static_cast<uint16_t>(rr.y >> 16));
+        v[0] += to_f32(static_cast<uint16_t>(rr.x & 0xffffu)); v[1] += to_f32(static_cast<uint16_t>(rr.x >> 16));
+        v[2] += to_f32(static_cast<uint16_t>(rr.y & 0xffffu)); v[3] += to_f32(static_cast<uint16_t>(rr.y >> 16));
       }
     }
     if constexpr (PAIRED) {
       *reinterpret_cast<uint32_t*>(static_cast<uint16_t*>(y) + (oi >> 1)) =
-          static_cast<uint32_t>(silu_mul_h(v[0], v[1])) | (static_cast<uint32_t>(silu_mul_h(v[2], v[3])) << 16);
+          static_cast<uint32_t>(silu_mul_t<BF>(v[0], v[1])) | (static_cast<uint32_t>(silu_mul_t<BF>(v[2], v[3])) << 16);
     } else if (out_f32) {
       *reinterpret_cast<float4*>(static_cast<float*>(y) + oi) = make_float4(v[0], v[1], v[2], v[3]);
     } else {
       uint2 o;
-      o.x = static_cast<uint32_t>(f2h(v[0])) | (static_cast<uint32_t>(f2h(v[1])) << 16);
-      o.y = static_cast<uint32_t>(f2h(v[2])) | (static_cast<uint32_t>(f2h(v[3])) << 16);
+      o.x = static_cast<uint32_t>(to_out(v[0])) | (static_cast<uint32_t>(to_out(v[1])) << 16);
+      o.y = static_cast<uint32_t>(to_out(v[2])) | (static_cast<uint32_t>(to_out(v[3])) << 16);
       *reinterpret_cast<uint2*>(static_cast<uint16_t*>(y) + oi) = o;
     }
   };
@@ -222,21 +247,32 @@ __global__ __launch_bounds__(KWL == 3 ? 512 : 256) void quadreg_kernel(const uin
           const uint32_t w8 = w[d] >> 8;
           lo[d][0] = and_or_c(w[d], 0x000f000fu, kMagic);
           lo[d][1] = and_or_c(w8, 0x000f000fu, kMagic);
-          hi[d][0] = and_or_c(w[d], 0x00f000f0u, kMagic);
-          hi[d][1] = and_or_c(w8, 0x00f000f0u, kMagic);
+          if constexpr (BF) {
+            hi[d][0] = and_or_c(w[d] >> 4, 0x000f000fu, kMagic);
+            hi[d][1] = and_or_c(w[d] >> 12, 0x000f000fu, kMagic);
+          } else {
+            hi[d][0] = and_or_c(w[d], 0x00f000f0u, kMagic);
+            hi[d][1] = and_or_c(w8, 0x00f000f0u, kMagic);
+          }
         } else {
           // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
           const uint32_t tt = (w[d] & 0x0000ffffu) | ((w[d] << 1) & 0xffff0000u);
           const uint32_t t9 = tt >> 9;
           lo[d][0] = and_or_c(tt, 0x00070007u, kMagic);   // fields (0,5)
           lo[d][1] = and_or_c(t9, 0x00070007u, kMagic);   // fields (3,8)
-          hi[d][0] = and_or_c(tt, 0x00380038u, kMagic);   // fields (1,6) x 8
-          hi[d][1] = and_or_c(t9, 0x00380038u, kMagic);   // fields (4,9) x 8
-          a64[d >> 1][d & 1] = and_or_c(tt, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+          if constexpr (BF) {
+            hi[d][0] = and_or_c(tt >> 3, 0x00070007u, kMagic);   // fields (1,6)
+            hi[d][1] = and_or_c(tt >> 12, 0x00070007u, kMagic);  // fields (4,9)
+            a64[d >> 1][d & 1] = and_or_c(tt >> 6, 0x00070007u, kMagic);  // fields (2,7)
+          } else {
+            hi[d][0] = and_or_c(tt, 0x00380038u, kMagic);   // fields (1,6) x 8
+            hi[d][1] = and_or_c(t9, 0x00380038u, kMagic);   // fields (4,9) x 8
+            a64[d >> 1][d & 1] = and_or_c(tt, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+          }
         }
       }
       // the four rows' scales of this block: lane 4b+i holds row i's (converted once, then broadcast)
-      const uint32_t s32 = __builtin_bit_cast(uint32_t, h2f(static_cast<uint16_t>(sc[u])));
+      const uint32_t s32 = __builtin_bit_cast(uint32_t, to_f32(static_cast<uint16_t>(sc[u])));
       float sv[4];
       sv[0] = __builtin_bit_cast(float, qr_dpp_u<0x00>(s32));
       sv[1] = __builtin_bit_cast(float, qr_dpp_u<0x55>(s32));
@@ -249,12 +285,12 @@ __global__ __launch_bounds__(KWL == 3 ? 512 : 256) void quadreg_kernel(const uin
         float4_t tacc = {c, c, c, c};
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          tacc = qr_mfma4(lo[d][0], lo[d][1], xo[bq][u][d].x, xo[bq][u][d].y, tacc);
-          tacc = qr_mfma4(hi[d][0], hi[d][1], xo[bq][u][d].z, xo[bq][u][d].w, tacc);
+          tacc = mm(lo[d][0], lo[d][1], xo[bq][u][d].x, xo[bq][u][d].y, tacc);
+          tacc = mm(hi[d][0], hi[d][1], xo[bq][u][d].z, xo[bq][u][d].w, tacc);
         }
         if constexpr (BITS == 3) {
-          tacc = qr_mfma4(a64[0][0], a64[0][1], xo[bq][u][CH - 1].x, xo[bq][u][CH - 1].y, tacc);
-          tacc = qr_mfma4(a64[1][0], a64[1][1], xo[bq][u][CH - 1].z, xo[bq][u][CH - 1].w, tacc);
+          tacc = mm(a64[0][0], a64[0][1], xo[bq][u][CH - 1].x, xo[bq][u][CH - 1].y, tacc);
+          tacc = mm(a64[1][0], a64[1][1], xo[bq][u][CH - 1].z, xo[bq][u][CH - 1].w, tacc);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[bq][i] = fmaf(sv[i], tacc[i], acc[bq][i]);
@@ -324,7 +360,7 @@ __global__ __launch_bounds__(KWL == 3 ? 512 : 256) void quadreg_kernel(const uin
   }
 }
 
-template <int BITS, int NBQ, int U, int KWL>
+template <int BITS, int NBQ, int U, int KWL, bool BF>
 hipError_t launch_mode(const GemmArgs& a, int nwalkers, int rounds, hipStream_t s) {
   constexpr int WPB = KWL == 3 ? 8 : 4;
   const int mode = a.paired ? 2 : ((a.bias != nullptr || a.residual != nullptr) ? 1 : 0);
@@ -336,10 +372,10 @@ hipError_t launch_mode(const GemmArgs& a, int nwalkers, int rounds, hipStream_t 
   const uint32_t w0 = static_cast<uint32_t>(nwalkers) | static_cast<uint32_t>(rounds) << 16;
   const uint32_t flags = a.out_f32 ? kQrOutF32 : 0u;
   const QuadRegTail t{a.bias, a.residual};
-  note_kernel("gq::quadreg_kernel<%d,%d,%d,%d,%d>", BITS, NBQ, U, KWL, mode);
+  note_kernel("gq::quadreg_kernel<%d,%d,%d,%d,%d%s>", BITS, NBQ, U, KWL, mode, BF ? ",true" : "");
   const int rows = static_cast<int>(a.rows), N = static_cast<int>(a.N), K = static_cast<int>(a.K);
 #define GQ_QR_LAUNCH(MODE_) \
-  hipLaunchKernelGGL((quadreg_kernel<BITS, NBQ, U, KWL, MODE_>), grid, block, lds, s, a.x, a.q_weight, a.q_scale, a.y, \
+  hipLaunchKernelGGL((quadreg_kernel<BITS, NBQ, U, KWL, MODE_, BF>), grid, block, lds, s, a.x, a.q_weight, a.q_scale, a.y, \
                      rows, N, K, w0, flags, t)
   if (mode == 2) GQ_QR_LAUNCH(2);
   else if (mode == 1) GQ_QR_LAUNCH(1);
@@ -348,10 +384,10 @@ hipError_t launch_mode(const GemmArgs& a, int nwalkers, int rounds, hipStream_t 
   return hipGetLastError();
 }
 
-template <int BITS, int NBQ>
+template <int BITS, int NBQ, bool BF = false>
 hipError_t launch_shape(const GemmArgs& a, int U, int kwl, int nwalkers, int rounds, hipStream_t s) {
 #define GQ_QR_CASE(U_, KWL_) \
-  if (U == U_ && kwl == KWL_) return launch_mode<BITS, NBQ, U_, KWL_>(a, nwalkers, rounds, s);
+  if (U == U_ && kwl == KWL_) return launch_mode<BITS, NBQ, U_, KWL_, BF>(a, nwalkers, rounds, s);
   GQ_QR_CASE(1, 0) GQ_QR_CASE(2, 0) GQ_QR_CASE(1, 1) GQ_QR_CASE(2, 1)
   GQ_QR_CASE(1, 2) GQ_QR_CASE(2, 2) GQ_QR_CASE(1, 3) GQ_QR_CASE(2, 3)
   if constexpr (NBQ == 1) {  // (two batch quads stop at two iterations per wave)
@@ -364,13 +400,14 @@ hipError_t launch_shape(const GemmArgs& a, int U, int kwl, int nwalkers, int rou
 
 }  // namespace
 
-// Plain linears (no expert segments, no gather) of up to 8 float16 activation rows with N % 4 == 0 and K % 8 == 0
+// Plain linears (no expert segments, no gather) of up to 8 float16 (q4: also bfloat16) activation rows with N % 4 == 0 and K % 8 == 0
 // and K of at most 16 iterations of 16 groups (q4: K <= 8192; q3: K <= 10240); hipErrorNotSupported otherwise.
 // Tuning overrides: quad_ksplit (log2 of the waves per quad), gemv_waves (waves in all).
 hipError_t launch_quadreg(const GemmArgs& a, int rows_max, hipStream_t s) {
   if (a.bits != 4 && a.bits != 3) return hipErrorNotSupported;
   const int G = a.bits == 4 ? 32 : 40;
-  if (a.group_size != G || a.indptr != nullptr || a.x_rows != nullptr || a.bf16) return hipErrorNotSupported;
+  if (a.group_size != G || a.indptr != nullptr || a.x_rows != nullptr) return hipErrorNotSupported;
+  if (a.bf16 && a.bits != 4) return hipErrorNotSupported;  // (the bfloat16 instances: q4bf16_*)
   if (a.rows == 0 || a.N == 0) return hipSuccess;
   if (rows_max > 8 || a.rows > 8 || (a.N & 3) != 0 || (a.K & 7) != 0 || a.K == 0) return hipErrorNotSupported;
   if ((reinterpret_cast<uintptr_t>(a.x) & 15) != 0 || (reinterpret_cast<uintptr_t>(a.y) & 15) != 0 ||
@@ -412,6 +449,7 @@ hipError_t launch_quadreg(const GemmArgs& a, int rows_max, hipStream_t s) {
   if (nwalkers > nquads) nwalkers = nquads;
   const int rounds = (nquads + nwalkers - 1) / nwalkers;
   nwalkers = (nquads + rounds - 1) / rounds;  // even share of quads per walker
+  if (a.bf16) return nbq == 1 ? launch_shape<4, 1, true>(a, U, kwl, nwalkers, rounds, s) : launch_shape<4, 2, true>(a, U, kwl, nwalkers, rounds, s);
   if (a.bits == 4) return nbq == 1 ? launch_shape<4, 1>(a, U, kwl, nwalkers, rounds, s) : launch_shape<4, 2>(a, U, kwl, nwalkers, rounds, s);
   return nbq == 1 ? launch_shape<3, 1>(a, U, kwl, nwalkers, rounds, s) : launch_shape<3, 2>(a, U, kwl, nwalkers, rounds, s);
 }

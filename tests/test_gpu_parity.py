@@ -1660,6 +1660,38 @@ def test_linear_other_model_dtypes(model_dtype, bits_name, m, n, k):
     assert np.array_equal(_carrier(y), o.round_to(y32.cpu().numpy(), model_dtype))
 
 
+@pytest.mark.parametrize("m", [3, 4, 8])
+@pytest.mark.parametrize("n,k", [(512, 4096), (132, 1000), (260, 8192)])
+def test_bfloat16_few_rows_take_the_register_fewrow_kernel(m, n, k):
+    """q4bf16_1 at 3..8 rows: the few-row kernel with x in registers on the bf16 4x4x4 matrix instruction (K up to 8192).
+    Float32 output exact against the unrounded-weight product (the kernel scales each group's integer dot product), the
+    bfloat16 output the same numbers rounded once; bias and residual; the fused gate/up form against the two steps."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(m * 100 + n)
+    w32 = o.round_to((rng.standard_normal((n, k)) * 0.05).astype(np.float32), "bfloat16")
+    x32 = o.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    b32 = o.round_to(rng.standard_normal(n).astype(np.float32), "bfloat16")
+    r32 = o.round_to(rng.standard_normal((m, n)).astype(np.float32), "bfloat16")
+    qw_ref, qs_ref = o.quantize_dt(w32, s, "bfloat16")
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).to(torch.bfloat16).to(DEV)
+    x, b, r = (torch.from_numpy(a).to(torch.bfloat16).to(DEV) for a in (x32, b32, r32))
+    y32 = ops.linear(x, qw, qs, 4, 32, None, out_dtype=torch.float32)
+    kern = gq._lib.last_kernel()
+    assert kern.startswith("gq::quadreg_kernel<4,") and kern.endswith(",true>"), kern
+    exact = o.linear_dt_fp64(x32, qw_ref, qs_ref, s, "bfloat16", None, unrounded_weights=True)
+    den = np.linalg.norm(exact)
+    assert np.linalg.norm(y32.double().cpu().numpy() - exact) / den <= 5e-6 + 1e-7 * np.sqrt(k)
+    y = ops.linear(x, qw, qs, 4, 32)
+    assert y.dtype == torch.bfloat16 and np.array_equal(_carrier(y), o.round_to(y32.cpu().numpy(), "bfloat16"))
+    yb = ops.linear(x, qw, qs, 4, 32, b, out_dtype=torch.float32, residual=r)
+    assert gq._lib.last_kernel().startswith("gq::quadreg_kernel<4,") and gq._lib.last_kernel().endswith("1,true>")
+    want = exact + b32.astype(np.float64) + r32.astype(np.float64)
+    assert np.linalg.norm(yb.double().cpu().numpy() - want) / np.linalg.norm(want) <= 5e-6 + 1e-7 * np.sqrt(k)
+    fused = ops.linear_silu_mul(x, qw, qs, 4, 32)
+    assert gq._lib.last_kernel().endswith("2,true>"), gq._lib.last_kernel()
+    assert torch.equal(fused, ops.silu_mul(y))
+
+
 def _assert_dt_matmul_ok(y: torch.Tensor, ref: np.ndarray, x32: np.ndarray, k: int, model_dtype: str, what=""):
     """Output in the model dtype against the exact product of the same operands: the fp32 accumulation
     (relative error of a sum of k terms grows like sqrt(k) * 2^-24) plus, for bfloat16, the one rounding of
