@@ -195,6 +195,178 @@ __global__ __launch_bounds__(256) void gemv_kn_kernel(const KnParams p) {
   }
 }
 
+// ---- up to 8 rows on the 4x4x4 matrix instruction, q4.  v_mfma_f32_4x4x4_16b_f16 multiplies 16 independent blocks;
+// here a block is 4 neighbouring columns (A rows) x 4 activation rows (B columns) and the 16 blocks of a wave are 16
+// different column quads of ONE quantisation group, so nothing is summed across lanes: lane (block q, j) ends with
+// y[row j][its block's four columns].  A lane loads one 128-bit piece of one word row (the same word of four columns; a
+// wave instruction covers 4 word rows x 256 contiguous bytes); the four lanes of a block then hold word rows 4g .. 4g + 3 of
+// the same four columns, and a 4 x 4 transpose inside the lane quad (two exchange steps) leaves every lane with the
+// four words, i.e. the whole group, of ONE column - the operand the NK few-row kernels load directly (gq_quadrow.hip),
+// whose unpack, operand classes and offset term this kernel shares.  x of the workgroup's K slice sits in LDS in operand
+// order; the 16 blocks read the same address (a broadcast).  A wave owns 64 columns and walks every group of the slice.
+typedef uint32_t kn_u2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float4_t kn_mfma4(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1, float4_t c) {
+  const kn_u2 a = {a0, a1}, b = {b0, b1};
+  return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, a), __builtin_bit_cast(half4_t, b), c, 0, 0, 0);
+}
+template <int CTRL>
+__device__ __forceinline__ uint32_t kn_dpp(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xf, 0xf, true));
+}
+// lane i of a quad holds (m[i][0..3]); afterwards it holds (m[0..3][i])
+__device__ __forceinline__ uint4 kn_quad_transpose(uint4 v, int lane) {
+  const bool odd = (lane & 1) != 0, hi = (lane & 2) != 0;
+  uint32_t r = kn_dpp<0xB1>(odd ? v.x : v.y);  // quad_perm [1,0,3,2]
+  if (odd) v.x = r; else v.y = r;
+  r = kn_dpp<0xB1>(odd ? v.z : v.w);
+  if (odd) v.z = r; else v.w = r;
+  r = kn_dpp<0x4E>(hi ? v.x : v.z);  // quad_perm [2,3,0,1]
+  if (hi) v.x = r; else v.z = r;
+  r = kn_dpp<0x4E>(hi ? v.y : v.w);
+  if (hi) v.y = r; else v.w = r;
+  return v;
+}
+
+// grid (column blocks of 256, K slices); NBQ batch quads (rows <= 4 * NBQ)
+template <int NBQ>
+__global__ __launch_bounds__(256) void kn_quad_kernel(const KnParams p, int rows) {
+  constexpr int G = 32, CH = 4, HP = 16, U = 2;
+  constexpr uint32_t kMagic = 0x64006400u;
+  extern __shared__ uint4 smem[];  // x of the slice in operand order [4 NBQ][gps][4 words], then the offset terms
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane & 3, q = lane >> 2;
+  const int g0 = blockIdx.y * p.gps;
+  const int gcount = min(p.gps, p.ng - g0);
+  float* const corr_lds = reinterpret_cast<float*>(smem + 4 * NBQ * p.gps * CH);
+
+  // ---- the first items' loads go out ahead of the staging of x
+  const int nq = blockIdx.x * 256 + wave * 64 + 4 * q;  // first column of this lane's quad
+  const bool col_ok = nq < p.N;                       // (N % 4 == 0: a quad is all inside or all outside)
+  const int nc = col_ok ? nq : 0;
+  uint4 wa[U], wb[U];
+  uint32_t sa[U], sb[U];
+  auto issue = [&](int gl, uint4 (&wn)[U], uint32_t (&sn)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int g = g0 + min(gl + u, gcount - 1);
+      wn[u] = *reinterpret_cast<const uint4*>(p.qw + static_cast<int64_t>(4 * g + li) * p.N + nc);
+      sn[u] = p.qs[static_cast<int64_t>(g) * p.N + nc + li];
+    }
+  };
+  issue(0, wa, sa);
+  issue(U, wb, sb);
+
+  // ---- stage this slice of x: one thread per (row, group); pair order, the odd fields' activations divided by 16 and
+  //      the offset term formed from the divided values (as gq_quadrow.hip)
+  for (int t = threadIdx.x; t < 4 * NBQ * gcount; t += 256) {
+    const int b = t / gcount, gl = t - b * gcount;
+    const int k0 = (g0 + gl) * G;
+    uint32_t nat[HP], xr[HP];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int k = k0 + 8 * c;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (b < rows && k + 8 <= p.K) v = *reinterpret_cast<const uint4*>(p.x + static_cast<int64_t>(b) * p.K + k);
+      nat[4 * c] = v.x; nat[4 * c + 1] = v.y; nat[4 * c + 2] = v.z; nat[4 * c + 3] = v.w;
+    }
+    permute_group<4>(nat, xr);
+    const half2_t r16 = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
+    float corr = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      xr[4 * c + 1] = as_u32(as_half2(xr[4 * c + 1]) * r16);
+      xr[4 * c + 3] = as_u32(as_half2(xr[4 * c + 3]) * r16);
+      corr = dot2(xr[4 * c + 0], 0x64076407u /* (1031, 1031) */, corr);
+      corr = dot2(xr[4 * c + 1], 0x64706470u /* (16 * 71, ..) */, corr);
+      corr = dot2(xr[4 * c + 2], 0x64076407u, corr);
+      corr = dot2(xr[4 * c + 3], 0x64706470u, corr);
+      smem[(b * p.gps + gl) * CH + c] = make_uint4(xr[4 * c + 0], xr[4 * c + 2], xr[4 * c + 1], xr[4 * c + 3]);
+    }
+    corr_lds[b * p.gps + gl] = -corr;
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // (the path around the staging loop would otherwise make the walk's first waits conservative)
+  __syncthreads();
+
+  float4_t acc[NBQ];
+#pragma unroll
+  for (int bq = 0; bq < NBQ; ++bq) acc[bq] = float4_t{0.f, 0.f, 0.f, 0.f};
+  auto compute = [&](int gl, const uint4 (&wc)[U], const uint32_t (&sc)[U]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bool live = gl + u < gcount;  // (uniform)
+      const int g = min(gl + u, gcount - 1);
+      const uint4 wt = kn_quad_transpose(wc[u], lane);  // the group's four words of column nq + li
+      const uint32_t w[4] = {wt.x, wt.y, wt.z, wt.w};
+      uint32_t lo[4][2], hi[4][2];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const uint32_t w8 = w[d] >> 8;
+        lo[d][0] = and_or_c(w[d], 0x000f000fu, kMagic);
+        lo[d][1] = and_or_c(w8, 0x000f000fu, kMagic);
+        hi[d][0] = and_or_c(w[d], 0x00f000f0u, kMagic);
+        hi[d][1] = and_or_c(w8, 0x00f000f0u, kMagic);
+      }
+      // the four columns' scales of this block: lane 4q + i holds column i's (a group past the slice adds nothing)
+      const uint32_t s32 = live ? __builtin_bit_cast(uint32_t, h2f(static_cast<uint16_t>(sc[u]))) : 0u;
+      float sv[4];
+      sv[0] = __builtin_bit_cast(float, kn_dpp<0x00>(s32));
+      sv[1] = __builtin_bit_cast(float, kn_dpp<0x55>(s32));
+      sv[2] = __builtin_bit_cast(float, kn_dpp<0xAA>(s32));
+      sv[3] = __builtin_bit_cast(float, kn_dpp<0xFF>(s32));
+#pragma unroll
+      for (int bq = 0; bq < NBQ; ++bq) {
+        const int e = (4 * bq + li) * p.gps + g;  // (activation row 4 bq + li, group): the same in every block
+        const float c = corr_lds[e];
+        float4_t tacc = {c, c, c, c};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint4 xv = smem[e * CH + d];
+          tacc = kn_mfma4(lo[d][0], lo[d][1], xv.x, xv.y, tacc);
+          tacc = kn_mfma4(hi[d][0], hi[d][1], xv.z, xv.w, tacc);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[bq][i] = fmaf(sv[i], tacc[i], acc[bq][i]);
+      }
+    }
+  };
+  for (int gl = 0; gl < gcount; gl += 2 * U) {
+    compute(gl, wa, sa);
+    issue(gl + 2 * U, wa, sa);
+    __builtin_amdgcn_sched_barrier(0);
+    compute(gl + U, wb, sb);  // past the slice: scale 0, adds nothing
+    issue(gl + 3 * U, wb, sb);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // lane (q, li): results of activation row 4 bq + li for the quad's four columns
+  if (!col_ok) return;
+#pragma unroll
+  for (int bq = 0; bq < NBQ; ++bq) {
+    const int b = 4 * bq + li;
+    if (b >= rows) continue;
+    float v[4] = {acc[bq][0], acc[bq][1], acc[bq][2], acc[bq][3]};
+    if (p.slices > 1) {  // fp32 partial sums [slice][row][N]; the reduction adds the bias
+      *reinterpret_cast<float4*>(static_cast<float*>(p.y) + (static_cast<int64_t>(blockIdx.y) * rows + b) * p.N + nq) =
+          make_float4(v[0], v[1], v[2], v[3]);
+      continue;
+    }
+    if (p.bias != nullptr) {
+      const uint2 bb = *reinterpret_cast<const uint2*>(p.bias + nq);
+      v[0] += h2f(static_cast<uint16_t>(bb.x & 0xffffu)); v[1] += h2f(static_cast<uint16_t>(bb.x >> 16));
+      v[2] += h2f(static_cast<uint16_t>(bb.y & 0xffffu)); v[3] += h2f(static_cast<uint16_t>(bb.y >> 16));
+    }
+    const int64_t oi = static_cast<int64_t>(b) * p.N + nq;
+    if (p.out_f32) {
+      *reinterpret_cast<float4*>(static_cast<float*>(p.y) + oi) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+      uint2 o;
+      o.x = static_cast<uint32_t>(f2h(v[0])) | (static_cast<uint32_t>(f2h(v[1])) << 16);
+      o.y = static_cast<uint32_t>(f2h(v[2])) | (static_cast<uint32_t>(f2h(v[3])) << 16);
+      *reinterpret_cast<uint2*>(static_cast<uint16_t*>(p.y) + oi) = o;
+    }
+  }
+}
+
 // y[i] = sum over slices of part[s][i] (+ bias), cast; i over M * N
 __global__ __launch_bounds__(256) void kn_reduce_kernel(const float* __restrict__ part, int slices, int64_t count, int N,
                                                         const uint16_t* __restrict__ bias, void* y, int out_f32) {
@@ -221,10 +393,56 @@ int kn_slices(int64_t M, int64_t N, int ng) {
   return static_cast<int>(slices);
 }
 
+// the matrix-instruction form above: q4, 16-byte aligned rows of x, 1..8 rows (a single row too: 4096 x 4096 7.8 us against
+// 8.6 for the GEMV below, 4096 x 14336 15.8 / 19.1, 28672 x 4096 18.0 / 18.3, 6144 x 4096 9.3 / 9.1); tuning override
+// gemv_variant 0: never
+hipError_t launch_kn_quad(const KnParams& p0, int M, void* workspace, int64_t workspace_bytes, void* y,
+                          const uint16_t* bias, hipStream_t s) {
+  const int gv = options().gemv_variant;
+  if (!p0.x_vec || gv == 0) return hipErrorNotSupported;
+  const int nbq = M <= 4 ? 1 : 2;
+  KnParams p = p0;
+  // K slices: about 512 workgroups, whole groups, the slice's x (68 bytes per row and group) within 48 KiB of LDS
+  const int64_t colblocks = (p.N + 255) / 256;
+  // (measured at 4 rows, graph replay over rotating weights: 4096 x 4096 at 8 / 16 / 32 slices 8.1 / 7.8 / 9.7 us, 6144 x 4096
+  //  at 6 / 8 / 11 / 22 slices 10.4 / 9.0 / 9.3 / 11.1, 4096 x 14336 at 8 / 16 / 32 19.2 / 16.0 / 20.3, 28672 x 4096 at 2 / 3 / 4 / 7
+  //  19.9 / 19.0 / 17.7 / 20.7: about one workgroup per CU, a little more where the column blocks alone are a third of that)
+  const int64_t want = options().gemv_waves > 0 ? options().gemv_waves / 4 : (colblocks >= 64 ? 448 : 256);
+  int64_t slices = (want + colblocks - 1) / colblocks;
+  if (slices > (p.ng + 3) / 4) slices = (p.ng + 3) / 4;
+  if (slices < 1) slices = 1;
+  const int64_t gmax = (48 * 1024) / (4 * nbq * 68);
+  if (slices < (p.ng + gmax - 1) / gmax) slices = (p.ng + gmax - 1) / gmax;
+  const int64_t part_bytes = slices * M * p.N * 4;
+  if (slices > 1 && (workspace == nullptr || workspace_bytes < part_bytes)) {
+    if (p.ng > gmax) return hipErrorNotSupported;
+    slices = 1;
+  }
+  p.gps = static_cast<int>((p.ng + slices - 1) / slices);
+  p.slices = (p.ng + p.gps - 1) / p.gps;
+  p.y = p.slices > 1 ? workspace : y;
+  p.bias = p.slices > 1 ? nullptr : bias;
+  const size_t lds = static_cast<size_t>(4 * nbq) * p.gps * 68;
+  const dim3 grid(static_cast<unsigned>(colblocks), static_cast<unsigned>(p.slices));
+  note_kernel("gq::kn_quad_kernel<%d> slices=%d", nbq, p.slices);
+  if (nbq == 1) hipLaunchKernelGGL(kn_quad_kernel<1>, grid, dim3(256), lds, s, p, M);
+  else hipLaunchKernelGGL(kn_quad_kernel<2>, grid, dim3(256), lds, s, p, M);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || p.slices == 1) return e;
+  const int64_t count = static_cast<int64_t>(M) * p.N;
+  hipLaunchKernelGGL(kn_reduce_kernel, dim3(static_cast<unsigned>((count + 255) / 256)), dim3(256), 0, s,
+                     static_cast<const float*>(workspace), p.slices, count, p.N, bias, y, p.out_f32);
+  return hipGetLastError();
+}
+
 template <int BITS>
 hipError_t launch_gemv_kn_bits(const KnParams& p0, int M, void* workspace, int64_t workspace_bytes, void* y,
                                const uint16_t* bias, hipStream_t s) {
   constexpr int CH = GemvTraits<BITS>::CH;
+  if constexpr (BITS == 4) {
+    const hipError_t e = launch_kn_quad(p0, M, workspace, workspace_bytes, y, bias, s);
+    if (e != hipErrorNotSupported) return e;
+  }
   KnParams p = p0;
   int slices = kn_slices(M, p.N, p.ng);
   const int64_t part_bytes = static_cast<int64_t>(slices) * M * p.N * 4;
@@ -282,8 +500,18 @@ int64_t gemv_kn_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits) {
   const int G = bits == 4 ? 32 : 40;
   const int ng = static_cast<int>((K + G - 1) / G);
   if (M < 1 || M > 8 || ng == 0) return 0;
-  const int slices = kn_slices(M, N, ng);
-  return slices > 1 ? static_cast<int64_t>(slices) * M * N * 4 : 0;
+  int64_t slices = kn_slices(M, N, ng);
+  if (bits == 4 && M >= 1) {  // the few-row form's split (launch_kn_quad)
+    const int nbq = M <= 4 ? 1 : 2;
+    const int64_t colblocks = (N + 255) / 256;
+    int64_t sq = ((colblocks >= 64 ? 448 : 256) + colblocks - 1) / colblocks;
+    if (sq > (ng + 3) / 4) sq = (ng + 3) / 4;
+    if (sq < 1) sq = 1;
+    const int64_t gmax = (48 * 1024) / (4 * nbq * 68);
+    if (sq < (ng + gmax - 1) / gmax) sq = (ng + gmax - 1) / gmax;
+    if (sq > slices) slices = sq;
+  }
+  return slices > 1 ? slices * M * N * 4 : 0;
 }
 
 // M <= 8 float16 rows, N % 4 == 0; hipErrorNotSupported otherwise (the caller transposes and runs the NK kernels)

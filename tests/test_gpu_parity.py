@@ -1042,7 +1042,18 @@ def test_kn_entry_points(name, n, k):
         ref = o.linear_fp32(x, qw[cols], qs[cols], s)
         y = ops.linear_kn(dev(x), qw_kn, qs_kn, s.bits, s.group_size)
         kern = gq._lib.last_kernel()
-        assert kern.startswith("gq::gemv_kn_kernel") == (m <= 8 and n % 4 == 0), (kern, m, n)
+        # q4 with 16-byte rows of x: the 4x4x4 matrix-instruction form; else the GEMV
+        quad = s.bits == 4 and m <= 8 and n % 4 == 0 and k % 8 == 0
+        assert kern.startswith("gq::kn_quad_kernel") == quad, (kern, m, n)
+        assert kern.startswith("gq::gemv_kn_kernel") == (m <= 8 and n % 4 == 0 and not quad), (kern, m, n)
+        if quad:  # ... against the GEMV on the same tensors (forced), and also for a single row (forced)
+            gq._lib.set_option("gemv_variant", 0)
+            try:
+                y_gemv = ops.linear_kn(dev(x), qw_kn, qs_kn, s.bits, s.group_size)
+                assert gq._lib.last_kernel().startswith("gq::gemv_kn_kernel")
+            finally:
+                gq._lib.set_option("gemv_variant", -1)
+            assert (y.float() - y_gemv.float()).abs().max().item() <= 2e-2 * max(1.0, y_gemv.float().abs().max().item())
         assert_linear_ok(y[:, torch.from_numpy(cols).to(DEV)], ref, x, k, f"linear_kn {name} {m}x{n}x{k} [{kern}]")
         y32 = ops.linear_kn(dev(x), qw_kn, qs_kn, s.bits, s.group_size, dev(b), torch.float32)
         assert_linear_ok(y32[:, torch.from_numpy(cols).to(DEV)], ref + b[cols].astype(np.float64), x, k,
