@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void gemv_kn_kernel(const KnParams p) {
   }
 }
 
-// ---- up to 8 rows on the 4x4x4 matrix instruction, q4.  v_mfma_f32_4x4x4_16b_f16 multiplies 16 independent blocks;
+// ---- up to 8 rows on the 4x4x4 matrix instruction.  v_mfma_f32_4x4x4_16b_f16 multiplies 16 independent blocks;
 // here a block is 4 neighbouring columns (A rows) x 4 activation rows (B columns) and the 16 blocks of a wave are 16
 // different column quads of ONE quantisation group, so nothing is summed across lanes: lane (block q, j) ends with
 // y[row j][its block's four columns].  A lane loads one 128-bit piece of one word row (the same word of four columns; a
@@ -228,9 +228,9 @@ __device__ __forceinline__ uint4 kn_quad_transpose(uint4 v, int lane) {
 }
 
 // grid (column blocks of 256, K slices); NBQ batch quads (rows <= 4 * NBQ)
-template <int NBQ>
+template <int BITS, int NBQ>
 __global__ __launch_bounds__(256) void kn_quad_kernel(const KnParams p, int rows) {
-  constexpr int G = 32, CH = 4, HP = 16, U = 2;
+  constexpr int G = GemvTraits<BITS>::G, CH = GemvTraits<BITS>::CH, HP = G / 2, U = 2;
   constexpr uint32_t kMagic = 0x64006400u;
   extern __shared__ uint4 smem[];  // x of the slice in operand order [4 NBQ][gps][4 words], then the offset terms
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -269,18 +269,38 @@ __global__ __launch_bounds__(256) void kn_quad_kernel(const KnParams p, int rows
       if (b < rows && k + 8 <= p.K) v = *reinterpret_cast<const uint4*>(p.x + static_cast<int64_t>(b) * p.K + k);
       nat[4 * c] = v.x; nat[4 * c + 1] = v.y; nat[4 * c + 2] = v.z; nat[4 * c + 3] = v.w;
     }
-    permute_group<4>(nat, xr);
+    permute_group<BITS>(nat, xr);
     const half2_t r16 = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
+    const half2_t r8 = {static_cast<_Float16>(0.125f), static_cast<_Float16>(0.125f)};
+    const half2_t r64 = {static_cast<_Float16>(0.015625f), static_cast<_Float16>(0.015625f)};
     float corr = 0.f;
+    if constexpr (BITS == 4) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      xr[4 * c + 1] = as_u32(as_half2(xr[4 * c + 1]) * r16);
-      xr[4 * c + 3] = as_u32(as_half2(xr[4 * c + 3]) * r16);
-      corr = dot2(xr[4 * c + 0], 0x64076407u /* (1031, 1031) */, corr);
-      corr = dot2(xr[4 * c + 1], 0x64706470u /* (16 * 71, ..) */, corr);
-      corr = dot2(xr[4 * c + 2], 0x64076407u, corr);
-      corr = dot2(xr[4 * c + 3], 0x64706470u, corr);
-      smem[(b * p.gps + gl) * CH + c] = make_uint4(xr[4 * c + 0], xr[4 * c + 2], xr[4 * c + 1], xr[4 * c + 3]);
+      for (int c = 0; c < 4; ++c) {
+        xr[4 * c + 1] = as_u32(as_half2(xr[4 * c + 1]) * r16);
+        xr[4 * c + 3] = as_u32(as_half2(xr[4 * c + 3]) * r16);
+        corr = dot2(xr[4 * c + 0], 0x64076407u /* (1031, 1031) */, corr);
+        corr = dot2(xr[4 * c + 1], 0x64706470u /* (16 * 71, ..) */, corr);
+        corr = dot2(xr[4 * c + 2], 0x64076407u, corr);
+        corr = dot2(xr[4 * c + 3], 0x64706470u, corr);
+        smem[(b * p.gps + gl) * CH + c] = make_uint4(xr[4 * c + 0], xr[4 * c + 2], xr[4 * c + 1], xr[4 * c + 3]);
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        xr[5 * c + 1] = as_u32(as_half2(xr[5 * c + 1]) * r8);
+        xr[5 * c + 4] = as_u32(as_half2(xr[5 * c + 4]) * r8);
+        xr[5 * c + 2] = as_u32(as_half2(xr[5 * c + 2]) * r64);
+        corr = dot2(xr[5 * c + 0], 0x64036403u /* (1027, 1027) */, corr);
+        corr = dot2(xr[5 * c + 1], 0x64186418u /* (8 * 131, ..) */, corr);
+        corr = dot2(xr[5 * c + 2], 0x64c064c0u /* (64 * 19, ..) */, corr);
+        corr = dot2(xr[5 * c + 3], 0x64036403u, corr);
+        corr = dot2(xr[5 * c + 4], 0x64186418u, corr);
+        // word c: fields (0,5)(3,8) meet the x1 operands, (1,6)(4,9) the x8 operands
+        smem[(b * p.gps + gl) * CH + c] = make_uint4(xr[5 * c + 0], xr[5 * c + 3], xr[5 * c + 1], xr[5 * c + 4]);
+      }
+      // fields (2,7) of all four words, the x64 class, share the fifth word
+      smem[(b * p.gps + gl) * CH + 4] = make_uint4(xr[2], xr[7], xr[12], xr[17]);
     }
     corr_lds[b * p.gps + gl] = -corr;
   }
@@ -297,14 +317,25 @@ __global__ __launch_bounds__(256) void kn_quad_kernel(const KnParams p, int rows
       const int g = min(gl + u, gcount - 1);
       const uint4 wt = kn_quad_transpose(wc[u], lane);  // the group's four words of column nq + li
       const uint32_t w[4] = {wt.x, wt.y, wt.z, wt.w};
-      uint32_t lo[4][2], hi[4][2];
+      uint32_t lo[4][2], hi[4][2], a64[2][2];
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
-        const uint32_t w8 = w[d] >> 8;
-        lo[d][0] = and_or_c(w[d], 0x000f000fu, kMagic);
-        lo[d][1] = and_or_c(w8, 0x000f000fu, kMagic);
-        hi[d][0] = and_or_c(w[d], 0x00f000f0u, kMagic);
-        hi[d][1] = and_or_c(w8, 0x00f000f0u, kMagic);
+        if constexpr (BITS == 4) {
+          const uint32_t w8 = w[d] >> 8;
+          lo[d][0] = and_or_c(w[d], 0x000f000fu, kMagic);
+          lo[d][1] = and_or_c(w8, 0x000f000fu, kMagic);
+          hi[d][0] = and_or_c(w[d], 0x00f000f0u, kMagic);
+          hi[d][1] = and_or_c(w8, 0x00f000f0u, kMagic);
+        } else {
+          // low half keeps fields 0-4, high half gets fields 5-9 aligned to bit 16
+          const uint32_t tt = (w[d] & 0x0000ffffu) | ((w[d] << 1) & 0xffff0000u);
+          const uint32_t t9 = tt >> 9;
+          lo[d][0] = and_or_c(tt, 0x00070007u, kMagic);   // fields (0,5)
+          lo[d][1] = and_or_c(t9, 0x00070007u, kMagic);   // fields (3,8)
+          hi[d][0] = and_or_c(tt, 0x00380038u, kMagic);   // fields (1,6) x 8
+          hi[d][1] = and_or_c(t9, 0x00380038u, kMagic);   // fields (4,9) x 8
+          a64[d >> 1][d & 1] = and_or_c(tt, 0x01c001c0u, kMagic);  // fields (2,7) x 64
+        }
       }
       // the four columns' scales of this block: lane 4q + i holds column i's (a group past the slice adds nothing)
       const uint32_t s32 = live ? __builtin_bit_cast(uint32_t, h2f(static_cast<uint16_t>(sc[u]))) : 0u;
@@ -323,6 +354,11 @@ __global__ __launch_bounds__(256) void kn_quad_kernel(const KnParams p, int rows
           const uint4 xv = smem[e * CH + d];
           tacc = kn_mfma4(lo[d][0], lo[d][1], xv.x, xv.y, tacc);
           tacc = kn_mfma4(hi[d][0], hi[d][1], xv.z, xv.w, tacc);
+        }
+        if constexpr (BITS == 3) {
+          const uint4 xv = smem[e * CH + 4];
+          tacc = kn_mfma4(a64[0][0], a64[0][1], xv.x, xv.y, tacc);
+          tacc = kn_mfma4(a64[1][0], a64[1][1], xv.z, xv.w, tacc);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[bq][i] = fmaf(sv[i], tacc[i], acc[bq][i]);
@@ -393,13 +429,19 @@ int kn_slices(int64_t M, int64_t N, int ng) {
   return static_cast<int>(slices);
 }
 
-// the matrix-instruction form above: q4, 16-byte aligned rows of x, 1..8 rows (a single row too: 4096 x 4096 7.8 us against
+// the matrix-instruction form above: 16-byte aligned rows of x, 1..8 rows (a single row too: 4096 x 4096 7.8 us against
 // 8.6 for the GEMV below, 4096 x 14336 15.8 / 19.1, 28672 x 4096 18.0 / 18.3, 6144 x 4096 9.3 / 9.1); tuning override
 // gemv_variant 0: never
+template <int BITS>
 hipError_t launch_kn_quad(const KnParams& p0, int M, void* workspace, int64_t workspace_bytes, void* y,
                           const uint16_t* bias, hipStream_t s) {
+  constexpr int kRowGroup = GemvTraits<BITS>::CH * 16 + 4;  // bytes of LDS per (activation row, group)
   const int gv = options().gemv_variant;
   if (!p0.x_vec || gv == 0) return hipErrorNotSupported;
+  // (a single row of q3 over a large matrix: the GEMV's dot products are ahead, 4096 x 14336 12.1 us against 13.0,
+  //  28672 x 4096 16.9 / 17.9; below that and from two rows on this form, 4096 x 4096 7.7 against 8.2, four rows of
+  //  28672 x 4096 17.2 against 25.8, eight 21.0 / 38.9)
+  if (BITS == 3 && M == 1 && gv < 0 && static_cast<int64_t>(p0.N) * p0.K >= (40ll << 20)) return hipErrorNotSupported;
   const int nbq = M <= 4 ? 1 : 2;
   KnParams p = p0;
   // K slices: about 512 workgroups, whole groups, the slice's x (68 bytes per row and group) within 48 KiB of LDS
@@ -411,7 +453,7 @@ hipError_t launch_kn_quad(const KnParams& p0, int M, void* workspace, int64_t wo
   int64_t slices = (want + colblocks - 1) / colblocks;
   if (slices > (p.ng + 3) / 4) slices = (p.ng + 3) / 4;
   if (slices < 1) slices = 1;
-  const int64_t gmax = (48 * 1024) / (4 * nbq * 68);
+  const int64_t gmax = (48 * 1024) / (4 * nbq * kRowGroup);
   if (slices < (p.ng + gmax - 1) / gmax) slices = (p.ng + gmax - 1) / gmax;
   const int64_t part_bytes = slices * M * p.N * 4;
   if (slices > 1 && (workspace == nullptr || workspace_bytes < part_bytes)) {
@@ -422,11 +464,11 @@ hipError_t launch_kn_quad(const KnParams& p0, int M, void* workspace, int64_t wo
   p.slices = (p.ng + p.gps - 1) / p.gps;
   p.y = p.slices > 1 ? workspace : y;
   p.bias = p.slices > 1 ? nullptr : bias;
-  const size_t lds = static_cast<size_t>(4 * nbq) * p.gps * 68;
+  const size_t lds = static_cast<size_t>(4 * nbq) * p.gps * kRowGroup;
   const dim3 grid(static_cast<unsigned>(colblocks), static_cast<unsigned>(p.slices));
-  note_kernel("gq::kn_quad_kernel<%d> slices=%d", nbq, p.slices);
-  if (nbq == 1) hipLaunchKernelGGL(kn_quad_kernel<1>, grid, dim3(256), lds, s, p, M);
-  else hipLaunchKernelGGL(kn_quad_kernel<2>, grid, dim3(256), lds, s, p, M);
+  note_kernel("gq::kn_quad_kernel<%d,%d> slices=%d", BITS, nbq, p.slices);
+  if (nbq == 1) hipLaunchKernelGGL((kn_quad_kernel<BITS, 1>), grid, dim3(256), lds, s, p, M);
+  else hipLaunchKernelGGL((kn_quad_kernel<BITS, 2>), grid, dim3(256), lds, s, p, M);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || p.slices == 1) return e;
   const int64_t count = static_cast<int64_t>(M) * p.N;
@@ -439,8 +481,8 @@ template <int BITS>
 hipError_t launch_gemv_kn_bits(const KnParams& p0, int M, void* workspace, int64_t workspace_bytes, void* y,
                                const uint16_t* bias, hipStream_t s) {
   constexpr int CH = GemvTraits<BITS>::CH;
-  if constexpr (BITS == 4) {
-    const hipError_t e = launch_kn_quad(p0, M, workspace, workspace_bytes, y, bias, s);
+  {
+    const hipError_t e = launch_kn_quad<BITS>(p0, M, workspace, workspace_bytes, y, bias, s);
     if (e != hipErrorNotSupported) return e;
   }
   KnParams p = p0;
@@ -501,13 +543,14 @@ int64_t gemv_kn_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits) {
   const int ng = static_cast<int>((K + G - 1) / G);
   if (M < 1 || M > 8 || ng == 0) return 0;
   int64_t slices = kn_slices(M, N, ng);
-  if (bits == 4 && M >= 1) {  // the few-row form's split (launch_kn_quad)
+  if (M >= 1) {  // the matrix-instruction form's split (launch_kn_quad)
     const int nbq = M <= 4 ? 1 : 2;
+    const int64_t row_group = (bits == 4 ? 4 : 5) * 16 + 4;
     const int64_t colblocks = (N + 255) / 256;
     int64_t sq = ((colblocks >= 64 ? 448 : 256) + colblocks - 1) / colblocks;
     if (sq > (ng + 3) / 4) sq = (ng + 3) / 4;
     if (sq < 1) sq = 1;
-    const int64_t gmax = (48 * 1024) / (4 * nbq * 68);
+    const int64_t gmax = (48 * 1024) / (4 * nbq * row_group);
     if (sq < (ng + gmax - 1) / gmax) sq = (ng + gmax - 1) / gmax;
     if (sq > slices) slices = sq;
   }

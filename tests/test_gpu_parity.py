@@ -1042,8 +1042,8 @@ def test_kn_entry_points(name, n, k):
         ref = o.linear_fp32(x, qw[cols], qs[cols], s)
         y = ops.linear_kn(dev(x), qw_kn, qs_kn, s.bits, s.group_size)
         kern = gq._lib.last_kernel()
-        # q4 with 16-byte rows of x: the 4x4x4 matrix-instruction form; else the GEMV
-        quad = s.bits == 4 and m <= 8 and n % 4 == 0 and k % 8 == 0
+        # 16-byte rows of x: the 4x4x4 matrix-instruction form; else the GEMV (and for one row of q3 over a large matrix)
+        quad = m <= 8 and n % 4 == 0 and k % 8 == 0 and not (s.bits == 3 and m == 1 and n * k >= 40 << 20)
         assert kern.startswith("gq::kn_quad_kernel") == quad, (kern, m, n)
         assert kern.startswith("gq::gemv_kn_kernel") == (m <= 8 and n % 4 == 0 and not quad), (kern, m, n)
         if quad:  # ... against the GEMV on the same tensors (forced), and also for a single row (forced)
