@@ -399,6 +399,18 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     const int64_t need = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
     q4_skinny_loses = need == 0 || (workspace != nullptr && workspace_bytes >= need);
   }
+  // q4, 9..16 rows of a K that one phase covers (up to 4096), from about 24 M weights on: the kernel that multiplies
+  // unscaled weight operands and scales the matrix instruction's result (28672 x 4096 at 9 / 16 rows 20.0 / 20.3 us
+  // against 27.8-28.1 for the GEMM's 32-row tile, 6144 x 4096 10.4 / 10.9 against 12.2 / 13.1 for the skinny kernel;
+  // 4096 x 4096 stays with the skinny kernel, 9.0-9.4 either way, and a longer K with the GEMM's tiles, 4096 x 14336
+  // 26-27 against 20).  The same test for the plain and the fused gate/up form: both must add in the same order.
+  const bool mid_rows = bits == 4 && M > 8 && M <= 16 && gq::options().gemm_variant < 0 &&
+                        (gq::options().gemv_variant < 0 || gq::options().gemv_variant == 10) && (K & 255) == 0 &&
+                        K <= 4096 && (N & 31) == 0 && N * K >= (24ll << 20);
+  if (mid_rows || gq::options().gemv_variant == 10) {  // (10: forced, whatever the shape)
+    const hipError_t e = gq::launch_midrow(g, static_cast<int>(M), as_stream(stream));
+    if (e != hipErrorNotSupported) return hip_result(e, "mid-row launch");
+  }
   if (paired) {
     // the regimes of the plain linear: register GEMV up to 2 rows, quad-row kernel up to 8 (q3: 16),
     // skinny kernel up to 16 (q4), else the pipelined GEMM
@@ -976,6 +988,17 @@ static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight
   //  its scales in bulk, and only a forced variant runs it on expert segments.  The same rows per expert hold for many
   //  experts: 64 experts x top-6 (2048 x 1408 projections), whole layer at 144 / 192 / 288 / 384 / 432 routed rows
   //  112 / 115 / 117 / 127 / 142 us against 137 / 141 / 146 / 143 / 144 on the GEMM's tiles)
+  // Between the quad-row kernel's few rows per expert and the GEMM's tiles: four to eight rows per expert on average (so that
+  // hardly a segment holds more than the 16 rows of one pass), up to 16 experts, q4, K % 256 == 0: the kernel that scales
+  // the matrix instruction's result.  Mixtral layer (8 experts x top-2) at 24 / 32 tokens: e1_e3 156 / 170 -> 115 / 117 us,
+  // e2 102 / 106 -> 76 / 78; at 16 tokens equal to the quad-row kernel (118 / 75 against 122 / 74), at 40 and beyond a
+  // segment of 17 rows or more takes a second pass over its expert's weights and the GEMM's tiles are ahead (203 / 131
+  // against 166 / 104).
+  if (gv == 10 || (gv < 0 && bits == 4 && gq::options().gemm_variant < 0 && num_experts <= 16 && rows > 4 * num_experts &&
+                   rows <= 8 * num_experts)) {
+    const hipError_t q = gq::launch_midrow(g, 16, as_stream(stream));
+    if (q != hipErrorNotSupported) return hip_result(q, "moe mid-row launch");
+  }
   const int64_t quad_rows = 7 * num_experts > 32 ? 7 * num_experts : 32;
   if ((rows <= 128 || rows <= 8 * num_experts) && gq::options().gemm_variant != 1 &&
       ((gv < 0 && rows <= quad_rows) || (gv >= 6 && gv <= 8))) {

@@ -97,6 +97,11 @@ hipError_t launch_quadrow(const GemmArgs& a, int rows_max, hipStream_t s);
 // hipErrorNotSupported when the shape does not fit.
 hipError_t launch_quadreg(const GemmArgs& a, int rows_max, hipStream_t s);
 
+// 16x16x32 matrix instruction on unscaled weight operands, the scale applied per group afterwards (q4f16_1, K % 256 == 0;
+// plain linears and expert segments); rows_max bounds the rows of any one segment; hipErrorNotSupported when the shape
+// does not fit.
+hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s);
+
 // KN-layout tensors (q_weight [nw, N], q_scale [ng, N]): both tensors transposed in one call (src_rows_w / src_rows_s rows
 // of src_cols columns each), the dequantisation to [K, N], and the decode GEMV (M <= 8, N % 4 == 0) with its workspace
 hipError_t launch_kn_transpose(const uint32_t* qw_src, const uint16_t* qs_src, int64_t src_rows_w, int64_t src_rows_s,

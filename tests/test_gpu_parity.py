@@ -358,6 +358,103 @@ def test_skinny_kernel_forms(mode, m, n, k):
     assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"skinny mode {mode} fp32 out")
 
 
+@pytest.mark.parametrize("form", [-1, 2, 4])  # ring of two tiles with the offsets kept, four without, three with
+@pytest.mark.parametrize("m", [1, 9, 16, 17, 40])  # one pass, a full one, and rows that take two and three passes
+@pytest.mark.parametrize("n,k", [(96, 256), (1000, 1024), (520, 4096), (72, 8192), (256, 14336), (16, 512)])
+def test_midrow_kernel(form, m, n, k):
+    """The kernel that feeds the matrix instruction unscaled weight operands and scales its result, forced (it runs by
+    default on large matrices at 9..16 rows): K of one to sixteen wave shares and of several phases, a last tile of
+    fewer than 16 weight rows, bias, residual and float32 output."""
+    s = SCHEMES["q4f16_1"]
+    x, qw, qs, b = _linear_case(s, m, n, k, 13 * m + n + k + form, bias=True)
+    res = np.random.default_rng(m + n).standard_normal((m, n)).astype(np.float16)
+    gq._lib.set_option("gemv_variant", 10)
+    gq._lib.set_option("gemv_rows_per_wave", form)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b))
+        kern = gq._lib.last_kernel()
+        y32 = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, None, torch.float32)
+        yr = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, dev(b), residual=dev(res))
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+        gq._lib.set_option("gemv_rows_per_wave", -1)
+    if k > 4096 and form == 2:  # (several phases exist for the default instance only: the shape falls through)
+        assert not kern.startswith("gq::midrow_kernel"), kern
+    else:
+        assert kern.startswith("gq::midrow_kernel<"), kern
+    ref = o.linear_fp32(x, qw, qs, s, b)
+    assert_linear_ok(y, ref, x, k, f"mid-row form {form} {m}x{n}x{k} [{kern}]")
+    assert_linear_ok(y32, ref - b.astype(np.float64), x, k, f"mid-row form {form} fp32 out")
+    assert_linear_ok(yr, ref + res.astype(np.float64), x, k, f"mid-row form {form} residual")
+
+
+@pytest.mark.parametrize("m", [9, 12, 16])
+@pytest.mark.parametrize("n,k", [(6144, 4096), (28672, 4096)])
+def test_midrow_kernel_is_the_default_on_large_matrices(m, n, k):
+    """9..16 rows of q4 on matrices of 24 M weights or more with K up to 4096: the default dispatch, against the oracle on
+    a sample of the columns; the fused gate/up form takes the same kernel and equals linear + silu_mul bit for bit."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(seed_of("midrow", m, n, k))
+    qw = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    qs = (rng.random((n, k // 32)) * 0.02 + 0.001).astype(np.float16)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    cols = np.unique(np.concatenate([[0, 1, n // 2, n - 1], rng.integers(0, n, 300)]))
+    y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32)
+    assert gq._lib.last_kernel().startswith("gq::midrow_kernel<"), gq._lib.last_kernel()
+    assert_linear_ok(y[:, torch.from_numpy(cols).to(DEV)], o.linear_fp32(x, qw[cols], qs[cols], s), x, k, f"mid-row {m}x{n}x{k}")
+    fused = ops.linear_silu_mul(dev(x), dev(qw), dev(qs), 4, 32)
+    assert gq._lib.last_kernel().startswith("gq::midrow_kernel<"), gq._lib.last_kernel()
+    assert torch.equal(fused, ops.silu_mul(y))
+
+
+@pytest.mark.parametrize("k", [1024, 4096, 14336])
+@pytest.mark.parametrize("paired", [False, True])
+def test_midrow_kernel_grouped(k, paired):
+    """Expert segments: an empty expert, one of a single row, one of 16 rows (a full pass) and one of 19 (two passes), the
+    gather of the activation rows folded in, int32 and int64 indptr; the fused gate/up form against linear + silu_mul of
+    the same kernel, bit for bit."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(63 + k)
+    ne, n = 5, 224
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    ip = np.array([0, 1, 1, 17, 36, 40], np.int32)
+    xs = rng.standard_normal((25, k)).astype(np.float16)
+    rows = rng.integers(0, 25, 40).astype(np.int32)
+    x = xs[rows]
+    gq._lib.set_option("gemv_variant", 10)
+    try:
+        out = ops.moe_experts(dev(xs), dev(rows), dev(qw), dev(qs), dev(ip), 4, 32, silu_mul_halves=paired)
+        kern = gq._lib.last_kernel()
+        out64 = ops.moe_experts(dev(x), None, dev(qw), dev(qs), dev(ip.astype(np.int64)), 4, 32, silu_mul_halves=paired)
+        plain = ops.moe_experts(dev(x), None, dev(qw), dev(qs), dev(ip), 4, 32)
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+    assert kern.startswith("gq::midrow_kernel<"), kern
+    assert torch.equal(out, out64)
+    assert_linear_ok(plain, o.dequantize_group_gemm_fp32(x, qw, qs, ip, s), x, k, f"grouped mid-row k={k}")
+    if paired:
+        assert torch.equal(out, ops.silu_mul(plain))
+    else:
+        assert torch.equal(out, plain)
+
+
+def test_midrow_kernel_is_the_default_between_few_rows_and_tiles():
+    """Four to eight rows per expert on average (up to 16 experts, q4): the default dispatch of the grouped matmul."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(64)
+    ne, n, k = 8, 96, 512
+    w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    ip = np.array([0, 4, 10, 15, 28, 37, 42, 55, 63], np.int32)
+    for rows, want in ((32, False), (33, True), (63, True)):
+        ipr = np.minimum(ip, rows).astype(np.int32)
+        x = rng.standard_normal((rows, k)).astype(np.float16)
+        out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ipr), 4, 32)
+        assert gq._lib.last_kernel().startswith("gq::midrow_kernel<") == want, (rows, gq._lib.last_kernel())
+        assert_linear_ok(out, o.dequantize_group_gemm_fp32(x, qw, qs, ipr, s), x, k, f"grouped, {rows} rows over 8 experts")
+
+
 @pytest.mark.parametrize("mode", [2, 3, 4])
 def test_skinny_kernel_forms_grouped(mode):
     s = SCHEMES["q4f16_1"]
