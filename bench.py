@@ -16,7 +16,7 @@ The JSON line also carries
                 over the 32 distinct gate_up weight sets;
   cpu_baseline  the C restatement of the reference's fused dequantize-matmul loop nest on the
                 host cores (a reported baseline, not the target);
-  extra         per-shape GEMV GB/s for batch 1/4/8 and prefill GEMM TFLOP/s at M = 2048.
+  extra         per-shape GEMV GB/s for batch 1/4/8/16 and prefill GEMM TFLOP/s at M = 2048.
 """
 
 from __future__ import annotations
@@ -201,9 +201,9 @@ def main() -> int:
         layers.append({name: make_weight(n, k, 1000 * layer + i) for i, (name, (n, k)) in enumerate(SHAPES.items())})
     lm_head = make_weight(*LM_HEAD, 999_999)
     gx = torch.Generator(device=dev).manual_seed(1)
-    x_in = {k: torch.randn((8, k), generator=gx, device=dev).half() for k in (4096, 14336)}
-    outs = {name: torch.empty((8, n), dtype=torch.float16, device=dev) for name, (n, _) in SHAPES.items()}
-    out_lm = torch.empty((8, LM_HEAD[0]), dtype=torch.float16, device=dev)
+    x_in = {k: torch.randn((16, k), generator=gx, device=dev).half() for k in (4096, 14336)}
+    outs = {name: torch.empty((16, n), dtype=torch.float16, device=dev) for name, (n, _) in SHAPES.items()}
+    out_lm = torch.empty((16, LM_HEAD[0]), dtype=torch.float16, device=dev)
     torch.cuda.synchronize()
 
     def run_linear(name, qw, qs, b, out):
@@ -246,7 +246,7 @@ def main() -> int:
     for name, (n, k) in list(SHAPES.items()) + [("lm_head", LM_HEAD)]:
         qw_, qs_ = lm_head if name == "lm_head" else layers[0][name]
         out_ = out_lm if name == "lm_head" else outs[name]
-        for b in (1, 4, 8):
+        for b in (1, 4, 8, 16):
             run_linear(name, qw_, qs_, b, out_)
             sampled_parity(f"{name} B={b}", out_[:b], x_in[k][:b], qw_, qs_, s4)
     run_linear("gate_up", *layers[0]["gate_up"], 1, outs["gate_up"])
@@ -345,12 +345,12 @@ def main() -> int:
                             "step_time_over_probe_step_time": round(ms_step / ms_probe_step, 3)},
     }
 
-    # ---------------------------------------------------------------- extra: per shape, batch 1/4/8, prefill GEMM
+    # ---------------------------------------------------------------- extra: per shape, batch 1/4/8/16, prefill GEMM
     extra = {}
     if not args.skip_extra:
         per_shape = {}
         for name, (n, k) in list(SHAPES.items()) + [("lm_head", LM_HEAD)]:
-            for b in (1, 4, 8):
+            for b in (1, 4, 8, 16):
                 if name == "lm_head":
                     # 8 launches on the one lm_head (296 MB: larger than the 256 MB infinity cache)
                     def sweep(b=b):
@@ -494,7 +494,7 @@ def main() -> int:
             del w13, w2
         g2 = torch.Generator(device=dev).manual_seed(2)
         moe_res = {}
-        for t in (1, 16, 512):
+        for t in (1, 16, 32, 512):
             xt = torch.randn((1, t, 4096), generator=gx, device=dev).half()
             logits = torch.randn((t, 8), generator=g2, device=dev).half()
             ms = timed(lambda: moe(xt, logits), 10, 2, use_graph)
