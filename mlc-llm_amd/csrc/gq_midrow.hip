@@ -165,22 +165,30 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
           sv[0] = v.x; sv[1] = v.y;
         }
       };
+      // ---- this wave's share of x goes out first (it is needed first, and loads retire in issue order): lane (i = c, j)
+      //      of batch tile bt reads x[row 16 bt + i][32 g + 8 j .. + 7]
+      uint4 xraw[NBT][U];
+      bool x_ok[NBT];
+#pragma unroll
+      for (int bt = 0; bt < NBT; ++bt) {
+        const int b = pass_lo + 16 * bt + c;
+        x_ok[bt] = k_live && b < seg_hi;
+        const uint16_t* xrow = p.x + x_row(p.x_rows, p.x_src_rows, x_ok[bt] ? b : seg_lo) * p.K + ga * 32 + 8 * j;
+#pragma unroll
+        for (int u = 0; u < U; ++u) xraw[bt][u] = *reinterpret_cast<const uint4*>(xrow + u * 32);
+      }
 #pragma unroll
       for (int r = 0; r < RT; ++r) issue(r, w[r], sc[r]);
 
-      // ---- this wave's share of x, in operand order: lane (i = c, j) of batch tile bt holds
-      //      x[row 16 bt + i][32 g + 8 j .. + 7] as (x0, x4) (x2, x6) (x1, x5) / 16 (x3, x7) / 16
+      // ---- x in operand order, (x0, x4) (x2, x6) (x1, x5) / 16 (x3, x7) / 16, and the offset terms
       mid_u4 xa[NBT][U];
       float4_t cc[KEEP_C ? NBT : 1][KEEP_C ? U : 1];
 #pragma unroll
       for (int bt = 0; bt < NBT; ++bt) {
-        const int b = pass_lo + 16 * bt + c;
-        const bool ok = k_live && b < seg_hi;
-        const uint16_t* xrow = p.x + x_row(p.x_rows, p.x_src_rows, ok ? b : seg_lo) * p.K + ga * 32 + 8 * j;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-          uint4 v = *reinterpret_cast<const uint4*>(xrow + u * 32);
-          if (!ok) v = make_uint4(0, 0, 0, 0);
+          uint4 v = xraw[bt][u];
+          if (!x_ok[bt]) v = make_uint4(0, 0, 0, 0);
           xa[bt][u][0] = __builtin_amdgcn_perm(v.z, v.x, kLoLo);
           xa[bt][u][1] = __builtin_amdgcn_perm(v.w, v.y, kLoLo);
           xa[bt][u][2] = as_u32(as_half2(__builtin_amdgcn_perm(v.z, v.x, kHiHi)) * r16);
