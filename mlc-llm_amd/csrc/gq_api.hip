@@ -993,10 +993,14 @@ static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight
   // the matrix instruction's result.  Mixtral layer (8 experts x top-2) at 24 / 32 tokens: e1_e3 156 / 170 -> 115 / 117 us,
   // e2 102 / 106 -> 76 / 78; at 16 tokens equal to the quad-row kernel (118 / 75 against 122 / 74), at 40 and beyond a
   // segment of 17 rows or more takes a second pass over its expert's weights and the GEMM's tiles are ahead (203 / 131
-  // against 166 / 104).
-  if (gv == 10 || (gv < 0 && bits == 4 && gq::options().gemm_variant < 0 && num_experts <= 16 && rows > 4 * num_experts &&
-                   rows <= 8 * num_experts)) {
-    const hipError_t q = gq::launch_midrow(g, 16, as_stream(stream));
+  // against 166 / 104).  From there to 24 rows per expert on average its instance with two batch tiles per pass, where K is
+  // one phase (up to 4096: e1_e3 at 40 / 64 / 96 tokens 166 / 167 / 195 -> 140 / 143 / 153 us; e2, K = 14336, 113-131 against the
+  // GEMM's 96-112, stays there).
+  const bool mid_ok = gv < 0 && bits == 4 && gq::options().gemm_variant < 0 && num_experts <= 16;
+  const bool mid_one = mid_ok && rows > 4 * num_experts && rows <= 8 * num_experts;
+  const bool mid_two = mid_ok && rows > 8 * num_experts && rows <= 24 * num_experts && K <= 4096;
+  if (gv == 10 || gv == 11 || mid_one || mid_two) {  // (10, 11: forced, one / two batch tiles)
+    const hipError_t q = gq::launch_midrow(g, (gv == 11 || mid_two) ? 32 : 16, as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "moe mid-row launch");
   }
   const int64_t quad_rows = 7 * num_experts > 32 ? 7 * num_experts : 32;

@@ -360,8 +360,8 @@ hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   p.paired = a.paired;
   p.ntiles = a.paired ? p.N / 32 : (p.N + 15) / 16;
   p.out_f32 = a.out_f32;
-  (void)rows_max;  // (one batch tile: segments of more than 16 rows take passes)
-  const int nbt = 1;
+  // batch tiles per pass: one for up to 16 rows per segment, else two (more rows: passes)
+  const int nbt = rows_max <= 16 ? 1 : 2;
   constexpr int U = 8;
   // waves that share a tile's K: as many as K has shares of U groups, at most 16
   int kwl = 4;
@@ -394,8 +394,10 @@ hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   p.rounds = ((rounds + p.chunks - 1) / p.chunks + unit - 1) / unit * unit;
   if (p.phases > 1) {
     if (form == 2) return hipErrorNotSupported;
+    if (nbt == 2) return launch_mid<2, 8, 2, false, true>(p, wgx, experts, s);
     return launch_mid<1, 8, 2, true, true>(p, wgx, experts, s);
   }
+  if (nbt == 2) return launch_mid<2, 8, 2, false, false>(p, wgx, experts, s);
   if (form == 2) return launch_mid<1, 8, 4, false, false>(p, wgx, experts, s);
   if (form == 4) return launch_mid<1, 8, 3, true, false>(p, wgx, experts, s);
   return launch_mid<1, 8, 2, true, false>(p, wgx, experts, s);

@@ -409,20 +409,21 @@ def test_midrow_kernel_is_the_default_on_large_matrices(m, n, k):
 
 @pytest.mark.parametrize("k", [1024, 4096, 14336])
 @pytest.mark.parametrize("paired", [False, True])
-def test_midrow_kernel_grouped(k, paired):
-    """Expert segments: an empty expert, one of a single row, one of 16 rows (a full pass) and one of 19 (two passes), the
-    gather of the activation rows folded in, int32 and int64 indptr; the fused gate/up form against linear + silu_mul of
-    the same kernel, bit for bit."""
+@pytest.mark.parametrize("tiles", [1, 2])  # batch tiles of 16 rows per pass
+def test_midrow_kernel_grouped(k, paired, tiles):
+    """Expert segments: an empty expert, one of a single row, one of 16 rows (a full pass of one batch tile), one of 19 (two
+    passes of one tile, one of two) and one of 40 (three passes / two), the gather of the activation rows folded in, int32 and
+    int64 indptr; the fused gate/up form against linear + silu_mul of the same kernel, bit for bit."""
     s = SCHEMES["q4f16_1"]
     rng = np.random.default_rng(63 + k)
     ne, n = 5, 224
     w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
     qw, qs = o.quantize(w, s)
-    ip = np.array([0, 1, 1, 17, 36, 40], np.int32)
+    ip = np.array([0, 1, 1, 17, 36, 76], np.int32)
     xs = rng.standard_normal((25, k)).astype(np.float16)
-    rows = rng.integers(0, 25, 40).astype(np.int32)
+    rows = rng.integers(0, 25, 76).astype(np.int32)
     x = xs[rows]
-    gq._lib.set_option("gemv_variant", 10)
+    gq._lib.set_option("gemv_variant", 9 + tiles)
     try:
         out = ops.moe_experts(dev(xs), dev(rows), dev(qw), dev(qs), dev(ip), 4, 32, silu_mul_halves=paired)
         kern = gq._lib.last_kernel()
@@ -430,7 +431,7 @@ def test_midrow_kernel_grouped(k, paired):
         plain = ops.moe_experts(dev(x), None, dev(qw), dev(qs), dev(ip), 4, 32)
     finally:
         gq._lib.set_option("gemv_variant", -1)
-    assert kern.startswith("gq::midrow_kernel<"), kern
+    assert kern.startswith(f"gq::midrow_kernel<{tiles},"), kern
     assert torch.equal(out, out64)
     assert_linear_ok(plain, o.dequantize_group_gemm_fp32(x, qw, qs, ip, s), x, k, f"grouped mid-row k={k}")
     if paired:
@@ -440,18 +441,22 @@ def test_midrow_kernel_grouped(k, paired):
 
 
 def test_midrow_kernel_is_the_default_between_few_rows_and_tiles():
-    """Four to eight rows per expert on average (up to 16 experts, q4): the default dispatch of the grouped matmul."""
+    """Four to eight rows per expert on average (up to 16 experts, q4) with one batch tile per pass, up to 24 with two where
+    K is one phase: the default dispatch of the grouped matmul."""
     s = SCHEMES["q4f16_1"]
     rng = np.random.default_rng(64)
     ne, n, k = 8, 96, 512
     w = (rng.standard_normal((ne, n, k)) * 0.02).astype(np.float16)
     qw, qs = o.quantize(w, s)
     ip = np.array([0, 4, 10, 15, 28, 37, 42, 55, 63], np.int32)
-    for rows, want in ((32, False), (33, True), (63, True)):
-        ipr = np.minimum(ip, rows).astype(np.int32)
+    for scale_rows, rows, want in ((1, 32, ""), (1, 33, "gq::midrow_kernel<1,"), (1, 63, "gq::midrow_kernel<1,"),
+                                   (3, 65, "gq::midrow_kernel<2,"), (3, 189, "gq::midrow_kernel<2,"), (4, 200, "")):
+        ipr = np.minimum(ip * scale_rows, rows).astype(np.int32)
+        ipr[-1] = rows
         x = rng.standard_normal((rows, k)).astype(np.float16)
         out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ipr), 4, 32)
-        assert gq._lib.last_kernel().startswith("gq::midrow_kernel<") == want, (rows, gq._lib.last_kernel())
+        kern = gq._lib.last_kernel()
+        assert (kern.startswith(want) if want else not kern.startswith("gq::midrow_kernel")), (rows, kern)
         assert_linear_ok(out, o.dequantize_group_gemm_fp32(x, qw, qs, ipr, s), x, k, f"grouped, {rows} rows over 8 experts")
 
 
