@@ -788,6 +788,18 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
       const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
       if (q != hipErrorNotSupported) return hip_result(q, "linear_dt quad-row launch");
     }
+    // 9..16 rows of q4 with K of one phase: the bfloat16 instance of the float16 linear's kernel for this range, from 4 M
+    // weights on (there is no bfloat16 skinny kernel: 6144 x 4096 at 16 rows 30.4 -> 10.8 us, 28672 x 4096 31.5 -> 20.3,
+    // 128256 x 4096 105 -> 71, 4096 x 4096 12.2 -> 9.4, 2048 x 2048 9.4 -> 8.8)
+    {
+      const int gvm = gq::options().gemv_variant;
+      const bool mid_rows = bits == 4 && M > 8 && M <= 16 && gq::options().gemm_variant < 0 && gvm < 0 && (K & 255) == 0 &&
+                            K <= 4096 && (N & 31) == 0 && N * K >= (4ll << 20);
+      if (mid_rows || gvm == 10) {
+        const hipError_t e = gq::launch_midrow(g, static_cast<int>(M), as_stream(stream));
+        if (e != hipErrorNotSupported) return hip_result(e, "linear_dt mid-row launch");
+      }
+    }
     // the float16 GEMM's tiles on the bf16 matrix instruction
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "linear_dt gemm launch");
@@ -1163,6 +1175,17 @@ static int moe_group_gemm_dt_impl(const void* x, int64_t rows, const void* q_wei
       if (e != hipErrorNotSupported) return hip_result(e, "moe_group_gemm_dt row GEMV launch");
       if (paired) return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul_dt: no fused GEMV for N=%lld K=%lld",
                               (long long)N, (long long)K);
+    }
+    // four to eight rows per expert on average, and up to 24 where K is one phase: as in float16 (the bfloat16 instance)
+    {
+      const int gvm = gq::options().gemv_variant;
+      const bool mid_ok = gvm < 0 && bits == 4 && gq::options().gemm_variant < 0 && num_experts <= 16;
+      const bool mid_one = mid_ok && rows > 4 * num_experts && rows <= 8 * num_experts;
+      const bool mid_two = mid_ok && rows > 8 * num_experts && rows <= 24 * num_experts && K <= 4096;
+      if (gvm == 10 || gvm == 11 || mid_one || mid_two) {
+        const hipError_t q = gq::launch_midrow(g, (gvm == 11 || mid_two) ? 32 : 16, as_stream(stream));
+        if (q != hipErrorNotSupported) return hip_result(q, "moe_group_gemm_dt mid-row launch");
+      }
     }
     // few rows in total: every expert streams its weights for a handful of rows (as in float16)
     const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;

@@ -1,4 +1,4 @@
-// Matmul for 9..64 activation rows against streamed q4f16_1 weights (batched decode, short prefill chunks):
+// Matmul for 9..64 activation rows against streamed q4f16_1 (q4bf16_1) weights (batched decode, short prefill chunks):
 // v_mfma_f32_16x16x32_f16 on UNSCALED weight operands, the group's scale applied to the matrix instruction's result,
 // the activations resident in registers.
 //
@@ -72,19 +72,28 @@ __device__ __forceinline__ void mid_transpose(uint32_t& r0, uint32_t& r1, uint32
 
 typedef uint32_t mid_u4 __attribute__((ext_vector_type(4)));
 
+template <bool BF>
 __device__ __forceinline__ float4_t mid_mfma(const mid_u4 a, const mid_u4 b, const float4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  if constexpr (BF) {
+    typedef __bf16 mid_bf8 __attribute__((ext_vector_type(8)));
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(mid_bf8, a), __builtin_bit_cast(mid_bf8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+  }
 }
 
 // NBT: batch tiles of 16 rows; U: groups of K a wave owns (4 or 8); RT: tiles of loads in flight per wave;
+// BF: bfloat16 model (x, scales, bias, residual and the 16-bit result are bfloat16): 0x4300 | q is the bfloat16 128 + q, so
+// every field is shifted down to bit 0 of its half (no x16 trick, x is not rescaled) and all carry the offset 128 + 7;
 // KEEP_C: the offset terms stay in registers (else the constant-operand instruction runs again in front of each group);
 // PHASED: K takes more than one phase (the sums of all of a wave's rounds stay in LDS between phases: one chunk of rounds);
 // else a wave's rounds come in chunks of p.rounds, each followed by the step that adds the K shares and stores, with x
 // and the ring of loads carried across
-template <int NBT, int U, int RT, bool KEEP_C, bool PHASED>
+template <int NBT, int U, int RT, bool KEEP_C, bool PHASED, bool BF = false>
 __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
   constexpr int STEPS = U / 4;
-  constexpr uint32_t kMagic = 0x64006400u;
+  constexpr uint32_t kMagic = BF ? 0x43004300u : 0x64006400u;
+  auto to_f32 = [](uint16_t bits) { return BF ? bf2f(bits) : h2f(bits); };
   extern __shared__ float4 res_lds[];  // [round][wave][NBT][64 lanes]
 
   // (the wave index in a scalar register: everything derived from it - K share, tiles, the loads' scalar offsets - is
@@ -139,7 +148,8 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
 
   constexpr uint32_t kLoLo = 0x05040100u, kHiHi = 0x07060302u;
   const half2_t r16 = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
-  const mid_u4 neg_off = {0xe407e407u /* -1031 */, 0xe407e407u, 0xe470e470u /* -16 * 71 */, 0xe470e470u};
+  const mid_u4 neg_off = BF ? mid_u4{0xc307c307u /* -135 */, 0xc307c307u, 0xc307c307u, 0xc307c307u}
+                            : mid_u4{0xe407e407u /* -1031 */, 0xe407e407u, 0xe470e470u /* -16 * 71 */, 0xe470e470u};
 
   for (int pass_lo = seg_lo; pass_lo < seg_hi; pass_lo += 16 * NBT) {
     for (int ph = 0; ph < (PHASED ? p.phases : 1); ++ph) {
@@ -191,9 +201,13 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
           if (!x_ok[bt]) v = make_uint4(0, 0, 0, 0);
           xa[bt][u][0] = __builtin_amdgcn_perm(v.z, v.x, kLoLo);
           xa[bt][u][1] = __builtin_amdgcn_perm(v.w, v.y, kLoLo);
-          xa[bt][u][2] = as_u32(as_half2(__builtin_amdgcn_perm(v.z, v.x, kHiHi)) * r16);
-          xa[bt][u][3] = as_u32(as_half2(__builtin_amdgcn_perm(v.w, v.y, kHiHi)) * r16);
-          if constexpr (KEEP_C) cc[bt][u] = mid_mfma(xa[bt][u], neg_off, float4_t{0.f, 0.f, 0.f, 0.f});
+          xa[bt][u][2] = __builtin_amdgcn_perm(v.z, v.x, kHiHi);
+          xa[bt][u][3] = __builtin_amdgcn_perm(v.w, v.y, kHiHi);
+          if constexpr (!BF) {
+            xa[bt][u][2] = as_u32(as_half2(xa[bt][u][2]) * r16);
+            xa[bt][u][3] = as_u32(as_half2(xa[bt][u][3]) * r16);
+          }
+          if constexpr (KEEP_C) cc[bt][u] = mid_mfma<BF>(xa[bt][u], neg_off, float4_t{0.f, 0.f, 0.f, 0.f});
         }
       }
 
@@ -219,15 +233,17 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
           for (int m = 0; m < 4; ++m) {
             const int u = 4 * st + m;
             const uint32_t w8 = r[m] >> 8;
-            const mid_u4 bw = {and_or_c(r[m], 0x000f000fu, kMagic), and_or_c(w8, 0x000f000fu, kMagic),
-                               and_or_c(r[m], 0x00f000f0u, kMagic), and_or_c(w8, 0x00f000f0u, kMagic)};
-            const float s = h2f(static_cast<uint16_t>((u & 1) ? sv[u >> 1] >> 16 : sv[u >> 1] & 0xffffu));
+            const mid_u4 bw = BF ? mid_u4{and_or_c(r[m], 0x000f000fu, kMagic), and_or_c(w8, 0x000f000fu, kMagic),
+                                          and_or_c(r[m] >> 4, 0x000f000fu, kMagic), and_or_c(r[m] >> 12, 0x000f000fu, kMagic)}
+                                 : mid_u4{and_or_c(r[m], 0x000f000fu, kMagic), and_or_c(w8, 0x000f000fu, kMagic),
+                                          and_or_c(r[m], 0x00f000f0u, kMagic), and_or_c(w8, 0x00f000f0u, kMagic)};
+            const float s = to_f32(static_cast<uint16_t>((u & 1) ? sv[u >> 1] >> 16 : sv[u >> 1] & 0xffffu));
 #pragma unroll
             for (int bt = 0; bt < NBT; ++bt) {
               float4_t c0;
               if constexpr (KEEP_C) c0 = cc[bt][u];
-              else c0 = mid_mfma(xa[bt][u], neg_off, zero4);
-              const float4_t d = mid_mfma(xa[bt][u], bw, c0);
+              else c0 = mid_mfma<BF>(xa[bt][u], neg_off, zero4);
+              const float4_t d = mid_mfma<BF>(xa[bt][u], bw, c0);
 #pragma unroll
               for (int q = 0; q < 4; ++q) acc[bt][q] = fmaf(s, d[q], acc[bt][q]);
             }
@@ -258,7 +274,7 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
             const int col = pair * 16 + cq, b = pass_lo + 16 * bt + jq;
             if (pair >= p.ntiles || b >= seg_hi) continue;
             const float gate = share_sum(2 * pr, tl, bt), up = share_sum(2 * pr + 1, tl, bt);
-            static_cast<uint16_t*>(p.y)[static_cast<int64_t>(b) * half + col] = silu_mul_h(gate, up);
+            static_cast<uint16_t*>(p.y)[static_cast<int64_t>(b) * half + col] = silu_mul_t<BF>(gate, up);
           }
         } else {
           const int items = p.rounds * tw * NBT;
@@ -269,10 +285,10 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
             if (t >= p.ntiles || col >= p.N || b >= seg_hi) continue;
             float v = share_sum(round, tl, bt);
             const int64_t oi = static_cast<int64_t>(b) * p.N + col;
-            if (p.bias != nullptr) v += h2f(p.bias[col]);
-            if (p.residual != nullptr) v += h2f(p.residual[oi]);
+            if (p.bias != nullptr) v += to_f32(p.bias[col]);
+            if (p.residual != nullptr) v += to_f32(p.residual[oi]);
             if (p.out_f32) static_cast<float*>(p.y)[oi] = v;
-            else static_cast<uint16_t*>(p.y)[oi] = f2h(v);
+            else static_cast<uint16_t*>(p.y)[oi] = BF ? f2bf(v) : f2h(v);
           }
         }
       };
@@ -312,34 +328,34 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
   }
 }
 
-template <int NBT, int U, int RT, bool KEEP_C, bool PHASED>
+template <int NBT, int U, int RT, bool KEEP_C, bool PHASED, bool BF = false>
 hipError_t launch_mid(const MidParams& p, int wgx, int experts, hipStream_t s) {
   const size_t lds = static_cast<size_t>(p.rounds) * 16 * NBT * 1024;
   if (lds > 160 * 1024) return hipErrorNotSupported;
   if (lds > 64 * 1024) {
     static bool raised = false;  // (idempotent; a race sets the same attribute twice)
     if (!raised) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&midrow_kernel<NBT, U, RT, KEEP_C, PHASED>),
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&midrow_kernel<NBT, U, RT, KEEP_C, PHASED, BF>),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return e;
       raised = true;
     }
   }
-  note_kernel("gq::midrow_kernel<%d,%d,%d,%d,%d> rounds=%d chunks=%d phases=%d kw=%d", NBT, U, RT, int(KEEP_C), int(PHASED),
-              p.rounds, p.chunks, p.phases, 1 << p.kw_log2);
-  hipLaunchKernelGGL((midrow_kernel<NBT, U, RT, KEEP_C, PHASED>), dim3(wgx, experts), dim3(1024), lds, s, p);
+  note_kernel("gq::midrow_kernel<%d,%d,%d,%d,%d%s> rounds=%d chunks=%d phases=%d kw=%d", NBT, U, RT, int(KEEP_C), int(PHASED),
+              BF ? ",true" : "", p.rounds, p.chunks, p.phases, 1 << p.kw_log2);
+  hipLaunchKernelGGL((midrow_kernel<NBT, U, RT, KEEP_C, PHASED, BF>), dim3(wgx, experts), dim3(1024), lds, s, p);
   return hipGetLastError();
 }
 
 }  // namespace
 
-// q4f16_1, float16 activations, K % 256 == 0 (a wave's eight groups: 16-byte runs of scales), N % 16 == 0 for expert
+// q4f16_1 / q4bf16_1 (float16 / bfloat16 activations, scales and results), K % 256 == 0 (a wave's eight groups: 16-byte runs of scales), N % 16 == 0 for expert
 // segments and N % 32 == 0 for the fused gate/up form; any number of rows (more than the batch tiles hold: passes that read
 // the weights again, so callers keep it to few rows per segment).  hipErrorNotSupported otherwise.  Tuning overrides:
 // quad_ksplit (log2 of the waves that share a tile's K, minus one), gemv_waves (workgroups per expert x 16),
 // gemv_rows_per_wave (1, 2: other one-batch-tile instances).
 hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s) {
-  if (a.bits != 4 || a.group_size != 32 || a.bf16) return hipErrorNotSupported;
+  if (a.bits != 4 || a.group_size != 32) return hipErrorNotSupported;
   if (a.rows < 1 || a.N < 16 || (a.K & 255) != 0 || a.K == 0) return hipErrorNotSupported;
   const bool grouped = a.indptr != nullptr;
   if (grouped && (a.N & 15) != 0) return hipErrorNotSupported;  // (an expert's tensor ends where the next begins)
@@ -392,6 +408,13 @@ hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   int rounds = (items * per_round + unit - 1) / unit * unit;
   p.chunks = (rounds + max_rounds - 1) / max_rounds;
   p.rounds = ((rounds + p.chunks - 1) / p.chunks + unit - 1) / unit * unit;
+  if (a.bf16) {  // (the bfloat16 instances: q4bf16_*)
+    if (p.phases > 1)
+      return nbt == 2 ? launch_mid<2, 8, 2, false, true, true>(p, wgx, experts, s)
+                      : launch_mid<1, 8, 2, true, true, true>(p, wgx, experts, s);
+    return nbt == 2 ? launch_mid<2, 8, 2, false, false, true>(p, wgx, experts, s)
+                    : launch_mid<1, 8, 2, true, false, true>(p, wgx, experts, s);
+  }
   if (p.phases > 1) {
     if (form == 2) return hipErrorNotSupported;
     if (nbt == 2) return launch_mid<2, 8, 2, false, true>(p, wgx, experts, s);

@@ -1805,6 +1805,63 @@ def test_bfloat16_few_rows_take_the_register_fewrow_kernel(m, n, k):
     assert torch.equal(fused, ops.silu_mul(y))
 
 
+@pytest.mark.parametrize("m", [9, 16, 23])  # one batch tile, a full one, two (forced)
+@pytest.mark.parametrize("n,k", [(512, 4096), (96, 1024), (160, 8192)])
+def test_bfloat16_midrow_kernel(m, n, k):
+    """q4bf16_1 on the kernel that scales the matrix instruction's result (its bfloat16 instance: every field shifted to
+    the low bits, offset 128 + 7, x as it is), forced on small shapes: float32 output exact against the unrounded-weight
+    product, the bfloat16 output the same numbers rounded once; bias and residual; the fused gate/up form against the two steps."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(m * 100 + n)
+    w32 = o.round_to((rng.standard_normal((n, k)) * 0.05).astype(np.float32), "bfloat16")
+    x32 = o.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    b32 = o.round_to(rng.standard_normal(n).astype(np.float32), "bfloat16")
+    r32 = o.round_to(rng.standard_normal((m, n)).astype(np.float32), "bfloat16")
+    qw_ref, qs_ref = o.quantize_dt(w32, s, "bfloat16")
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).to(torch.bfloat16).to(DEV)
+    x, b, r = (torch.from_numpy(a).to(torch.bfloat16).to(DEV) for a in (x32, b32, r32))
+    gq._lib.set_option("gemv_variant", 10)
+    try:
+        y32 = ops.linear(x, qw, qs, 4, 32, None, out_dtype=torch.float32)
+        kern = gq._lib.last_kernel()
+        y = ops.linear(x, qw, qs, 4, 32)
+        yb = ops.linear(x, qw, qs, 4, 32, b, out_dtype=torch.float32, residual=r)
+        fused = ops.linear_silu_mul(x, qw, qs, 4, 32)
+        kern_fused = gq._lib.last_kernel()
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+    assert kern.startswith(f"gq::midrow_kernel<{1 if m <= 16 else 2},") and ",true>" in kern, kern
+    assert kern_fused.startswith("gq::midrow_kernel<") and ",true>" in kern_fused, kern_fused
+    exact = o.linear_dt_fp64(x32, qw_ref, qs_ref, s, "bfloat16", None, unrounded_weights=True)
+    assert np.linalg.norm(y32.double().cpu().numpy() - exact) / np.linalg.norm(exact) <= 5e-6 + 1e-7 * np.sqrt(k)
+    assert y.dtype == torch.bfloat16 and np.array_equal(_carrier(y), o.round_to(y32.cpu().numpy(), "bfloat16"))
+    want = exact + b32.astype(np.float64) + r32.astype(np.float64)
+    assert np.linalg.norm(yb.double().cpu().numpy() - want) / np.linalg.norm(want) <= 5e-6 + 1e-7 * np.sqrt(k)
+    assert torch.equal(fused, ops.silu_mul(y))
+
+
+def test_bfloat16_midrow_kernel_grouped_default():
+    """q4bf16_1 expert segments at six and at sixteen rows per expert on average: the default dispatch takes the bfloat16
+    instance (one and two batch tiles per pass); against the exact product, and the fused gate/up form bit for bit."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(71)
+    ne, n, k = 4, 96, 1024
+    w32 = o.round_to((rng.standard_normal((ne, n, k)) * 0.05).astype(np.float32), "bfloat16")
+    qw_ref, qs_ref = o.quantize_dt(w32, s, "bfloat16")
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).to(torch.bfloat16).to(DEV)
+    for ip, tiles in ((np.array([0, 3, 3, 20, 24], np.int32), 1), (np.array([0, 30, 31, 45, 64], np.int32), 2)):
+        rows = int(ip[-1])
+        x32 = o.round_to(rng.standard_normal((rows, k)).astype(np.float32), "bfloat16")
+        x = torch.from_numpy(x32).to(torch.bfloat16).to(DEV)
+        out = ops.moe_experts(x, None, qw, qs, dev(ip), 4, 32)
+        kern = gq._lib.last_kernel()
+        assert kern.startswith(f"gq::midrow_kernel<{tiles},") and ",true>" in kern, kern
+        ref = o.dequantize_group_gemm_dt_fp64(x32, qw_ref, qs_ref, ip, s, "bfloat16")
+        _assert_dt_matmul_ok(out, ref, x32, k, "bfloat16", f"grouped bf16 mid-row, {tiles} tile(s)")
+        fused = ops.moe_experts(x, None, qw, qs, dev(ip), 4, 32, silu_mul_halves=True)
+        assert torch.equal(fused, ops.silu_mul(out))
+
+
 def _assert_dt_matmul_ok(y: torch.Tensor, ref: np.ndarray, x32: np.ndarray, k: int, model_dtype: str, what=""):
     """Output in the model dtype against the exact product of the same operands: the fp32 accumulation
     (relative error of a sum of k terms grows like sqrt(k) * 2^-24) plus, for bfloat16, the one rounding of
