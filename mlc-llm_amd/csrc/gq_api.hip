@@ -952,6 +952,30 @@ static hipError_t moe_row_gemv(const gq::GemmArgs& g, hipStream_t s) {
   return gq::launch_gemv(a, s);
 }
 
+// Expert segments on the kernel that scales the matrix instruction's result (gq_midrow.hip): rows per pass (16 or 32), or
+// 0 where the quad-row kernel (fewer rows) or the GEMM's tiles (more) stay ahead.  A segment longer than a pass takes
+// another pass over its expert's weights while the other experts' workgroups are done, so the bounds keep the longest
+// segment inside one pass: with 8 experts 4 to 8 rows per expert on average for 16-row passes, with 64 experts (whose
+// longest segment is further above the average: 12 at an average of 6, 17 at 9) 2 to 6; beyond that, up to 24 resp. 16 on
+// average, the two-tile instance where K is one phase.  Measured, 8 experts x top-2 (Mixtral, e1_e3 / e2 in us): 24 tokens
+// 156 / 102 -> 115 / 76, 32 tokens 170 / 106 -> 117 / 78, 16 tokens 118 / 75 against the quad-row kernel's 122 / 74, 40 tokens
+// with 16-row passes 203 / 131 against the GEMM's 166 / 104; two tiles at 40 / 64 / 96 tokens 166 / 167 / 195 -> 140 / 143 / 153
+// for e1_e3 (e2, K = 14336 in phases, 113-131 against 96-112: stays with the GEMM).  64 experts x top-6, 2816 x 2048 / 2048 x
+// 1536 / 5120 x 3584 at 144..384 rows: 55-64 / 46-49 / 142-197 -> 51-53 / 34-35 / 142-145; at 576 rows (two tiles) 83 / 49 / 211
+// -> 69 / 48 / 191.
+static int midrow_rows_per_pass(int64_t rows, int64_t num_experts, int64_t K, int bits) {
+  const int gv = gq::options().gemv_variant;
+  if (gv == 10) return 16;  // (forced)
+  if (gv == 11) return 32;
+  if (gv >= 0 || bits != 4 || gq::options().gemm_variant >= 0) return 0;
+  const bool many = num_experts > 16;
+  const int64_t lo = (many ? 2 : 4) * num_experts, mid = (many ? 6 : 8) * num_experts,
+                hi = (many ? 16 : 24) * num_experts;
+  if (rows > lo && rows <= mid) return 16;
+  if (rows > mid && rows <= hi && K <= 4096) return 32;
+  return 0;
+}
+
 static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight, const void* q_scale,
                                const void* indptr, int indptr_dtype, int64_t num_experts, int64_t N,
                                int64_t K, int bits, int group_size, void* out, mi355gq_stream_t stream,
@@ -1000,19 +1024,8 @@ static int moe_group_gemm_impl(const void* x, int64_t rows, const void* q_weight
   //  its scales in bulk, and only a forced variant runs it on expert segments.  The same rows per expert hold for many
   //  experts: 64 experts x top-6 (2048 x 1408 projections), whole layer at 144 / 192 / 288 / 384 / 432 routed rows
   //  112 / 115 / 117 / 127 / 142 us against 137 / 141 / 146 / 143 / 144 on the GEMM's tiles)
-  // Between the quad-row kernel's few rows per expert and the GEMM's tiles: four to eight rows per expert on average (so that
-  // hardly a segment holds more than the 16 rows of one pass), up to 16 experts, q4, K % 256 == 0: the kernel that scales
-  // the matrix instruction's result.  Mixtral layer (8 experts x top-2) at 24 / 32 tokens: e1_e3 156 / 170 -> 115 / 117 us,
-  // e2 102 / 106 -> 76 / 78; at 16 tokens equal to the quad-row kernel (118 / 75 against 122 / 74), at 40 and beyond a
-  // segment of 17 rows or more takes a second pass over its expert's weights and the GEMM's tiles are ahead (203 / 131
-  // against 166 / 104).  From there to 24 rows per expert on average its instance with two batch tiles per pass, where K is
-  // one phase (up to 4096: e1_e3 at 40 / 64 / 96 tokens 166 / 167 / 195 -> 140 / 143 / 153 us; e2, K = 14336, 113-131 against the
-  // GEMM's 96-112, stays there).
-  const bool mid_ok = gv < 0 && bits == 4 && gq::options().gemm_variant < 0 && num_experts <= 16;
-  const bool mid_one = mid_ok && rows > 4 * num_experts && rows <= 8 * num_experts;
-  const bool mid_two = mid_ok && rows > 8 * num_experts && rows <= 24 * num_experts && K <= 4096;
-  if (gv == 10 || gv == 11 || mid_one || mid_two) {  // (10, 11: forced, one / two batch tiles)
-    const hipError_t q = gq::launch_midrow(g, (gv == 11 || mid_two) ? 32 : 16, as_stream(stream));
+  if (const int per_pass = midrow_rows_per_pass(rows, num_experts, K, bits)) {
+    const hipError_t q = gq::launch_midrow(g, per_pass, as_stream(stream));
     if (q != hipErrorNotSupported) return hip_result(q, "moe mid-row launch");
   }
   const int64_t quad_rows = 7 * num_experts > 32 ? 7 * num_experts : 32;
@@ -1176,16 +1189,10 @@ static int moe_group_gemm_dt_impl(const void* x, int64_t rows, const void* q_wei
       if (paired) return fail(MI355GQ_ERR_UNSUPPORTED, "moe_group_gemm_silu_mul_dt: no fused GEMV for N=%lld K=%lld",
                               (long long)N, (long long)K);
     }
-    // four to eight rows per expert on average, and up to 24 where K is one phase: as in float16 (the bfloat16 instance)
-    {
-      const int gvm = gq::options().gemv_variant;
-      const bool mid_ok = gvm < 0 && bits == 4 && gq::options().gemm_variant < 0 && num_experts <= 16;
-      const bool mid_one = mid_ok && rows > 4 * num_experts && rows <= 8 * num_experts;
-      const bool mid_two = mid_ok && rows > 8 * num_experts && rows <= 24 * num_experts && K <= 4096;
-      if (gvm == 10 || gvm == 11 || mid_one || mid_two) {
-        const hipError_t q = gq::launch_midrow(g, (gvm == 11 || mid_two) ? 32 : 16, as_stream(stream));
-        if (q != hipErrorNotSupported) return hip_result(q, "moe_group_gemm_dt mid-row launch");
-      }
+    // between the few-row kernel and the tiles: as in float16 (the bfloat16 instance)
+    if (const int per_pass = midrow_rows_per_pass(rows, num_experts, K, bits)) {
+      const hipError_t q = gq::launch_midrow(g, per_pass, as_stream(stream));
+      if (q != hipErrorNotSupported) return hip_result(q, "moe_group_gemm_dt mid-row launch");
     }
     // few rows in total: every expert streams its weights for a handful of rows (as in float16)
     const int64_t quad_rows = 6 * num_experts > 32 ? 6 * num_experts : 32;

@@ -379,9 +379,10 @@ hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   // batch tiles per pass: one for up to 16 rows per segment, else two (more rows: passes)
   const int nbt = rows_max <= 16 ? 1 : 2;
   constexpr int U = 8;
-  // waves that share a tile's K: as many as K has shares of U groups, at most 16
-  int kwl = 4;
-  while (kwl > 0 && (p.ng / U) < (1 << kwl)) --kwl;
+  // waves that share a tile's K: the power of two that covers K's shares of U groups, at most 16 (a wave whose share lies
+  // past K idles: one phase with 14 of 16 waves at work is ahead of two phases of 8)
+  int kwl = 0;
+  while (kwl < 4 && (1 << kwl) < p.ng / U) ++kwl;
   if (options().quad_ksplit >= 0) kwl = options().quad_ksplit + 1;  // (tuning override: 2, 4, 8 or 16 waves)
   p.kw_log2 = kwl;
   const int phase_groups = (1 << kwl) * U;

@@ -457,7 +457,20 @@ def test_midrow_kernel_is_the_default_between_few_rows_and_tiles():
         out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ipr), 4, 32)
         kern = gq._lib.last_kernel()
         assert (kern.startswith(want) if want else not kern.startswith("gq::midrow_kernel")), (rows, kern)
-        assert_linear_ok(out, o.dequantize_group_gemm_fp32(x, qw, qs, ipr, s), x, k, f"grouped, {rows} rows over 8 experts")
+        assert_linear_ok(out, o.dequantize_group_gemm_fp32(x, qw, qs, ipr, s), x, k, f"grouped, {rows} rows over {ne} experts")
+    # many experts (their longest segment is further above the average): 2 to 6 rows per expert with one batch tile, up to 16 with two
+    ne = 40
+    w = (rng.standard_normal((ne, 32, k)) * 0.02).astype(np.float16)
+    qw, qs = o.quantize(w, s)
+    for rows, want in ((80, ""), (90, "gq::midrow_kernel<1,"), (240, "gq::midrow_kernel<1,"), (250, "gq::midrow_kernel<2,"),
+                       (640, "gq::midrow_kernel<2,"), (650, "")):
+        cuts = np.sort(rng.integers(0, rows + 1, ne - 1))
+        ipr = np.concatenate([[0], cuts, [rows]]).astype(np.int32)
+        x = rng.standard_normal((rows, k)).astype(np.float16)
+        out = ops.moe_group_gemm(dev(x), dev(qw), dev(qs), dev(ipr), 4, 32)
+        kern = gq._lib.last_kernel()
+        assert (kern.startswith(want) if want else not kern.startswith("gq::midrow_kernel")), (rows, kern)
+        assert_linear_ok(out, o.dequantize_group_gemm_fp32(x, qw, qs, ipr, s), x, k, f"grouped, {rows} rows over {ne} experts")
 
 
 @pytest.mark.parametrize("mode", [2, 3, 4])
