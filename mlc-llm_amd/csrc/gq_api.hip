@@ -399,14 +399,16 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
     const int64_t need = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
     q4_skinny_loses = need == 0 || (workspace != nullptr && workspace_bytes >= need);
   }
-  // q4, 9..16 rows of a K that one phase covers (up to 4096), from about 24 M weights on: the kernel that multiplies
+  // q4, 9..16 rows of a K that one phase covers (up to 4096; two phases: below), from about 24 M weights on: the kernel that multiplies
   // unscaled weight operands and scales the matrix instruction's result (28672 x 4096 at 9 / 16 rows 20.0 / 20.3 us
   // against 27.8-28.1 for the GEMM's 32-row tile, 6144 x 4096 10.4 / 10.9 against 12.2 / 13.1 for the skinny kernel;
   // 4096 x 4096 stays with the skinny kernel, 9.0-9.4 either way, and a longer K with the GEMM's tiles, 4096 x 14336
   // 26-27 against 20).  The same test for the plain and the fused gate/up form: both must add in the same order.
+  // (K of two phases, up to 8192, from 48 M weights on: 10240 x 8192 28 -> 21-22 us, 8192 x 8192 21 -> 17-18.5, 57344 x 8192
+  //  100-106 -> 74-78, 15360 x 5120 24.5 -> 21-22, 27648 x 5120 33.4-34.4 -> 32.4-33.8)
   const bool mid_rows = bits == 4 && M > 8 && M <= 16 && gq::options().gemm_variant < 0 &&
                         (gq::options().gemv_variant < 0 || gq::options().gemv_variant == 10) && (K & 255) == 0 &&
-                        K <= 4096 && (N & 31) == 0 && N * K >= (24ll << 20);
+                        (N & 31) == 0 && ((K <= 4096 && N * K >= (24ll << 20)) || (K <= 8192 && N * K >= (48ll << 20)));
   if (mid_rows || gq::options().gemv_variant == 10) {  // (10: forced, whatever the shape)
     const hipError_t e = gq::launch_midrow(g, static_cast<int>(M), as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "mid-row launch");
@@ -794,7 +796,7 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
     {
       const int gvm = gq::options().gemv_variant;
       const bool mid_rows = bits == 4 && M > 8 && M <= 16 && gq::options().gemm_variant < 0 && gvm < 0 && (K & 255) == 0 &&
-                            K <= 4096 && (N & 31) == 0 && N * K >= (4ll << 20);
+                            (N & 31) == 0 && ((K <= 4096 && N * K >= (4ll << 20)) || (K <= 8192 && N * K >= (48ll << 20)));
       if (mid_rows || gvm == 10) {
         const hipError_t e = gq::launch_midrow(g, static_cast<int>(M), as_stream(stream));
         if (e != hipErrorNotSupported) return hip_result(e, "linear_dt mid-row launch");

@@ -389,10 +389,11 @@ def test_midrow_kernel(form, m, n, k):
 
 
 @pytest.mark.parametrize("m", [9, 12, 16])
-@pytest.mark.parametrize("n,k", [(6144, 4096), (28672, 4096)])
+@pytest.mark.parametrize("n,k", [(6144, 4096), (28672, 4096), (8192, 8192)])
 def test_midrow_kernel_is_the_default_on_large_matrices(m, n, k):
-    """9..16 rows of q4 on matrices of 24 M weights or more with K up to 4096: the default dispatch, against the oracle on
-    a sample of the columns; the fused gate/up form takes the same kernel and equals linear + silu_mul bit for bit."""
+    """9..16 rows of q4 on matrices of 24 M weights or more with K up to 4096 (48 M with K up to 8192, two phases): the default
+    dispatch, against the oracle on a sample of the columns; the fused gate/up form takes the same kernel and equals
+    linear + silu_mul bit for bit."""
     s = SCHEMES["q4f16_1"]
     rng = np.random.default_rng(seed_of("midrow", m, n, k))
     qw = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
