@@ -388,6 +388,27 @@ def test_midrow_kernel(form, m, n, k):
     assert_linear_ok(yr, ref + res.astype(np.float64), x, k, f"mid-row form {form} residual")
 
 
+def test_midrow_kernel_random_shapes():
+    """Forty random shapes through the forced kernel against the oracle: rows 1..48 (one to three passes of one or two batch
+    tiles), N from 16 up (whole and ragged last tiles), K of 1 to 40 wave shares (1, 2, 4, 8, 16 waves per tile, one to three
+    phases), with and without bias."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(20250)
+    for case in range(40):
+        m = int(rng.integers(1, 49))
+        n = int(rng.choice([16, 31, 48, 100, 257, 512, 1000, 1552, 3000]))
+        k = 256 * int(rng.choice([1, 2, 3, 4, 5, 8, 13, 16, 17, 24, 40]))
+        x, qw, qs, b = _linear_case(s, m, n, k, 1000 + case, bias=bool(case & 1))
+        gq._lib.set_option("gemv_variant", 10)
+        try:
+            y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, None if b is None else dev(b))
+            kern = gq._lib.last_kernel()
+        finally:
+            gq._lib.set_option("gemv_variant", -1)
+        assert kern.startswith("gq::midrow_kernel<"), (m, n, k, kern)
+        assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"mid-row random case {case}: {m}x{n}x{k} [{kern}]")
+
+
 @pytest.mark.parametrize("m", [9, 12, 16])
 @pytest.mark.parametrize("n,k", [(6144, 4096), (28672, 4096), (8192, 8192)])
 def test_midrow_kernel_is_the_default_on_large_matrices(m, n, k):
