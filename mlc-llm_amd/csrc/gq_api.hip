@@ -406,9 +406,15 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   // 26-27 against 20).  The same test for the plain and the fused gate/up form: both must add in the same order.
   // (K of two phases, up to 8192, from 48 M weights on: 10240 x 8192 28 -> 21-22 us, 8192 x 8192 21 -> 17-18.5, 57344 x 8192
   //  100-106 -> 74-78, 15360 x 5120 24.5 -> 21-22, 27648 x 5120 33.4-34.4 -> 32.4-33.8)
-  const bool mid_rows = bits == 4 && M > 8 && M <= 16 && gq::options().gemm_variant < 0 &&
+  // 17..32 rows (two batch tiles per pass, the offsets subtracted from the weight operand): one phase and 48 M weights or more
+  // (14336 x 4096 at 17 / 24 / 32 rows 19.4 / 19.9 / 20.4 -> 16.9 / 17.9 / 19.0 us, 28672 x 4096 28.3 / 28.0 / 27.9 -> 26.0 / 26.1 / 27.5, 128256 x
+  //  4096 99-101 -> 84-87; 6144 x 4096 13.4-14.4 against 12.3-14.1 and 4096 x 4096 stay with the GEMM's tile, as does K = 8192 in
+  //  two phases: 57344 x 8192 92-97 against 112-126)
+  const bool mid_size = (M > 8 && M <= 16 && ((K <= 4096 && N * K >= (24ll << 20)) || (K <= 8192 && N * K >= (48ll << 20)))) ||
+                        (M > 16 && M <= 32 && K <= 4096 && N * K >= (48ll << 20));
+  const bool mid_rows = bits == 4 && mid_size && gq::options().gemm_variant < 0 &&
                         (gq::options().gemv_variant < 0 || gq::options().gemv_variant == 10) && (K & 255) == 0 &&
-                        (N & 31) == 0 && ((K <= 4096 && N * K >= (24ll << 20)) || (K <= 8192 && N * K >= (48ll << 20)));
+                        (N & 31) == 0;
   if (mid_rows || gq::options().gemv_variant == 10) {  // (10: forced, whatever the shape)
     const hipError_t e = gq::launch_midrow(g, static_cast<int>(M), as_stream(stream));
     if (e != hipErrorNotSupported) return hip_result(e, "mid-row launch");

@@ -238,12 +238,24 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
                                  : mid_u4{and_or_c(r[m], 0x000f000fu, kMagic), and_or_c(w8, 0x000f000fu, kMagic),
                                           and_or_c(r[m], 0x00f000f0u, kMagic), and_or_c(w8, 0x00f000f0u, kMagic)};
             const float s = to_f32(static_cast<uint16_t>((u & 1) ? sv[u >> 1] >> 16 : sv[u >> 1] & 0xffffu));
+            // (float16 without the kept offsets: the offsets come off the weight operand instead, exactly - 1024 + q - 1031
+            //  and 1024 + 16 q - 16 * 71 are small integers -, four packed adds per group whatever the batch tiles, in place
+            //  of one more matrix instruction per group and batch tile)
+            constexpr bool SUB = !KEEP_C && !BF;
+            mid_u4 bo = bw;
+            if constexpr (SUB) {
+              const half2_t o_lo = {static_cast<_Float16>(-1031.f), static_cast<_Float16>(-1031.f)};
+              const half2_t o_hi = {static_cast<_Float16>(-1136.f), static_cast<_Float16>(-1136.f)};
+              bo[0] = as_u32(as_half2(bw[0]) + o_lo); bo[1] = as_u32(as_half2(bw[1]) + o_lo);
+              bo[2] = as_u32(as_half2(bw[2]) + o_hi); bo[3] = as_u32(as_half2(bw[3]) + o_hi);
+            }
 #pragma unroll
             for (int bt = 0; bt < NBT; ++bt) {
               float4_t c0;
               if constexpr (KEEP_C) c0 = cc[bt][u];
+              else if constexpr (SUB) c0 = float4_t{0.f, 0.f, 0.f, 0.f};
               else c0 = mid_mfma<BF>(xa[bt][u], neg_off, zero4);
-              const float4_t d = mid_mfma<BF>(xa[bt][u], bw, c0);
+              const float4_t d = mid_mfma<BF>(xa[bt][u], SUB ? bo : bw, c0);
 #pragma unroll
               for (int q = 0; q < 4; ++q) acc[bt][q] = fmaf(s, d[q], acc[bt][q]);
             }

@@ -409,11 +409,11 @@ def test_midrow_kernel_random_shapes():
         assert_linear_ok(y, o.linear_fp32(x, qw, qs, s, b), x, k, f"mid-row random case {case}: {m}x{n}x{k} [{kern}]")
 
 
-@pytest.mark.parametrize("m", [9, 12, 16])
+@pytest.mark.parametrize("m", [9, 12, 16, 17, 32])
 @pytest.mark.parametrize("n,k", [(6144, 4096), (28672, 4096), (8192, 8192)])
 def test_midrow_kernel_is_the_default_on_large_matrices(m, n, k):
-    """9..16 rows of q4 on matrices of 24 M weights or more with K up to 4096 (48 M with K up to 8192, two phases): the default
-    dispatch, against the oracle on a sample of the columns; the fused gate/up form takes the same kernel and equals
+    """9..16 rows of q4 on matrices of 24 M weights or more with K up to 4096 (48 M with K up to 8192, two phases), 17..32 rows
+    from 48 M weights on with K up to 4096: the default dispatch, against the oracle on a sample of the columns; the fused gate/up form takes the same kernel and equals
     linear + silu_mul bit for bit."""
     s = SCHEMES["q4f16_1"]
     rng = np.random.default_rng(seed_of("midrow", m, n, k))
@@ -421,11 +421,13 @@ def test_midrow_kernel_is_the_default_on_large_matrices(m, n, k):
     qs = (rng.random((n, k // 32)) * 0.02 + 0.001).astype(np.float16)
     x = rng.standard_normal((m, k)).astype(np.float16)
     cols = np.unique(np.concatenate([[0, 1, n // 2, n - 1], rng.integers(0, n, 300)]))
+    # (17..32 rows: two batch tiles, from 48 M weights on and with K of one phase only)
+    want = m <= 16 or (n * k >= 48 << 20 and k <= 4096)
     y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32)
-    assert gq._lib.last_kernel().startswith("gq::midrow_kernel<"), gq._lib.last_kernel()
+    assert gq._lib.last_kernel().startswith(f"gq::midrow_kernel<{1 if m <= 16 else 2},") == want, gq._lib.last_kernel()
     assert_linear_ok(y[:, torch.from_numpy(cols).to(DEV)], o.linear_fp32(x, qw[cols], qs[cols], s), x, k, f"mid-row {m}x{n}x{k}")
     fused = ops.linear_silu_mul(dev(x), dev(qw), dev(qs), 4, 32)
-    assert gq._lib.last_kernel().startswith("gq::midrow_kernel<"), gq._lib.last_kernel()
+    assert gq._lib.last_kernel().startswith("gq::midrow_kernel<") == want, gq._lib.last_kernel()
     assert torch.equal(fused, ops.silu_mul(y))
 
 
