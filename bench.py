@@ -494,7 +494,7 @@ def main() -> int:
             del w13, w2
         g2 = torch.Generator(device=dev).manual_seed(2)
         moe_res = {}
-        for t in (1, 16, 32, 512):
+        for t in (1, 16, 32, 64, 512):
             xt = torch.randn((1, t, 4096), generator=gx, device=dev).half()
             logits = torch.randn((t, 8), generator=g2, device=dev).half()
             ms = timed(lambda: moe(xt, logits), 10, 2, use_graph)
