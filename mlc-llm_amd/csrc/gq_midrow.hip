@@ -13,7 +13,7 @@
 // field pair, odd fields come out times 16 and meet activations divided by 16), one instruction per quantisation
 // group, so that the group's scale multiplies four accumulator values per lane afterwards and the offset
 // -(1024 + 7) * sum(x) of the group enters as the instruction's C operand: the arithmetic of the 4x4x4 kernels
-// (gq_quadrow.hip), about 1.3 vector instructions per weight and lane at 16 rows.
+// (gq_quadrow.hip), about ten vector instructions per group of 512 weights and wave at 16 rows.
 //
 // B operand of instruction g = group g of 16 weight rows (a "tile"): lane (c = lane % 16, j = lane / 16) supplies the
 // 8 k of storage word j of row c.  A lane LOADS a whole group (128 bits: lane (c, j) group 4 * step + j of row c, so a
