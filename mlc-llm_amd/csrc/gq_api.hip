@@ -320,11 +320,14 @@ int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits
   if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
       N >= kMaxDim || K >= kMaxDim)
     return 0;
+  // q4 at 9..32 rows of a K beyond 4096: the K slices of the kernel on unscaled weight operands (see linear_impl)
+  const int64_t mid = (bits == 4 && M > 8 && M <= 32) ? gq::midrow_workspace_bytes(M, N, K) : 0;
   // only the few-row GEMM (more rows than the GEMV / skinny kernels take, at most 256) splits K
   // (q4 at 9..16 rows: the skinny kernel, except on matrices of 40 M to 256 M weights, see linear_impl)
-  if (M <= 16 && bits == 4 && !(M > 8 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return 0;
+  if (M <= 16 && bits == 4 && !(M > 8 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return mid;
   if (M <= 8) return 0;
-  return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+  const int64_t gemm = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+  return gemm > mid ? gemm : mid;
 }
 
 int64_t mi355gq_linear_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size,
@@ -333,18 +336,24 @@ int64_t mi355gq_linear_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int b
   if (model_dtype != MI355GQ_BF16 || check_scheme(bits, group_size) != MI355GQ_OK || M < 2 || N < 0 || K < 0 ||
       M >= kMaxDim || N >= kMaxDim || K >= kMaxDim)
     return 0;
-  // bfloat16: every batch from two rows on may run the few-row GEMM (there are no bf16 skinny kernels)
-  return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+  // bfloat16: every batch from two rows on may run the few-row GEMM (there are no bf16 skinny kernels); 9..16 rows of a
+  // long K: the K slices of the kernel on unscaled weight operands
+  const int64_t mid = (bits == 4 && M > 8 && M <= 16) ? gq::midrow_workspace_bytes(M, N, K) : 0;
+  const int64_t gemm = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+  return gemm > mid ? gemm : mid;
 }
 
 int64_t mi355gq_linear_silu_mul_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
   if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
       N >= kMaxDim || K >= kMaxDim)
     return 0;
+  // q4 at 9..32 rows of a K beyond 4096: the K slices of the kernel on unscaled weight operands (as the plain linear)
+  const int64_t mid = (bits == 4 && M > 8 && M <= 32 && (N % 32) == 0) ? gq::midrow_workspace_bytes(M, N, K) : 0;
   // GEMV / few-row kernels, or a shape that never splits
-  if (M <= 8 || (N % 64) != 0) return 0;
-  if (M <= 16 && !(bits == 4 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return 0;
-  return gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+  if (M <= 8 || (N % 64) != 0) return M <= 8 ? 0 : mid;
+  if (M <= 16 && !(bits == 4 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return mid;
+  const int64_t gemm = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
+  return gemm > mid ? gemm : mid;
 }
 
 // paired: the fused gate/up form (y fp16 [M, N / 2]); a shape no fused kernel takes is an
@@ -408,10 +417,17 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   //  100-106 -> 74-78, 15360 x 5120 24.5 -> 21-22, 27648 x 5120 33.4-34.4 -> 32.4-33.8)
   // 17..32 rows (two batch tiles per pass, the offsets subtracted from the weight operand): one phase and 48 M weights or more
   // (14336 x 4096 at 17 / 24 / 32 rows 19.4 / 19.9 / 20.4 -> 16.9 / 17.9 / 19.0 us, 28672 x 4096 28.3 / 28.0 / 27.9 -> 26.0 / 26.1 / 27.5, 128256 x
-  //  4096 99-101 -> 84-87; 6144 x 4096 13.4-14.4 against 12.3-14.1 and 4096 x 4096 stay with the GEMM's tile, as does K = 8192 in
-  //  two phases: 57344 x 8192 92-97 against 112-126)
-  const bool mid_size = (M > 8 && M <= 16 && ((K <= 4096 && N * K >= (24ll << 20)) || (K <= 8192 && N * K >= (48ll << 20)))) ||
-                        (M > 16 && M <= 32 && K <= 4096 && N * K >= (48ll << 20));
+  //  4096 99-101 -> 84-87; 6144 x 4096 13.4-14.4 against 12.3-14.1 and 4096 x 4096 stay with the GEMM's tile).
+  // A longer K runs as K slices over workgroups where the caller brings the scratch for their partial sums
+  // (mi355gq_linear_workspace_bytes), ahead of the phases everywhere and of the GEMM's tiles at 9..16 rows from 24 M weights
+  // on (4096 x 14336 20.1 / 19.5 -> 16.5 / 17.2 us at 9 / 16 rows, 5120 x 13824 24.2 / 24.7 -> 18.7 / 19.4, 8192 x 28672 49.7 / 51.9 -> 38.7 / 39.8,
+  //  57344 x 8192 72.9 / 77.4 in phases -> 64.5 / 68.1) and at 17..32 rows from 256 M weights on (57344 x 8192 97 -> 85; 4096 x 14336
+  //  20.0 against 22.1 and 8192 x 28672 52 against 52 stay with the tiles).
+  const bool slices_ok = K > 4096 && workspace != nullptr && aligned16(workspace) &&
+                         workspace_bytes >= gq::midrow_workspace_bytes(M, N, K) && gq::options().gemv_ksplit != 0;
+  const bool mid_size =
+      (M > 8 && M <= 16 && N * K >= (24ll << 20) && (K <= 4096 || slices_ok || (K <= 8192 && N * K >= (48ll << 20)))) ||
+      (M > 16 && M <= 32 && ((K <= 4096 && N * K >= (48ll << 20)) || (slices_ok && N * K >= (256ll << 20))));
   const bool mid_rows = bits == 4 && mid_size && gq::options().gemm_variant < 0 &&
                         (gq::options().gemv_variant < 0 || gq::options().gemv_variant == 10) && (K & 255) == 0 &&
                         (N & 31) == 0;
@@ -801,8 +817,12 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
     // 128256 x 4096 105 -> 71, 4096 x 4096 12.2 -> 9.4, 2048 x 2048 9.4 -> 8.8)
     {
       const int gvm = gq::options().gemv_variant;
+      const bool slices_ok = K > 4096 && workspace != nullptr && aligned16(workspace) &&
+                             workspace_bytes >= gq::midrow_workspace_bytes(M, N, K) && gq::options().gemv_ksplit != 0;
       const bool mid_rows = bits == 4 && M > 8 && M <= 16 && gq::options().gemm_variant < 0 && gvm < 0 && (K & 255) == 0 &&
-                            (N & 31) == 0 && ((K <= 4096 && N * K >= (4ll << 20)) || (K <= 8192 && N * K >= (48ll << 20)));
+                            (N & 31) == 0 &&
+                            ((K <= 4096 && N * K >= (4ll << 20)) || (slices_ok && N * K >= (24ll << 20)) ||
+                             (K <= 8192 && N * K >= (48ll << 20)));
       if (mid_rows || gvm == 10) {
         const hipError_t e = gq::launch_midrow(g, static_cast<int>(M), as_stream(stream));
         if (e != hipErrorNotSupported) return hip_result(e, "linear_dt mid-row launch");
@@ -830,7 +850,13 @@ int mi355gq_linear_dt(const void* x, const void* q_weight, const void* q_scale, 
 int64_t mi355gq_linear_silu_mul_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size,
                                                    int model_dtype) {
   if (model_dtype == MI355GQ_F16) return mi355gq_linear_silu_mul_workspace_bytes(M, N, K, bits, group_size);
-  if ((N % 64) != 0) return 0;  // the partial sums of the fused form need whole 32 + 32 column blocks
+  // (the GEMM's partial sums of the fused form need whole 32 + 32 column blocks; the K slices of the kernel on unscaled
+  //  weight operands, 9..16 rows, do not)
+  if ((N % 64) != 0)
+    return (model_dtype == MI355GQ_BF16 && check_scheme(bits, group_size) == MI355GQ_OK && bits == 4 && M > 8 && M <= 16 &&
+            N > 0 && K > 0 && N < kMaxDim && K < kMaxDim && (N % 32) == 0)
+               ? gq::midrow_workspace_bytes(M, N, K)
+               : 0;
   return mi355gq_linear_dt_workspace_bytes(M, N, K, bits, group_size, model_dtype);
 }
 

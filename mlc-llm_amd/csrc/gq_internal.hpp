@@ -101,6 +101,7 @@ hipError_t launch_quadreg(const GemmArgs& a, int rows_max, hipStream_t s);
 // plain linears and expert segments); rows_max bounds the rows of any one segment; hipErrorNotSupported when the shape
 // does not fit.
 hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s);
+int64_t midrow_workspace_bytes(int64_t rows, int64_t N, int64_t K);
 
 // KN-layout tensors (q_weight [nw, N], q_scale [ng, N]): both tensors transposed in one call (src_rows_w / src_rows_s rows
 // of src_cols columns each), the dequantisation to [K, N], and the decode GEMV (M <= 8, N % 4 == 0) with its workspace

@@ -57,6 +57,8 @@ struct MidParams {
   int rounds;              // tiles a wave walks per chunk (a multiple of the tiles in flight; the fused form: even)
   int chunks;              // chunks of rounds (1 when K takes phases)
   int phases;              // passes over K (a workgroup covers KW * U groups per phase)
+  int slices;              // workgroups along K (plain linears with a workspace: grid z; each covers one phase's worth of
+                           // K and leaves fp32 partial sums [slice][rows][N] in y for the reduction kernel)
   int kw_log2;             // log2 of the waves that share a tile's K
   int out_f32, paired, indptr_i64, x_src_rows;
 };
@@ -153,7 +155,7 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
 
   for (int pass_lo = seg_lo; pass_lo < seg_hi; pass_lo += 16 * NBT) {
     for (int ph = 0; ph < (PHASED ? p.phases : 1); ++ph) {
-      const int ga_raw = (ph * kw + ks) * U;
+      const int ga_raw = ((static_cast<int>(blockIdx.z) + ph) * kw + ks) * U;  // (slices > 1: one phase each)
       const bool k_live = ga_raw < p.ng;  // (uniform; ng % U == 0: a share is whole or empty)
       const int ga = k_live ? ga_raw : p.ng - U;
       const int w_lane = (c * p.nw + 4 * (ga + j)) * 4, s_lane = (c * p.ng + ga) * 2;
@@ -297,6 +299,10 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
             if (t >= p.ntiles || col >= p.N || b >= seg_hi) continue;
             float v = share_sum(round, tl, bt);
             const int64_t oi = static_cast<int64_t>(b) * p.N + col;
+            if (p.slices > 1) {  // (bias, residual and the cast belong to the reduction)
+              static_cast<float*>(p.y)[static_cast<int64_t>(blockIdx.z) * p.rows * p.N + oi] = v;
+              continue;
+            }
             if (p.bias != nullptr) v += to_f32(p.bias[col]);
             if (p.residual != nullptr) v += to_f32(p.residual[oi]);
             if (p.out_f32) static_cast<float*>(p.y)[oi] = v;
@@ -340,6 +346,23 @@ __global__ __launch_bounds__(1024) void midrow_kernel(const MidParams p) {
   }
 }
 
+// y[b][j] = silu(sum over slices of part[s][b][j]) * (sum over slices of part[s][b][N / 2 + j]), in the model dtype
+__global__ __launch_bounds__(256) void mid_reduce_silu_kernel(const float* __restrict__ part, int slices, int64_t rows, int N,
+                                                              uint16_t* __restrict__ y, int bf16) {
+  const int half = N >> 1;
+  const int64_t count = rows * N, outs = rows * half;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < outs; i += static_cast<int64_t>(gridDim.x) * 256) {
+    const int64_t b = i / half;
+    const int64_t at = b * N + (i - b * half);
+    float g = 0.f, u = 0.f;
+    for (int sl = 0; sl < slices; ++sl) {
+      g += part[sl * count + at];
+      u += part[sl * count + at + half];
+    }
+    y[i] = bf16 ? silu_mul_bf(g, u) : silu_mul_h(g, u);
+  }
+}
+
 template <int NBT, int U, int RT, bool KEEP_C, bool PHASED, bool BF = false>
 hipError_t launch_mid(const MidParams& p, int wgx, int experts, hipStream_t s) {
   const size_t lds = static_cast<size_t>(p.rounds) * 16 * NBT * 1024;
@@ -353,9 +376,9 @@ hipError_t launch_mid(const MidParams& p, int wgx, int experts, hipStream_t s) {
       raised = true;
     }
   }
-  note_kernel("gq::midrow_kernel<%d,%d,%d,%d,%d%s> rounds=%d chunks=%d phases=%d kw=%d", NBT, U, RT, int(KEEP_C), int(PHASED),
-              BF ? ",true" : "", p.rounds, p.chunks, p.phases, 1 << p.kw_log2);
-  hipLaunchKernelGGL((midrow_kernel<NBT, U, RT, KEEP_C, PHASED, BF>), dim3(wgx, experts), dim3(1024), lds, s, p);
+  note_kernel("gq::midrow_kernel<%d,%d,%d,%d,%d%s> rounds=%d chunks=%d phases=%d slices=%d kw=%d", NBT, U, RT, int(KEEP_C),
+              int(PHASED), BF ? ",true" : "", p.rounds, p.chunks, p.phases, p.slices, 1 << p.kw_log2);
+  hipLaunchKernelGGL((midrow_kernel<NBT, U, RT, KEEP_C, PHASED, BF>), dim3(wgx, experts, p.slices), dim3(1024), lds, s, p);
   return hipGetLastError();
 }
 
@@ -399,17 +422,37 @@ hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   p.kw_log2 = kwl;
   const int phase_groups = (1 << kwl) * U;
   p.phases = (p.ng + phase_groups - 1) / phase_groups;
+  // A plain linear whose K takes several phases and whose caller brings the scratch: one workgroup row per phase's worth of
+  // K instead (x stays in registers for all of a workgroup's tiles, the walk comes in chunks), fp32 partial sums in the
+  // workspace and a second, small launch that adds them; the fused gate/up form then runs as a plain one and the reduction
+  // folds the activation in.  Tuning override: gemv_ksplit 0 keeps the phases.
+  p.slices = 1;
+  bool fold_silu = false;
+  if (p.phases > 1 && !grouped && p.phases <= 64 && options().gemv_ksplit != 0 && a.workspace != nullptr &&
+      a.workspace_bytes >= static_cast<int64_t>(p.phases) * p.rows * p.N * 4 &&
+      (reinterpret_cast<uintptr_t>(a.workspace) & 15) == 0) {
+    p.slices = p.phases;
+    p.phases = 1;
+    p.y = a.workspace;
+    p.bias = nullptr; p.residual = nullptr; p.out_f32 = 1;
+    if (p.paired) {
+      fold_silu = true;
+      p.paired = 0;
+      p.ntiles = (p.N + 15) / 16;
+    }
+  }
+  const bool paired_walk = p.paired != 0;
   const int tw = 16 >> kwl;
   const int form = options().gemv_rows_per_wave;  // (tuning override: which one-batch-tile instance)
   const int rt = form == 2 ? 4 : (form == 4 ? 3 : 2);
   // workgroups in all: one per CU (sixteen waves of up to 128 registers fill it), each with at most 128 KiB of sums in LDS
   const int want_wg = options().gemv_waves > 0 ? options().gemv_waves / 16 : 256;
-  int wgx = want_wg / experts;
+  int wgx = want_wg / (experts * p.slices);
   if (wgx < 1) wgx = 1;
-  const int per_round = a.paired ? 2 : 1;           // rounds per walked item
+  const int per_round = paired_walk ? 2 : 1;           // rounds per walked item
   const int sets = (p.ntiles + tw - 1) / tw;        // items per tile lane
   if (wgx > sets) wgx = sets;
-  const int unit = a.paired ? (rt % 2 == 0 ? rt : 2 * rt) : rt;  // rounds come in whole rings (and whole pairs)
+  const int unit = paired_walk ? (rt % 2 == 0 ? rt : 2 * rt) : rt;  // rounds come in whole rings (and whole pairs)
   const int max_rounds = (128 / (16 * nbt)) / unit * unit;
   if (max_rounds < unit) return hipErrorNotSupported;
   int items = (sets + wgx - 1) / wgx;               // items per wave
@@ -421,22 +464,45 @@ hipError_t launch_midrow(const GemmArgs& a, int rows_max, hipStream_t s) {
   int rounds = (items * per_round + unit - 1) / unit * unit;
   p.chunks = (rounds + max_rounds - 1) / max_rounds;
   p.rounds = ((rounds + p.chunks - 1) / p.chunks + unit - 1) / unit * unit;
-  if (a.bf16) {  // (the bfloat16 instances: q4bf16_*)
-    if (p.phases > 1)
-      return nbt == 2 ? launch_mid<2, 8, 2, false, true, true>(p, wgx, experts, s)
-                      : launch_mid<1, 8, 2, true, true, true>(p, wgx, experts, s);
-    return nbt == 2 ? launch_mid<2, 8, 2, false, false, true>(p, wgx, experts, s)
-                    : launch_mid<1, 8, 2, true, false, true>(p, wgx, experts, s);
+  auto run = [&]() -> hipError_t {
+    if (a.bf16) {  // (the bfloat16 instances: q4bf16_*)
+      if (p.phases > 1)
+        return nbt == 2 ? launch_mid<2, 8, 2, false, true, true>(p, wgx, experts, s)
+                        : launch_mid<1, 8, 2, true, true, true>(p, wgx, experts, s);
+      return nbt == 2 ? launch_mid<2, 8, 2, false, false, true>(p, wgx, experts, s)
+                      : launch_mid<1, 8, 2, true, false, true>(p, wgx, experts, s);
+    }
+    if (p.phases > 1) {
+      if (form == 2) return hipErrorNotSupported;
+      if (nbt == 2) return launch_mid<2, 8, 2, false, true>(p, wgx, experts, s);
+      return launch_mid<1, 8, 2, true, true>(p, wgx, experts, s);
+    }
+    if (nbt == 2) return launch_mid<2, 8, 2, false, false>(p, wgx, experts, s);
+    if (form == 2) return launch_mid<1, 8, 4, false, false>(p, wgx, experts, s);
+    if (form == 4) return launch_mid<1, 8, 3, true, false>(p, wgx, experts, s);
+    return launch_mid<1, 8, 2, true, false>(p, wgx, experts, s);
+  };
+  const hipError_t e = run();
+  if (e != hipSuccess || p.slices == 1) return e;
+  const int64_t count = static_cast<int64_t>(p.rows) * p.N;
+  if (fold_silu) {
+    const int64_t outs = count / 2;
+    hipLaunchKernelGGL(mid_reduce_silu_kernel, dim3(static_cast<unsigned>((outs + 255) / 256 > 4096 ? 4096 : (outs + 255) / 256)),
+                       dim3(256), 0, s, static_cast<const float*>(a.workspace), p.slices, static_cast<int64_t>(p.rows), p.N,
+                       static_cast<uint16_t*>(a.y), a.bf16);
+  } else {
+    const int64_t blocks = ((p.N & 3) == 0 ? (count / 4 + 255) / 256 : (count + 255) / 256);
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s,
+                       static_cast<const float*>(a.workspace), p.slices, count, p.N, a.bias, a.residual, a.y, a.out_f32, a.bf16);
   }
-  if (p.phases > 1) {
-    if (form == 2) return hipErrorNotSupported;
-    if (nbt == 2) return launch_mid<2, 8, 2, false, true>(p, wgx, experts, s);
-    return launch_mid<1, 8, 2, true, true>(p, wgx, experts, s);
-  }
-  if (nbt == 2) return launch_mid<2, 8, 2, false, false>(p, wgx, experts, s);
-  if (form == 2) return launch_mid<1, 8, 4, false, false>(p, wgx, experts, s);
-  if (form == 4) return launch_mid<1, 8, 3, true, false>(p, wgx, experts, s);
-  return launch_mid<1, 8, 2, true, false>(p, wgx, experts, s);
+  return hipGetLastError();
+}
+
+// scratch for the K slices of a plain linear (0: K is one phase)
+int64_t midrow_workspace_bytes(int64_t rows, int64_t N, int64_t K) {
+  if (rows < 1 || N < 16 || K <= 0 || (K & 255) != 0) return 0;
+  const int64_t phases = (K / 32 + 127) / 128;
+  return phases > 1 ? phases * rows * N * 4 : 0;
 }
 
 }  // namespace gq

@@ -378,8 +378,9 @@ def test_midrow_kernel(form, m, n, k):
     finally:
         gq._lib.set_option("gemv_variant", -1)
         gq._lib.set_option("gemv_rows_per_wave", -1)
-    if k > 4096 and form == 2:  # (several phases exist for the default instance only: the shape falls through)
-        assert not kern.startswith("gq::midrow_kernel"), kern
+    if k > 4096 and form == 2:  # (several phases exist for the default instance only: K slices where the call's scratch
+        #                          holds their partial sums, else the shape falls through)
+        assert not kern.startswith("gq::midrow_kernel") or " phases=1 " in kern, kern
     else:
         assert kern.startswith("gq::midrow_kernel<"), kern
     ref = o.linear_fp32(x, qw, qs, s, b)
@@ -429,6 +430,52 @@ def test_midrow_kernel_is_the_default_on_large_matrices(m, n, k):
     fused = ops.linear_silu_mul(dev(x), dev(qw), dev(qs), 4, 32)
     assert gq._lib.last_kernel().startswith("gq::midrow_kernel<") == want, gq._lib.last_kernel()
     assert torch.equal(fused, ops.silu_mul(y))
+
+
+@pytest.mark.parametrize("m,n,k", [(9, 4096, 14336), (16, 4096, 14336), (32, 4096, 14336), (12, 5120, 13824), (16, 8192, 28672),
+                                   (9, 10240, 8192), (24, 32768, 8192), (32, 2048, 8192)])
+def test_midrow_kernel_k_slices(m, n, k):
+    """A K of several phases on a plain linear whose caller brings the scratch: one workgroup row per phase's worth of K,
+    fp32 partial sums, a reduction that adds bias and residual and casts.  The default at 9..16 rows from 24 M weights on and
+    at 17..32 rows from 256 M; forced elsewhere.  Against the oracle on a sample of the columns, with bias, residual and
+    float32 output; the fused gate/up form equals linear + silu_mul bit for bit; without the scratch the call still answers
+    (phases inside the workgroup, or the GEMM's tiles)."""
+    s = SCHEMES["q4f16_1"]
+    rng = np.random.default_rng(seed_of("midrow-slices", m, n, k))
+    qw = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    qs = (rng.random((n, k // 32)) * 0.02 + 0.001).astype(np.float16)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    bias = rng.standard_normal(n).astype(np.float16)
+    res = rng.standard_normal((m, n)).astype(np.float16)
+    cols = np.unique(np.concatenate([[0, 1, n // 2, n - 1], rng.integers(0, n, 200)]))
+    pick = torch.from_numpy(cols).to(DEV)
+    default = (m <= 16 and n * k >= 24 << 20) or n * k >= 256 << 20
+    phases = -(-(k // 32) // 128)
+    if not default:
+        gq._lib.set_option("gemv_variant", 10)
+    try:
+        y = ops.linear(dev(x), dev(qw), dev(qs), 4, 32)
+        kern = gq._lib.last_kernel()
+        yb = ops.linear(dev(x), dev(qw), dev(qs), 4, 32, bias=dev(bias), residual=dev(res), out_dtype=torch.float32)
+        fused = ops.linear_silu_mul(dev(x), dev(qw), dev(qs), 4, 32)
+        kern_fused = gq._lib.last_kernel()
+    finally:
+        gq._lib.set_option("gemv_variant", -1)
+    assert kern.startswith(f"gq::midrow_kernel<{1 if m <= 16 else 2},") and f"slices={phases} " in kern, kern
+    assert kern_fused.startswith("gq::midrow_kernel<") and f"slices={phases} " in kern_fused, kern_fused
+    ref = o.linear_fp32(x, qw[cols], qs[cols], s)
+    assert_linear_ok(y[:, pick], ref, x, k, f"mid-row slices {m}x{n}x{k}")
+    assert_linear_ok(yb[:, pick], ref + bias[cols].astype(np.float32) + res[:, cols].astype(np.float32), x, k,
+                     f"mid-row slices, bias + residual, f32 {m}x{n}x{k}")
+    assert torch.equal(fused, ops.silu_mul(y))
+    # no scratch: the same call answers without the slices
+    out = torch.empty((m, n), dtype=torch.float16, device=DEV)
+    dx, dqw, dqs = dev(x), dev(qw), dev(qs)
+    gq._lib.call("mi355gq_linear", dx.data_ptr(), dqw.data_ptr(), dqs.data_ptr(), None, m, n, k, 4, 32, gq._lib.F16,
+                 out.data_ptr(), None, 0, ops._stream())
+    torch.cuda.synchronize()
+    assert "slices=" not in gq._lib.last_kernel() or "slices=1 " in gq._lib.last_kernel(), gq._lib.last_kernel()
+    assert_linear_ok(out[:, pick], ref, x, k, f"no scratch {m}x{n}x{k}")
 
 
 @pytest.mark.parametrize("k", [1024, 4096, 14336])
@@ -1843,7 +1890,7 @@ def test_bfloat16_few_rows_take_the_register_fewrow_kernel(m, n, k):
 
 
 @pytest.mark.parametrize("m", [9, 16, 23])  # one batch tile, a full one, two (forced)
-@pytest.mark.parametrize("n,k", [(512, 4096), (96, 1024), (160, 8192)])
+@pytest.mark.parametrize("n,k", [(512, 4096), (96, 1024), (160, 8192), (224, 14336)])  # (the last two: K slices at 9 and 16 rows)
 def test_bfloat16_midrow_kernel(m, n, k):
     """q4bf16_1 on the kernel that scales the matrix instruction's result (its bfloat16 instance: every field shifted to
     the low bits, offset 128 + 7, x as it is), forced on small shapes: float32 output exact against the unrounded-weight
