@@ -109,8 +109,9 @@ MI355GQ_API int mi355gq_embedding_take_dt(const void* ids, int64_t T, const void
  * M <= 8 runs the decode GEMV / few-row kernels, larger M the MFMA GEMM (the regime split of
  * compiler_pass/low_batch_specialization.py:22-57).
  * workspace: device scratch, 16-byte aligned, of at least mi355gq_linear_workspace_bytes()
- * bytes for the shape; only the GEMM with 17..256 rows asks for any (fp32 partial sums of its
- * split along K).  NULL or too small is not an error: the same tiles run unsplit, slower.
+ * bytes for the shape; the GEMM with 17..256 rows asks for some (fp32 partial sums of its
+ * split along K), and so does q4 at 9..32 rows with K beyond 4096 (partial sums of K slices that
+ * run on separate workgroups).  NULL or too small is not an error: the shape runs unsplit, slower.
  * Its contents are undefined afterwards; calls that share a workspace must be stream-ordered.
  */
 MI355GQ_API int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size);
@@ -121,8 +122,8 @@ MI355GQ_API int mi355gq_linear(const void* x, const void* q_weight, const void* 
 /*
  * mi355gq_linear for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose VM allocates workspaces
- * itself.  Same arguments and results as mi355gq_linear without the workspace: the split-K partial sums of the
- * few-row GEMM go to a device array inside the library (mi355gq_linear_static_scratch_max_bytes() = 32 MiB, held
+ * itself.  Same arguments and results as mi355gq_linear without the workspace: the partial sums of a split
+ * along K go to a device array inside the library (mi355gq_linear_static_scratch_max_bytes() = 32 MiB, held
  * by every GPU the library runs on until the process ends), so the call allocates nothing.  Shapes whose split
  * would want more return MI355GQ_ERR_WORKSPACE (nothing is launched).  All calls on one GPU share the array:
  * calls that overlap on one GPU (different streams, different threads) race on it; stream-ordered calls do not.
