@@ -110,8 +110,8 @@ MI355GQ_API int mi355gq_embedding_take_dt(const void* ids, int64_t T, const void
  * compiler_pass/low_batch_specialization.py:22-57).
  * workspace: device scratch, 16-byte aligned, of at least mi355gq_linear_workspace_bytes()
  * bytes for the shape; the GEMM with 17..256 rows asks for some (fp32 partial sums of its
- * split along K), and so does q4 at 9..32 rows with K beyond 4096 (partial sums of K slices that
- * run on separate workgroups).  NULL or too small is not an error: the shape runs unsplit, slower.
+ * split along K), and so does q4 at 9..32 rows with K beyond 4096 and at 5..8 rows with K beyond
+ * 8192 (partial sums of K slices that run on separate workgroups).  NULL or too small is not an error: the shape runs unsplit, slower.
  * Its contents are undefined afterwards; calls that share a workspace must be stream-ordered.
  */
 MI355GQ_API int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size);

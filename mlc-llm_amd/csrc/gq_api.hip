@@ -320,12 +320,13 @@ int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits
   if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
       N >= kMaxDim || K >= kMaxDim)
     return 0;
-  // q4 at 9..32 rows of a K beyond 4096: the K slices of the kernel on unscaled weight operands (see linear_impl)
-  const int64_t mid = (bits == 4 && M > 8 && M <= 32) ? gq::midrow_workspace_bytes(M, N, K) : 0;
+  // q4 at 9..32 rows of a K beyond 4096, at 5..8 rows of a K beyond 8192: the K slices of the kernel on unscaled weight
+  // operands (see linear_impl)
+  const int64_t mid = (bits == 4 && M <= 32 && (M > 8 || (M > 4 && K > 8192))) ? gq::midrow_workspace_bytes(M, N, K) : 0;
   // only the few-row GEMM (more rows than the GEMV / skinny kernels take, at most 256) splits K
   // (q4 at 9..16 rows: the skinny kernel, except on matrices of 40 M to 256 M weights, see linear_impl)
   if (M <= 16 && bits == 4 && !(M > 8 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return mid;
-  if (M <= 8) return 0;
+  if (M <= 8) return mid;
   const int64_t gemm = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
   return gemm > mid ? gemm : mid;
 }
@@ -347,10 +348,13 @@ int64_t mi355gq_linear_silu_mul_workspace_bytes(int64_t M, int64_t N, int64_t K,
   if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
       N >= kMaxDim || K >= kMaxDim)
     return 0;
-  // q4 at 9..32 rows of a K beyond 4096: the K slices of the kernel on unscaled weight operands (as the plain linear)
-  const int64_t mid = (bits == 4 && M > 8 && M <= 32 && (N % 32) == 0) ? gq::midrow_workspace_bytes(M, N, K) : 0;
+  // q4 at 9..32 rows of a K beyond 4096, at 5..8 rows of a K beyond 8192: the K slices of the kernel on unscaled weight
+  // operands (as the plain linear)
+  const int64_t mid = (bits == 4 && M <= 32 && (M > 8 || (M > 4 && K > 8192)) && (N % 32) == 0)
+                          ? gq::midrow_workspace_bytes(M, N, K)
+                          : 0;
   // GEMV / few-row kernels, or a shape that never splits
-  if (M <= 8 || (N % 64) != 0) return M <= 8 ? 0 : mid;
+  if (M <= 8 || (N % 64) != 0) return mid;
   if (M <= 16 && !(bits == 4 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return mid;
   const int64_t gemm = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
   return gemm > mid ? gemm : mid;
@@ -425,7 +429,11 @@ static int linear_impl(const void* x, const void* q_weight, const void* q_scale,
   //  20.0 against 22.1 and 8192 x 28672 52 against 52 stay with the tiles).
   const bool slices_ok = K > 4096 && workspace != nullptr && aligned16(workspace) &&
                          workspace_bytes >= gq::midrow_workspace_bytes(M, N, K) && gq::options().gemv_ksplit != 0;
+  // 5..8 rows of a K beyond 8192 from 64 M weights on, as K slices: the quad-row kernels read x once per four rows and K
+  // share there (8192 x 28672 at 5 / 8 rows 46.1 / 47.3 -> 37.0 us, 5120 x 13824 22.3 / 23.2 -> 18.2 / 18.6; 4096 x 14336 15.3-16.1 against
+  // 15.9-16.2 and up to four rows, 36.6 against 36.5 and 17.2 against 18.4, stay with them)
   const bool mid_size =
+      (M > 4 && M <= 8 && slices_ok && K > 8192 && N * K >= (64ll << 20)) ||
       (M > 8 && M <= 16 && N * K >= (24ll << 20) && (K <= 4096 || slices_ok || (K <= 8192 && N * K >= (48ll << 20)))) ||
       (M > 16 && M <= 32 && ((K <= 4096 && N * K >= (48ll << 20)) || (slices_ok && N * K >= (256ll << 20))));
   const bool mid_rows = bits == 4 && mid_size && gq::options().gemm_variant < 0 &&

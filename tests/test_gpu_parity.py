@@ -433,11 +433,12 @@ def test_midrow_kernel_is_the_default_on_large_matrices(m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(9, 4096, 14336), (16, 4096, 14336), (32, 4096, 14336), (12, 5120, 13824), (16, 8192, 28672),
-                                   (9, 10240, 8192), (24, 32768, 8192), (32, 2048, 8192)])
+                                   (9, 10240, 8192), (24, 32768, 8192), (32, 2048, 8192), (5, 5120, 13824), (8, 8192, 28672),
+                                   (7, 4096, 14336)])
 def test_midrow_kernel_k_slices(m, n, k):
     """A K of several phases on a plain linear whose caller brings the scratch: one workgroup row per phase's worth of K,
-    fp32 partial sums, a reduction that adds bias and residual and casts.  The default at 9..16 rows from 24 M weights on and
-    at 17..32 rows from 256 M; forced elsewhere.  Against the oracle on a sample of the columns, with bias, residual and
+    fp32 partial sums, a reduction that adds bias and residual and casts.  The default at 9..16 rows from 24 M weights on, at
+    17..32 rows from 256 M and at 5..8 rows of a K beyond 8192 from 64 M; forced elsewhere.  Against the oracle on a sample of the columns, with bias, residual and
     float32 output; the fused gate/up form equals linear + silu_mul bit for bit; without the scratch the call still answers
     (phases inside the workgroup, or the GEMM's tiles)."""
     s = SCHEMES["q4f16_1"]
@@ -449,7 +450,7 @@ def test_midrow_kernel_k_slices(m, n, k):
     res = rng.standard_normal((m, n)).astype(np.float16)
     cols = np.unique(np.concatenate([[0, 1, n // 2, n - 1], rng.integers(0, n, 200)]))
     pick = torch.from_numpy(cols).to(DEV)
-    default = (m <= 16 and n * k >= 24 << 20) or n * k >= 256 << 20
+    default = (8 < m <= 16 and n * k >= 24 << 20) or (m > 16 and n * k >= 256 << 20) or (m <= 8 and k > 8192 and n * k >= 64 << 20)
     phases = -(-(k // 32) // 128)
     if not default:
         gq._lib.set_option("gemv_variant", 10)
