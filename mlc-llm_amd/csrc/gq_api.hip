@@ -339,7 +339,7 @@ int64_t mi355gq_linear_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int b
     return 0;
   // bfloat16: every batch from two rows on may run the few-row GEMM (there are no bf16 skinny kernels); 9..16 rows of a
   // long K: the K slices of the kernel on unscaled weight operands
-  const int64_t mid = (bits == 4 && M > 8 && M <= 16) ? gq::midrow_workspace_bytes(M, N, K) : 0;
+  const int64_t mid = (bits == 4 && M <= 16 && (M > 8 || (M > 4 && K > 8192))) ? gq::midrow_workspace_bytes(M, N, K) : 0;
   const int64_t gemm = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
   return gemm > mid ? gemm : mid;
 }
@@ -809,6 +809,26 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
     g.workspace = workspace; g.workspace_bytes = workspace ? workspace_bytes : 0;
     g.bf16 = 1;
     g.paired = paired;
+    // 9..16 rows of q4: the bfloat16 instance of the float16 linear's kernel for this range (ahead of the few-row kernels
+    // below because a long K takes it from five rows on); K of one phase from 4 M
+    // weights on (there is no bfloat16 skinny kernel: 6144 x 4096 at 16 rows 30.4 -> 10.8 us, 28672 x 4096 31.5 -> 20.3,
+    // 128256 x 4096 105 -> 71, 4096 x 4096 12.2 -> 9.4, 2048 x 2048 9.4 -> 8.8)
+    {
+      const int gvm = gq::options().gemv_variant;
+      const bool slices_ok = K > 4096 && workspace != nullptr && aligned16(workspace) &&
+                             workspace_bytes >= gq::midrow_workspace_bytes(M, N, K) && gq::options().gemv_ksplit != 0;
+      // (5..8 rows of a K beyond 8192 from 64 M weights on, as K slices, like the float16 linear: 8192 x 28672 at 5 / 8 rows
+      //  49.1 / 50.6 -> 38.0 / 37.5 us, 5120 x 13824 23.1 / 23.7 -> 18.6 / 18.2; 4096 x 14336 15.5-16.3 against 15.7-16.1 stays)
+      const bool mid_size =
+          (M > 4 && M <= 8 && slices_ok && K > 8192 && N * K >= (64ll << 20)) ||
+          (M > 8 && M <= 16 &&
+           ((K <= 4096 && N * K >= (4ll << 20)) || (slices_ok && N * K >= (24ll << 20)) || (K <= 8192 && N * K >= (48ll << 20))));
+      const bool mid_rows = bits == 4 && mid_size && gq::options().gemm_variant < 0 && gvm < 0 && (K & 255) == 0 && (N & 31) == 0;
+      if (mid_rows || gvm == 10) {
+        const hipError_t e = gq::launch_midrow(g, static_cast<int>(M), as_stream(stream));
+        if (e != hipErrorNotSupported) return hip_result(e, "linear_dt mid-row launch");
+      }
+    }
     // up to 8 rows: the float16 path's quad-row kernels on the bf16 4x4x4 matrix instruction (x in registers where that
     // form applies, as in the float16 linear)
     if (M <= 8) {
@@ -819,22 +839,6 @@ static int linear_dt_impl(const void* x, const void* q_weight, const void* q_sca
       }
       const hipError_t q = gq::launch_quadrow(g, static_cast<int>(M), as_stream(stream));
       if (q != hipErrorNotSupported) return hip_result(q, "linear_dt quad-row launch");
-    }
-    // 9..16 rows of q4 with K of one phase: the bfloat16 instance of the float16 linear's kernel for this range, from 4 M
-    // weights on (there is no bfloat16 skinny kernel: 6144 x 4096 at 16 rows 30.4 -> 10.8 us, 28672 x 4096 31.5 -> 20.3,
-    // 128256 x 4096 105 -> 71, 4096 x 4096 12.2 -> 9.4, 2048 x 2048 9.4 -> 8.8)
-    {
-      const int gvm = gq::options().gemv_variant;
-      const bool slices_ok = K > 4096 && workspace != nullptr && aligned16(workspace) &&
-                             workspace_bytes >= gq::midrow_workspace_bytes(M, N, K) && gq::options().gemv_ksplit != 0;
-      const bool mid_rows = bits == 4 && M > 8 && M <= 16 && gq::options().gemm_variant < 0 && gvm < 0 && (K & 255) == 0 &&
-                            (N & 31) == 0 &&
-                            ((K <= 4096 && N * K >= (4ll << 20)) || (slices_ok && N * K >= (24ll << 20)) ||
-                             (K <= 8192 && N * K >= (48ll << 20)));
-      if (mid_rows || gvm == 10) {
-        const hipError_t e = gq::launch_midrow(g, static_cast<int>(M), as_stream(stream));
-        if (e != hipErrorNotSupported) return hip_result(e, "linear_dt mid-row launch");
-      }
     }
     // the float16 GEMM's tiles on the bf16 matrix instruction
     const hipError_t e = gq::launch_gemm(g, as_stream(stream));
@@ -861,7 +865,8 @@ int64_t mi355gq_linear_silu_mul_dt_workspace_bytes(int64_t M, int64_t N, int64_t
   // (the GEMM's partial sums of the fused form need whole 32 + 32 column blocks; the K slices of the kernel on unscaled
   //  weight operands, 9..16 rows, do not)
   if ((N % 64) != 0)
-    return (model_dtype == MI355GQ_BF16 && check_scheme(bits, group_size) == MI355GQ_OK && bits == 4 && M > 8 && M <= 16 &&
+    return (model_dtype == MI355GQ_BF16 && check_scheme(bits, group_size) == MI355GQ_OK && bits == 4 && M <= 16 &&
+            (M > 8 || (M > 4 && K > 8192)) &&
             N > 0 && K > 0 && N < kMaxDim && K < kMaxDim && (N % 32) == 0)
                ? gq::midrow_workspace_bytes(M, N, K)
                : 0;

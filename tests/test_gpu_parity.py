@@ -1925,6 +1925,32 @@ def test_bfloat16_midrow_kernel(m, n, k):
     assert torch.equal(fused, ops.silu_mul(y))
 
 
+@pytest.mark.parametrize("m", [6, 12])
+def test_bfloat16_midrow_kernel_k_slices_default(m):
+    """q4bf16_1, 5120 x 13824 (a K of four phases, 68 M weights): five rows and more take the K slices of the kernel on unscaled
+    weight operands by default; a sample of the columns against the exact product, the fused gate/up form against the two steps."""
+    s = SCHEMES["q4f16_1"]
+    n, k = 5120, 13824
+    rng = np.random.default_rng(90 + m)
+    qw_ref = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    qs_ref = o.round_to((rng.random((n, k // 32)) * 0.02 + 0.001).astype(np.float32), "bfloat16")
+    x32 = o.round_to(rng.standard_normal((m, k)).astype(np.float32), "bfloat16")
+    qw, qs = dev(qw_ref), torch.from_numpy(qs_ref).to(torch.bfloat16).to(DEV)
+    x = torch.from_numpy(x32).to(torch.bfloat16).to(DEV)
+    cols = np.unique(np.concatenate([[0, 1, n // 2, n - 1], rng.integers(0, n, 200)]))
+    y32 = ops.linear(x, qw, qs, 4, 32, None, out_dtype=torch.float32)
+    kern = gq._lib.last_kernel()
+    assert kern.startswith("gq::midrow_kernel<1,") and ",true>" in kern and "slices=4 " in kern, kern
+    y = ops.linear(x, qw, qs, 4, 32)
+    fused = ops.linear_silu_mul(x, qw, qs, 4, 32)
+    assert gq._lib.last_kernel().startswith("gq::midrow_kernel<1,"), gq._lib.last_kernel()
+    exact = o.linear_dt_fp64(x32, qw_ref[cols], qs_ref[cols], s, "bfloat16", None, unrounded_weights=True)
+    got = y32[:, torch.from_numpy(cols).to(DEV)].double().cpu().numpy()
+    assert np.linalg.norm(got - exact) / np.linalg.norm(exact) <= 5e-6 + 1e-7 * np.sqrt(k)
+    assert np.array_equal(_carrier(y), o.round_to(y32.cpu().numpy(), "bfloat16"))
+    assert torch.equal(fused, ops.silu_mul(y))
+
+
 def test_bfloat16_midrow_kernel_grouped_default():
     """q4bf16_1 expert segments at six and at sixteen rows per expert on average: the default dispatch takes the bfloat16
     instance (one and two batch tiles per pass); against the exact product, and the fused gate/up form bit for bit."""
