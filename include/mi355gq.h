@@ -125,7 +125,8 @@ MI355GQ_API int mi355gq_linear(const void* x, const void* q_weight, const void* 
  * itself.  Same arguments and results as mi355gq_linear without the workspace: the partial sums of a split
  * along K go to a device array inside the library (mi355gq_linear_static_scratch_max_bytes() = 32 MiB, held
  * by every GPU the library runs on until the process ends), so the call allocates nothing.  Shapes whose split
- * would want more return MI355GQ_ERR_WORKSPACE (nothing is launched).  All calls on one GPU share the array:
+ * would want more return MI355GQ_ERR_WORKSPACE (nothing is launched); the K slices of 5..32 rows are dropped first
+ * where only their sums do not fit (the shape then runs as it does without a workspace for them).  All calls on one GPU share the array:
  * calls that overlap on one GPU (different streams, different threads) race on it; stream-ordered calls do not.
  * The first use on a device looks the array's address up (and may load it with the code object): call
  * mi355gq_linear_static_scratch_init() once per device, with that device current, before a region that must not

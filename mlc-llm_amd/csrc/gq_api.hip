@@ -316,19 +316,26 @@ int mi355gq_embedding_take_dt(const void* ids, int64_t T, const void* q_weight, 
                     "embedding_take_dt launch");
 }
 
-int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
+// with_slices false: what the shape needs when the K slices of the kernel on unscaled weight operands go without
+static int64_t linear_workspace_need(int64_t M, int64_t N, int64_t K, int bits, int group_size, bool with_slices) {
   if (check_scheme(bits, group_size) != MI355GQ_OK || M < 0 || N < 0 || K < 0 || M >= kMaxDim ||
       N >= kMaxDim || K >= kMaxDim)
     return 0;
   // q4 at 9..32 rows of a K beyond 4096, at 5..8 rows of a K beyond 8192: the K slices of the kernel on unscaled weight
   // operands (see linear_impl)
-  const int64_t mid = (bits == 4 && M <= 32 && (M > 8 || (M > 4 && K > 8192))) ? gq::midrow_workspace_bytes(M, N, K) : 0;
+  const int64_t mid = (with_slices && bits == 4 && M <= 32 && (M > 8 || (M > 4 && K > 8192)))
+                          ? gq::midrow_workspace_bytes(M, N, K)
+                          : 0;
   // only the few-row GEMM (more rows than the GEMV / skinny kernels take, at most 256) splits K
   // (q4 at 9..16 rows: the skinny kernel, except on matrices of 40 M to 256 M weights, see linear_impl)
   if (M <= 16 && bits == 4 && !(M > 8 && N * K >= (40ll << 20) && N * K < (256ll << 20))) return mid;
   if (M <= 8) return mid;
   const int64_t gemm = gq::gemm_workspace_bytes(M, N, K, bits, group_size);
   return gemm > mid ? gemm : mid;
+}
+
+int64_t mi355gq_linear_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size) {
+  return linear_workspace_need(M, N, K, bits, group_size, true);
 }
 
 int64_t mi355gq_linear_dt_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits, int group_size,
@@ -571,7 +578,9 @@ int mi355gq_linear_static_scratch_init(void) {
 int mi355gq_linear_static_scratch(const void* x, const void* q_weight, const void* q_scale, const void* bias,
                                   int64_t M, int64_t N, int64_t K, int bits, int group_size, int out_dtype,
                                   void* y, mi355gq_stream_t stream) {
-  const int64_t need = mi355gq_linear_workspace_bytes(M, N, K, bits, group_size);
+  // (the K slices of 5..32 rows are an option of the dispatch: where their sums do not fit, the shape runs without them)
+  int64_t need = linear_workspace_need(M, N, K, bits, group_size, true);
+  if (need > kStaticScratchBytes) need = linear_workspace_need(M, N, K, bits, group_size, false);
   if (need > kStaticScratchBytes)
     return fail(MI355GQ_ERR_WORKSPACE,
                 "linear_static_scratch: M=%lld N=%lld K=%lld wants %lld bytes of split-K partial sums, the library's "

@@ -55,7 +55,7 @@ def test_static_scratch_linear_two_calls_in_a_row():
     # matmul that splits into fewer, smaller partial tiles and finds the first call's sums still in the array;
     # then one-row and large-M calls that need no scratch at all
     cases = [(64, 1024, 8192, lib.F16), (24, 520, 4096, lib.F16), (40, 260, 8192, lib.F32), (1, 384, 1024, lib.F16),
-             (300, 256, 512, lib.F16)]
+             (300, 256, 512, lib.F16), (12, 2048, 14336, lib.F16)]  # (the last: K slices of the 9..16-row kernel)
     needs = []
     lib.call("mi355gq_linear_static_scratch_init")  # the per-device set-up (address look-up), outside any call that must not allocate
     for i, (m, n, k, od) in enumerate(cases):
@@ -65,7 +65,7 @@ def test_static_scratch_linear_two_calls_in_a_row():
         assert torch.equal(got, want), (m, n, k)
         err, bound, rel = o.check_linear(got.float().cpu().numpy(), o.linear_fp32(x, qw, qs, s, b), x, k)
         assert err <= bound and rel <= 2e-3, (m, n, k, err, bound, rel)
-    assert needs[0] > needs[1] > 0 and needs[3] == 0  # the cases do what the comments say
+    assert needs[0] > needs[1] > 0 and needs[3] == 0 and needs[5] == 4 * 12 * 2048 * 4  # the cases do what the comments say
 
 
 def test_static_scratch_linear_rejects_what_does_not_fit():
@@ -86,3 +86,29 @@ def test_static_scratch_linear_rejects_what_does_not_fit():
     finally:
         lib.set_option("gemm_split_k", -1)
     assert ei.value.code == lib.ERR_WORKSPACE and "partial sums" in str(ei.value)
+
+
+def test_static_scratch_linear_runs_without_the_k_slices_where_they_do_not_fit():
+    """32 rows of 16416 x 65536: the K slices of the 17..32-row kernel would keep 16 x 32 x 16416 floats, just over the array;
+    they are an option of the dispatch, so the call answers on the GEMM's tiles (whose own split fits) instead of
+    rejecting the shape.  A sample of the columns against the oracle."""
+    lib = gq._lib
+    s = o.SCHEMES["q4f16_1"]
+    m, n, k = 32, 16416, 65536
+    cap = lib.lib().mi355gq_linear_static_scratch_max_bytes()
+    assert lib.lib().mi355gq_linear_workspace_bytes(m, n, k, 4, 32) > cap
+    rng = np.random.default_rng(7)
+    qw = rng.integers(0, 2**32, (n, k // 8), dtype=np.uint32)
+    qs = (rng.random((n, k // 32)) * 0.02 + 0.001).astype(np.float16)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    xd = torch.from_numpy(x).to(DEV)
+    qwd, qsd = torch.from_numpy(qw.view(np.int32)).to(DEV), torch.from_numpy(qs).to(DEV)
+    got = torch.full((m, n), 3.0, dtype=torch.float16, device=DEV)
+    lib.call("mi355gq_linear_static_scratch", xd.data_ptr(), qwd.data_ptr(), qsd.data_ptr(), None, m, n, k, 4, 32, lib.F16,
+             got.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert not lib.last_kernel().startswith("gq::midrow_kernel"), lib.last_kernel()
+    cols = np.unique(np.concatenate([[0, 1, n - 1], rng.integers(0, n, 60)]))
+    ref = o.linear_fp32(x, qw[cols], qs[cols], s)
+    err, bound, rel = o.check_linear(got[:, torch.from_numpy(cols).to(DEV)].float().cpu().numpy(), ref, x, k)
+    assert err <= bound and rel <= 2e-3, (err, bound, rel)
